@@ -1,0 +1,321 @@
+/*
+ * hipq.h -- C ABI of libhipq.so: the int8 quantized-inference kernels for AMD gfx950 (MI355X).
+ *
+ * This is the seam between the C++ host side (the nGraph "HIP" backend plugin, which never includes
+ * a HIP header) and the hand-written HIP kernels.  Every entry point takes plain pointers and
+ * sizes; pointers named data/filter/out/scale/... are DEVICE pointers unless a comment says host.
+ * All functions return HIPQ_OK (0) or an error code; hipq_last_error() gives the message of the
+ * last failure on the calling thread.  A launch is asynchronous on `stream` (a hipStream_t passed
+ * as void*, NULL = the default stream of the current device).
+ *
+ * Each compute entry point replaces one kernel of the nGraph reference and keeps its arithmetic.
+ * Paths cited below are relative to the nGraph source tree.
+ */
+#ifndef HIPQ_H
+#define HIPQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(_WIN32)
+#define HIPQ_API
+#else
+#define HIPQ_API __attribute__((visibility("default")))
+#endif
+
+/* ---------------------------------------------------------------- status */
+enum
+{
+    HIPQ_OK = 0,
+    HIPQ_ERR_INVALID = 1,     /* malformed argument (null pointer, bad rank, shape mismatch) */
+    HIPQ_ERR_UNSUPPORTED = 2, /* element-type combination the reference has no kernel for either */
+    HIPQ_ERR_HIP = 3,         /* a HIP runtime call failed */
+    HIPQ_ERR_LIMIT = 4        /* size beyond a documented maximum */
+};
+
+/* element types; the quantized ones are u8, i8, i32 (src/ngraph/type/element_type.cpp:83-88) */
+typedef enum
+{
+    HIPQ_U8 = 0,
+    HIPQ_I8 = 1,
+    HIPQ_I32 = 2,
+    HIPQ_F32 = 3,
+    HIPQ_F64 = 4
+} hipq_dtype_t;
+
+/* same order as op::v0::Quantize::RoundMode (src/ngraph/op/quantize.hpp:38-81) */
+typedef enum
+{
+    HIPQ_ROUND_NEAREST_TOWARD_INFINITY = 0,
+    HIPQ_ROUND_NEAREST_TOWARD_ZERO = 1,
+    HIPQ_ROUND_NEAREST_UPWARD = 2,
+    HIPQ_ROUND_NEAREST_DOWNWARD = 3,
+    HIPQ_ROUND_NEAREST_TOWARD_EVEN = 4,
+    HIPQ_ROUND_TOWARD_INFINITY = 5,
+    HIPQ_ROUND_TOWARD_ZERO = 6,
+    HIPQ_ROUND_UP = 7,
+    HIPQ_ROUND_DOWN = 8
+} hipq_round_mode_t;
+
+/* tensor layouts for convolution data / output.  NCX is the reference's (batch, channel,
+ * spatial...) order; NXC is channels-last, the order the MFMA kernels consume natively. */
+typedef enum
+{
+    HIPQ_LAYOUT_NCX = 0,
+    HIPQ_LAYOUT_NXC = 1
+} hipq_layout_t;
+
+#define HIPQ_MAX_RANK 8
+#define HIPQ_MAX_SPATIAL 3
+
+/* ---------------------------------------------------------------- runtime plumbing */
+
+typedef struct hipq_device_info
+{
+    char name[64];
+    char arch[32];           /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
+    int32_t compute_units;   /* CUs */
+    int32_t clock_mhz;       /* peak engine clock */
+    int32_t lds_bytes_per_cu;
+    int32_t reserved;
+    uint64_t hbm_bytes;      /* total device memory */
+} hipq_device_info_t;
+
+HIPQ_API const char* hipq_last_error(void);
+HIPQ_API int hipq_version(void);
+HIPQ_API int hipq_device_count(int* count);
+HIPQ_API int hipq_set_device(int ordinal);
+HIPQ_API int hipq_get_device_info(hipq_device_info_t* info);
+HIPQ_API int hipq_malloc(void** dptr, size_t bytes);
+HIPQ_API int hipq_free(void* dptr);
+HIPQ_API int hipq_memcpy_h2d(void* dst_dev, const void* src_host, size_t bytes, void* stream);
+HIPQ_API int hipq_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes, void* stream);
+HIPQ_API int hipq_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
+/* byte fill done by a kernel (not a memset node), safe to record into a HIP graph */
+HIPQ_API int hipq_fill_bytes(void* dst_dev, int value, size_t bytes, void* stream);
+HIPQ_API int hipq_stream_create(void** stream);
+HIPQ_API int hipq_stream_destroy(void* stream);
+HIPQ_API int hipq_stream_sync(void* stream);
+HIPQ_API int hipq_event_create(void** event);
+HIPQ_API int hipq_event_destroy(void* event);
+HIPQ_API int hipq_event_record(void* event, void* stream);
+HIPQ_API int hipq_event_sync(void* event);
+HIPQ_API int hipq_event_elapsed_ms(void* start, void* stop, float* ms);
+
+/* ---------------------------------------------------------------- Quantize / Dequantize */
+
+/*
+ * Shape of the real/quantized tensor plus the axes the scale / zero-point tensors are laid along:
+ * bit a of axes_mask set <=> axis a is in the op's AxisSet.  scale and zero_point are dense
+ * row-major tensors whose shape is `shape` restricted to those axes (scalar when axes_mask == 0).
+ */
+typedef struct hipq_quant_desc
+{
+    int32_t real_t;     /* HIPQ_F32 or HIPQ_F64: input of quantize / output of dequantize */
+    int32_t quant_t;    /* HIPQ_U8, HIPQ_I8 or HIPQ_I32 */
+    int32_t rank;       /* 0..HIPQ_MAX_RANK */
+    int32_t round_mode; /* hipq_round_mode_t; quantize only */
+    uint32_t axes_mask;
+    uint32_t reserved;
+    int64_t shape[HIPQ_MAX_RANK];
+} hipq_quant_desc_t;
+
+/*
+ * out = (QUANT) clamp(round_mode(in / scale[j]) + zero_point[j])        j = coordinate on `axes`
+ * Replaces runtime::reference::quantize<REAL,QUANT>
+ * (src/ngraph/runtime/reference/quantize.hpp:29-117, dispatched at
+ * src/ngraph/runtime/interpreter/int_executable.hpp:1405-1451).
+ * scale has type real_t, zero_point has type quant_t.  Bit-exact with the reference for finite
+ * inputs (true IEEE division, the reference's floor/ceil rounding formulas, clamp in REAL).
+ */
+HIPQ_API int hipq_quantize(const hipq_quant_desc_t* desc,
+                           const void* in,
+                           const void* scale,
+                           const void* zero_point,
+                           void* out,
+                           void* stream);
+
+/*
+ * out = (REAL)(in - zero_point[j]) * scale[j]
+ * Replaces runtime::reference::dequantize<QUANT,REAL>
+ * (src/ngraph/runtime/reference/dequantize.hpp:31-53, dispatched at int_executable.hpp:830-863).
+ */
+HIPQ_API int hipq_dequantize(const hipq_quant_desc_t* desc,
+                             const void* in,
+                             const void* scale,
+                             const void* zero_point,
+                             void* out,
+                             void* stream);
+
+/* ---------------------------------------------------------------- QuantizedConvolution */
+
+typedef struct hipq_conv_desc
+{
+    int32_t n_spatial;   /* 1..HIPQ_MAX_SPATIAL */
+    int32_t data_t;      /* HIPQ_U8 (the reference's only data type) or HIPQ_I8 */
+    int32_t filter_t;    /* HIPQ_I8 or HIPQ_U8 */
+    int32_t out_t;       /* HIPQ_I8, HIPQ_U8 or HIPQ_I32 */
+    int32_t data_layout; /* hipq_layout_t of `data` (and of `sum_in`) */
+    int32_t out_layout;  /* hipq_layout_t of `out` */
+    int64_t N, C, K;     /* batch, input channels, output channels; filter is always K,C,spatial */
+    int64_t in_sp[HIPQ_MAX_SPATIAL];
+    int64_t f_sp[HIPQ_MAX_SPATIAL];
+    int64_t out_sp[HIPQ_MAX_SPATIAL]; /* must equal hipq_conv_infer_output()'s result */
+    int64_t stride[HIPQ_MAX_SPATIAL];        /* window_movement_strides */
+    int64_t dilation[HIPQ_MAX_SPATIAL];      /* window_dilation_strides */
+    int64_t data_dilation[HIPQ_MAX_SPATIAL]; /* data_dilation_strides */
+    int64_t pad_below[HIPQ_MAX_SPATIAL];     /* may be negative */
+    int64_t pad_above[HIPQ_MAX_SPATIAL];
+} hipq_conv_desc_t;
+
+/* Fills desc->out_sp with the reference's inferred output extent:
+ * ((in-1)*data_dilation+1 + pad_below + pad_above - ((f-1)*dilation+1)) / stride + 1
+ * (infer_convolution_forward, src/ngraph/validation_util.cpp).  HIPQ_ERR_INVALID if not positive. */
+HIPQ_API int hipq_conv_infer_output(hipq_conv_desc_t* desc);
+
+/*
+ * Prepacked filter for the MFMA path.  hipq_conv_packed_filter_bytes returns 0 when the shape /
+ * type combination is not eligible for that path (the call then runs on the direct kernel and
+ * `packed` may be NULL).  The packed blob holds the filter reordered to K,spatial,C plus a
+ * per-output-channel table of 128*sum(filter) used to run u8 data on the signed i8 MFMA.
+ */
+HIPQ_API size_t hipq_conv_packed_filter_bytes(const hipq_conv_desc_t* desc);
+HIPQ_API int hipq_conv_pack_filter(const hipq_conv_desc_t* desc,
+                                   const void* filter,
+                                   void* packed,
+                                   void* stream);
+
+/*
+ * op::v0::QuantizedConvolution.  Replaces runtime::reference::convolution<IN,FILT,OUT,int32_t>
+ * (src/ngraph/runtime/reference/convolution.hpp:55-265,267-313; dispatched at
+ * int_executable.hpp:1453-1558) with the INTERPRETER's arithmetic:
+ *   acc   = sum over in-bounds taps of (data - *data_zp) * (filter - *filter_zp)      int32
+ *   scale = (*data_scale * *filter_scale) / *out_scale                                f32
+ *   out   = (OUT) roundf((float)acc * scale) + *out_zp      half away from zero, narrowing wraps
+ * The six scale / zero-point arguments are DEVICE pointers to scalars (they may be graph
+ * Parameters), zero points typed like the tensor they belong to.
+ */
+HIPQ_API int hipq_quantized_convolution(const hipq_conv_desc_t* desc,
+                                        const void* data,
+                                        const void* filter,
+                                        const void* packed_filter, /* may be NULL */
+                                        const float* data_scale,
+                                        const void* data_zp,
+                                        const float* filter_scale,
+                                        const void* filter_zp,
+                                        const float* out_scale,
+                                        const void* out_zp,
+                                        void* out,
+                                        void* stream);
+
+/* Post-ops of the fused ops.  The arithmetic is oneDNN's as driven by the nGraph CPU backend:
+ *   v = scale[k or 0] * ((float)acc + (float)bias[k]);  v = fmaf(sum_scale, (float)sum_in, v);
+ *   v = relu ? max(v, 0) : v;  out = saturate<OUT>(nearbyintf(v))        round-half-to-even
+ */
+typedef struct hipq_fused_desc
+{
+    int32_t has_bias;    /* bias: int32[K] */
+    int32_t has_sum;     /* sum_in: tensor shaped and laid out like out */
+    int32_t sum_t;       /* HIPQ_U8 or HIPQ_I8 (QuantizedConvolutionBiasSignedAdd reads i8) */
+    int32_t with_relu;
+    int64_t scale_count; /* 1, or K for per-output-channel requantization scales */
+} hipq_fused_desc_t;
+
+/*
+ * op::v0::QuantizedConvolutionBias / ...Relu / ...BiasAdd / ...BiasSignedAdd
+ * (src/ngraph/op/experimental/quantized_conv_bias.cpp:26-237, quantized_conv_relu.cpp:25-80;
+ * executed by src/ngraph/runtime/cpu/builder/quantized_conv.cpp:332-766 with the attributes of
+ * src/ngraph/runtime/cpu/dnnl_emitter.hpp:668-706).  data must be u8 or i8, filter i8, zero points
+ * are all 0; out_t is desc->out_t.  sum_in may alias out.
+ */
+HIPQ_API int hipq_quantized_convolution_fused(const hipq_conv_desc_t* desc,
+                                              const hipq_fused_desc_t* fused,
+                                              const void* data,
+                                              const void* filter,
+                                              const void* packed_filter, /* may be NULL */
+                                              const int32_t* bias,
+                                              const void* sum_in,
+                                              const float* scale,
+                                              const float* sum_scale,
+                                              void* out,
+                                              void* stream);
+
+/* ---------------------------------------------------------------- QuantizedDot */
+
+typedef enum
+{
+    HIPQ_B_KN = 0, /* second operand is [K,N] row-major: op::v0::QuantizedDot */
+    HIPQ_B_NK = 1  /* second operand is [N,K] row-major: op::v0::QuantizedDotBias weights */
+} hipq_b_layout_t;
+
+typedef struct hipq_dot_desc
+{
+    int32_t a_t;      /* HIPQ_U8 or HIPQ_I8 */
+    int32_t b_t;      /* HIPQ_I8 or HIPQ_U8 */
+    int32_t out_t;    /* HIPQ_I8, HIPQ_U8, HIPQ_I32, or HIPQ_F32 (QuantizedDotBias, no requantize) */
+    int32_t b_layout; /* hipq_b_layout_t */
+    int64_t M, K, N;
+} hipq_dot_desc_t;
+
+/*
+ * Optional per-weight-matrix table for the MFMA path: int32[N] holding 128*sum_k(b[k,n]).
+ * hipq_dot_prepare computes it on the device; pass it as `bsum` (NULL = compute per call into an
+ * internal workspace).
+ */
+HIPQ_API int hipq_dot_prepare(const hipq_dot_desc_t* desc, const void* b, int32_t* bsum, void* stream);
+
+/*
+ * op::v0::QuantizedDot with one reduction axis.  Replaces runtime::reference::dot<IN0,IN1,OUT,int32_t>
+ * (src/ngraph/runtime/reference/dot.hpp:34-167; dispatched at int_executable.hpp:1565-1653),
+ * INTERPRETER arithmetic as for hipq_quantized_convolution.  a is [M,K], b is [K,N].
+ */
+HIPQ_API int hipq_quantized_dot(const hipq_dot_desc_t* desc,
+                                const void* a,
+                                const void* b,
+                                const int32_t* bsum, /* may be NULL */
+                                const float* a_scale,
+                                const void* a_zp,
+                                const float* b_scale,
+                                const void* b_zp,
+                                const float* out_scale,
+                                const void* out_zp,
+                                void* out,
+                                void* stream);
+
+/*
+ * op::v0::QuantizedDotBias (src/ngraph/op/experimental/quantized_dot_bias.cpp:27-56; executed by
+ * src/ngraph/runtime/cpu/builder/quantized_dot.cpp:36-125, attributes dnnl_emitter.hpp:737-761).
+ * a is u8 or i8 [M,K], w is i8 [N,K], bias int32[N] (has_bias), scale f32[scale_count].
+ * out_t F32: out = relu?(scale * (acc + bias));  I8/U8: saturate(nearbyint(that)).
+ * has_sum must be 0.
+ */
+HIPQ_API int hipq_quantized_dot_bias(const hipq_dot_desc_t* desc,
+                                     const hipq_fused_desc_t* fused,
+                                     const void* a,
+                                     const void* w,
+                                     const int32_t* wsum, /* may be NULL */
+                                     const int32_t* bias,
+                                     const float* scale,
+                                     void* out,
+                                     void* stream);
+
+/* ---------------------------------------------------------------- layout helpers */
+
+/* [N,C,X] -> [N,X,C] and back for elem_bytes in {1,4}; X = product of spatial extents. */
+HIPQ_API int hipq_transpose_ncx_to_nxc(
+    const void* in, void* out, int64_t N, int64_t C, int64_t X, int32_t elem_bytes, void* stream);
+HIPQ_API int hipq_transpose_nxc_to_ncx(
+    const void* in, void* out, int64_t N, int64_t C, int64_t X, int32_t elem_bytes, void* stream);
+
+/* Which kernel the last hipq_quantized_* call on this thread used: "mfma", "direct", ... (host
+ * string, never NULL).  For tests and profiles. */
+HIPQ_API const char* hipq_last_kernel(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIPQ_H */

@@ -1,0 +1,465 @@
+"""ctypes view of libhipq.so (declared in include/hipq.h).
+
+Plumbing for the Python tests and the benchmark: descriptor structs, dtype codes and a loader
+that fails loudly when the HIP library has not been built.  There is no CPU fallback here or
+anywhere else in the package.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "csrc", "libhipq.so")
+
+U8, I8, I32, F32, F64 = 0, 1, 2, 3, 4
+NCX, NXC = 0, 1
+B_KN, B_NK = 0, 1
+OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_LIMIT = 0, 1, 2, 3, 4
+
+ROUND_MODES = [
+    "ROUND_NEAREST_TOWARD_INFINITY",
+    "ROUND_NEAREST_TOWARD_ZERO",
+    "ROUND_NEAREST_UPWARD",
+    "ROUND_NEAREST_DOWNWARD",
+    "ROUND_NEAREST_TOWARD_EVEN",
+    "ROUND_TOWARD_INFINITY",
+    "ROUND_TOWARD_ZERO",
+    "ROUND_UP",
+    "ROUND_DOWN",
+]
+RNE = ROUND_MODES.index("ROUND_NEAREST_TOWARD_EVEN")
+
+NP_OF = {U8: np.uint8, I8: np.int8, I32: np.int32, F32: np.float32, F64: np.float64}
+CODE_OF = {np.dtype(v): k for k, v in NP_OF.items()}
+NAME_OF = {U8: "u8", I8: "i8", I32: "i32", F32: "f32", F64: "f64"}
+CODE_OF_NAME = {v: k for k, v in NAME_OF.items()}
+
+
+def dtype_code(x) -> int:
+    if isinstance(x, str):
+        return CODE_OF_NAME[x]
+    if isinstance(x, int):
+        return x
+    return CODE_OF[np.dtype(x)]
+
+
+class QuantDesc(C.Structure):
+    _fields_ = [
+        ("real_t", C.c_int32),
+        ("quant_t", C.c_int32),
+        ("rank", C.c_int32),
+        ("round_mode", C.c_int32),
+        ("axes_mask", C.c_uint32),
+        ("reserved", C.c_uint32),
+        ("shape", C.c_int64 * 8),
+    ]
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [
+        ("n_spatial", C.c_int32),
+        ("data_t", C.c_int32),
+        ("filter_t", C.c_int32),
+        ("out_t", C.c_int32),
+        ("data_layout", C.c_int32),
+        ("out_layout", C.c_int32),
+        ("N", C.c_int64),
+        ("C", C.c_int64),
+        ("K", C.c_int64),
+        ("in_sp", C.c_int64 * 3),
+        ("f_sp", C.c_int64 * 3),
+        ("out_sp", C.c_int64 * 3),
+        ("stride", C.c_int64 * 3),
+        ("dilation", C.c_int64 * 3),
+        ("data_dilation", C.c_int64 * 3),
+        ("pad_below", C.c_int64 * 3),
+        ("pad_above", C.c_int64 * 3),
+    ]
+
+    def out_shape(self):
+        sp = [int(self.out_sp[i]) for i in range(self.n_spatial)]
+        if self.out_layout == NXC:
+            return [int(self.N)] + sp + [int(self.K)]
+        return [int(self.N), int(self.K)] + sp
+
+    def data_shape(self):
+        sp = [int(self.in_sp[i]) for i in range(self.n_spatial)]
+        if self.data_layout == NXC:
+            return [int(self.N)] + sp + [int(self.C)]
+        return [int(self.N), int(self.C)] + sp
+
+    def filter_shape(self):
+        return [int(self.K), int(self.C)] + [int(self.f_sp[i]) for i in range(self.n_spatial)]
+
+    def ops(self):
+        """2 * MACs of the dense contraction (padding taps counted, as rooflines do)."""
+        n = 2 * int(self.N) * int(self.K) * int(self.C)
+        for i in range(self.n_spatial):
+            n *= int(self.out_sp[i]) * int(self.f_sp[i])
+        return n
+
+
+class FusedDesc(C.Structure):
+    _fields_ = [
+        ("has_bias", C.c_int32),
+        ("has_sum", C.c_int32),
+        ("sum_t", C.c_int32),
+        ("with_relu", C.c_int32),
+        ("scale_count", C.c_int64),
+    ]
+
+
+class DotDesc(C.Structure):
+    _fields_ = [
+        ("a_t", C.c_int32),
+        ("b_t", C.c_int32),
+        ("out_t", C.c_int32),
+        ("b_layout", C.c_int32),
+        ("M", C.c_int64),
+        ("K", C.c_int64),
+        ("N", C.c_int64),
+    ]
+
+
+class DeviceInfo(C.Structure):
+    _fields_ = [
+        ("name", C.c_char * 64),
+        ("arch", C.c_char * 32),
+        ("compute_units", C.c_int32),
+        ("clock_mhz", C.c_int32),
+        ("lds_bytes_per_cu", C.c_int32),
+        ("reserved", C.c_int32),
+        ("hbm_bytes", C.c_uint64),
+    ]
+
+
+def make_quant_desc(shape, axes, real_t, quant_t, round_mode=RNE) -> QuantDesc:
+    d = QuantDesc()
+    d.real_t, d.quant_t = dtype_code(real_t), dtype_code(quant_t)
+    d.rank = len(shape)
+    d.round_mode = round_mode if isinstance(round_mode, int) else ROUND_MODES.index(round_mode)
+    d.axes_mask = sum(1 << int(a) for a in axes)
+    for i, s in enumerate(shape):
+        d.shape[i] = int(s)
+    return d
+
+
+def make_conv_desc(
+    N,
+    C_,
+    K,
+    in_sp,
+    f_sp,
+    stride=None,
+    dilation=None,
+    pad_below=None,
+    pad_above=None,
+    data_dilation=None,
+    data_t=U8,
+    filter_t=I8,
+    out_t=I8,
+    data_layout=NCX,
+    out_layout=NCX,
+) -> ConvDesc:
+    ns = len(in_sp)
+    d = ConvDesc()
+    d.n_spatial = ns
+    d.data_t, d.filter_t, d.out_t = dtype_code(data_t), dtype_code(filter_t), dtype_code(out_t)
+    d.data_layout, d.out_layout = data_layout, out_layout
+    d.N, d.C, d.K = N, C_, K
+    for i in range(3):
+        d.in_sp[i] = d.f_sp[i] = d.out_sp[i] = 1
+        d.stride[i] = d.dilation[i] = d.data_dilation[i] = 1
+        d.pad_below[i] = d.pad_above[i] = 0
+    for i in range(ns):
+        d.in_sp[i] = in_sp[i]
+        d.f_sp[i] = f_sp[i]
+        d.stride[i] = (stride or [1] * ns)[i]
+        d.dilation[i] = (dilation or [1] * ns)[i]
+        d.data_dilation[i] = (data_dilation or [1] * ns)[i]
+        d.pad_below[i] = (pad_below or [0] * ns)[i]
+        d.pad_above[i] = (pad_above or [0] * ns)[i]
+    for i in range(ns):
+        eff_in = (d.in_sp[i] - 1) * d.data_dilation[i] + 1 + d.pad_below[i] + d.pad_above[i]
+        eff_f = (d.f_sp[i] - 1) * d.dilation[i] + 1
+        if eff_in < eff_f:
+            raise ValueError("convolution window larger than padded input")
+        d.out_sp[i] = (eff_in - eff_f) // d.stride[i] + 1
+    return d
+
+
+def make_fused_desc(has_bias=True, has_sum=False, sum_t=U8, with_relu=False, scale_count=1) -> FusedDesc:
+    f = FusedDesc()
+    f.has_bias, f.has_sum, f.sum_t = int(has_bias), int(has_sum), dtype_code(sum_t)
+    f.with_relu, f.scale_count = int(with_relu), int(scale_count)
+    return f
+
+
+def make_dot_desc(M, K, N, a_t=U8, b_t=I8, out_t=I8, b_layout=B_KN) -> DotDesc:
+    d = DotDesc()
+    d.a_t, d.b_t, d.out_t, d.b_layout = dtype_code(a_t), dtype_code(b_t), dtype_code(out_t), b_layout
+    d.M, d.K, d.N = M, K, N
+    return d
+
+
+EXPORTS = [
+    "hipq_last_error",
+    "hipq_version",
+    "hipq_device_count",
+    "hipq_set_device",
+    "hipq_get_device_info",
+    "hipq_malloc",
+    "hipq_free",
+    "hipq_memcpy_h2d",
+    "hipq_memcpy_d2h",
+    "hipq_memcpy_d2d",
+    "hipq_fill_bytes",
+    "hipq_stream_create",
+    "hipq_stream_destroy",
+    "hipq_stream_sync",
+    "hipq_event_create",
+    "hipq_event_destroy",
+    "hipq_event_record",
+    "hipq_event_sync",
+    "hipq_event_elapsed_ms",
+    "hipq_quantize",
+    "hipq_dequantize",
+    "hipq_conv_infer_output",
+    "hipq_conv_packed_filter_bytes",
+    "hipq_conv_pack_filter",
+    "hipq_quantized_convolution",
+    "hipq_quantized_convolution_fused",
+    "hipq_dot_prepare",
+    "hipq_quantized_dot",
+    "hipq_quantized_dot_bias",
+    "hipq_transpose_ncx_to_nxc",
+    "hipq_transpose_nxc_to_ncx",
+    "hipq_last_kernel",
+]
+
+_lib = None
+
+
+class HipqError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__(f"hipq error {code}: {msg}")
+        self.code = code
+
+
+def load():
+    """dlopen libhipq.so (built by __graft_entry__.build()); raises if it is not there."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build the HIP library first (python -c 'import __graft_entry__ as g; g.build()')"
+        )
+    lib = C.CDLL(LIB_PATH)
+    vp, i64, i32 = C.c_void_p, C.c_int64, C.c_int32
+    lib.hipq_last_error.restype = C.c_char_p
+    lib.hipq_last_kernel.restype = C.c_char_p
+    lib.hipq_conv_packed_filter_bytes.restype = C.c_size_t
+    lib.hipq_conv_packed_filter_bytes.argtypes = [C.POINTER(ConvDesc)]
+    lib.hipq_device_count.argtypes = [C.POINTER(C.c_int)]
+    lib.hipq_set_device.argtypes = [C.c_int]
+    lib.hipq_get_device_info.argtypes = [C.POINTER(DeviceInfo)]
+    lib.hipq_malloc.argtypes = [C.POINTER(vp), C.c_size_t]
+    lib.hipq_free.argtypes = [vp]
+    for n in ("hipq_memcpy_h2d", "hipq_memcpy_d2h", "hipq_memcpy_d2d"):
+        getattr(lib, n).argtypes = [vp, vp, C.c_size_t, vp]
+    lib.hipq_fill_bytes.argtypes = [vp, C.c_int, C.c_size_t, vp]
+    lib.hipq_stream_create.argtypes = [C.POINTER(vp)]
+    lib.hipq_stream_destroy.argtypes = [vp]
+    lib.hipq_stream_sync.argtypes = [vp]
+    lib.hipq_event_create.argtypes = [C.POINTER(vp)]
+    lib.hipq_event_destroy.argtypes = [vp]
+    lib.hipq_event_record.argtypes = [vp, vp]
+    lib.hipq_event_sync.argtypes = [vp]
+    lib.hipq_event_elapsed_ms.argtypes = [vp, vp, C.POINTER(C.c_float)]
+    lib.hipq_quantize.argtypes = [C.POINTER(QuantDesc), vp, vp, vp, vp, vp]
+    lib.hipq_dequantize.argtypes = [C.POINTER(QuantDesc), vp, vp, vp, vp, vp]
+    lib.hipq_conv_infer_output.argtypes = [C.POINTER(ConvDesc)]
+    lib.hipq_conv_pack_filter.argtypes = [C.POINTER(ConvDesc), vp, vp, vp]
+    lib.hipq_quantized_convolution.argtypes = [C.POINTER(ConvDesc)] + [vp] * 11
+    lib.hipq_quantized_convolution_fused.argtypes = [C.POINTER(ConvDesc), C.POINTER(FusedDesc)] + [vp] * 9
+    lib.hipq_dot_prepare.argtypes = [C.POINTER(DotDesc), vp, vp, vp]
+    lib.hipq_quantized_dot.argtypes = [C.POINTER(DotDesc)] + [vp] * 11
+    lib.hipq_quantized_dot_bias.argtypes = [C.POINTER(DotDesc), C.POINTER(FusedDesc)] + [vp] * 7
+    for n in ("hipq_transpose_ncx_to_nxc", "hipq_transpose_nxc_to_ncx"):
+        getattr(lib, n).argtypes = [vp, vp, i64, i64, i64, i32, vp]
+    _lib = lib
+    return lib
+
+
+def check(rc):
+    if rc != OK:
+        raise HipqError(rc, load().hipq_last_error().decode())
+
+
+def last_kernel() -> str:
+    return load().hipq_last_kernel().decode()
+
+
+class DeviceBuffer:
+    """Device allocation owned through hipq_malloc / hipq_free."""
+
+    def __init__(self, nbytes: int):
+        self.nbytes = int(nbytes)
+        p = C.c_void_p()
+        check(load().hipq_malloc(C.byref(p), max(self.nbytes, 1)))
+        self.ptr = p.value
+
+    @classmethod
+    def from_numpy(cls, a: np.ndarray) -> "DeviceBuffer":
+        a = np.ascontiguousarray(a)
+        b = cls(a.nbytes)
+        if a.nbytes:
+            check(load().hipq_memcpy_h2d(b.ptr, a.ctypes.data, a.nbytes, None))
+        return b
+
+    def to_numpy(self, dtype, shape) -> np.ndarray:
+        out = np.empty(shape, dtype=dtype)
+        assert out.nbytes <= self.nbytes
+        if out.nbytes:
+            check(load().hipq_memcpy_d2h(out.ctypes.data, self.ptr, out.nbytes, None))
+        return out
+
+    def free(self):
+        if self.ptr:
+            load().hipq_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def _dev(x):
+    """numpy array / scalar -> DeviceBuffer (None stays None)."""
+    if x is None:
+        return None
+    return DeviceBuffer.from_numpy(np.asarray(x))
+
+
+def _p(b):
+    return None if b is None else b.ptr
+
+
+# ---- numpy-in / numpy-out conveniences (one call = upload, launch, sync, download) ----------
+
+
+def quantize(x, scale, zp, quant_t, axes=(), round_mode=RNE):
+    x = np.ascontiguousarray(x)
+    qt = dtype_code(quant_t)
+    d = make_quant_desc(x.shape, axes, x.dtype, qt, round_mode)
+    bx, bs, bz = _dev(x), _dev(np.asarray(scale, dtype=x.dtype)), _dev(np.asarray(zp, dtype=NP_OF[qt]))
+    out = DeviceBuffer(x.size * np.dtype(NP_OF[qt]).itemsize)
+    check(load().hipq_quantize(C.byref(d), bx.ptr, bs.ptr, bz.ptr, out.ptr, None))
+    check(load().hipq_stream_sync(None))
+    return out.to_numpy(NP_OF[qt], x.shape)
+
+
+def dequantize(q, scale, zp, real_t=F32, axes=()):
+    q = np.ascontiguousarray(q)
+    rt = dtype_code(real_t)
+    d = make_quant_desc(q.shape, axes, rt, q.dtype)
+    bq, bs, bz = _dev(q), _dev(np.asarray(scale, dtype=NP_OF[rt])), _dev(np.asarray(zp, dtype=q.dtype))
+    out = DeviceBuffer(q.size * np.dtype(NP_OF[rt]).itemsize)
+    check(load().hipq_dequantize(C.byref(d), bq.ptr, bs.ptr, bz.ptr, out.ptr, None))
+    check(load().hipq_stream_sync(None))
+    return out.to_numpy(NP_OF[rt], q.shape)
+
+
+def pack_filter(desc: ConvDesc, filter_dev: DeviceBuffer):
+    """Returns the packed-filter DeviceBuffer, or None when the MFMA path does not apply."""
+    n = load().hipq_conv_packed_filter_bytes(C.byref(desc))
+    if n == 0:
+        return None
+    packed = DeviceBuffer(n)
+    check(load().hipq_conv_pack_filter(C.byref(desc), filter_dev.ptr, packed.ptr, None))
+    return packed
+
+
+def quantized_convolution(desc, data, filt, data_scale, data_zp, filter_scale, filter_zp, out_scale, out_zp, use_packed=True):
+    lib = load()
+    bd, bf = _dev(data), _dev(filt)
+    packed = pack_filter(desc, bf) if use_packed else None
+    s = [_dev(np.float32(v)) for v in (data_scale, filter_scale, out_scale)]
+    z = [
+        _dev(np.asarray(data_zp, dtype=NP_OF[desc.data_t])),
+        _dev(np.asarray(filter_zp, dtype=NP_OF[desc.filter_t])),
+        _dev(np.asarray(out_zp, dtype=NP_OF[desc.out_t])),
+    ]
+    oshape = desc.out_shape()
+    out = DeviceBuffer(int(np.prod(oshape)) * np.dtype(NP_OF[desc.out_t]).itemsize)
+    check(
+        lib.hipq_quantized_convolution(
+            C.byref(desc), bd.ptr, bf.ptr, _p(packed), s[0].ptr, z[0].ptr, s[1].ptr, z[1].ptr, s[2].ptr, z[2].ptr, out.ptr, None
+        )
+    )
+    check(lib.hipq_stream_sync(None))
+    return out.to_numpy(NP_OF[desc.out_t], oshape)
+
+
+def quantized_convolution_fused(desc, fused, data, filt, bias, sum_in, scale, sum_scale, use_packed=True):
+    lib = load()
+    bd, bf = _dev(data), _dev(filt)
+    packed = pack_filter(desc, bf) if use_packed else None
+    bb = _dev(None if bias is None else np.asarray(bias, dtype=np.int32))
+    bsc = _dev(np.asarray(scale, dtype=np.float32))
+    bss = _dev(None if sum_scale is None else np.float32(sum_scale))
+    oshape = desc.out_shape()
+    nbytes = int(np.prod(oshape)) * np.dtype(NP_OF[desc.out_t]).itemsize
+    out = DeviceBuffer(nbytes)
+    bsum = _dev(sum_in)
+    check(
+        lib.hipq_quantized_convolution_fused(
+            C.byref(desc), C.byref(fused), bd.ptr, bf.ptr, _p(packed), _p(bb), _p(bsum), bsc.ptr, _p(bss), out.ptr, None
+        )
+    )
+    check(lib.hipq_stream_sync(None))
+    return out.to_numpy(NP_OF[desc.out_t], oshape)
+
+
+def quantized_dot(desc, a, b, a_scale, a_zp, b_scale, b_zp, out_scale, out_zp, prepare=True):
+    lib = load()
+    ba, bb = _dev(a), _dev(b)
+    bsum = None
+    if prepare:
+        bsum = DeviceBuffer(4 * max(int(desc.N), 1))
+        check(lib.hipq_dot_prepare(C.byref(desc), bb.ptr, bsum.ptr, None))
+    s = [_dev(np.float32(v)) for v in (a_scale, b_scale, out_scale)]
+    z = [
+        _dev(np.asarray(a_zp, dtype=NP_OF[desc.a_t])),
+        _dev(np.asarray(b_zp, dtype=NP_OF[desc.b_t])),
+        _dev(np.asarray(out_zp, dtype=NP_OF[desc.out_t])),
+    ]
+    out = DeviceBuffer(int(desc.M * desc.N) * np.dtype(NP_OF[desc.out_t]).itemsize)
+    check(
+        lib.hipq_quantized_dot(
+            C.byref(desc), ba.ptr, bb.ptr, _p(bsum), s[0].ptr, z[0].ptr, s[1].ptr, z[1].ptr, s[2].ptr, z[2].ptr, out.ptr, None
+        )
+    )
+    check(lib.hipq_stream_sync(None))
+    return out.to_numpy(NP_OF[desc.out_t], (int(desc.M), int(desc.N)))
+
+
+def quantized_dot_bias(desc, fused, a, w, bias, scale, prepare=True):
+    lib = load()
+    ba, bw = _dev(a), _dev(w)
+    wsum = None
+    if prepare:
+        wsum = DeviceBuffer(4 * max(int(desc.N), 1))
+        check(lib.hipq_dot_prepare(C.byref(desc), bw.ptr, wsum.ptr, None))
+    bb = _dev(None if bias is None else np.asarray(bias, dtype=np.int32))
+    bsc = _dev(np.asarray(scale, dtype=np.float32))
+    out = DeviceBuffer(int(desc.M * desc.N) * np.dtype(NP_OF[desc.out_t]).itemsize)
+    check(
+        lib.hipq_quantized_dot_bias(C.byref(desc), C.byref(fused), ba.ptr, bw.ptr, _p(wsum), _p(bb), bsc.ptr, out.ptr, None)
+    )
+    check(lib.hipq_stream_sync(None))
+    return out.to_numpy(NP_OF[desc.out_t], (int(desc.M), int(desc.N)))

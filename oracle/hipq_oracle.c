@@ -1,0 +1,748 @@
+/*
+ * hipq_oracle.c -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * A plain-C, CPU restatement of the arithmetic of the nGraph kernels that libhipq.so replaces.
+ * It exists so that the parity tests, the smoke check and the benchmark's cpu_baseline leg have
+ * something that travels to a machine where the nGraph sources are absent.  Nothing in the
+ * product (the HIP library, the backend plugin, the Python binding) links, loads or calls it.
+ *
+ * Every function mirrors one entry point of include/hipq.h (same descriptor structs, host
+ * pointers instead of device pointers) and cites the reference lines it restates (paths relative
+ * to the nGraph source tree).
+ *
+ * How each function is pinned (tests/test_oracle_*.py):
+ *   orc_quantize / orc_dequantize   the 28 literal vectors of test/backend/quantize_dequantize.in.cpp,
+ *                                   the builder vectors of test/builder_quantization.cpp:679-847, and
+ *                                   the compiled reference templates (oracle/_ref) on seeded tensors.
+ *   orc_quantized_convolution       test/backend/quantized_convolution.in.cpp:31-134, the ONNX
+ *                                   QLinearConv byte fixtures (non-zero zero points), oracle/_ref on
+ *                                   seeded shapes (strides, dilations, negative pads, 1-D..3-D), and
+ *                                   a brute-force int64 convolution written independently in numpy.
+ *   orc_quantized_dot               test/backend/quantized_dot.in.cpp:31-115, the QLinearMatMul vector
+ *                                   of test/onnx/onnx_import_quant.in.cpp:296-312, oracle/_ref, numpy.
+ *   orc_quantized_convolution_fused,
+ *   orc_quantized_dot_bias          the oneDNN-backed ops have no runnable reference here (oneDNN
+ *                                   v1.6.2 is fetched at build time, cmake/external/onednn.cmake:120-124).
+ *                                   Pinned by the reference's own known answers at that boundary
+ *                                   (test/builder_quantization.cpp:51-677,995-1098), which fix
+ *                                   round-half-even (78.5 -> 78), saturation (134 -> 127) and the
+ *                                   float order scale*(acc+bias).  Outside those vectors (per-channel
+ *                                   scales, |acc+bias| > 2^24, fused-multiply-add of the sum term)
+ *                                   PARITY IS UNPINNED and defined by the closed form below.
+ *   orc_get_*scale                  the same builder tests (they feed min/max, not scales).
+ */
+#include "../include/hipq.h"
+
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#if defined(_OPENMP)
+#include <omp.h>
+#endif
+
+#define ORC_API __attribute__((visibility("default")))
+
+static int g_threads = 1;
+
+/* number of OpenMP threads the loops below may use (1 = scalar port) */
+ORC_API void orc_set_threads(int n)
+{
+    g_threads = n < 1 ? 1 : n;
+}
+
+ORC_API int orc_get_threads(void)
+{
+    return g_threads;
+}
+
+/* ------------------------------------------------------------------------------------------
+ * x86-64 narrowing semantics of the reference build (g++, SSE): float -> integer goes through
+ * cvttss2si, which yields INT32_MIN for NaN and anything outside [-2^31, 2^31); 8-bit results
+ * are the low byte of that.
+ * ------------------------------------------------------------------------------------------ */
+static int32_t cvtt_f32(float v)
+{
+    if (!(v < 2147483648.0f) || v < -2147483648.0f)
+    {
+        return INT32_MIN;
+    }
+    return (int32_t)v;
+}
+
+static int32_t cvtt_f64(double v)
+{
+    if (!(v < 2147483648.0) || v <= -2147483649.0)
+    {
+        return INT32_MIN;
+    }
+    return (int32_t)v;
+}
+
+static size_t dtype_size(int t)
+{
+    switch (t)
+    {
+    case HIPQ_U8:
+    case HIPQ_I8: return 1;
+    case HIPQ_I32:
+    case HIPQ_F32: return 4;
+    case HIPQ_F64: return 8;
+    default: return 0;
+    }
+}
+
+static int32_t load_q(const void* p, int t, size_t i)
+{
+    switch (t)
+    {
+    case HIPQ_U8: return ((const uint8_t*)p)[i];
+    case HIPQ_I8: return ((const int8_t*)p)[i];
+    default: return ((const int32_t*)p)[i];
+    }
+}
+
+static void store_q_wrap(void* p, int t, size_t i, int32_t v)
+{
+    switch (t)
+    {
+    case HIPQ_U8: ((uint8_t*)p)[i] = (uint8_t)(uint32_t)v; break;
+    case HIPQ_I8: ((int8_t*)p)[i] = (int8_t)(uint8_t)(uint32_t)v; break;
+    default: ((int32_t*)p)[i] = v; break;
+    }
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Quantize: src/ngraph/runtime/reference/quantize.hpp:29-117
+ * ------------------------------------------------------------------------------------------ */
+static float round_mode_f32(float q, int mode)
+{
+    switch (mode)
+    {
+    case HIPQ_ROUND_NEAREST_TOWARD_INFINITY: /* quantize.hpp:51-58 */
+    {
+        float a = floorf(fabsf(q) + 0.5f);
+        return (q < 0.0f) ? -a : a;
+    }
+    case HIPQ_ROUND_NEAREST_TOWARD_ZERO: /* :59-66 */
+    {
+        float a = ceilf(fabsf(q) - 0.5f);
+        return (q < 0.0f) ? -a : a;
+    }
+    case HIPQ_ROUND_NEAREST_UPWARD: return floorf(q + 0.5f);   /* :67-70 */
+    case HIPQ_ROUND_NEAREST_DOWNWARD: return ceilf(q - 0.5f);  /* :71-74 */
+    case HIPQ_ROUND_NEAREST_TOWARD_EVEN:                       /* :75-81 */
+    {
+        float up = floorf(q + 0.5f);
+        float dn = ceilf(q - 0.5f);
+        double rem = fmod((double)up, 2.0);
+        return (rem == 0.0) ? up : dn;
+    }
+    case HIPQ_ROUND_TOWARD_INFINITY: /* :82-88 */
+    {
+        float a = ceilf(fabsf(q));
+        return (q < 0.0f) ? -a : a;
+    }
+    case HIPQ_ROUND_TOWARD_ZERO: /* :89-95 */
+    {
+        float a = floorf(fabsf(q));
+        return (q < 0.0f) ? -a : a;
+    }
+    case HIPQ_ROUND_UP: return ceilf(q);    /* :96-99 */
+    case HIPQ_ROUND_DOWN: return floorf(q); /* :100-103 */
+    default: return q;
+    }
+}
+
+static double round_mode_f64(double q, int mode)
+{
+    switch (mode)
+    {
+    case HIPQ_ROUND_NEAREST_TOWARD_INFINITY:
+    {
+        double a = floor(fabs(q) + 0.5);
+        return (q < 0.0) ? -a : a;
+    }
+    case HIPQ_ROUND_NEAREST_TOWARD_ZERO:
+    {
+        double a = ceil(fabs(q) - 0.5);
+        return (q < 0.0) ? -a : a;
+    }
+    case HIPQ_ROUND_NEAREST_UPWARD: return floor(q + 0.5);
+    case HIPQ_ROUND_NEAREST_DOWNWARD: return ceil(q - 0.5);
+    case HIPQ_ROUND_NEAREST_TOWARD_EVEN:
+    {
+        double up = floor(q + 0.5);
+        double dn = ceil(q - 0.5);
+        double rem = fmod(up, 2.0);
+        return (rem == 0.0) ? up : dn;
+    }
+    case HIPQ_ROUND_TOWARD_INFINITY:
+    {
+        double a = ceil(fabs(q));
+        return (q < 0.0) ? -a : a;
+    }
+    case HIPQ_ROUND_TOWARD_ZERO:
+    {
+        double a = floor(fabs(q));
+        return (q < 0.0) ? -a : a;
+    }
+    case HIPQ_ROUND_UP: return ceil(q);
+    case HIPQ_ROUND_DOWN: return floor(q);
+    default: return q;
+    }
+}
+
+static void quant_limits(int t, double* lo, double* hi)
+{
+    switch (t)
+    {
+    case HIPQ_U8: *lo = 0.0; *hi = 255.0; break;
+    case HIPQ_I8: *lo = -128.0; *hi = 127.0; break;
+    default: *lo = -2147483648.0; *hi = 2147483647.0; break;
+    }
+}
+
+/* index into the scale / zero-point tensor of the element with flat index `i`:
+ * project(coordinate, axes) then row-major index (shape_util.hpp project, quantize.hpp:44) */
+static size_t project_index(const hipq_quant_desc_t* d, size_t i)
+{
+    size_t coord[HIPQ_MAX_RANK];
+    for (int a = d->rank - 1; a >= 0; --a)
+    {
+        coord[a] = i % (size_t)d->shape[a];
+        i /= (size_t)d->shape[a];
+    }
+    size_t j = 0;
+    for (int a = 0; a < d->rank; ++a)
+    {
+        if (d->axes_mask & (1u << a))
+        {
+            j = j * (size_t)d->shape[a] + coord[a];
+        }
+    }
+    return j;
+}
+
+static int check_quant_desc(const hipq_quant_desc_t* d)
+{
+    if (!d || d->rank < 0 || d->rank > HIPQ_MAX_RANK)
+        return HIPQ_ERR_INVALID;
+    if (d->real_t != HIPQ_F32 && d->real_t != HIPQ_F64)
+        return HIPQ_ERR_UNSUPPORTED;
+    if (d->quant_t != HIPQ_U8 && d->quant_t != HIPQ_I8 && d->quant_t != HIPQ_I32)
+        return HIPQ_ERR_UNSUPPORTED;
+    if (d->rank < 32 && (d->axes_mask >> d->rank) != 0)
+        return HIPQ_ERR_INVALID;
+    return HIPQ_OK;
+}
+
+static size_t quant_count(const hipq_quant_desc_t* d)
+{
+    size_t n = 1;
+    for (int a = 0; a < d->rank; ++a)
+        n *= (size_t)d->shape[a];
+    return n;
+}
+
+ORC_API int orc_quantize(
+    const hipq_quant_desc_t* d, const void* in, const void* scale, const void* zp, void* out)
+{
+    int rc = check_quant_desc(d);
+    if (rc)
+        return rc;
+    size_t n = quant_count(d);
+    double lo, hi;
+    quant_limits(d->quant_t, &lo, &hi);
+    long long i;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (i = 0; i < (long long)n; ++i)
+    {
+        size_t j = d->axes_mask ? project_index(d, (size_t)i) : 0;
+        int32_t z = load_q(zp, d->quant_t, j);
+        int32_t r;
+        if (d->real_t == HIPQ_F32)
+        {
+            float q = ((const float*)in)[i] / ((const float*)scale)[j]; /* quantize.hpp:47-48 */
+            q = round_mode_f32(q, d->round_mode);
+            q += (float)z;                                  /* :106 */
+            q = (q < (float)lo) ? (float)lo : q;            /* :109-110 std::max */
+            q = ((float)hi < q) ? (float)hi : q;            /* :111-112 std::min */
+            r = cvtt_f32(q);                                /* :115 */
+        }
+        else
+        {
+            double q = ((const double*)in)[i] / ((const double*)scale)[j];
+            q = round_mode_f64(q, d->round_mode);
+            q += (double)z;
+            q = (q < lo) ? lo : q;
+            q = (hi < q) ? hi : q;
+            r = cvtt_f64(q);
+        }
+        store_q_wrap(out, d->quant_t, (size_t)i, r);
+    }
+    return HIPQ_OK;
+}
+
+/* Dequantize: src/ngraph/runtime/reference/dequantize.hpp:31-53 */
+ORC_API int orc_dequantize(
+    const hipq_quant_desc_t* d, const void* in, const void* scale, const void* zp, void* out)
+{
+    int rc = check_quant_desc(d);
+    if (rc)
+        return rc;
+    size_t n = quant_count(d);
+    long long i;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (i = 0; i < (long long)n; ++i)
+    {
+        size_t j = d->axes_mask ? project_index(d, (size_t)i) : 0;
+        /* integer subtract after promotion; int32 wraps (dequantize.hpp:46-50) */
+        int32_t diff =
+            (int32_t)((uint32_t)load_q(in, d->quant_t, (size_t)i) - (uint32_t)load_q(zp, d->quant_t, j));
+        if (d->real_t == HIPQ_F32)
+            ((float*)out)[i] = (float)diff * ((const float*)scale)[j];
+        else
+            ((double*)out)[i] = (double)diff * ((const double*)scale)[j];
+    }
+    return HIPQ_OK;
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Requantization epilogues
+ * ------------------------------------------------------------------------------------------ */
+
+/* INTERPRETER policy: convolution.hpp:252-258, dot.hpp:152-159.
+ *   out = static_cast<OUT>(std::round(float(acc) * scale)) + *out_zp   (narrowing store) */
+static int32_t requant_interp(int32_t acc, float scale, int32_t ozp, int out_t)
+{
+    float v = roundf((float)acc * scale);
+    int32_t t = cvtt_f32(v);
+    if (out_t == HIPQ_U8)
+        t = (uint8_t)(uint32_t)t;
+    else if (out_t == HIPQ_I8)
+        t = (int8_t)(uint8_t)(uint32_t)t;
+    return (int32_t)((uint32_t)t + (uint32_t)ozp);
+}
+
+/* oneDNN policy as the nGraph CPU backend drives it (dnnl_emitter.hpp:668-706,737-761):
+ * output scale, then post-ops sum, then relu, then round-to-nearest-even with saturation. */
+static float fused_value(
+    int32_t acc, int has_bias, int32_t bias, float scale, int has_sum, float sum_scale, int32_t sum_v, int relu)
+{
+    float v = (float)acc;
+    if (has_bias)
+        v += (float)bias;
+    v *= scale;
+    if (has_sum)
+        v = fmaf(sum_scale, (float)sum_v, v);
+    if (relu)
+        v = (v > 0.0f) ? v : v * -0.0f; /* eltwise_relu with negative slope -0.f */
+    return v;
+}
+
+static int32_t saturate_rne(float v, int out_t)
+{
+    float lo = (out_t == HIPQ_U8) ? 0.0f : (out_t == HIPQ_I8 ? -128.0f : -2147483648.0f);
+    float hi = (out_t == HIPQ_U8) ? 255.0f : (out_t == HIPQ_I8 ? 127.0f : 2147483520.0f);
+    v = (v < lo) ? lo : v;
+    v = (hi < v) ? hi : v;
+    return (int32_t)nearbyintf(v);
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Convolution accumulator: convolution.hpp:102-251 with the membership rule of
+ * CoordinateTransform::has_source_coordinate (coordinate_transform.cpp:326-370): a tap
+ * contributes only if it lands on a real input element, i.e. not in the padding and not in a
+ * data-dilation gap.  Skipped taps add nothing, they are not (0 - zero_point).
+ * ------------------------------------------------------------------------------------------ */
+typedef struct conv_dims
+{
+    int64_t N, C, K;
+    int64_t in[3], f[3], out[3], st[3], dl[3], dd[3], pb[3];
+} conv_dims_t;
+
+static int normalise_conv(const hipq_conv_desc_t* d, conv_dims_t* c)
+{
+    if (!d || d->n_spatial < 1 || d->n_spatial > HIPQ_MAX_SPATIAL)
+        return HIPQ_ERR_INVALID;
+    int lead = 3 - d->n_spatial;
+    c->N = d->N;
+    c->C = d->C;
+    c->K = d->K;
+    for (int i = 0; i < 3; ++i)
+    {
+        c->in[i] = c->f[i] = c->out[i] = c->st[i] = c->dl[i] = c->dd[i] = 1;
+        c->pb[i] = 0;
+    }
+    for (int i = 0; i < d->n_spatial; ++i)
+    {
+        c->in[lead + i] = d->in_sp[i];
+        c->f[lead + i] = d->f_sp[i];
+        c->out[lead + i] = d->out_sp[i];
+        c->st[lead + i] = d->stride[i];
+        c->dl[lead + i] = d->dilation[i];
+        c->dd[lead + i] = d->data_dilation[i];
+        c->pb[lead + i] = d->pad_below[i];
+        if (d->in_sp[i] < 1 || d->f_sp[i] < 1 || d->out_sp[i] < 1 || d->stride[i] < 1 ||
+            d->dilation[i] < 1 || d->data_dilation[i] < 1)
+            return HIPQ_ERR_INVALID;
+    }
+    if (d->N < 1 || d->C < 1 || d->K < 1)
+        return HIPQ_ERR_INVALID;
+    return HIPQ_OK;
+}
+
+ORC_API int orc_conv_infer_output(hipq_conv_desc_t* d)
+{
+    if (!d || d->n_spatial < 1 || d->n_spatial > HIPQ_MAX_SPATIAL)
+        return HIPQ_ERR_INVALID;
+    for (int i = 0; i < d->n_spatial; ++i)
+    {
+        int64_t in_eff = (d->in_sp[i] - 1) * d->data_dilation[i] + 1 + d->pad_below[i] + d->pad_above[i];
+        int64_t f_eff = (d->f_sp[i] - 1) * d->dilation[i] + 1;
+        if (in_eff < f_eff || d->stride[i] < 1)
+            return HIPQ_ERR_INVALID;
+        d->out_sp[i] = (in_eff - f_eff) / d->stride[i] + 1;
+    }
+    return HIPQ_OK;
+}
+
+static size_t act_index(int layout, const int64_t* sp, int64_t Cn, int64_t n, int64_t c, int64_t z, int64_t y, int64_t x)
+{
+    size_t s = (size_t)((z * sp[1] + y) * sp[2] + x);
+    size_t S = (size_t)(sp[0] * sp[1] * sp[2]);
+    if (layout == HIPQ_LAYOUT_NXC)
+        return ((size_t)n * S + s) * (size_t)Cn + (size_t)c;
+    return ((size_t)n * (size_t)Cn + (size_t)c) * S + s;
+}
+
+static int32_t conv_acc_one(const hipq_conv_desc_t* d,
+                            const conv_dims_t* c,
+                            const void* data,
+                            const void* filter,
+                            int32_t dzp,
+                            int32_t fzp,
+                            int64_t n,
+                            int64_t k,
+                            int64_t oz,
+                            int64_t oy,
+                            int64_t ox)
+{
+    int32_t acc = 0;
+    for (int64_t fz = 0; fz < c->f[0]; ++fz)
+    {
+        int64_t pz = oz * c->st[0] + fz * c->dl[0] - c->pb[0];
+        if (pz < 0 || pz > (c->in[0] - 1) * c->dd[0] || pz % c->dd[0] != 0)
+            continue;
+        for (int64_t fy = 0; fy < c->f[1]; ++fy)
+        {
+            int64_t py = oy * c->st[1] + fy * c->dl[1] - c->pb[1];
+            if (py < 0 || py > (c->in[1] - 1) * c->dd[1] || py % c->dd[1] != 0)
+                continue;
+            for (int64_t fx = 0; fx < c->f[2]; ++fx)
+            {
+                int64_t px = ox * c->st[2] + fx * c->dl[2] - c->pb[2];
+                if (px < 0 || px > (c->in[2] - 1) * c->dd[2] || px % c->dd[2] != 0)
+                    continue;
+                for (int64_t ch = 0; ch < c->C; ++ch)
+                {
+                    size_t di = act_index(
+                        d->data_layout, c->in, c->C, n, ch, pz / c->dd[0], py / c->dd[1], px / c->dd[2]);
+                    size_t fi = (size_t)((((k * c->C + ch) * c->f[0] + fz) * c->f[1] + fy) * c->f[2] + fx);
+                    int32_t a = load_q(data, d->data_t, di) - dzp;
+                    int32_t b = load_q(filter, d->filter_t, fi) - fzp;
+                    acc = (int32_t)((uint32_t)acc + (uint32_t)(a * b));
+                }
+            }
+        }
+    }
+    return acc;
+}
+
+/* raw int32 accumulators, laid out like the output tensor (d->out_layout) */
+ORC_API int orc_conv_accumulate(const hipq_conv_desc_t* d,
+                                const void* data,
+                                const void* filter,
+                                int32_t data_zp,
+                                int32_t filter_zp,
+                                int32_t* acc)
+{
+    conv_dims_t c;
+    int rc = normalise_conv(d, &c);
+    if (rc)
+        return rc;
+    long long total = (long long)(c.N * c.K * c.out[0] * c.out[1] * c.out[2]);
+    long long t;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (t = 0; t < total; ++t)
+    {
+        int64_t r = t;
+        int64_t ox = r % c.out[2];
+        r /= c.out[2];
+        int64_t oy = r % c.out[1];
+        r /= c.out[1];
+        int64_t oz = r % c.out[0];
+        r /= c.out[0];
+        int64_t k = r % c.K;
+        int64_t n = r / c.K;
+        size_t oi = act_index(d->out_layout, c.out, c.K, n, k, oz, oy, ox);
+        acc[oi] = conv_acc_one(d, &c, data, filter, data_zp, filter_zp, n, k, oz, oy, ox);
+    }
+    return HIPQ_OK;
+}
+
+static int conv_types_ok(const hipq_conv_desc_t* d)
+{
+    /* combinations the INTERPRETER dispatches: int_executable.hpp:1461-1549 (+ i8 data, which the
+     * CPU backend's fused ops accept) */
+    if (d->data_t != HIPQ_U8 && d->data_t != HIPQ_I8)
+        return 0;
+    if (d->filter_t != HIPQ_I8 && d->filter_t != HIPQ_U8)
+        return 0;
+    if (d->out_t != HIPQ_I8 && d->out_t != HIPQ_U8 && d->out_t != HIPQ_I32)
+        return 0;
+    return 1;
+}
+
+/* op::v0::QuantizedConvolution, INTERPRETER arithmetic */
+ORC_API int orc_quantized_convolution(const hipq_conv_desc_t* d,
+                                      const void* data,
+                                      const void* filter,
+                                      const float* data_scale,
+                                      const void* data_zp,
+                                      const float* filter_scale,
+                                      const void* filter_zp,
+                                      const float* out_scale,
+                                      const void* out_zp,
+                                      void* out)
+{
+    conv_dims_t c;
+    int rc = normalise_conv(d, &c);
+    if (rc)
+        return rc;
+    if (!conv_types_ok(d))
+        return HIPQ_ERR_UNSUPPORTED;
+    size_t total = (size_t)(c.N * c.K * c.out[0] * c.out[1] * c.out[2]);
+    int32_t* acc = (int32_t*)malloc(total * sizeof(int32_t));
+    if (!acc)
+        return HIPQ_ERR_LIMIT;
+    int32_t dzp = load_q(data_zp, d->data_t, 0);
+    int32_t fzp = load_q(filter_zp, d->filter_t, 0);
+    int32_t ozp = load_q(out_zp, d->out_t, 0);
+    orc_conv_accumulate(d, data, filter, dzp, fzp, acc);
+    float scale = *data_scale * *filter_scale / *out_scale; /* convolution.hpp:254 */
+    for (size_t i = 0; i < total; ++i)
+        store_q_wrap(out, d->out_t, i, requant_interp(acc[i], scale, ozp, d->out_t));
+    free(acc);
+    return HIPQ_OK;
+}
+
+/* QuantizedConvolutionBias / Relu / BiasAdd / BiasSignedAdd, oneDNN arithmetic.
+ * sum_in may alias out: every element is read before it is written. */
+ORC_API int orc_quantized_convolution_fused(const hipq_conv_desc_t* d,
+                                            const hipq_fused_desc_t* f,
+                                            const void* data,
+                                            const void* filter,
+                                            const int32_t* bias,
+                                            const void* sum_in,
+                                            const float* scale,
+                                            const float* sum_scale,
+                                            void* out)
+{
+    conv_dims_t c;
+    int rc = normalise_conv(d, &c);
+    if (rc)
+        return rc;
+    if (!f || !conv_types_ok(d) || d->filter_t != HIPQ_I8)
+        return HIPQ_ERR_UNSUPPORTED;
+    if (f->scale_count != 1 && f->scale_count != c.K)
+        return HIPQ_ERR_INVALID;
+    size_t total = (size_t)(c.N * c.K * c.out[0] * c.out[1] * c.out[2]);
+    size_t S = (size_t)(c.out[0] * c.out[1] * c.out[2]);
+    int32_t* acc = (int32_t*)malloc(total * sizeof(int32_t));
+    if (!acc)
+        return HIPQ_ERR_LIMIT;
+    orc_conv_accumulate(d, data, filter, 0, 0, acc);
+    float ss = f->has_sum ? *sum_scale : 0.0f;
+    for (size_t i = 0; i < total; ++i)
+    {
+        size_t k = (d->out_layout == HIPQ_LAYOUT_NXC) ? (i % (size_t)c.K) : ((i / S) % (size_t)c.K);
+        float sc = scale[f->scale_count == 1 ? 0 : k];
+        int32_t sv = f->has_sum ? load_q(sum_in, f->sum_t, i) : 0;
+        float v = fused_value(acc[i], f->has_bias, f->has_bias ? bias[k] : 0, sc, f->has_sum, ss, sv, f->with_relu);
+        store_q_wrap(out, d->out_t, i, saturate_rne(v, d->out_t));
+    }
+    free(acc);
+    return HIPQ_OK;
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Dot: dot.hpp:93-150 with reduction_axes_count = 1 (int_executable.hpp:1583)
+ * ------------------------------------------------------------------------------------------ */
+ORC_API int orc_dot_accumulate(
+    const hipq_dot_desc_t* d, const void* a, const void* b, int32_t a_zp, int32_t b_zp, int32_t* acc)
+{
+    if (!d || d->M < 0 || d->N < 0 || d->K < 0)
+        return HIPQ_ERR_INVALID;
+    long long m;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (m = 0; m < (long long)d->M; ++m)
+    {
+        for (int64_t n = 0; n < d->N; ++n)
+        {
+            int32_t s = 0;
+            for (int64_t k = 0; k < d->K; ++k)
+            {
+                size_t bi = (d->b_layout == HIPQ_B_NK) ? (size_t)(n * d->K + k) : (size_t)(k * d->N + n);
+                int32_t x = load_q(a, d->a_t, (size_t)(m * d->K + k)) - a_zp;
+                int32_t y = load_q(b, d->b_t, bi) - b_zp;
+                s = (int32_t)((uint32_t)s + (uint32_t)(x * y));
+            }
+            acc[m * d->N + n] = s;
+        }
+    }
+    return HIPQ_OK;
+}
+
+ORC_API int orc_quantized_dot(const hipq_dot_desc_t* d,
+                              const void* a,
+                              const void* b,
+                              const float* a_scale,
+                              const void* a_zp,
+                              const float* b_scale,
+                              const void* b_zp,
+                              const float* out_scale,
+                              const void* out_zp,
+                              void* out)
+{
+    if (!d)
+        return HIPQ_ERR_INVALID;
+    if ((d->a_t != HIPQ_U8 && d->a_t != HIPQ_I8) || (d->b_t != HIPQ_I8 && d->b_t != HIPQ_U8) ||
+        (d->out_t != HIPQ_I8 && d->out_t != HIPQ_U8 && d->out_t != HIPQ_I32))
+        return HIPQ_ERR_UNSUPPORTED;
+    size_t total = (size_t)(d->M * d->N);
+    int32_t* acc = (int32_t*)malloc((total ? total : 1) * sizeof(int32_t));
+    if (!acc)
+        return HIPQ_ERR_LIMIT;
+    int32_t azp = load_q(a_zp, d->a_t, 0);
+    int32_t bzp = load_q(b_zp, d->b_t, 0);
+    int32_t ozp = load_q(out_zp, d->out_t, 0);
+    orc_dot_accumulate(d, a, b, azp, bzp, acc);
+    float scale = *a_scale * *b_scale / *out_scale; /* dot.hpp:154 */
+    for (size_t i = 0; i < total; ++i)
+        store_q_wrap(out, d->out_t, i, requant_interp(acc[i], scale, ozp, d->out_t));
+    free(acc);
+    return HIPQ_OK;
+}
+
+/* op::v0::QuantizedDotBias: weights [N,K] (quantized_dot_bias.cpp:43-44), oneDNN inner product */
+ORC_API int orc_quantized_dot_bias(const hipq_dot_desc_t* d,
+                                   const hipq_fused_desc_t* f,
+                                   const void* a,
+                                   const void* w,
+                                   const int32_t* bias,
+                                   const float* scale,
+                                   void* out)
+{
+    if (!d || !f)
+        return HIPQ_ERR_INVALID;
+    if ((d->a_t != HIPQ_U8 && d->a_t != HIPQ_I8) || d->b_t != HIPQ_I8 || f->has_sum)
+        return HIPQ_ERR_UNSUPPORTED;
+    if (d->out_t != HIPQ_I8 && d->out_t != HIPQ_U8 && d->out_t != HIPQ_F32)
+        return HIPQ_ERR_UNSUPPORTED;
+    if (f->scale_count != 1 && f->scale_count != d->N)
+        return HIPQ_ERR_INVALID;
+    size_t total = (size_t)(d->M * d->N);
+    int32_t* acc = (int32_t*)malloc((total ? total : 1) * sizeof(int32_t));
+    if (!acc)
+        return HIPQ_ERR_LIMIT;
+    orc_dot_accumulate(d, a, w, 0, 0, acc);
+    for (size_t i = 0; i < total; ++i)
+    {
+        size_t n = i % (size_t)d->N;
+        float sc = scale[f->scale_count == 1 ? 0 : n];
+        float v = fused_value(acc[i], f->has_bias, f->has_bias ? bias[n] : 0, sc, 0, 0.0f, 0, f->with_relu);
+        if (d->out_t == HIPQ_F32)
+            ((float*)out)[i] = v;
+        else
+            store_q_wrap(out, d->out_t, i, saturate_rne(v, d->out_t));
+    }
+    free(acc);
+    return HIPQ_OK;
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Builder scale algebra: src/ngraph/builder/quantization_utils.cpp:33-174, evaluated in f32 the
+ * way the scale sub-graph (Abs / Maximum / Minimum / Add / Divide / Multiply on f32) evaluates.
+ * ------------------------------------------------------------------------------------------ */
+static float quant_range(int quant_t)
+{
+    /* quantization_utils.cpp:69-71 */
+    switch (quant_t)
+    {
+    case HIPQ_U8: return 255.0f;
+    case HIPQ_I8: return 127.0f;
+    default: return (float)2147483647.0; /* i32: 2^31-1 rounds to 2^31 in f32 */
+    }
+}
+
+ORC_API float orc_get_scale(float min_range, float max_range, int quant_t, int bump_by_eps)
+{
+    float mn = min_range, mx = max_range;
+    if (bump_by_eps) /* :52-66 */
+    {
+        mn = fminf(0.0f, min_range);
+        float max_abs_in = fmaxf(fabsf(min_range), fabsf(max_range));
+        float eps = fmaxf(1.0f, max_abs_in) / 100.0f;
+        mx = fmaxf(max_range, mn + eps);
+        mx = fmaxf(0.0f, mx);
+    }
+    return fmaxf(fabsf(mn), fabsf(mx)) / quant_range(quant_t);
+}
+
+ORC_API float orc_get_bias_scale(float min_in, float max_in, float min_f, float max_f)
+{
+    /* :81-109 */
+    return (fmaxf(fabsf(min_in), fabsf(max_in)) * fmaxf(fabsf(min_f), fabsf(max_f))) / (255.0f * 127.0f);
+}
+
+ORC_API float orc_get_sum_scale(float min_out, float max_out, float min_sum, float max_sum)
+{
+    /* :111-135 */
+    return fmaxf(fabsf(min_sum), fabsf(max_sum)) / fmaxf(fabsf(min_out), fabsf(max_out));
+}
+
+ORC_API float orc_get_dot_scale(float min_in,
+                                float max_in,
+                                float min_f,
+                                float max_f,
+                                float min_out,
+                                float max_out,
+                                int input_t,
+                                int output_t,
+                                int requantize)
+{
+    /* :137-174 */
+    float ds = orc_get_scale(min_in, max_in, input_t, 0);
+    float ws = orc_get_scale(min_f, max_f, HIPQ_I8, 0);
+    float os = orc_get_scale(min_out, max_out, output_t, 0);
+    return requantize ? ds * ws / os : ds * ws;
+}
+
+/* requantization scale of the fused convolution builders: input_scale * filter_scale / output_scale
+ * (src/ngraph/builder/quantized_conv_builder.cpp:100-106) */
+ORC_API float orc_get_conv_requant_scale(
+    float min_in, float max_in, int data_t, float min_f, float max_f, int filter_t, float min_out, float max_out, int out_t)
+{
+    float is = orc_get_scale(min_in, max_in, data_t, 0);
+    float fs = orc_get_scale(min_f, max_f, filter_t, 0);
+    float os = orc_get_scale(min_out, max_out, out_t, 0);
+    return is * fs / os;
+}
+
+ORC_API size_t orc_dtype_size(int t)
+{
+    return dtype_size(t);
+}

@@ -1,0 +1,244 @@
+"""ctypes access to the test oracle: oracle/libhipq_oracle.so (the C restatement) and, where it was
+built, oracle/_ref/libngraph_ref.so (the real nGraph reference kernels).
+
+Only tests, the smoke check and the benchmark's cpu_baseline leg import this module.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+from ngraph_amd import hipq as H
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PORT_PATH = os.path.join(ROOT, "oracle", "libhipq_oracle.so")
+REF_PATH = os.path.join(ROOT, "oracle", "_ref", "libngraph_ref.so")
+
+_port = None
+_ref = None
+
+
+def port():
+    global _port
+    if _port is None:
+        if not os.path.exists(PORT_PATH):
+            subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle"), "port"])
+        lib = C.CDLL(PORT_PATH)
+        vp = C.c_void_p
+        lib.orc_set_threads.argtypes = [C.c_int]
+        lib.orc_quantize.argtypes = [C.POINTER(H.QuantDesc), vp, vp, vp, vp]
+        lib.orc_dequantize.argtypes = [C.POINTER(H.QuantDesc), vp, vp, vp, vp]
+        lib.orc_conv_infer_output.argtypes = [C.POINTER(H.ConvDesc)]
+        lib.orc_conv_accumulate.argtypes = [C.POINTER(H.ConvDesc), vp, vp, C.c_int32, C.c_int32, vp]
+        lib.orc_quantized_convolution.argtypes = [C.POINTER(H.ConvDesc)] + [vp] * 9
+        lib.orc_quantized_convolution_fused.argtypes = [C.POINTER(H.ConvDesc), C.POINTER(H.FusedDesc)] + [vp] * 7
+        lib.orc_dot_accumulate.argtypes = [C.POINTER(H.DotDesc), vp, vp, C.c_int32, C.c_int32, vp]
+        lib.orc_quantized_dot.argtypes = [C.POINTER(H.DotDesc)] + [vp] * 9
+        lib.orc_quantized_dot_bias.argtypes = [C.POINTER(H.DotDesc), C.POINTER(H.FusedDesc)] + [vp] * 5
+        f = C.c_float
+        lib.orc_get_scale.restype = f
+        lib.orc_get_scale.argtypes = [f, f, C.c_int, C.c_int]
+        lib.orc_get_bias_scale.restype = f
+        lib.orc_get_bias_scale.argtypes = [f] * 4
+        lib.orc_get_sum_scale.restype = f
+        lib.orc_get_sum_scale.argtypes = [f] * 4
+        lib.orc_get_dot_scale.restype = f
+        lib.orc_get_dot_scale.argtypes = [f] * 6 + [C.c_int] * 3
+        lib.orc_get_conv_requant_scale.restype = f
+        lib.orc_get_conv_requant_scale.argtypes = [f, f, C.c_int, f, f, C.c_int, f, f, C.c_int]
+        _port = lib
+    return _port
+
+
+def have_ref() -> bool:
+    return os.path.exists(REF_PATH)
+
+
+def ref():
+    global _ref
+    if _ref is None:
+        lib = C.CDLL(REF_PATH)
+        vp, i64p = C.c_void_p, C.POINTER(C.c_int64)
+        lib.ref_quantized_convolution.argtypes = [C.c_int] + [i64p] * 8 + [C.c_int] * 3 + [vp] * 9
+        lib.ref_quantized_dot.argtypes = [C.c_int64] * 3 + [C.c_int] * 3 + [vp] * 9
+        lib.ref_quantize.argtypes = [C.c_int, i64p, C.c_uint32, C.c_int, C.c_int, C.c_int] + [vp] * 4
+        lib.ref_dequantize.argtypes = [C.c_int, i64p, C.c_uint32, C.c_int, C.c_int] + [vp] * 4
+        _ref = lib
+    return _ref
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data
+
+
+def _arr(x, dtype):
+    return np.ascontiguousarray(np.asarray(x, dtype=dtype))
+
+
+def _ok(rc):
+    if rc != 0:
+        raise RuntimeError(f"oracle returned status {rc}")
+
+
+# ------------------------------------------------------------------ C restatement
+
+
+def quantize(x, scale, zp, quant_t, axes=(), round_mode=H.RNE):
+    x = np.ascontiguousarray(x)
+    qt = H.dtype_code(quant_t)
+    d = H.make_quant_desc(x.shape, axes, x.dtype, qt, round_mode)
+    s, z = _arr(scale, x.dtype), _arr(zp, H.NP_OF[qt])
+    out = np.empty(x.shape, dtype=H.NP_OF[qt])
+    _ok(port().orc_quantize(C.byref(d), _ptr(x), _ptr(s), _ptr(z), _ptr(out)))
+    return out
+
+
+def dequantize(q, scale, zp, real_t=H.F32, axes=()):
+    q = np.ascontiguousarray(q)
+    rt = H.dtype_code(real_t)
+    d = H.make_quant_desc(q.shape, axes, rt, q.dtype)
+    s, z = _arr(scale, H.NP_OF[rt]), _arr(zp, q.dtype)
+    out = np.empty(q.shape, dtype=H.NP_OF[rt])
+    _ok(port().orc_dequantize(C.byref(d), _ptr(q), _ptr(s), _ptr(z), _ptr(out)))
+    return out
+
+
+def conv_accumulate(desc, data, filt, data_zp=0, filter_zp=0):
+    data, filt = np.ascontiguousarray(data), np.ascontiguousarray(filt)
+    out = np.empty(desc.out_shape(), dtype=np.int32)
+    _ok(port().orc_conv_accumulate(C.byref(desc), _ptr(data), _ptr(filt), int(data_zp), int(filter_zp), _ptr(out)))
+    return out
+
+
+def quantized_convolution(desc, data, filt, data_scale, data_zp, filter_scale, filter_zp, out_scale, out_zp):
+    data, filt = np.ascontiguousarray(data), np.ascontiguousarray(filt)
+    s = [_arr(v, np.float32) for v in (data_scale, filter_scale, out_scale)]
+    z = [_arr(data_zp, H.NP_OF[desc.data_t]), _arr(filter_zp, H.NP_OF[desc.filter_t]), _arr(out_zp, H.NP_OF[desc.out_t])]
+    out = np.empty(desc.out_shape(), dtype=H.NP_OF[desc.out_t])
+    _ok(
+        port().orc_quantized_convolution(
+            C.byref(desc), _ptr(data), _ptr(filt), _ptr(s[0]), _ptr(z[0]), _ptr(s[1]), _ptr(z[1]), _ptr(s[2]), _ptr(z[2]), _ptr(out)
+        )
+    )
+    return out
+
+
+def quantized_convolution_fused(desc, fused, data, filt, bias, sum_in, scale, sum_scale):
+    data, filt = np.ascontiguousarray(data), np.ascontiguousarray(filt)
+    b = None if bias is None else _arr(bias, np.int32)
+    sm = None if sum_in is None else np.ascontiguousarray(sum_in)
+    sc = _arr(scale, np.float32)
+    ss = None if sum_scale is None else _arr(sum_scale, np.float32)
+    out = np.empty(desc.out_shape(), dtype=H.NP_OF[desc.out_t])
+    _ok(
+        port().orc_quantized_convolution_fused(
+            C.byref(desc), C.byref(fused), _ptr(data), _ptr(filt), _ptr(b), _ptr(sm), _ptr(sc), _ptr(ss), _ptr(out)
+        )
+    )
+    return out
+
+
+def dot_accumulate(desc, a, b, a_zp=0, b_zp=0):
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    out = np.empty((int(desc.M), int(desc.N)), dtype=np.int32)
+    _ok(port().orc_dot_accumulate(C.byref(desc), _ptr(a), _ptr(b), int(a_zp), int(b_zp), _ptr(out)))
+    return out
+
+
+def quantized_dot(desc, a, b, a_scale, a_zp, b_scale, b_zp, out_scale, out_zp):
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    s = [_arr(v, np.float32) for v in (a_scale, b_scale, out_scale)]
+    z = [_arr(a_zp, H.NP_OF[desc.a_t]), _arr(b_zp, H.NP_OF[desc.b_t]), _arr(out_zp, H.NP_OF[desc.out_t])]
+    out = np.empty((int(desc.M), int(desc.N)), dtype=H.NP_OF[desc.out_t])
+    _ok(
+        port().orc_quantized_dot(
+            C.byref(desc), _ptr(a), _ptr(b), _ptr(s[0]), _ptr(z[0]), _ptr(s[1]), _ptr(z[1]), _ptr(s[2]), _ptr(z[2]), _ptr(out)
+        )
+    )
+    return out
+
+
+def quantized_dot_bias(desc, fused, a, w, bias, scale):
+    a, w = np.ascontiguousarray(a), np.ascontiguousarray(w)
+    b = None if bias is None else _arr(bias, np.int32)
+    sc = _arr(scale, np.float32)
+    out = np.empty((int(desc.M), int(desc.N)), dtype=H.NP_OF[desc.out_t])
+    _ok(port().orc_quantized_dot_bias(C.byref(desc), C.byref(fused), _ptr(a), _ptr(w), _ptr(b), _ptr(sc), _ptr(out)))
+    return out
+
+
+# ------------------------------------------------------------------ real reference (oracle/_ref)
+
+
+def _i64(v):
+    return (C.c_int64 * len(v))(*[int(x) for x in v])
+
+
+def ref_quantized_convolution(desc, data, filt, data_scale, data_zp, filter_scale, filter_zp, out_scale, out_zp):
+    """desc must use the reference's NCX layouts."""
+    assert desc.data_layout == H.NCX and desc.out_layout == H.NCX
+    ns = desc.n_spatial
+    data, filt = np.ascontiguousarray(data), np.ascontiguousarray(filt)
+    s = [_arr(v, np.float32) for v in (data_scale, filter_scale, out_scale)]
+    z = [_arr(data_zp, H.NP_OF[desc.data_t]), _arr(filter_zp, H.NP_OF[desc.filter_t]), _arr(out_zp, H.NP_OF[desc.out_t])]
+    out = np.empty(desc.out_shape(), dtype=H.NP_OF[desc.out_t])
+    rc = ref().ref_quantized_convolution(
+        ns,
+        _i64(desc.data_shape()),
+        _i64(desc.filter_shape()),
+        _i64(desc.out_shape()),
+        _i64(list(desc.stride)[:ns]),
+        _i64(list(desc.dilation)[:ns]),
+        _i64(list(desc.pad_below)[:ns]),
+        _i64(list(desc.pad_above)[:ns]),
+        _i64(list(desc.data_dilation)[:ns]),
+        desc.data_t,
+        desc.filter_t,
+        desc.out_t,
+        _ptr(data),
+        _ptr(filt),
+        _ptr(s[0]),
+        _ptr(z[0]),
+        _ptr(s[1]),
+        _ptr(z[1]),
+        _ptr(s[2]),
+        _ptr(z[2]),
+        _ptr(out),
+    )
+    _ok(rc)
+    return out
+
+
+def ref_quantized_dot(desc, a, b, a_scale, a_zp, b_scale, b_zp, out_scale, out_zp):
+    assert desc.b_layout == H.B_KN
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    s = [_arr(v, np.float32) for v in (a_scale, b_scale, out_scale)]
+    z = [_arr(a_zp, H.NP_OF[desc.a_t]), _arr(b_zp, H.NP_OF[desc.b_t]), _arr(out_zp, H.NP_OF[desc.out_t])]
+    out = np.empty((int(desc.M), int(desc.N)), dtype=H.NP_OF[desc.out_t])
+    rc = ref().ref_quantized_dot(
+        desc.M, desc.K, desc.N, desc.a_t, desc.b_t, desc.out_t, _ptr(a), _ptr(b), _ptr(s[0]), _ptr(z[0]), _ptr(s[1]), _ptr(z[1]), _ptr(s[2]), _ptr(z[2]), _ptr(out)
+    )
+    _ok(rc)
+    return out
+
+
+def ref_quantize(x, scale, zp, quant_t, axes=(), round_mode=H.RNE):
+    x = np.ascontiguousarray(x)
+    qt = H.dtype_code(quant_t)
+    s, z = _arr(scale, x.dtype), _arr(zp, H.NP_OF[qt])
+    out = np.empty(x.shape, dtype=H.NP_OF[qt])
+    mask = sum(1 << int(a) for a in axes)
+    rm = round_mode if isinstance(round_mode, int) else H.ROUND_MODES.index(round_mode)
+    _ok(ref().ref_quantize(x.ndim, _i64(x.shape), mask, H.dtype_code(x.dtype), qt, rm, _ptr(x), _ptr(s), _ptr(z), _ptr(out)))
+    return out
+
+
+def ref_dequantize(q, scale, zp, real_t=H.F32, axes=()):
+    q = np.ascontiguousarray(q)
+    rt = H.dtype_code(real_t)
+    s, z = _arr(scale, H.NP_OF[rt]), _arr(zp, q.dtype)
+    out = np.empty(q.shape, dtype=H.NP_OF[rt])
+    mask = sum(1 << int(a) for a in axes)
+    _ok(ref().ref_dequantize(q.ndim, _i64(q.shape), mask, rt, H.dtype_code(q.dtype), _ptr(q), _ptr(s), _ptr(z), _ptr(out)))
+    return out

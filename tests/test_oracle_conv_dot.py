@@ -1,0 +1,255 @@
+"""Pins orc_quantized_convolution / orc_quantized_dot and the fused (oneDNN-semantics) variants."""
+import numpy as np
+import pytest
+
+import cases
+import oracle_lib as O
+from ngraph_amd import hipq as H
+from ngraph_amd import synth
+
+
+def _scales_for(k, d, lib):
+    if k.get("via_builder"):
+        # QuantizedConvolutionBuilder: three get_scale() calls, zero points 0
+        # (src/ngraph/builder/quantized_conv_builder.cpp:46-57)
+        s = [
+            lib.orc_get_scale(k["in_range"][0], k["in_range"][1], d.data_t, 0),
+            lib.orc_get_scale(k["filter_range"][0], k["filter_range"][1], d.filter_t, 0),
+            lib.orc_get_scale(k["out_range"][0], k["out_range"][1], d.out_t, 0),
+        ]
+        return s, [0, 0, 0]
+    return k["scales"], k["zps"]
+
+
+def test_conv_kats(kats):
+    lib = O.port()
+    for k in kats["conv"]:
+        d, data, filt, exp = cases.kat_conv(k)
+        s, z = _scales_for(k, d, lib)
+        got = O.quantized_convolution(d, data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
+        if k.get("policy") == "dnnl":
+            # vector produced by the CPU backend's oneDNN path (round-half-even): the INTERPRETER
+            # arithmetic differs from it exactly at the .5 ties, and the fused entry point (no
+            # bias, no relu) reproduces it bit for bit
+            diff = np.flatnonzero(got.reshape(-1).astype(np.int64) != exp.astype(np.int64))
+            acc = O.conv_accumulate(H.make_conv_desc(1, 1, 1, (9, 9), (3, 3), pad_below=(1, 1), pad_above=(1, 1), out_t="i32"), data, filt)
+            ties = np.flatnonzero((acc.reshape(-1) % 16 == 8) & ((acc.reshape(-1) // 16) % 2 == 0))
+            assert diff.tolist() == ties.tolist() and len(ties) > 0
+            f = H.make_fused_desc(has_bias=False)
+            rs = np.float32(np.float32(s[0]) * np.float32(s[1])) / np.float32(s[2])
+            got = O.quantized_convolution_fused(d, f, data, filt, None, None, rs, None)
+        assert got.reshape(-1).astype(np.int64).tolist() == exp.astype(np.int64).tolist(), k["name"]
+
+
+@pytest.mark.skipif(not O.have_ref(), reason="oracle/_ref not built (reference tree absent)")
+def test_ref_build_conv_kats(kats):
+    lib = O.port()
+    for k in kats["conv"]:
+        d, data, filt, exp = cases.kat_conv(k)
+        s, z = _scales_for(k, d, lib)
+        if k.get("policy") == "dnnl":
+            continue
+        got = O.ref_quantized_convolution(d, data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
+        assert got.reshape(-1).astype(np.int64).tolist() == exp.astype(np.int64).tolist(), k["name"]
+
+
+def test_conv_reference_vectors(ref_vectors):
+    """compiled-reference outputs on seeded shapes: C1 (wrapping), strides, dilations, negative
+    pads, data dilation, 1-D / 3-D, non-zero zero points, all four type combinations"""
+    manifest, arrays = ref_vectors
+    n = 0
+    for m in manifest:
+        if m["kind"] != "conv":
+            continue
+        d, data, filt, s, z = cases.conv_from_manifest(m)
+        got = O.quantized_convolution(d, data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
+        assert np.array_equal(got, arrays[m["name"]]), m["name"]
+        n += 1
+    assert n >= 15
+
+
+def test_c1_wraps_like_the_reference(ref_vectors):
+    """BASELINE config 1: most outputs are out of int8 range and wrap mod 256 (no saturation)"""
+    manifest, arrays = ref_vectors
+    m = next(x for x in manifest if x["name"] == "c1")
+    d, data, filt, s, z = cases.conv_from_manifest(m)
+    di = H.make_conv_desc(1, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1), out_t="i32")
+    acc = O.conv_accumulate(di, data, filt)
+    scale = np.float32(np.float32(np.float32(0.02) * np.float32(0.005)) / np.float32(0.1))
+    v = np.round(acc.astype(np.float32) * scale)  # no ties at this config; checked below
+    frac = np.abs(acc.astype(np.float32) * scale - np.trunc(acc.astype(np.float32) * scale))
+    assert not np.any(frac == 0.5)
+    wrapped = v.astype(np.int64).astype(np.uint8).astype(np.int8)
+    assert np.array_equal(wrapped, arrays["c1"])
+    assert np.mean(np.abs(v) > 128) > 0.5
+
+
+def test_conv_accumulator_brute_force():
+    """independent numpy convolution (explicit pad / dilate / crop) on a shape grid"""
+    grid = [
+        dict(N=2, C=3, K=4, in_sp=(7, 6), f_sp=(3, 3), pad_below=(1, 1), pad_above=(1, 1)),
+        dict(N=1, C=5, K=2, in_sp=(9, 8), f_sp=(3, 2), stride=(2, 3), pad_below=(2, 0), pad_above=(0, 1)),
+        dict(N=1, C=2, K=3, in_sp=(8, 8), f_sp=(2, 3), dilation=(3, 2), pad_below=(1, 2), pad_above=(2, 1)),
+        dict(N=1, C=2, K=2, in_sp=(4, 5), f_sp=(3, 3), data_dilation=(2, 2), pad_below=(1, 1), pad_above=(1, 1)),
+        dict(N=1, C=2, K=2, in_sp=(9, 9), f_sp=(3, 3), pad_below=(-2, 1), pad_above=(1, -1), stride=(2, 1)),
+        dict(N=2, C=3, K=2, in_sp=(11,), f_sp=(4,), stride=(2,), pad_below=(3,), pad_above=(0,)),
+        dict(N=1, C=2, K=2, in_sp=(4, 5, 3), f_sp=(2, 2, 2), pad_below=(1, 0, 1), pad_above=(0, 1, 0), dilation=(1, 2, 1)),
+    ]
+    for i, g in enumerate(grid):
+        for (dt, ft, dzp, fzp) in (("u8", "i8", 0, 0), ("u8", "u8", 17, 201), ("u8", "i8", 128, -5)):
+            d = H.make_conv_desc(data_t=dt, filter_t=ft, out_t="i32", **{("C_" if k == "C" else k): v for k, v in g.items()})
+            data = synth.uniform_int(50 + i, d.data_shape(), 0, 255, np.uint8)
+            lo, hi = (-128, 127) if ft == "i8" else (0, 255)
+            filt = synth.uniform_int(70 + i, d.filter_shape(), lo, hi, H.NP_OF[d.filter_t])
+            got = O.conv_accumulate(d, data, filt, dzp, fzp)
+            exp = cases.brute_conv_acc(d, data, filt, dzp, fzp)
+            assert np.array_equal(got.astype(np.int64), exp), (i, dt, ft)
+
+
+def test_conv_layouts_agree():
+    """channels-last descriptors index the same tensor: NXC in/out == transposed NCX in/out"""
+    g = dict(N=2, C_=8, K=6, in_sp=(7, 5), f_sp=(3, 3), stride=(2, 1), pad_below=(1, 1), pad_above=(1, 1))
+    d0 = H.make_conv_desc(out_t="i8", **g)
+    d1 = H.make_conv_desc(out_t="i8", data_layout=H.NXC, out_layout=H.NXC, **g)
+    d2 = H.make_conv_desc(out_t="i8", data_layout=H.NXC, out_layout=H.NCX, **g)
+    data = synth.uniform_int(5, d0.data_shape(), 0, 255, np.uint8)
+    filt = synth.uniform_int(6, d0.filter_shape(), -127, 127, np.int8)
+    a = O.quantized_convolution(d0, data, filt, 0.02, 0, 0.005, 0, 0.3, 3)
+    b = O.quantized_convolution(d1, cases.to_nxc(data), filt, 0.02, 0, 0.005, 0, 0.3, 3)
+    c = O.quantized_convolution(d2, cases.to_nxc(data), filt, 0.02, 0, 0.005, 0, 0.3, 3)
+    assert np.array_equal(a, cases.to_ncx(b))
+    assert np.array_equal(a, c)
+
+
+def test_requant_interp_closed_form():
+    """half-away-from-zero + mod-256 wrap, independent of the C code: numpy on exact ties"""
+    d = H.make_dot_desc(1, 1, 9, a_t="u8", b_t="i8", out_t="i8")
+    a = np.uint8([[1]])
+    b = np.int8([[1, 3, 5, -1, -3, -5, 127, -127, 101]])
+    # scale 0.5 * 1 / 1: acc/2 -> .5 ties round away from zero
+    got = O.quantized_dot(d, a, b, 0.5, 0, 1.0, 0, 1.0, 0)
+    assert got.tolist() == [[1, 2, 3, -1, -2, -3, 64, -64, 51]]
+    # scale 100: 127*100 = 12700 -> 12700 mod 256 = 156 -> int8 -100 ; plus zero point 7
+    got = O.quantized_dot(d, a, b, 100.0, 0, 1.0, 0, 1.0, 7)
+    exp = ((b.astype(np.int64) * 100) & 0xFF).astype(np.uint8).astype(np.int8).astype(np.int64) + 7
+    exp = (exp & 0xFF).astype(np.uint8).astype(np.int8)
+    assert np.array_equal(got, exp)
+
+
+def test_dot_kats(kats):
+    for k in kats["dot"]:
+        M, K = k["a_shape"]
+        N = k["b_shape"][1]
+        d = H.make_dot_desc(M, K, N, a_t=k["a_t"], b_t=k["b_t"], out_t=k["out_t"])
+        a = np.array(k["a"], dtype=H.NP_OF[d.a_t]).reshape(M, K)
+        b = np.array(k["b"], dtype=H.NP_OF[d.b_t]).reshape(K, N)
+        s, z = k["scales"], k["zps"]
+        got = O.quantized_dot(d, a, b, s[0], z[0], s[1], z[1], s[2], z[2])
+        assert got.reshape(-1).tolist() == k["expected"], k["name"]
+        if O.have_ref():
+            got = O.ref_quantized_dot(d, a, b, s[0], z[0], s[1], z[1], s[2], z[2])
+            assert got.reshape(-1).tolist() == k["expected"], k["name"]
+
+
+def test_dot_reference_vectors(ref_vectors):
+    manifest, arrays = ref_vectors
+    n = 0
+    for m in manifest:
+        if m["kind"] != "dot":
+            continue
+        d, a, b, s, z = cases.dot_from_manifest(m)
+        got = O.quantized_dot(d, a, b, s[0], z[0], s[1], z[1], s[2], z[2])
+        assert np.array_equal(got, arrays[m["name"]]), m["name"]
+        n += 1
+    assert n >= 6
+
+
+def test_dot_accumulator_numpy():
+    a = synth.uniform_int(1, (7, 130), 0, 255, np.uint8)
+    b = synth.uniform_int(2, (130, 9), -128, 127, np.int8)
+    d = H.make_dot_desc(7, 130, 9, out_t="i32")
+    assert np.array_equal(O.dot_accumulate(d, a, b, 3, -4), (a.astype(np.int64) - 3) @ (b.astype(np.int64) + 4))
+    dn = H.make_dot_desc(7, 130, 9, out_t="i32", b_layout=H.B_NK)
+    assert np.array_equal(O.dot_accumulate(dn, a, np.ascontiguousarray(b.T)), a.astype(np.int64) @ b.astype(np.int64))
+
+
+# ---------------------------------------------------------------- fused (oneDNN semantics)
+
+
+def _fused_scales(k, lib, out_code):
+    rs = lib.orc_get_conv_requant_scale(
+        k["in_range"][0], k["in_range"][1], H.U8, k["filter_range"][0], k["filter_range"][1], H.I8, k["out_range"][0], k["out_range"][1], out_code
+    )
+    return rs
+
+
+def test_fused_conv_kats(kats):
+    """test/builder_quantization.cpp:51-677: RNE (78.5 -> 78, 114.5 -> 114), saturation
+    (134 -> 127), bias, sum post-op before ReLU, signed sum with doubled scale, f32 bias"""
+    lib = O.port()
+    for k in kats["fused_conv"]:
+        d, data, filt, exp = cases.kat_conv(k)
+        builder_out_t = H.U8 if k["with_relu"] else H.I8  # quantized_conv_builder.cpp:100,173,275
+        scale = _fused_scales(k, lib, builder_out_t)
+        bias = k.get("bias")
+        if "bias_f32" in k:  # builder quantizes an f32 bias with RNE at get_bias_scale (:111-123)
+            bs = lib.orc_get_bias_scale(k["in_range"][0], k["in_range"][1], k["filter_range"][0], k["filter_range"][1])
+            bias = O.quantize(np.float32(k["bias_f32"]), bs, 0, "i32", (), H.RNE).tolist()
+        has_sum = "sum" in k
+        sum_scale = None
+        sum_in = None
+        if has_sum:
+            sum_scale = lib.orc_get_sum_scale(k["out_range"][0], k["out_range"][1], k["sum_range"][0], k["sum_range"][1])
+            if k["op"] == "QuantizedConvolutionBiasSignedAdd" and builder_out_t == H.U8:
+                sum_scale = np.float32(2.0) * np.float32(sum_scale)  # :283-288
+            sum_in = np.array(k["sum"], dtype=H.NP_OF[H.dtype_code(k["sum_t"])]).reshape(d.out_shape())
+        f = H.make_fused_desc(has_bias=bias is not None, has_sum=has_sum, sum_t=k.get("sum_t", "u8"), with_relu=k["with_relu"])
+        got = O.quantized_convolution_fused(d, f, data, filt, bias, sum_in, scale, sum_scale)
+        if k["out_t"] == "u8_via_i8_convert":
+            got = got.astype(np.uint8)  # builder appends Convert(u8), :319
+        assert got.reshape(-1).astype(np.int64).tolist() == exp.tolist(), k["name"]
+
+
+def test_dot_bias_kat(kats):
+    """test/builder_quantization.cpp:995-1098: f32 output pins the float order scale*(acc+bias)"""
+    k = kats["dot_bias"]
+    lib = O.port()
+    M, K = k["a_shape"]
+    N = k["w_shape"][0]
+    a = np.array(k["a"], dtype=np.uint8).reshape(M, K)
+    w = np.array(k["w"], dtype=np.int8).reshape(N, K)
+    r = k["in_range"] + k["filter_range"] + k["out_range"]
+    for requant, relu, key, out_t in ((0, 0, "expected_f32", "f32"), (0, 1, "expected_f32_relu", "f32"), (1, 0, "expected_i8", "i8"), (1, 1, "expected_u8_relu", "u8")):
+        scale = lib.orc_get_dot_scale(*r, H.U8, H.U8 if relu else H.I8, requant)
+        d = H.make_dot_desc(M, K, N, out_t=out_t, b_layout=H.B_NK)
+        f = H.make_fused_desc(has_bias=True, with_relu=bool(relu))
+        got = O.quantized_dot_bias(d, f, a, w, k["bias"], scale)
+        exp = np.array(k[key], dtype=got.dtype).reshape(M, N)
+        assert np.array_equal(got, exp), key
+
+
+def test_fused_matches_decomposed_graph():
+    """the INTERPRETER-runnable decomposition: conv(i32, unit scales) -> +bias -> f32 -> *scale ->
+    [+ sum_scale*sum] -> [relu] -> Quantize(RNE) (whose clamp is the saturation); exact-arithmetic
+    region only (|acc+bias| < 2^24 and a sum term whose product is exact)"""
+    g = dict(N=1, C_=16, K=8, in_sp=(6, 6), f_sp=(3, 3), pad_below=(1, 1), pad_above=(1, 1))
+    di = H.make_conv_desc(out_t="i32", **g)
+    data = synth.uniform_int(11, di.data_shape(), 0, 255, np.uint8)
+    filt = synth.uniform_int(12, di.filter_shape(), -127, 127, np.int8)
+    bias = synth.uniform_int(13, (8,), -5000, 5000, np.int32)
+    scales = synth.uniform_f32(14, (8,), 1e-4, 2e-3)
+    acc = O.quantized_convolution(di, data, filt, 1.0, 0, 1.0, 0, 1.0, 0)
+    summ = synth.uniform_int(15, di.out_shape(), 0, 255, np.uint8)
+    for relu in (False, True):
+        for has_sum in (False, True):
+            out_t = "u8" if relu else "i8"
+            v = (acc + bias[None, :, None, None]).astype(np.float32) * scales[None, :, None, None]
+            if has_sum:
+                v = v + np.float32(0.5) * summ.astype(np.float32)  # 0.5*integer is exact: fma == mul+add
+            if relu:
+                v = np.maximum(v, np.float32(0))
+            exp = O.quantize(v.astype(np.float32), 1.0, 0, out_t, (), H.RNE)
+            d = H.make_conv_desc(out_t=out_t, **g)
+            f = H.make_fused_desc(has_bias=True, has_sum=has_sum, sum_t="u8", with_relu=relu, scale_count=8)
+            got = O.quantized_convolution_fused(d, f, data, filt, bias, summ if has_sum else None, scales, 0.5 if has_sum else None)
+            assert np.array_equal(got, exp), (relu, has_sum)

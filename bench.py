@@ -1,0 +1,251 @@
+#!/usr/bin/env python3
+"""Benchmark of the int8 hot path on one MI355X.
+
+Headline step: one op::v0::QuantizedConvolution call on the layer of BASELINE config 1
+(u8 [N,64,56,56] x i8 [64,64,3,3] -> i8, stride 1, pad 1) through the C ABI with the reference's
+NCHW tensors already resident in HBM, filter prepacked once (as a backend does at compile time).
+The batch defaults to 128, where a matrix-core fraction is meaningful; the N=1 and N=32 results
+of the same layer, the int8 GEMM of config 2 and the Quantize/Dequantize chain of config 3 are
+reported in the "results" object of the same JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch N] [--quick]
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+from ngraph_amd import hipq as H  # noqa: E402
+from ngraph_amd import synth  # noqa: E402
+
+PEAK_I8_TOPS = 5000.0  # MI355X dense int8 MFMA, published
+PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published
+
+
+class Timer:
+    """HIP events on the stream the kernels are launched on."""
+
+    def __init__(self, lib, stream):
+        self.lib, self.stream = lib, stream
+        self.a, self.b = C.c_void_p(), C.c_void_p()
+        H.check(lib.hipq_event_create(C.byref(self.a)))
+        H.check(lib.hipq_event_create(C.byref(self.b)))
+
+    def run(self, fn, steps, warmup):
+        """-> (wall ms per step, event ms per step)"""
+        for _ in range(warmup):
+            fn()
+        H.check(self.lib.hipq_stream_sync(self.stream))
+        H.check(self.lib.hipq_event_record(self.a, self.stream))
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        H.check(self.lib.hipq_event_record(self.b, self.stream))
+        H.check(self.lib.hipq_stream_sync(self.stream))
+        t1 = time.perf_counter()
+        ms = C.c_float()
+        H.check(self.lib.hipq_event_elapsed_ms(self.a, self.b, C.byref(ms)))
+        return (t1 - t0) * 1e3 / steps, ms.value / steps
+
+
+def dev(a):
+    return H.DeviceBuffer.from_numpy(np.ascontiguousarray(a))
+
+
+def scalar(v, dt):
+    return dev(np.asarray(v, dtype=dt))
+
+
+def bench_conv(lib, stream, timer, N, steps, warmup, layout):
+    d = H.make_conv_desc(N, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1), data_layout=layout, out_layout=layout)
+    one = H.make_conv_desc(1, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1), data_layout=layout, out_layout=layout)
+    img = synth.uniform_int(1001, one.data_shape(), 0, 255, np.uint8)
+    data = dev(np.ascontiguousarray(np.broadcast_to(img, d.data_shape())))
+    filt = dev(synth.uniform_int(1002, d.filter_shape(), -127, 127, np.int8))
+    packed = H.pack_filter(d, filt)
+    assert packed is not None
+    s = [scalar(v, np.float32) for v in (0.02, 0.005, 0.1)]
+    z = [scalar(0, np.uint8), scalar(0, np.int8), scalar(0, np.int8)]
+    out = H.DeviceBuffer(int(np.prod(d.out_shape())))
+
+    def step():
+        rc = lib.hipq_quantized_convolution(C.byref(d), data.ptr, filt.ptr, packed.ptr, s[0].ptr, z[0].ptr, s[1].ptr, z[1].ptr, s[2].ptr, z[2].ptr, out.ptr, stream)
+        if rc:
+            H.check(rc)
+
+    wall, ev = timer.run(step, steps, warmup)
+    kern = H.last_kernel()
+    ops = d.ops()
+    return dict(N=N, layout="NCHW" if layout == H.NCX else "NHWC", ops=ops, ms_wall=wall, ms_event=ev, tops=ops / (wall * 1e-3) / 1e12, tops_event=ops / (ev * 1e-3) / 1e12, kernel=kern)
+
+
+def bench_gemm(lib, stream, timer, M, steps, warmup):
+    K = N = 4096
+    d = H.make_dot_desc(M, K, N, out_t="i8", b_layout=H.B_NK)
+    f = H.make_fused_desc(has_bias=True, with_relu=False, scale_count=N)
+    a = dev(synth.uniform_int(2001, (M, K), 0, 255, np.uint8))
+    w = dev(synth.uniform_int(2002, (N, K), -127, 127, np.int8))
+    bias = dev(synth.uniform_int(2003, (N,), -(2**15), 2**15, np.int32))
+    scale = dev(synth.uniform_f32(2004, (N,), 0.001, 0.01))
+    packed = H.pack_dot(d, w)
+    out = H.DeviceBuffer(M * N)
+
+    def step():
+        rc = lib.hipq_quantized_dot_bias(C.byref(d), C.byref(f), a.ptr, w.ptr, packed.ptr, bias.ptr, scale.ptr, out.ptr, stream)
+        if rc:
+            H.check(rc)
+
+    wall, ev = timer.run(step, steps, warmup)
+    ops = 2 * M * K * N
+    nbytes = K * N + M * K + M * N + 4 * N + 4 * N
+    return dict(M=M, ops=ops, bytes=nbytes, ms_wall=wall, ms_event=ev, tops=ops / (ev * 1e-3) / 1e12, gbs=nbytes / (ev * 1e-3) / 1e9, kernel=H.last_kernel())
+
+
+def bench_qdq(lib, stream, timer, steps, warmup):
+    shape = (64, 1024, 1024)
+    n = int(np.prod(shape))
+    block = synth.normal_f32(3001, (4, 1024, 1024))
+    scale = (np.abs(block).max(axis=(0, 2)) / np.float32(127)).astype(np.float32)
+    bx = H.DeviceBuffer(n * 4)
+    for i in range(16):
+        H.check(lib.hipq_memcpy_h2d(bx.ptr + i * block.nbytes, block.ctypes.data, block.nbytes, None))
+    bs, bz = dev(scale), dev(np.zeros(1024, np.int8))
+    bq, bdq = H.DeviceBuffer(n), H.DeviceBuffer(n * 4)
+    d = H.make_quant_desc(shape, (1,), "f32", "i8")
+
+    def q():
+        rc = lib.hipq_quantize(C.byref(d), bx.ptr, bs.ptr, bz.ptr, bq.ptr, stream)
+        if rc:
+            H.check(rc)
+
+    def dq():
+        rc = lib.hipq_dequantize(C.byref(d), bq.ptr, bs.ptr, bz.ptr, bdq.ptr, stream)
+        if rc:
+            H.check(rc)
+
+    _, evq = timer.run(q, steps, warmup)
+    kq = H.last_kernel()
+    _, evd = timer.run(dq, steps, warmup)
+    kd = H.last_kernel()
+    nbytes = 5 * n
+    return dict(
+        elements=n,
+        quantize=dict(ms_event=evq, gbs=nbytes / (evq * 1e-3) / 1e9, frac_hbm=nbytes / (evq * 1e-3) / 1e9 / PEAK_HBM_GBS, kernel=kq),
+        dequantize=dict(ms_event=evd, gbs=nbytes / (evd * 1e-3) / 1e9, frac_hbm=nbytes / (evd * 1e-3) / 1e9 / PEAK_HBM_GBS, kernel=kd),
+    )
+
+
+def cpu_baseline(seconds=12.0):
+    """The reference's own convolution kernel (oracle/_ref, compiled from the nGraph tree) when it
+    was built, else the C restatement; BASELINE config 1 at N=1 on one host core."""
+    import oracle_lib as O
+
+    d = H.make_conv_desc(1, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1))
+    data = synth.uniform_int(1001, d.data_shape(), 0, 255, np.uint8)
+    filt = synth.uniform_int(1002, d.filter_shape(), -127, 127, np.int8)
+    kind = "reference" if O.have_ref() else "port"
+    fn = O.ref_quantized_convolution if kind == "reference" else O.quantized_convolution
+    O.port().orc_set_threads(1)
+    calls, t0 = 0, time.perf_counter()
+    while True:
+        fn(d, data, filt, 0.02, 0, 0.005, 0, 0.1, 0)
+        calls += 1
+        el = time.perf_counter() - t0
+        if el >= seconds or calls >= 200:
+            break
+    return dict(
+        value=d.ops() * calls / el / 1e12,
+        unit="TOP/s",
+        cores=1,
+        kind=kind,
+        sample="%d calls of QuantizedConvolution u8[1,64,56,56] x i8[64,64,3,3] -> i8 (config 1, N=1), %.1f s, %s"
+        % (calls, el, "runtime::reference::convolution compiled from the nGraph tree" if kind == "reference" else "C restatement of it"),
+    )
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--batch", type=int, default=128)
+    ap.add_argument("--quick", action="store_true", help="headline workload only, no CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    lib = H.load()
+    H.check(lib.hipq_set_device(0))
+    info = H.DeviceInfo()
+    H.check(lib.hipq_get_device_info(C.byref(info)))
+    sp = C.c_void_p()
+    H.check(lib.hipq_stream_create(C.byref(sp)))
+    stream = sp.value
+    timer = Timer(lib, stream)
+
+    # headline: the reference's NCHW tensors in, NCHW out
+    head = bench_conv(lib, stream, timer, args.batch, args.steps, args.warmup, H.NCX)
+    # dominant kernel alone (channels-last in and out: the call launches only the MFMA kernel)
+    kern = bench_conv(lib, stream, timer, args.batch, args.steps, args.warmup, H.NXC)
+
+    results = {"conv_nchw": [head], "conv_nhwc_kernel": [kern]}
+    cpu = None
+    if not args.quick:
+        small = max(20, args.steps // 4)
+        for n in (1, 32):
+            results["conv_nchw"].append(bench_conv(lib, stream, timer, n, args.steps, args.warmup, H.NCX))
+            results["conv_nhwc_kernel"].append(bench_conv(lib, stream, timer, n, args.steps, args.warmup, H.NXC))
+        results["gemm_config2"] = [bench_gemm(lib, stream, timer, m, small, 5) for m in (1, 32, 256)]
+        results["quantize_dequantize_config3"] = bench_qdq(lib, stream, timer, small, 5)
+        cpu = cpu_baseline()
+
+    derived_peak = info.compute_units * info.clock_mhz * 1e6 * 8192 / 1e12
+    line = {
+        "metric": "QuantizedConvolution int8 TOPS",
+        "value": head["tops"],
+        "unit": "TOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_wall"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "i8",
+        "data": "synthetic",
+        "config": {
+            "workload": "op::v0::QuantizedConvolution u8[%d,64,56,56] x i8[64,64,3,3] -> i8, stride 1, pad 1 (BASELINE config 1 layer at batch %d), NCHW in / NCHW out through the C ABI, filter prepacked"
+            % (args.batch, args.batch),
+            "ops_per_step": head["ops"],
+            "device": info.name.decode(),
+            "compute_units": info.compute_units,
+            "clock_mhz": info.clock_mhz,
+            "derived_i8_peak_tops": derived_peak,
+        },
+        "roofline": {
+            "bound": "mfma",
+            "kernel": kern["kernel"],
+            "achieved": kern["tops_event"],
+            "peak": PEAK_I8_TOPS,
+            "unit": "TOP/s",
+            "frac": kern["tops_event"] / PEAK_I8_TOPS,
+            "traffic": None,
+            "kernel_ms": kern["ms_event"],
+        },
+        "cpu_baseline": cpu,
+        "results": results,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -181,7 +181,10 @@ HIPQ_API int hipq_conv_infer_output(hipq_conv_desc_t* desc);
  * Prepacked filter for the MFMA path.  hipq_conv_packed_filter_bytes returns 0 when the shape /
  * type combination is not eligible for that path (the call then runs on the direct kernel and
  * `packed` may be NULL).  The packed blob holds the filter reordered to K,spatial,C plus a
- * per-output-channel table of 128*sum(filter) used to run u8 data on the signed i8 MFMA.
+ * per-output-channel table of sum(filter) used to run u8 data on the signed i8 MFMA.
+ * Pass the blob to a convolution call only when the filter zero point is zero (the nGraph CPU
+ * backend makes the same demand of its fast path, src/ngraph/runtime/cpu/pass/cpu_assignment.cpp:
+ * 801-825); a non-zero one is still computed correctly, by a slow in-kernel path.
  */
 HIPQ_API size_t hipq_conv_packed_filter_bytes(const hipq_conv_desc_t* desc);
 HIPQ_API int hipq_conv_pack_filter(const hipq_conv_desc_t* desc,
@@ -262,11 +265,15 @@ typedef struct hipq_dot_desc
 } hipq_dot_desc_t;
 
 /*
- * Optional per-weight-matrix table for the MFMA path: int32[N] holding 128*sum_k(b[k,n]).
- * hipq_dot_prepare computes it on the device; pass it as `bsum` (NULL = compute per call into an
- * internal workspace).
+ * Prepacked second operand for the MFMA path.  hipq_dot_packed_bytes returns 0 when the shape /
+ * type combination is not eligible for that path.  The blob holds the operand as [N,K] (a
+ * transposed copy for HIPQ_B_KN, nothing for HIPQ_B_NK, which is used in place) followed by a
+ * table int32[N] of sum_k(b[k,n]) used to run u8 activations on the signed i8 MFMA.  Passing
+ * NULL for `packed_b` makes the call build the same data in an internal workspace every time.
+ * Like the packed filter, it is only valid while the second operand's zero point is zero.
  */
-HIPQ_API int hipq_dot_prepare(const hipq_dot_desc_t* desc, const void* b, int32_t* bsum, void* stream);
+HIPQ_API size_t hipq_dot_packed_bytes(const hipq_dot_desc_t* desc);
+HIPQ_API int hipq_dot_pack(const hipq_dot_desc_t* desc, const void* b, void* packed, void* stream);
 
 /*
  * op::v0::QuantizedDot with one reduction axis.  Replaces runtime::reference::dot<IN0,IN1,OUT,int32_t>
@@ -276,7 +283,7 @@ HIPQ_API int hipq_dot_prepare(const hipq_dot_desc_t* desc, const void* b, int32_
 HIPQ_API int hipq_quantized_dot(const hipq_dot_desc_t* desc,
                                 const void* a,
                                 const void* b,
-                                const int32_t* bsum, /* may be NULL */
+                                const void* packed_b, /* may be NULL */
                                 const float* a_scale,
                                 const void* a_zp,
                                 const float* b_scale,
@@ -297,7 +304,7 @@ HIPQ_API int hipq_quantized_dot_bias(const hipq_dot_desc_t* desc,
                                      const hipq_fused_desc_t* fused,
                                      const void* a,
                                      const void* w,
-                                     const int32_t* wsum, /* may be NULL */
+                                     const void* packed_w, /* may be NULL */
                                      const int32_t* bias,
                                      const float* scale,
                                      void* out,

@@ -1,0 +1,232 @@
+// Internal declarations shared by the translation units of libhipq.so.  gfx950 only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/hipq.h"
+
+namespace hipq
+{
+    // ---- host-side error plumbing ------------------------------------------------------------
+    int fail(int code, const char* fmt, ...);
+    void set_last_kernel(const char* name);
+
+#define HIPQ_HIP(call)                                                                             \
+    do                                                                                             \
+    {                                                                                              \
+        hipError_t e_ = (call);                                                                    \
+        if (e_ != hipSuccess)                                                                      \
+            return ::hipq::fail(HIPQ_ERR_HIP, "%s failed: %s", #call, hipGetErrorString(e_));      \
+    } while (0)
+
+#define HIPQ_REQUIRE(cond, ...)                                                                    \
+    do                                                                                             \
+    {                                                                                              \
+        if (!(cond))                                                                               \
+            return ::hipq::fail(HIPQ_ERR_INVALID, __VA_ARGS__);                                    \
+    } while (0)
+
+    inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+    int check_launch(const char* kernel);
+
+    // Grow-only device workspace, one per device, shared by every call on that device (calls that
+    // need it and overlap on different streams would race; the backend serialises per executable).
+    int workspace(size_t bytes, void** ptr);
+
+    inline size_t dtype_size(int t)
+    {
+        switch (t)
+        {
+        case HIPQ_U8:
+        case HIPQ_I8: return 1;
+        case HIPQ_I32:
+        case HIPQ_F32: return 4;
+        case HIPQ_F64: return 8;
+        default: return 0;
+        }
+    }
+
+    inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+    // ---- convolution geometry normalised to three spatial dims ------------------------------------
+    struct ConvGeom
+    {
+        int64_t N, C, K;
+        int64_t in[3], f[3], out[3], st[3], dl[3], dd[3], pb[3];
+        int data_t, filter_t, out_t, data_layout, out_layout;
+        __host__ __device__ int64_t out_count() const { return N * K * out[0] * out[1] * out[2]; }
+        __host__ __device__ int64_t in_count() const { return N * C * in[0] * in[1] * in[2]; }
+        __host__ __device__ int64_t taps() const { return f[0] * f[1] * f[2]; }
+    };
+    int make_geom(const hipq_conv_desc_t* d, ConvGeom* g);
+
+    // ---- requantization epilogue, passed to kernels by value ----------------------------------
+    enum
+    {
+        EPI_INTERP = 0, // INTERPRETER: half away from zero, narrowing wraps
+        EPI_FUSED = 1   // oneDNN: bias, scale, sum, relu, half to even, saturate
+    };
+
+    struct Epilogue
+    {
+        int mode;
+        int out_t;
+        // EPI_INTERP: device scalars; scale = (*s_data * *s_filter) / *s_out
+        const float* s_data;
+        const float* s_filter;
+        const float* s_out;
+        const void* out_zp;
+        // EPI_FUSED
+        const int32_t* bias; // may be null
+        const float* scale;  // [scale_count]
+        const float* sum_scale;
+        const void* sum_in; // may be null; indexed like out
+        int sum_t;
+        int relu;
+        int per_channel; // scale_count > 1
+    };
+
+    // zero points of the accumulation, device scalars typed like their tensors (null = 0)
+    struct ZeroPoints
+    {
+        const void* data_zp;
+        const void* filter_zp;
+        int data_t;
+        int filter_t;
+    };
+
+#if defined(__HIPCC__)
+    __device__ __forceinline__ int32_t load_q(const void* p, int t, size_t i)
+    {
+        switch (t)
+        {
+        case HIPQ_U8: return static_cast<const uint8_t*>(p)[i];
+        case HIPQ_I8: return static_cast<const int8_t*>(p)[i];
+        default: return static_cast<const int32_t*>(p)[i];
+        }
+    }
+
+    __device__ __forceinline__ int32_t load_zp(const void* p, int t)
+    {
+        return p ? load_q(p, t, 0) : 0;
+    }
+
+    // float -> int32 the way x86 cvttss2si does it: NaN and out-of-range give INT32_MIN
+    __device__ __forceinline__ int32_t cvtt_x86(float v)
+    {
+        if (!(v < 2147483648.0f) || v < -2147483648.0f)
+            return INT32_MIN;
+        return static_cast<int32_t>(v);
+    }
+
+    // Resolved per-thread view of an Epilogue (scalars loaded once).
+    struct EpiRegs
+    {
+        float scale;     // interp scale, or fused scalar scale
+        float sum_scale; // fused
+        int32_t ozp;     // interp
+    };
+
+    __device__ __forceinline__ EpiRegs epi_load(const Epilogue& e)
+    {
+        EpiRegs r;
+        r.sum_scale = 0.0f;
+        r.ozp = 0;
+        if (e.mode == EPI_INTERP)
+        {
+            // src/ngraph/runtime/reference/convolution.hpp:254 : two f32 roundings, this order
+            r.scale = __fdiv_rn(__fmul_rn(*e.s_data, *e.s_filter), *e.s_out);
+            r.ozp = load_zp(e.out_zp, e.out_t);
+        }
+        else
+        {
+            r.scale = e.scale[0];
+            if (e.sum_in)
+                r.sum_scale = *e.sum_scale;
+        }
+        return r;
+    }
+
+    // acc -> output value as int32 bits (for F32 outputs: the float's bit pattern).
+    // k = output channel (bias / per-channel scale index), idx = flat output index (sum_in index).
+    __device__ __forceinline__ int32_t epi_apply(const Epilogue& e, const EpiRegs& r, int32_t acc, int64_t k, int64_t idx)
+    {
+        if (e.mode == EPI_INTERP)
+        {
+            float v = roundf(__fmul_rn(static_cast<float>(acc), r.scale));
+            int32_t t = cvtt_x86(v);
+            if (e.out_t == HIPQ_U8)
+                t = t & 0xFF;
+            else if (e.out_t == HIPQ_I8)
+                t = static_cast<int8_t>(t);
+            return static_cast<int32_t>(static_cast<uint32_t>(t) + static_cast<uint32_t>(r.ozp));
+        }
+        float v = static_cast<float>(acc);
+        if (e.bias)
+            v = __fadd_rn(v, static_cast<float>(e.bias[k]));
+        v = __fmul_rn(v, e.per_channel ? e.scale[k] : r.scale);
+        if (e.sum_in)
+            v = fmaf(r.sum_scale, static_cast<float>(load_q(e.sum_in, e.sum_t, idx)), v);
+        if (e.relu)
+            v = (v > 0.0f) ? v : __fmul_rn(v, -0.0f);
+        if (e.out_t == HIPQ_F32)
+            return __float_as_int(v);
+        float lo = (e.out_t == HIPQ_U8) ? 0.0f : (e.out_t == HIPQ_I8 ? -128.0f : -2147483648.0f);
+        float hi = (e.out_t == HIPQ_U8) ? 255.0f : (e.out_t == HIPQ_I8 ? 127.0f : 2147483520.0f);
+        v = (v < lo) ? lo : v;
+        v = (hi < v) ? hi : v;
+        return static_cast<int32_t>(rintf(v));
+    }
+
+    __device__ __forceinline__ void store_out(void* out, int out_t, int64_t idx, int32_t v)
+    {
+        if (out_t == HIPQ_U8 || out_t == HIPQ_I8)
+            static_cast<uint8_t*>(out)[idx] = static_cast<uint8_t>(v);
+        else
+            static_cast<int32_t*>(out)[idx] = v;
+    }
+#endif
+
+    // ---- launchers implemented in the kernel translation units (host side) ------------------
+    int launch_conv_direct(const ConvGeom& g,
+                           const void* data,
+                           const void* filter,
+                           const ZeroPoints& zp,
+                           const Epilogue& epi,
+                           void* out,
+                           hipStream_t s);
+    int launch_dot_direct(const hipq_dot_desc_t& d,
+                          const void* a,
+                          const void* b,
+                          const ZeroPoints& zp,
+                          const Epilogue& epi,
+                          void* out,
+                          hipStream_t s);
+
+    // MFMA implicit-GEMM convolution on channels-last data (both data and out NXC).
+    bool conv_mfma_eligible(const ConvGeom& g);
+    int launch_conv_mfma(const ConvGeom& g,
+                         const void* data_nxc,
+                         const void* packed,
+                         const ZeroPoints& zp,
+                         const Epilogue& epi,
+                         void* out_nxc,
+                         hipStream_t s);
+    bool dot_mfma_eligible(const hipq_dot_desc_t& d);
+    int launch_dot_mfma(const hipq_dot_desc_t& d,
+                        const void* a,
+                        const void* w_nk,      // [N,K] weights
+                        const int32_t* wsum,   // [N]
+                        const ZeroPoints& zp,
+                        const Epilogue& epi,
+                        void* out,
+                        hipStream_t s);
+
+    int launch_transpose(const void* in, void* out, int64_t N, int64_t R, int64_t Cc, int elem_bytes, hipStream_t s);
+    int launch_row_sums_i8(const void* w, int64_t rows, int64_t cols, int32_t* sums, hipStream_t s);
+}

@@ -1,0 +1,326 @@
+// Entry points of the quantized convolution / dot family: argument checks, choice between the
+// MFMA kernels and the direct kernels, layout conversion through the device workspace.
+#include "hipq_common.h"
+
+namespace hipq
+{
+    static bool is_quant8(int t) { return t == HIPQ_U8 || t == HIPQ_I8; }
+
+    static int check_conv_types(const ConvGeom& g, bool fused)
+    {
+        // INTERPRETER combinations: int_executable.hpp:1461-1549 (data is u8 there); i8 data is
+        // accepted as well because the oneDNN-backed fused ops take it.
+        if (!is_quant8(g.data_t) || !is_quant8(g.filter_t))
+            return fail(HIPQ_ERR_UNSUPPORTED, "data and filter must be u8 or i8");
+        if (!is_quant8(g.out_t) && g.out_t != HIPQ_I32)
+            return fail(HIPQ_ERR_UNSUPPORTED, "convolution output must be i8, u8 or i32");
+        if (fused && g.filter_t != HIPQ_I8)
+            return fail(HIPQ_ERR_UNSUPPORTED, "fused convolutions take i8 filters");
+        return HIPQ_OK;
+    }
+
+    // Runs the convolution with whatever layouts the descriptor names.
+    static int run_conv(const ConvGeom& g,
+                        const void* data,
+                        const void* filter,
+                        const void* packed,
+                        const ZeroPoints& zp,
+                        Epilogue epi,
+                        void* out,
+                        hipStream_t s)
+    {
+        if (!packed || !conv_mfma_eligible(g))
+            return launch_conv_direct(g, data, filter, zp, epi, out, s);
+
+        const size_t out_eb = dtype_size(g.out_t);
+        const int64_t in_sp = g.in[1] * g.in[2], out_sp = g.out[1] * g.out[2];
+        const size_t in_bytes = align_up(static_cast<size_t>(g.in_count()), 256);
+        const size_t out_bytes = align_up(static_cast<size_t>(g.out_count()) * out_eb, 256);
+        const size_t sum_bytes = epi.sum_in ? align_up(static_cast<size_t>(g.out_count()), 256) : 0;
+        const bool tr_in = g.data_layout == HIPQ_LAYOUT_NCX && g.C > 1;
+        const bool tr_out = g.out_layout == HIPQ_LAYOUT_NCX && g.K > 1;
+        const void* x = data;
+        void* y = out;
+        if (tr_in || tr_out)
+        {
+            uint8_t* ws = nullptr;
+            size_t need = (tr_in ? in_bytes : 0) + (tr_out ? out_bytes + sum_bytes : 0);
+            int rc = workspace(need, reinterpret_cast<void**>(&ws));
+            if (rc)
+                return rc;
+            if (tr_in)
+            {
+                rc = launch_transpose(data, ws, g.N, g.C, in_sp, 1, s);
+                if (rc)
+                    return rc;
+                x = ws;
+                ws += in_bytes;
+            }
+            if (tr_out)
+            {
+                y = ws;
+                ws += out_bytes;
+                if (epi.sum_in)
+                {
+                    rc = launch_transpose(epi.sum_in, ws, g.N, g.K, out_sp, 1, s);
+                    if (rc)
+                        return rc;
+                    epi.sum_in = ws;
+                }
+            }
+        }
+        int rc = launch_conv_mfma(g, x, packed, zp, epi, y, s);
+        if (rc)
+            return rc;
+        if (tr_out)
+        {
+            rc = launch_transpose(y, out, g.N, out_sp, g.K, static_cast<int>(out_eb), s);
+            if (rc)
+                return rc;
+            set_last_kernel("conv_mfma_i8_32x32x32");
+        }
+        return HIPQ_OK;
+    }
+
+    static int fused_epilogue(const hipq_fused_desc_t* f,
+                              int out_t,
+                              int64_t channels,
+                              const int32_t* bias,
+                              const void* sum_in,
+                              const float* scale,
+                              const float* sum_scale,
+                              Epilogue* e)
+    {
+        HIPQ_REQUIRE(f, "fused descriptor is null");
+        HIPQ_REQUIRE(scale, "scale is null");
+        HIPQ_REQUIRE(f->scale_count == 1 || f->scale_count == channels,
+                     "scale_count %lld is neither 1 nor the channel count %lld",
+                     (long long)f->scale_count,
+                     (long long)channels);
+        HIPQ_REQUIRE(!f->has_bias || bias, "has_bias set but bias is null");
+        HIPQ_REQUIRE(!f->has_sum || (sum_in && sum_scale), "has_sum set but sum_in / sum_scale is null");
+        if (f->has_sum && !is_quant8(f->sum_t))
+            return fail(HIPQ_ERR_UNSUPPORTED, "sum input must be u8 or i8");
+        memset(e, 0, sizeof(*e));
+        e->mode = EPI_FUSED;
+        e->out_t = out_t;
+        e->bias = f->has_bias ? bias : nullptr;
+        e->scale = scale;
+        e->per_channel = f->scale_count > 1;
+        e->sum_in = f->has_sum ? sum_in : nullptr;
+        e->sum_scale = f->has_sum ? sum_scale : nullptr;
+        e->sum_t = f->sum_t;
+        e->relu = f->with_relu;
+        return HIPQ_OK;
+    }
+
+    // weights [N,K] + column sums for the MFMA dot, either prepacked or built in the workspace
+    static int dot_operands(const hipq_dot_desc_t& d, const void* b, const void* packed, const void** w, const int32_t** wsum, hipStream_t s)
+    {
+        const size_t wbytes = d.b_layout == HIPQ_B_KN ? align_up(static_cast<size_t>(d.N * d.K), 256) : 0;
+        const uint8_t* blob = static_cast<const uint8_t*>(packed);
+        if (!blob)
+        {
+            uint8_t* ws = nullptr;
+            int rc = workspace(wbytes + static_cast<size_t>(d.N) * sizeof(int32_t), reinterpret_cast<void**>(&ws));
+            if (rc)
+                return rc;
+            rc = hipq_dot_pack(&d, b, ws, s);
+            if (rc)
+                return rc;
+            blob = ws;
+        }
+        *w = d.b_layout == HIPQ_B_KN ? static_cast<const void*>(blob) : b;
+        *wsum = reinterpret_cast<const int32_t*>(blob + wbytes);
+        return HIPQ_OK;
+    }
+
+    static int run_dot(const hipq_dot_desc_t& d,
+                       const void* a,
+                       const void* b,
+                       const void* packed,
+                       const ZeroPoints& zp,
+                       const Epilogue& epi,
+                       void* out,
+                       hipStream_t s)
+    {
+        if (d.M == 0 || d.N == 0)
+            return HIPQ_OK;
+        HIPQ_REQUIRE(out && (d.K == 0 || (a && b)), "null tensor pointer");
+        if (!dot_mfma_eligible(d) || (reinterpret_cast<uintptr_t>(a) & 15) || (reinterpret_cast<uintptr_t>(b) & 15) ||
+            (reinterpret_cast<uintptr_t>(out) & 15))
+            return launch_dot_direct(d, a, b, zp, epi, out, s);
+        const void* w = nullptr;
+        const int32_t* wsum = nullptr;
+        int rc = dot_operands(d, b, packed, &w, &wsum, s);
+        if (rc)
+            return rc;
+        return launch_dot_mfma(d, a, w, wsum, zp, epi, out, s);
+    }
+}
+
+using namespace hipq;
+
+extern "C" {
+
+int hipq_conv_infer_output(hipq_conv_desc_t* d)
+{
+    HIPQ_REQUIRE(d, "descriptor is null");
+    HIPQ_REQUIRE(d->n_spatial >= 1 && d->n_spatial <= HIPQ_MAX_SPATIAL, "n_spatial %d out of range", d->n_spatial);
+    for (int i = 0; i < d->n_spatial; ++i)
+    {
+        HIPQ_REQUIRE(d->in_sp[i] >= 1 && d->f_sp[i] >= 1 && d->stride[i] >= 1 && d->dilation[i] >= 1 && d->data_dilation[i] >= 1,
+                     "non-positive extent, stride or dilation on spatial axis %d", i);
+        int64_t in_eff = (d->in_sp[i] - 1) * d->data_dilation[i] + 1 + d->pad_below[i] + d->pad_above[i];
+        int64_t f_eff = (d->f_sp[i] - 1) * d->dilation[i] + 1;
+        HIPQ_REQUIRE(in_eff >= f_eff, "window larger than padded data on spatial axis %d", i);
+        d->out_sp[i] = (in_eff - f_eff) / d->stride[i] + 1;
+    }
+    return HIPQ_OK;
+}
+
+int hipq_quantized_convolution(const hipq_conv_desc_t* desc,
+                               const void* data,
+                               const void* filter,
+                               const void* packed_filter,
+                               const float* data_scale,
+                               const void* data_zp,
+                               const float* filter_scale,
+                               const void* filter_zp,
+                               const float* out_scale,
+                               const void* out_zp,
+                               void* out,
+                               void* stream)
+{
+    ConvGeom g;
+    int rc = make_geom(desc, &g);
+    if (rc)
+        return rc;
+    rc = check_conv_types(g, false);
+    if (rc)
+        return rc;
+    HIPQ_REQUIRE(data && filter && out, "null tensor pointer");
+    HIPQ_REQUIRE(data_scale && data_zp && filter_scale && filter_zp && out_scale && out_zp, "null scale or zero point");
+    Epilogue e;
+    memset(&e, 0, sizeof(e));
+    e.mode = EPI_INTERP;
+    e.out_t = g.out_t;
+    e.s_data = data_scale;
+    e.s_filter = filter_scale;
+    e.s_out = out_scale;
+    e.out_zp = out_zp;
+    ZeroPoints zp{data_zp, filter_zp, g.data_t, g.filter_t};
+    return run_conv(g, data, filter, packed_filter, zp, e, out, as_stream(stream));
+}
+
+int hipq_quantized_convolution_fused(const hipq_conv_desc_t* desc,
+                                     const hipq_fused_desc_t* fused,
+                                     const void* data,
+                                     const void* filter,
+                                     const void* packed_filter,
+                                     const int32_t* bias,
+                                     const void* sum_in,
+                                     const float* scale,
+                                     const float* sum_scale,
+                                     void* out,
+                                     void* stream)
+{
+    ConvGeom g;
+    int rc = make_geom(desc, &g);
+    if (rc)
+        return rc;
+    rc = check_conv_types(g, true);
+    if (rc)
+        return rc;
+    HIPQ_REQUIRE(data && filter && out, "null tensor pointer");
+    Epilogue e;
+    rc = fused_epilogue(fused, g.out_t, g.K, bias, sum_in, scale, sum_scale, &e);
+    if (rc)
+        return rc;
+    ZeroPoints zp{nullptr, nullptr, g.data_t, g.filter_t};
+    return run_conv(g, data, filter, packed_filter, zp, e, out, as_stream(stream));
+}
+
+size_t hipq_dot_packed_bytes(const hipq_dot_desc_t* d)
+{
+    if (!d || !dot_mfma_eligible(*d))
+        return 0;
+    size_t wbytes = d->b_layout == HIPQ_B_KN ? align_up(static_cast<size_t>(d->N * d->K), 256) : 0;
+    return wbytes + static_cast<size_t>(d->N) * sizeof(int32_t);
+}
+
+int hipq_dot_pack(const hipq_dot_desc_t* d, const void* b, void* packed, void* stream)
+{
+    HIPQ_REQUIRE(d && b && packed, "null pointer");
+    if (!dot_mfma_eligible(*d))
+        return fail(HIPQ_ERR_UNSUPPORTED, "shape is not eligible for the MFMA path (hipq_dot_packed_bytes is 0)");
+    hipStream_t s = as_stream(stream);
+    uint8_t* blob = static_cast<uint8_t*>(packed);
+    const void* w = b;
+    size_t wbytes = 0;
+    if (d->b_layout == HIPQ_B_KN)
+    {
+        wbytes = align_up(static_cast<size_t>(d->N * d->K), 256);
+        int rc = launch_transpose(b, blob, 1, d->K, d->N, 1, s); // [K][N] -> [N][K]
+        if (rc)
+            return rc;
+        w = blob;
+    }
+    return launch_row_sums_i8(w, d->N, d->K, reinterpret_cast<int32_t*>(blob + wbytes), s);
+}
+
+int hipq_quantized_dot(const hipq_dot_desc_t* d,
+                       const void* a,
+                       const void* b,
+                       const void* packed_b,
+                       const float* a_scale,
+                       const void* a_zp,
+                       const float* b_scale,
+                       const void* b_zp,
+                       const float* out_scale,
+                       const void* out_zp,
+                       void* out,
+                       void* stream)
+{
+    HIPQ_REQUIRE(d, "descriptor is null");
+    HIPQ_REQUIRE(d->M >= 0 && d->N >= 0 && d->K >= 0, "negative extent");
+    HIPQ_REQUIRE(d->b_layout == HIPQ_B_KN || d->b_layout == HIPQ_B_NK, "bad b_layout");
+    if (!is_quant8(d->a_t) || !is_quant8(d->b_t) || (!is_quant8(d->out_t) && d->out_t != HIPQ_I32))
+        return fail(HIPQ_ERR_UNSUPPORTED, "QuantizedDot takes u8/i8 operands and gives i8, u8 or i32");
+    HIPQ_REQUIRE(a_scale && a_zp && b_scale && b_zp && out_scale && out_zp, "null scale or zero point");
+    Epilogue e;
+    memset(&e, 0, sizeof(e));
+    e.mode = EPI_INTERP;
+    e.out_t = d->out_t;
+    e.s_data = a_scale;
+    e.s_filter = b_scale;
+    e.s_out = out_scale;
+    e.out_zp = out_zp;
+    ZeroPoints zp{a_zp, b_zp, d->a_t, d->b_t};
+    return run_dot(*d, a, b, packed_b, zp, e, out, as_stream(stream));
+}
+
+int hipq_quantized_dot_bias(const hipq_dot_desc_t* d,
+                            const hipq_fused_desc_t* fused,
+                            const void* a,
+                            const void* w,
+                            const void* packed_w,
+                            const int32_t* bias,
+                            const float* scale,
+                            void* out,
+                            void* stream)
+{
+    HIPQ_REQUIRE(d, "descriptor is null");
+    HIPQ_REQUIRE(d->M >= 0 && d->N >= 0 && d->K >= 0, "negative extent");
+    HIPQ_REQUIRE(d->b_layout == HIPQ_B_KN || d->b_layout == HIPQ_B_NK, "bad b_layout");
+    if (!is_quant8(d->a_t) || d->b_t != HIPQ_I8 || (!is_quant8(d->out_t) && d->out_t != HIPQ_F32))
+        return fail(HIPQ_ERR_UNSUPPORTED, "QuantizedDotBias takes u8/i8 data, i8 weights and gives i8, u8 or f32");
+    HIPQ_REQUIRE(fused && !fused->has_sum, "QuantizedDotBias has no sum input");
+    Epilogue e;
+    int rc = fused_epilogue(fused, d->out_t, d->N, bias, nullptr, scale, nullptr, &e);
+    if (rc)
+        return rc;
+    ZeroPoints zp{nullptr, nullptr, d->a_t, d->b_t};
+    return run_dot(*d, a, w, packed_w, zp, e, out, as_stream(stream));
+}
+}

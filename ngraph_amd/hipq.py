@@ -230,7 +230,8 @@ EXPORTS = [
     "hipq_conv_pack_filter",
     "hipq_quantized_convolution",
     "hipq_quantized_convolution_fused",
-    "hipq_dot_prepare",
+    "hipq_dot_packed_bytes",
+    "hipq_dot_pack",
     "hipq_quantized_dot",
     "hipq_quantized_dot_bias",
     "hipq_transpose_ncx_to_nxc",
@@ -284,7 +285,9 @@ def load():
     lib.hipq_conv_pack_filter.argtypes = [C.POINTER(ConvDesc), vp, vp, vp]
     lib.hipq_quantized_convolution.argtypes = [C.POINTER(ConvDesc)] + [vp] * 11
     lib.hipq_quantized_convolution_fused.argtypes = [C.POINTER(ConvDesc), C.POINTER(FusedDesc)] + [vp] * 9
-    lib.hipq_dot_prepare.argtypes = [C.POINTER(DotDesc), vp, vp, vp]
+    lib.hipq_dot_packed_bytes.restype = C.c_size_t
+    lib.hipq_dot_packed_bytes.argtypes = [C.POINTER(DotDesc)]
+    lib.hipq_dot_pack.argtypes = [C.POINTER(DotDesc), vp, vp, vp]
     lib.hipq_quantized_dot.argtypes = [C.POINTER(DotDesc)] + [vp] * 11
     lib.hipq_quantized_dot_bias.argtypes = [C.POINTER(DotDesc), C.POINTER(FusedDesc)] + [vp] * 7
     for n in ("hipq_transpose_ncx_to_nxc", "hipq_transpose_nxc_to_ncx"):
@@ -384,6 +387,16 @@ def pack_filter(desc: ConvDesc, filter_dev: DeviceBuffer):
     return packed
 
 
+def pack_dot(desc: DotDesc, b_dev: DeviceBuffer):
+    """Returns the packed second operand, or None when the MFMA path does not apply."""
+    n = load().hipq_dot_packed_bytes(C.byref(desc))
+    if n == 0:
+        return None
+    packed = DeviceBuffer(n)
+    check(load().hipq_dot_pack(C.byref(desc), b_dev.ptr, packed.ptr, None))
+    return packed
+
+
 def quantized_convolution(desc, data, filt, data_scale, data_zp, filter_scale, filter_zp, out_scale, out_zp, use_packed=True):
     lib = load()
     bd, bf = _dev(data), _dev(filt)
@@ -428,10 +441,7 @@ def quantized_convolution_fused(desc, fused, data, filt, bias, sum_in, scale, su
 def quantized_dot(desc, a, b, a_scale, a_zp, b_scale, b_zp, out_scale, out_zp, prepare=True):
     lib = load()
     ba, bb = _dev(a), _dev(b)
-    bsum = None
-    if prepare:
-        bsum = DeviceBuffer(4 * max(int(desc.N), 1))
-        check(lib.hipq_dot_prepare(C.byref(desc), bb.ptr, bsum.ptr, None))
+    bsum = pack_dot(desc, bb) if prepare else None
     s = [_dev(np.float32(v)) for v in (a_scale, b_scale, out_scale)]
     z = [
         _dev(np.asarray(a_zp, dtype=NP_OF[desc.a_t])),
@@ -451,10 +461,7 @@ def quantized_dot(desc, a, b, a_scale, a_zp, b_scale, b_zp, out_scale, out_zp, p
 def quantized_dot_bias(desc, fused, a, w, bias, scale, prepare=True):
     lib = load()
     ba, bw = _dev(a), _dev(w)
-    wsum = None
-    if prepare:
-        wsum = DeviceBuffer(4 * max(int(desc.N), 1))
-        check(lib.hipq_dot_prepare(C.byref(desc), bw.ptr, wsum.ptr, None))
+    wsum = pack_dot(desc, bw) if prepare else None
     bb = _dev(None if bias is None else np.asarray(bias, dtype=np.int32))
     bsc = _dev(np.asarray(scale, dtype=np.float32))
     out = DeviceBuffer(int(desc.M * desc.N) * np.dtype(NP_OF[desc.out_t]).itemsize)

@@ -1,0 +1,483 @@
+"""Parity of the HIP library (through the C ABI) with the oracle, on a real MI355X.
+
+Bars: bit-exact for every integer output (int32 accumulators, int8 / uint8 results); Dequantize
+f32 outputs within 1e-5 relative (they are in fact required to be bit-exact below, which is
+stricter).  Every case prints its name before it touches the GPU.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import cases
+import oracle_lib as O
+from ngraph_amd import hipq as H
+from ngraph_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+
+
+# ------------------------------------------------------------------ Quantize / Dequantize
+
+
+def test_quantize_dequantize_kats(gpu_lib, qdq_kats):
+    for t in qdq_kats:
+        say(t["name"])
+        shape = t["shape"]
+        x = np.array(t["input"], dtype=H.NP_OF[H.dtype_code(t["input_type"])]).reshape(shape)
+        if t["op"] == "quantize":
+            got = H.quantize(x, t["scale"], t["offset"], t["output_type"], t["axes"], t["round_mode"])
+            assert got.reshape(-1).astype(np.int64).tolist() == t["expected"], t["name"]
+        else:
+            got = H.dequantize(x, t["scale"], t["offset"], t["output_type"], t["axes"])
+            assert np.array_equal(got.reshape(-1), np.array(t["expected"], dtype=got.dtype)), t["name"]
+
+
+def test_quantize_reference_vectors(gpu_lib, ref_vectors):
+    manifest, arrays = ref_vectors
+    for m in manifest:
+        if m["kind"] != "quantize":
+            continue
+        say(m["name"])
+        x, s, z = arrays[m["name"] + "__x"], arrays[m["name"] + "__scale"], arrays[m["name"] + "__zp"]
+        got = H.quantize(x, s, z, m["quant_t"], m["axes"], m["round_mode"])
+        assert np.array_equal(got, arrays[m["name"]]), m["name"]
+        dq = H.dequantize(got, s, z, m["real_t"], m["axes"])
+        assert np.array_equal(dq, arrays[m["name"] + "__dq"]), m["name"]
+
+
+@pytest.mark.parametrize("mode", range(9))
+@pytest.mark.parametrize("qt", ["i8", "u8", "i32"])
+def test_quantize_round_modes_dense(gpu_lib, mode, qt):
+    """every half-integer neighbourhood, vectorised kernel (count % 4 == 0) and generic kernel"""
+    base = np.arange(-600, 600, dtype=np.float32) * 0.25
+    eps = np.float32(2.0**-20)
+    x = np.concatenate([base, base + eps, base - eps, np.float32([8388607.5, 8388609.0, -8388609.0, 1e9, -1e9, 0.49999997, -0.49999997, 3e38])])
+    assert x.size % 4 == 0
+    for (s, z) in ((1.0, 0), (0.3, 3)):
+        say("round modes", mode, qt, s, z)
+        assert np.array_equal(H.quantize(x, s, z, qt, (), mode), O.quantize(x, s, z, qt, (), mode))
+        assert np.array_equal(H.quantize(x[:-1], s, z, qt, (), mode), O.quantize(x[:-1], s, z, qt, (), mode))
+
+
+@pytest.mark.parametrize(
+    "shape,axes",
+    [((8, 64, 128), (1,)), ((5, 7, 12), (1,)), ((6, 40), (0,)), ((6, 40), (1,)), ((3, 4, 5, 8), (1, 2)), ((3, 4, 5), (0, 2)), ((2, 3, 5, 7), ()), ((4096,), (0,))],
+)
+def test_quantize_axes_patterns(gpu_lib, shape, axes):
+    say("axes", shape, axes)
+    x = synth.normal_f32(7, shape) * 30
+    sshape = [shape[a] for a in axes]
+    scale = synth.uniform_f32(8, sshape, 0.05, 1.5)
+    for qt in ("i8", "u8"):
+        lo, hi = (-20, 20) if qt == "i8" else (0, 40)
+        zp = synth.uniform_int(9, sshape, lo, hi, H.NP_OF[H.dtype_code(qt)])
+        got = H.quantize(x, scale, zp, qt, axes)
+        exp = O.quantize(x, scale, zp, qt, axes)
+        assert np.array_equal(got, exp)
+        dq = H.dequantize(got, scale, zp, "f32", axes)
+        dexp = O.dequantize(exp, scale, zp, "f32", axes)
+        assert np.array_equal(dq, dexp)
+        # the 1e-5 relative bar of the specification, stated explicitly
+        assert np.allclose(dq, dexp, rtol=1e-5, atol=0)
+
+
+def test_quantize_dequantize_config3_shape(gpu_lib):
+    """[8,1024,1024] slice of BASELINE config 3 (per-channel scales on axis 1 = max|x|/127, RNE)
+    against the oracle, bit for bit"""
+    shape = (8, 1024, 1024)
+    say("config3 slice", shape)
+    x = synth.normal_f32(11, shape)
+    scale = (np.abs(x).max(axis=(0, 2)) / np.float32(127)).astype(np.float32)
+    zp = np.zeros(1024, np.int8)
+    O.port().orc_set_threads(8)
+    got = H.quantize(x, scale, zp, "i8", (1,))
+    assert H.last_kernel() == "quantize_vec4"
+    exp = O.quantize(x, scale, zp, "i8", (1,))
+    assert np.array_equal(got, exp)
+    dq = H.dequantize(got, scale, zp, "f32", (1,))
+    assert H.last_kernel() == "dequantize_vec4"
+    assert np.array_equal(dq, O.dequantize(exp, scale, zp, "f32", (1,)))
+    O.port().orc_set_threads(1)
+
+
+def test_quantize_dequantize_config3_full_size_properties(gpu_lib):
+    """full [64,1024,1024] of config 3 on the device: size-independent properties.
+    |dq - x| <= scale/2 (+ rounding slack) inside the clamp range, re-quantizing the dequantized
+    tensor reproduces q exactly (idempotence), and the 8 slices agree with the oracle-checked kernel
+    run slice by slice (same kernel, different launch geometry)."""
+    lib = gpu_lib
+    shape = (64, 1024, 1024)
+    say("config3 full", shape)
+    n = int(np.prod(shape))
+    x = synth.normal_f32(12, (8, 1024, 1024))
+    scale = (np.abs(x).max(axis=(0, 2)) / np.float32(127)).astype(np.float32)
+    zp = np.zeros(1024, np.int8)
+    bx = H.DeviceBuffer(n * 4)
+    for i in range(8):  # tile the 8-image block eight times
+        H.check(lib.hipq_memcpy_h2d(bx.ptr + i * x.nbytes, x.ctypes.data, x.nbytes, None))
+    bs, bz = H.DeviceBuffer.from_numpy(scale), H.DeviceBuffer.from_numpy(zp)
+    bq, bdq, bq2 = H.DeviceBuffer(n), H.DeviceBuffer(n * 4), H.DeviceBuffer(n)
+    d = H.make_quant_desc(shape, (1,), "f32", "i8")
+    H.check(lib.hipq_quantize(C.byref(d), bx.ptr, bs.ptr, bz.ptr, bq.ptr, None))
+    H.check(lib.hipq_dequantize(C.byref(d), bq.ptr, bs.ptr, bz.ptr, bdq.ptr, None))
+    H.check(lib.hipq_quantize(C.byref(d), bdq.ptr, bs.ptr, bz.ptr, bq2.ptr, None))
+    H.check(lib.hipq_stream_sync(None))
+    q = bq.to_numpy(np.int8, shape)
+    q2 = bq2.to_numpy(np.int8, shape)
+    assert np.array_equal(q, q2)
+    part = H.quantize(x, scale, zp, "i8", (1,))
+    for i in range(8):
+        assert np.array_equal(q[8 * i : 8 * i + 8], part)
+    dq = bdq.to_numpy(np.float32, shape)[:8]
+    err = np.abs(dq - x)
+    # half a quantization step, plus the f32 roundings of x/scale and q*scale (a few ulp of |x| <= 127*scale)
+    bound = scale[None, :, None] * np.float32(0.5 + 127 * 4 * 2.0**-24)
+    assert np.all(err <= bound)
+
+
+def test_quantize_empty_and_scalar(gpu_lib):
+    say("empty / rank-0")
+    assert H.quantize(np.zeros((0, 3), np.float32), 1.0, 0, "i8").shape == (0, 3)
+    assert H.quantize(np.float32(5.0).reshape(()), 2.0, 1, "u8").item() == 3
+    assert H.dequantize(np.int8(-4).reshape(()), 0.5, 2, "f32").item() == -3.0
+
+
+# ------------------------------------------------------------------ QuantizedConvolution
+
+
+def _conv_both(desc, data, filt, s, z):
+    """direct kernel and (where eligible) MFMA kernel"""
+    outs = []
+    got = H.quantized_convolution(desc, data, filt, s[0], z[0], s[1], z[1], s[2], z[2], use_packed=False)
+    outs.append(("direct", got, H.last_kernel()))
+    if H.load().hipq_conv_packed_filter_bytes(C.byref(desc)):
+        got = H.quantized_convolution(desc, data, filt, s[0], z[0], s[1], z[1], s[2], z[2], use_packed=True)
+        outs.append(("mfma", got, H.last_kernel()))
+    return outs
+
+
+def test_conv_kats(gpu_lib, kats):
+    lib = O.port()
+    for k in kats["conv"]:
+        if k.get("policy") == "dnnl":
+            continue
+        say(k["name"])
+        d, data, filt, exp = cases.kat_conv(k)
+        if k.get("via_builder"):
+            s = [lib.orc_get_scale(*k["in_range"], d.data_t, 0), lib.orc_get_scale(*k["filter_range"], d.filter_t, 0), lib.orc_get_scale(*k["out_range"], d.out_t, 0)]
+            z = [0, 0, 0]
+        else:
+            s, z = k["scales"], k["zps"]
+        for name, got, kern in _conv_both(d, data, filt, s, z):
+            assert got.reshape(-1).astype(np.int64).tolist() == exp.astype(np.int64).tolist(), (k["name"], name)
+
+
+def test_conv_reference_vectors(gpu_lib, ref_vectors):
+    """compiled-reference outputs, including BASELINE config 1 with its wrapped outputs"""
+    manifest, arrays = ref_vectors
+    used = set()
+    for m in manifest:
+        if m["kind"] != "conv":
+            continue
+        say(m["name"])
+        d, data, filt, s, z = cases.conv_from_manifest(m)
+        for name, got, kern in _conv_both(d, data, filt, s, z):
+            assert np.array_equal(got, arrays[m["name"]]), (m["name"], name, kern)
+            used.add(kern)
+        # channels-last descriptors on the same tensors (2-D MFMA-eligible cases included)
+        dl = cases.conv_from_manifest(m, H.NXC, H.NXC)[0]
+        for name, got, kern in _conv_both(dl, cases.to_nxc(data), filt, s, z):
+            assert np.array_equal(cases.to_ncx(got), arrays[m["name"]]), (m["name"], name, "nxc")
+    assert "conv_direct" in used and any(k.startswith("conv_mfma") for k in used), used
+
+
+MFMA_SHAPES = [
+    # N, C, K, in_sp, f_sp, kw : ResNet-50-like layers and ragged edges (K, pixels not multiples of the tile)
+    (1, 64, 64, (56, 56), (3, 3), dict(pad_below=(1, 1), pad_above=(1, 1))),
+    (3, 64, 64, (20, 20), (3, 3), dict(pad_below=(1, 1), pad_above=(1, 1))),
+    (2, 64, 256, (14, 14), (1, 1), dict()),
+    (2, 256, 64, (14, 14), (1, 1), dict()),
+    (1, 128, 128, (28, 28), (3, 3), dict(stride=(2, 2), pad_below=(1, 1), pad_above=(1, 1))),
+    (2, 256, 512, (14, 14), (1, 1), dict(stride=(2, 2))),
+    (1, 16, 24, (9, 7), (3, 3), dict(pad_below=(1, 1), pad_above=(1, 1))),
+    (1, 48, 40, (11, 13), (3, 2), dict(stride=(2, 1), dilation=(1, 2), pad_below=(2, 0), pad_above=(0, 3))),
+    (2, 32, 200, (10, 10), (5, 5), dict(pad_below=(2, 2), pad_above=(2, 2))),
+    (1, 80, 17, (6, 6), (3, 3), dict(pad_below=(-1, 1), pad_above=(1, -1))),
+    (2, 32, 8, (33,), (5,), dict(stride=(2,), pad_below=(2,), pad_above=(2,))),
+    (1, 512, 512, (7, 7), (3, 3), dict(pad_below=(1, 1), pad_above=(1, 1))),
+]
+
+
+@pytest.mark.parametrize("i", range(len(MFMA_SHAPES)))
+def test_conv_mfma_shapes(gpu_lib, i):
+    N, Cc, K, in_sp, f_sp, kw = MFMA_SHAPES[i]
+    say("mfma conv", MFMA_SHAPES[i])
+    for out_t, s, z in (("i32", (1.0, 1.0, 1.0), (0, 0, 0)), ("i8", (0.02, 0.005, 0.9), (0, 0, -3)), ("i8", (0.02, 0.005, 0.7), (131, 0, 0))):
+        d = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t=out_t, data_layout=H.NXC, out_layout=H.NXC, **kw)
+        data = synth.uniform_int(100 + i, d.data_shape(), 0, 255, np.uint8)
+        filt = synth.uniform_int(200 + i, d.filter_shape(), -128, 127, np.int8)
+        O.port().orc_set_threads(8)
+        exp = O.quantized_convolution(d, data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
+        O.port().orc_set_threads(1)
+        got = H.quantized_convolution(d, data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
+        assert H.last_kernel().startswith("conv_mfma"), H.last_kernel()
+        assert np.array_equal(got, exp), (out_t, z)
+    # reference layouts in and out (transposed through the workspace)
+    d = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t="i8", **kw)
+    data = synth.uniform_int(100 + i, d.data_shape(), 0, 255, np.uint8)
+    O.port().orc_set_threads(8)
+    exp = O.quantized_convolution(d, data, filt, 0.02, 0, 0.005, 0, 0.9, 0)
+    O.port().orc_set_threads(1)
+    got = H.quantized_convolution(d, data, filt, 0.02, 0, 0.005, 0, 0.9, 0)
+    assert H.last_kernel().startswith("conv_mfma"), H.last_kernel()
+    assert np.array_equal(got, exp)
+
+
+def test_conv_mfma_nonzero_filter_zero_point(gpu_lib):
+    """packed filter handed over although the filter zero point is not zero: the kernel's slow
+    in-kernel path must still give the reference's numbers"""
+    say("mfma conv, filter zp != 0")
+    d = H.make_conv_desc(1, 32, 40, (9, 9), (3, 3), pad_below=(1, 1), pad_above=(1, 1), data_layout=H.NXC, out_layout=H.NXC)
+    data = synth.uniform_int(31, d.data_shape(), 0, 255, np.uint8)
+    filt = synth.uniform_int(32, d.filter_shape(), -128, 127, np.int8)
+    exp = O.quantized_convolution(d, data, filt, 0.02, 7, 0.005, -9, 0.9, 1)
+    got = H.quantized_convolution(d, data, filt, 0.02, 7, 0.005, -9, 0.9, 1)
+    assert np.array_equal(got, exp)
+
+
+def test_conv_i8_data(gpu_lib):
+    say("i8 data")
+    d = H.make_conv_desc(1, 32, 48, (9, 9), (3, 3), pad_below=(1, 1), pad_above=(1, 1), data_t="i8", out_t="i32", data_layout=H.NXC, out_layout=H.NXC)
+    data = synth.uniform_int(41, d.data_shape(), -128, 127, np.int8)
+    filt = synth.uniform_int(42, d.filter_shape(), -128, 127, np.int8)
+    for zpd in (0, -5):
+        exp = O.quantized_convolution(d, data, filt, 1.0, zpd, 1.0, 0, 1.0, 0)
+        for packed in (False, True):
+            got = H.quantized_convolution(d, data, filt, 1.0, zpd, 1.0, 0, 1.0, 0, use_packed=packed)
+            assert np.array_equal(got, exp), (zpd, packed, H.last_kernel())
+
+
+def test_conv_linearity_at_config1_batch(gpu_lib):
+    """BASELINE config 1's layer at batch 32 (too slow for the CPU oracle in a test): int32
+    accumulators are linear in the filter, conv(f1) + conv(f2) == conv(f1 + f2), and image 0
+    equals the oracle-checked single-image result"""
+    say("config1 batch 32 linearity")
+    kw = dict(pad_below=(1, 1), pad_above=(1, 1), out_t="i32", data_layout=H.NXC, out_layout=H.NXC)
+    d = H.make_conv_desc(32, 64, 64, (56, 56), (3, 3), **kw)
+    data = synth.uniform_int(51, d.data_shape(), 0, 255, np.uint8)
+    f1 = synth.uniform_int(52, d.filter_shape(), -60, 60, np.int8)
+    f2 = synth.uniform_int(53, d.filter_shape(), -60, 60, np.int8)
+    a = H.quantized_convolution(d, data, f1, 1.0, 0, 1.0, 0, 1.0, 0).astype(np.int64)
+    b = H.quantized_convolution(d, data, f2, 1.0, 0, 1.0, 0, 1.0, 0).astype(np.int64)
+    c = H.quantized_convolution(d, data, (f1 + f2).astype(np.int8), 1.0, 0, 1.0, 0, 1.0, 0).astype(np.int64)
+    assert H.last_kernel().startswith("conv_mfma")
+    assert np.array_equal(a + b, c)
+    d1 = H.make_conv_desc(1, 64, 64, (56, 56), (3, 3), **kw)
+    O.port().orc_set_threads(8)
+    exp0 = O.quantized_convolution(d1, data[:1], f1, 1.0, 0, 1.0, 0, 1.0, 0)
+    exp31 = O.quantized_convolution(d1, data[31:], f1, 1.0, 0, 1.0, 0, 1.0, 0)
+    O.port().orc_set_threads(1)
+    assert np.array_equal(a[:1], exp0) and np.array_equal(a[31:], exp31)
+
+
+# ------------------------------------------------------------------ fused convolutions
+
+
+def test_fused_conv_kats(gpu_lib, kats):
+    lib = O.port()
+    for k in kats["fused_conv"]:
+        say(k["name"])
+        d, data, filt, exp = cases.kat_conv(k)
+        builder_out_t = H.U8 if k["with_relu"] else H.I8
+        scale = lib.orc_get_conv_requant_scale(*k["in_range"], H.U8, *k["filter_range"], H.I8, *k["out_range"], builder_out_t)
+        bias = k.get("bias")
+        if "bias_f32" in k:
+            bs = lib.orc_get_bias_scale(*k["in_range"], *k["filter_range"])
+            bias = H.quantize(np.float32(k["bias_f32"]), bs, 0, "i32", (), H.RNE).tolist()
+        has_sum = "sum" in k
+        sum_scale = sum_in = None
+        if has_sum:
+            sum_scale = lib.orc_get_sum_scale(*k["out_range"], *k["sum_range"])
+            if k["op"] == "QuantizedConvolutionBiasSignedAdd" and builder_out_t == H.U8:
+                sum_scale = np.float32(2.0) * np.float32(sum_scale)
+            sum_in = np.array(k["sum"], dtype=H.NP_OF[H.dtype_code(k["sum_t"])]).reshape(d.out_shape())
+        f = H.make_fused_desc(has_bias=bias is not None, has_sum=has_sum, sum_t=k.get("sum_t", "u8"), with_relu=k["with_relu"])
+        got = H.quantized_convolution_fused(d, f, data, filt, bias, sum_in, scale, sum_scale)
+        if k["out_t"] == "u8_via_i8_convert":
+            got = got.astype(np.uint8)
+        assert got.reshape(-1).astype(np.int64).tolist() == exp.tolist(), k["name"]
+
+
+def test_quant_conv_linear_rne_kat(gpu_lib, kats):
+    """ONNX QLinearConv vector (round-half-even): the fused entry point without bias"""
+    k = next(x for x in kats["conv"] if x.get("policy") == "dnnl")
+    say(k["name"])
+    d, data, filt, exp = cases.kat_conv(k)
+    f = H.make_fused_desc(has_bias=False)
+    got = H.quantized_convolution_fused(d, f, data, filt, None, None, np.float32(1.0 / 16.0), None)
+    assert got.reshape(-1).astype(np.int64).tolist() == exp.tolist()
+
+
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("has_sum", [False, True])
+@pytest.mark.parametrize("layout", [H.NCX, H.NXC])
+def test_fused_conv_random(gpu_lib, relu, has_sum, layout):
+    """ResNet-style bottleneck piece: per-channel scales, bias, residual sum, relu; both kernels"""
+    say("fused conv", relu, has_sum, layout)
+    out_t = "u8" if relu else "i8"
+    for (Cc, K, sp, fs, kw) in ((64, 96, (12, 12), (3, 3), dict(pad_below=(1, 1), pad_above=(1, 1))), (3, 16, (17, 17), (7, 7), dict(stride=(2, 2), pad_below=(3, 3), pad_above=(3, 3)))):
+        d = H.make_conv_desc(2, Cc, K, sp, fs, out_t=out_t, data_layout=layout, out_layout=layout, **kw)
+        dn = H.make_conv_desc(2, Cc, K, sp, fs, out_t=out_t, **kw)
+        data = synth.uniform_int(61, dn.data_shape(), 0, 255, np.uint8)
+        filt = synth.uniform_int(62, d.filter_shape(), -127, 127, np.int8)
+        bias = synth.uniform_int(63, (K,), -20000, 20000, np.int32)
+        scales = synth.uniform_f32(64, (K,), 2e-4, 9e-4)
+        summ = synth.uniform_int(65, dn.out_shape(), 0, 255, np.uint8) if has_sum else None
+        if layout == H.NXC:
+            data = cases.to_nxc(data)
+            summ = cases.to_nxc(summ) if has_sum else None
+        f = H.make_fused_desc(has_bias=True, has_sum=has_sum, sum_t="u8", with_relu=relu, scale_count=K)
+        ss = 0.37 if has_sum else None
+        exp = O.quantized_convolution_fused(d, f, data, filt, bias, summ, scales, ss)
+        for packed in (False, True):
+            got = H.quantized_convolution_fused(d, f, data, filt, bias, summ, scales, ss, use_packed=packed)
+            assert np.array_equal(got, exp), (Cc, packed, H.last_kernel())
+    # signed sum input, scalar scale, output stays i8 (QuantizedConvolutionBiasSignedAdd)
+    d = H.make_conv_desc(1, 32, 32, (8, 8), (1, 1), out_t="i8", data_layout=layout, out_layout=layout)
+    data = synth.uniform_int(71, d.data_shape(), 0, 255, np.uint8)
+    filt = synth.uniform_int(72, d.filter_shape(), -127, 127, np.int8)
+    summ = synth.uniform_int(73, d.out_shape(), -128, 127, np.int8)
+    f = H.make_fused_desc(has_bias=False, has_sum=True, sum_t="i8", with_relu=relu)
+    exp = O.quantized_convolution_fused(d, f, data, filt, None, summ, 1.5e-3, 0.8)
+    got = H.quantized_convolution_fused(d, f, data, filt, None, summ, 1.5e-3, 0.8)
+    assert np.array_equal(got, exp)
+
+
+# ------------------------------------------------------------------ QuantizedDot
+
+
+def test_dot_kats(gpu_lib, kats):
+    for k in kats["dot"]:
+        say(k["name"])
+        M, K = k["a_shape"]
+        N = k["b_shape"][1]
+        d = H.make_dot_desc(M, K, N, a_t=k["a_t"], b_t=k["b_t"], out_t=k["out_t"])
+        a = np.array(k["a"], dtype=H.NP_OF[d.a_t]).reshape(M, K)
+        b = np.array(k["b"], dtype=H.NP_OF[d.b_t]).reshape(K, N)
+        s, z = k["scales"], k["zps"]
+        got = H.quantized_dot(d, a, b, s[0], z[0], s[1], z[1], s[2], z[2])
+        assert got.reshape(-1).tolist() == k["expected"], k["name"]
+
+
+def test_dot_reference_vectors(gpu_lib, ref_vectors):
+    manifest, arrays = ref_vectors
+    used = set()
+    for m in manifest:
+        if m["kind"] != "dot":
+            continue
+        say(m["name"])
+        d, a, b, s, z = cases.dot_from_manifest(m)
+        for prepare in (False, True):
+            got = H.quantized_dot(d, a, b, s[0], z[0], s[1], z[1], s[2], z[2], prepare=prepare)
+            used.add(H.last_kernel())
+            assert np.array_equal(got, arrays[m["name"]]), (m["name"], prepare, H.last_kernel())
+    assert "dot_direct" in used and any(k.startswith("dot_mfma") for k in used), used
+
+
+@pytest.mark.parametrize("M", [1, 32, 256, 130])
+def test_dot_mfma_vs_oracle(gpu_lib, M):
+    say("dot mfma M", M)
+    K, N = 512, 384
+    a = synth.uniform_int(81, (M, K), 0, 255, np.uint8)
+    b = synth.uniform_int(82, (K, N), -127, 127, np.int8)
+    O.port().orc_set_threads(8)
+    for out_t, s, z in (("i32", (1.0, 1.0, 1.0), (0, 0, 0)), ("i8", (0.01, 0.01, 2.5), (0, 0, 4)), ("i8", (0.01, 0.01, 2.5), (9, 0, 0)), ("i8", (0.01, 0.01, 2.5), (9, 3, 0))):
+        d = H.make_dot_desc(M, K, N, out_t=out_t)
+        exp = O.quantized_dot(d, a, b, s[0], z[0], s[1], z[1], s[2], z[2])
+        got = H.quantized_dot(d, a, b, s[0], z[0], s[1], z[1], s[2], z[2])
+        assert H.last_kernel().startswith("dot_mfma")
+        assert np.array_equal(got, exp), (out_t, z)
+    O.port().orc_set_threads(1)
+
+
+def test_dot_bias_kat(gpu_lib, kats):
+    k = kats["dot_bias"]
+    say(k["name"])
+    lib = O.port()
+    M, K = k["a_shape"]
+    N = k["w_shape"][0]
+    a = np.array(k["a"], dtype=np.uint8).reshape(M, K)
+    w = np.array(k["w"], dtype=np.int8).reshape(N, K)
+    r = k["in_range"] + k["filter_range"] + k["out_range"]
+    for requant, relu, key, out_t in ((0, 0, "expected_f32", "f32"), (0, 1, "expected_f32_relu", "f32"), (1, 0, "expected_i8", "i8"), (1, 1, "expected_u8_relu", "u8")):
+        scale = lib.orc_get_dot_scale(*r, H.U8, H.U8 if relu else H.I8, requant)
+        d = H.make_dot_desc(M, K, N, out_t=out_t, b_layout=H.B_NK)
+        f = H.make_fused_desc(has_bias=True, with_relu=bool(relu))
+        got = H.quantized_dot_bias(d, f, a, w, k["bias"], scale)
+        assert np.array_equal(got, np.array(k[key], dtype=got.dtype).reshape(M, N)), key
+
+
+@pytest.mark.parametrize("M", [1, 32, 256])
+def test_dot_bias_config2_shape(gpu_lib, M):
+    """BASELINE config 2 at K = N = 1024 (the oracle needs minutes at 4096): per-output-channel
+    scales, int32 bias, requantize to i8; and the f32 / relu variants"""
+    say("config2 M", M)
+    K = N = 1024
+    a = synth.uniform_int(91, (M, K), 0, 255, np.uint8)
+    w = synth.uniform_int(92, (N, K), -127, 127, np.int8)
+    bias = synth.uniform_int(93, (N,), -(2**15), 2**15, np.int32)
+    scales = synth.uniform_f32(94, (N,), 0.001, 0.01) * np.float32(0.02)
+    O.port().orc_set_threads(8)
+    for out_t, relu in (("i8", False), ("u8", True), ("f32", False), ("f32", True)):
+        d = H.make_dot_desc(M, K, N, out_t=out_t, b_layout=H.B_NK)
+        f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
+        exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
+        got = H.quantized_dot_bias(d, f, a, w, bias, scales)
+        assert H.last_kernel().startswith("dot_mfma")
+        assert np.array_equal(got, exp), (out_t, relu)
+        assert len(np.unique(exp)) > 20  # the case is not degenerate (all saturated)
+    O.port().orc_set_threads(1)
+
+
+def test_dot_config2_full_size_properties(gpu_lib):
+    """config 2 at its real size [256,4096] x [4096,4096]: rows of the M=256 result equal the
+    M=1 / M=32 results (launch geometry independence), and int32 accumulators of a row subset
+    match numpy's int64 matmul"""
+    say("config2 full size")
+    K = N = 4096
+    a = synth.uniform_int(95, (256, K), 0, 255, np.uint8)
+    w = synth.uniform_int(96, (N, K), -127, 127, np.int8)
+    d = H.make_dot_desc(256, K, N, out_t="i32", b_layout=H.B_NK)
+    got = H.quantized_dot(d, a, w, 1.0, 0, 1.0, 0, 1.0, 0)
+    assert H.last_kernel().startswith("dot_mfma")
+    rows = [0, 1, 31, 32, 127, 128, 255]
+    exp = a[rows].astype(np.int64) @ w.astype(np.int64).T
+    assert np.array_equal(got[rows].astype(np.int64), exp)
+    for M in (1, 32):
+        dm = H.make_dot_desc(M, K, N, out_t="i32", b_layout=H.B_NK)
+        gm = H.quantized_dot(dm, a[:M], w, 1.0, 0, 1.0, 0, 1.0, 0)
+        assert np.array_equal(gm, got[:M])
+
+
+# ------------------------------------------------------------------ layout helpers
+
+
+@pytest.mark.parametrize("eb", [1, 4])
+def test_transposes(gpu_lib, eb):
+    say("transpose", eb)
+    dt = np.uint8 if eb == 1 else np.int32
+    for (N, Cc, X) in ((2, 64, 3136), (3, 5, 7), (1, 130, 67)):
+        a = synth.uniform_int(5, (N, Cc, X), 0, 255, np.uint8).astype(dt)
+        src = H.DeviceBuffer.from_numpy(a)
+        dst = H.DeviceBuffer(a.nbytes)
+        H.check(gpu_lib.hipq_transpose_ncx_to_nxc(src.ptr, dst.ptr, N, Cc, X, eb, None))
+        t = dst.to_numpy(dt, (N, X, Cc))
+        assert np.array_equal(t, np.transpose(a, (0, 2, 1)))
+        back = H.DeviceBuffer(a.nbytes)
+        H.check(gpu_lib.hipq_transpose_nxc_to_ncx(dst.ptr, back.ptr, N, Cc, X, eb, None))
+        assert np.array_equal(back.to_numpy(dt, (N, Cc, X)), a)

@@ -318,6 +318,59 @@ HIPQ_API int hipq_transpose_ncx_to_nxc(
 HIPQ_API int hipq_transpose_nxc_to_ncx(
     const void* in, void* out, int64_t N, int64_t C, int64_t X, int32_t elem_bytes, void* stream);
 
+/* ---------------------------------------------------------------- glue ops
+ * The small elementwise / shape ops that surround the quantized ops in a graph: the f32 scale
+ * sub-graphs the builders emit (src/ngraph/builder/quantization_utils.cpp:33-174), and the integer
+ * glue of quantized networks.  Arithmetic is the reference's (src/ngraph/runtime/reference/
+ * {abs,relu,add,subtract,multiply,divide,maximum,minimum,convert,broadcast,reshape}.hpp): plain C++
+ * operators on the element type, so 8-bit sums wrap and Convert is a static_cast. */
+typedef enum
+{
+    HIPQ_OP_ADD = 0,
+    HIPQ_OP_SUBTRACT = 1,
+    HIPQ_OP_MULTIPLY = 2,
+    HIPQ_OP_DIVIDE = 3,
+    HIPQ_OP_MAXIMUM = 4,
+    HIPQ_OP_MINIMUM = 5
+} hipq_binary_op_t;
+
+typedef enum
+{
+    HIPQ_OP_ABS = 0,
+    HIPQ_OP_RELU = 1,
+    HIPQ_OP_COPY = 2
+} hipq_unary_op_t;
+
+/* out[i] = a[i or 0] (op) b[i or 0]; a_count and b_count are each `count` or 1 (broadcast scalar) */
+HIPQ_API int hipq_binary(int32_t op,
+                         int32_t dtype,
+                         const void* a,
+                         int64_t a_count,
+                         const void* b,
+                         int64_t b_count,
+                         void* out,
+                         int64_t count,
+                         void* stream);
+HIPQ_API int hipq_unary(int32_t op, int32_t dtype, const void* in, void* out, int64_t count, void* stream);
+/* out[i] = static_cast<OUT>(in[i]) with the x86 narrowing of the reference build */
+HIPQ_API int hipq_convert(int32_t in_t, int32_t out_t, const void* in, void* out, int64_t count, void* stream);
+/* op::v0::Broadcast: `in` has out_shape minus the axes in axes_mask */
+HIPQ_API int hipq_broadcast(int32_t elem_bytes,
+                            const void* in,
+                            void* out,
+                            int32_t out_rank,
+                            const int64_t* out_shape, /* host */
+                            uint32_t axes_mask,
+                            void* stream);
+/* op::v0::Reshape's transposition: out = in with axes read in `order` (out dim i = in dim order[i]) */
+HIPQ_API int hipq_permute(int32_t elem_bytes,
+                          const void* in,
+                          void* out,
+                          int32_t rank,
+                          const int64_t* in_shape, /* host */
+                          const int32_t* order,    /* host */
+                          void* stream);
+
 /* Which kernel the last hipq_quantized_* call on this thread used: "mfma", "direct", ... (host
  * string, never NULL).  For tests and profiles. */
 HIPQ_API const char* hipq_last_kernel(void);

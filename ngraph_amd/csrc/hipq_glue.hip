@@ -1,0 +1,312 @@
+// Elementwise and shape glue around the quantized ops (tiny f32 scale tensors, integer glue).
+#include "hipq_common.h"
+
+namespace hipq
+{
+    template <typename T>
+    __device__ __forceinline__ T binary_apply(int op, T a, T b)
+    {
+        switch (op)
+        {
+        case HIPQ_OP_ADD: return static_cast<T>(a + b);
+        case HIPQ_OP_SUBTRACT: return static_cast<T>(a - b);
+        case HIPQ_OP_MULTIPLY: return static_cast<T>(a * b);
+        case HIPQ_OP_DIVIDE: return static_cast<T>(a / b);
+        case HIPQ_OP_MAXIMUM: return a > b ? a : b;
+        default: return a < b ? a : b;
+        }
+    }
+    template <>
+    __device__ __forceinline__ float binary_apply<float>(int op, float a, float b)
+    {
+        switch (op)
+        {
+        case HIPQ_OP_ADD: return __fadd_rn(a, b);
+        case HIPQ_OP_SUBTRACT: return __fsub_rn(a, b);
+        case HIPQ_OP_MULTIPLY: return __fmul_rn(a, b);
+        case HIPQ_OP_DIVIDE: return __fdiv_rn(a, b);
+        case HIPQ_OP_MAXIMUM: return a > b ? a : b;
+        default: return a < b ? a : b;
+        }
+    }
+    // integer division by zero has no defined result in the reference either; keep the GPU quiet
+    template <>
+    __device__ __forceinline__ int32_t binary_apply<int32_t>(int op, int32_t a, int32_t b)
+    {
+        switch (op)
+        {
+        case HIPQ_OP_ADD: return static_cast<int32_t>(static_cast<uint32_t>(a) + static_cast<uint32_t>(b));
+        case HIPQ_OP_SUBTRACT: return static_cast<int32_t>(static_cast<uint32_t>(a) - static_cast<uint32_t>(b));
+        case HIPQ_OP_MULTIPLY: return static_cast<int32_t>(static_cast<uint32_t>(a) * static_cast<uint32_t>(b));
+        case HIPQ_OP_DIVIDE: return b == 0 ? 0 : (a == INT32_MIN && b == -1 ? INT32_MIN : a / b);
+        case HIPQ_OP_MAXIMUM: return a > b ? a : b;
+        default: return a < b ? a : b;
+        }
+    }
+
+    template <typename T>
+    __global__ __launch_bounds__(256) void binary_kernel(int op, const T* a, int64_t an, const T* b, int64_t bn, T* out, int64_t n)
+    {
+        int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+        const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+        for (; i < n; i += step)
+        {
+            T x = a[an == 1 ? 0 : i], y = b[bn == 1 ? 0 : i];
+            if (sizeof(T) == 1 && op == HIPQ_OP_DIVIDE && y == 0)
+                out[i] = 0;
+            else
+                out[i] = binary_apply<T>(op, x, y);
+        }
+    }
+
+    template <typename T>
+    __global__ __launch_bounds__(256) void unary_kernel(int op, const T* in, T* out, int64_t n)
+    {
+        int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+        const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+        for (; i < n; i += step)
+        {
+            T x = in[i];
+            if (op == HIPQ_OP_ABS)
+                out[i] = x < T(0) ? static_cast<T>(-x) : x; // reference::abs: (x < 0 ? -x : x)
+            else if (op == HIPQ_OP_RELU)
+                out[i] = x > T(0) ? x : T(0); // reference::relu
+            else
+                out[i] = x;
+        }
+    }
+
+    template <typename TO>
+    __device__ __forceinline__ TO convert_from_f(double v, bool from_f32)
+    {
+        return static_cast<TO>(v);
+    }
+
+    template <typename TI, typename TO>
+    __global__ __launch_bounds__(256) void convert_kernel(const TI* in, TO* out, int64_t n)
+    {
+        int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+        const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+        for (; i < n; i += step)
+        {
+            TI x = in[i];
+            if (std::is_floating_point<TI>::value && std::is_integral<TO>::value)
+            {
+                // x86: cvttss2si / cvttsd2si to 32 bits, then the low bits
+                double d = static_cast<double>(x);
+                int32_t t = (!(d < 2147483648.0) || d <= -2147483649.0) ? INT32_MIN : static_cast<int32_t>(d);
+                out[i] = static_cast<TO>(t);
+            }
+            else
+                out[i] = static_cast<TO>(x);
+        }
+    }
+
+    struct BroadcastInfo
+    {
+        int32_t rank;
+        uint32_t axes_mask;
+        int64_t shape[HIPQ_MAX_RANK];
+    };
+
+    template <typename T>
+    __global__ __launch_bounds__(256) void broadcast_kernel(const T* in, T* out, int64_t n, BroadcastInfo bi)
+    {
+        int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+        const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+        for (; i < n; i += step)
+        {
+            int64_t r = i, coord[HIPQ_MAX_RANK];
+            for (int a = bi.rank - 1; a >= 0; --a)
+            {
+                coord[a] = r % bi.shape[a];
+                r /= bi.shape[a];
+            }
+            int64_t j = 0;
+            for (int a = 0; a < bi.rank; ++a)
+                if (!(bi.axes_mask & (1u << a)))
+                    j = j * bi.shape[a] + coord[a];
+            out[i] = in[j];
+        }
+    }
+
+    struct PermuteInfo
+    {
+        int32_t rank;
+        int64_t out_shape[HIPQ_MAX_RANK];
+        int64_t in_stride[HIPQ_MAX_RANK]; // stride in the input of output axis i
+    };
+
+    template <typename T>
+    __global__ __launch_bounds__(256) void permute_kernel(const T* in, T* out, int64_t n, PermuteInfo pi)
+    {
+        int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+        const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+        for (; i < n; i += step)
+        {
+            int64_t r = i, j = 0;
+            for (int a = pi.rank - 1; a >= 0; --a)
+            {
+                j += (r % pi.out_shape[a]) * pi.in_stride[a];
+                r /= pi.out_shape[a];
+            }
+            out[i] = in[j];
+        }
+    }
+
+    static unsigned blocks_for(int64_t n)
+    {
+        int64_t b = (n + 255) / 256;
+        return static_cast<unsigned>(b < 1 ? 1 : (b > 65536 ? 65536 : b));
+    }
+}
+
+using namespace hipq;
+
+extern "C" {
+
+int hipq_binary(int32_t op, int32_t dtype, const void* a, int64_t an, const void* b, int64_t bn, void* out, int64_t n, void* stream)
+{
+    HIPQ_REQUIRE(op >= HIPQ_OP_ADD && op <= HIPQ_OP_MINIMUM, "binary op %d unknown", op);
+    HIPQ_REQUIRE(n >= 0 && (an == n || an == 1) && (bn == n || bn == 1), "operand counts must be the output count or 1");
+    if (n == 0)
+        return HIPQ_OK;
+    HIPQ_REQUIRE(a && b && out, "null tensor pointer");
+    hipStream_t s = as_stream(stream);
+#define LAUNCH_B(T) binary_kernel<T><<<blocks_for(n), 256, 0, s>>>(op, static_cast<const T*>(a), an, static_cast<const T*>(b), bn, static_cast<T*>(out), n)
+    switch (dtype)
+    {
+    case HIPQ_U8: LAUNCH_B(uint8_t); break;
+    case HIPQ_I8: LAUNCH_B(int8_t); break;
+    case HIPQ_I32: LAUNCH_B(int32_t); break;
+    case HIPQ_F32: LAUNCH_B(float); break;
+    case HIPQ_F64: LAUNCH_B(double); break;
+    default: return fail(HIPQ_ERR_UNSUPPORTED, "element type %d", dtype);
+    }
+#undef LAUNCH_B
+    return check_launch("binary");
+}
+
+int hipq_unary(int32_t op, int32_t dtype, const void* in, void* out, int64_t n, void* stream)
+{
+    HIPQ_REQUIRE(op >= HIPQ_OP_ABS && op <= HIPQ_OP_COPY, "unary op %d unknown", op);
+    HIPQ_REQUIRE(n >= 0, "negative count");
+    if (n == 0)
+        return HIPQ_OK;
+    HIPQ_REQUIRE(in && out, "null tensor pointer");
+    hipStream_t s = as_stream(stream);
+#define LAUNCH_U(T) unary_kernel<T><<<blocks_for(n), 256, 0, s>>>(op, static_cast<const T*>(in), static_cast<T*>(out), n)
+    switch (dtype)
+    {
+    case HIPQ_U8: LAUNCH_U(uint8_t); break;
+    case HIPQ_I8: LAUNCH_U(int8_t); break;
+    case HIPQ_I32: LAUNCH_U(int32_t); break;
+    case HIPQ_F32: LAUNCH_U(float); break;
+    case HIPQ_F64: LAUNCH_U(double); break;
+    default: return fail(HIPQ_ERR_UNSUPPORTED, "element type %d", dtype);
+    }
+#undef LAUNCH_U
+    return check_launch("unary");
+}
+
+int hipq_convert(int32_t in_t, int32_t out_t, const void* in, void* out, int64_t n, void* stream)
+{
+    HIPQ_REQUIRE(n >= 0, "negative count");
+    if (n == 0)
+        return HIPQ_OK;
+    HIPQ_REQUIRE(in && out, "null tensor pointer");
+    hipStream_t s = as_stream(stream);
+#define LAUNCH_C(TI, TO) convert_kernel<TI, TO><<<blocks_for(n), 256, 0, s>>>(static_cast<const TI*>(in), static_cast<TO*>(out), n)
+#define CONVERT_TO(TI)                                                                             \
+    switch (out_t)                                                                                 \
+    {                                                                                              \
+    case HIPQ_U8: LAUNCH_C(TI, uint8_t); break;                                                    \
+    case HIPQ_I8: LAUNCH_C(TI, int8_t); break;                                                     \
+    case HIPQ_I32: LAUNCH_C(TI, int32_t); break;                                                   \
+    case HIPQ_F32: LAUNCH_C(TI, float); break;                                                     \
+    case HIPQ_F64: LAUNCH_C(TI, double); break;                                                    \
+    default: return fail(HIPQ_ERR_UNSUPPORTED, "element type %d", out_t);                          \
+    }
+    switch (in_t)
+    {
+    case HIPQ_U8: CONVERT_TO(uint8_t); break;
+    case HIPQ_I8: CONVERT_TO(int8_t); break;
+    case HIPQ_I32: CONVERT_TO(int32_t); break;
+    case HIPQ_F32: CONVERT_TO(float); break;
+    case HIPQ_F64: CONVERT_TO(double); break;
+    default: return fail(HIPQ_ERR_UNSUPPORTED, "element type %d", in_t);
+    }
+#undef CONVERT_TO
+#undef LAUNCH_C
+    return check_launch("convert");
+}
+
+int hipq_broadcast(int32_t elem_bytes, const void* in, void* out, int32_t rank, const int64_t* shape, uint32_t axes_mask, void* stream)
+{
+    HIPQ_REQUIRE(rank >= 0 && rank <= HIPQ_MAX_RANK, "rank %d out of range", rank);
+    HIPQ_REQUIRE(rank == 0 || shape, "shape is null");
+    BroadcastInfo bi;
+    bi.rank = rank;
+    bi.axes_mask = axes_mask;
+    int64_t n = 1;
+    for (int i = 0; i < HIPQ_MAX_RANK; ++i)
+    {
+        bi.shape[i] = i < rank ? shape[i] : 1;
+        HIPQ_REQUIRE(bi.shape[i] >= 0, "negative extent");
+        n *= bi.shape[i];
+    }
+    if (n == 0)
+        return HIPQ_OK;
+    HIPQ_REQUIRE(in && out, "null tensor pointer");
+    hipStream_t s = as_stream(stream);
+    switch (elem_bytes)
+    {
+    case 1: broadcast_kernel<uint8_t><<<blocks_for(n), 256, 0, s>>>(static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), n, bi); break;
+    case 4: broadcast_kernel<uint32_t><<<blocks_for(n), 256, 0, s>>>(static_cast<const uint32_t*>(in), static_cast<uint32_t*>(out), n, bi); break;
+    case 8: broadcast_kernel<uint64_t><<<blocks_for(n), 256, 0, s>>>(static_cast<const uint64_t*>(in), static_cast<uint64_t*>(out), n, bi); break;
+    default: return fail(HIPQ_ERR_UNSUPPORTED, "%d-byte elements", elem_bytes);
+    }
+    return check_launch("broadcast");
+}
+
+int hipq_permute(int32_t elem_bytes, const void* in, void* out, int32_t rank, const int64_t* in_shape, const int32_t* order, void* stream)
+{
+    HIPQ_REQUIRE(rank >= 0 && rank <= HIPQ_MAX_RANK, "rank %d out of range", rank);
+    HIPQ_REQUIRE(rank == 0 || (in_shape && order), "shape or order is null");
+    int64_t stride[HIPQ_MAX_RANK];
+    int64_t n = 1;
+    for (int i = rank - 1; i >= 0; --i)
+    {
+        HIPQ_REQUIRE(in_shape[i] >= 0, "negative extent");
+        stride[i] = n;
+        n *= in_shape[i];
+    }
+    PermuteInfo pi;
+    pi.rank = rank;
+    uint32_t seen = 0;
+    for (int i = 0; i < HIPQ_MAX_RANK; ++i)
+    {
+        pi.out_shape[i] = 1;
+        pi.in_stride[i] = 0;
+    }
+    for (int i = 0; i < rank; ++i)
+    {
+        HIPQ_REQUIRE(order[i] >= 0 && order[i] < rank && !(seen & (1u << order[i])), "order is not a permutation");
+        seen |= 1u << order[i];
+        pi.out_shape[i] = in_shape[order[i]];
+        pi.in_stride[i] = stride[order[i]];
+    }
+    if (n == 0)
+        return HIPQ_OK;
+    HIPQ_REQUIRE(in && out, "null tensor pointer");
+    hipStream_t s = as_stream(stream);
+    switch (elem_bytes)
+    {
+    case 1: permute_kernel<uint8_t><<<blocks_for(n), 256, 0, s>>>(static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), n, pi); break;
+    case 4: permute_kernel<uint32_t><<<blocks_for(n), 256, 0, s>>>(static_cast<const uint32_t*>(in), static_cast<uint32_t*>(out), n, pi); break;
+    case 8: permute_kernel<uint64_t><<<blocks_for(n), 256, 0, s>>>(static_cast<const uint64_t*>(in), static_cast<uint64_t*>(out), n, pi); break;
+    default: return fail(HIPQ_ERR_UNSUPPORTED, "%d-byte elements", elem_bytes);
+    }
+    return check_launch("permute");
+}
+}

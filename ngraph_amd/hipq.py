@@ -236,6 +236,11 @@ EXPORTS = [
     "hipq_quantized_dot_bias",
     "hipq_transpose_ncx_to_nxc",
     "hipq_transpose_nxc_to_ncx",
+    "hipq_binary",
+    "hipq_unary",
+    "hipq_convert",
+    "hipq_broadcast",
+    "hipq_permute",
     "hipq_last_kernel",
 ]
 
@@ -292,6 +297,11 @@ def load():
     lib.hipq_quantized_dot_bias.argtypes = [C.POINTER(DotDesc), C.POINTER(FusedDesc)] + [vp] * 7
     for n in ("hipq_transpose_ncx_to_nxc", "hipq_transpose_nxc_to_ncx"):
         getattr(lib, n).argtypes = [vp, vp, i64, i64, i64, i32, vp]
+    lib.hipq_binary.argtypes = [i32, i32, vp, i64, vp, i64, vp, i64, vp]
+    lib.hipq_unary.argtypes = [i32, i32, vp, vp, i64, vp]
+    lib.hipq_convert.argtypes = [i32, i32, vp, vp, i64, vp]
+    lib.hipq_broadcast.argtypes = [i32, vp, vp, i32, C.POINTER(C.c_int64), C.c_uint32, vp]
+    lib.hipq_permute.argtypes = [i32, vp, vp, i32, C.POINTER(C.c_int64), C.POINTER(C.c_int32), vp]
     _lib = lib
     return lib
 

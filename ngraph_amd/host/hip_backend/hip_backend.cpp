@@ -1,0 +1,723 @@
+// The "HIP" nGraph backend: runtime::Backend / Executable / Tensor over the C ABI of libhipq.so.
+//
+// This file never includes a HIP header; the GPU is reached only through include/hipq.h.
+// Structure follows the reference's minimal plugins (src/runtime/nop/nop_backend.cpp:36-81 for the
+// registration seam, src/ngraph/runtime/interpreter/int_executable.cpp:63-278 for compile / call):
+// compile() clones the function, folds the constant scale sub-graphs, and lowers the ordered ops to
+// a flat list of launches over device buffers; call() binds parameter / result tensors and replays
+// the list on one stream.
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <unordered_map>
+
+#include "hipq.h"
+#include "ngraph/ngraph.hpp"
+
+using namespace std;
+using namespace ngraph;
+
+#define HIP_BACKEND_API __attribute__((visibility("default")))
+
+namespace
+{
+    void check(int rc, const char* what)
+    {
+        if (rc != HIPQ_OK)
+        {
+            string msg = string(what) + ": " + hipq_last_error();
+            if (rc == HIPQ_ERR_UNSUPPORTED)
+                throw unsupported_op(msg);
+            throw ngraph_error(msg);
+        }
+    }
+
+    int dtype_of(const element::Type& t)
+    {
+        switch (t.get_type_enum())
+        {
+        case element::Type_t::u8:
+        case element::Type_t::boolean: return HIPQ_U8;
+        case element::Type_t::i8: return HIPQ_I8;
+        case element::Type_t::i32: return HIPQ_I32;
+        case element::Type_t::f32: return HIPQ_F32;
+        case element::Type_t::f64: return HIPQ_F64;
+        default: throw unsupported_op("HIP backend: unsupported element type " + t.get_type_name());
+        }
+    }
+
+    // ------------------------------------------------------------------ tensor
+    class HIPTensor : public runtime::Tensor
+    {
+    public:
+        HIPTensor(const element::Type& et, const Shape& shape, void* device_memory = nullptr)
+            : runtime::Tensor(make_shared<descriptor::Tensor>(et, shape, "external")), m_ptr(device_memory), m_owned(device_memory == nullptr)
+        {
+            if (m_owned)
+                check(hipq_malloc(&m_ptr, get_size_in_bytes()), "HIPTensor allocation");
+        }
+        ~HIPTensor() override
+        {
+            if (m_owned)
+                hipq_free(m_ptr);
+        }
+        void write(const void* p, size_t n) override
+        {
+            if (n != get_size_in_bytes())
+                throw out_of_range("partial tensor write not supported");
+            if (n && !p)
+                throw runtime_error("HIPTensor::write: null source");
+            check(hipq_memcpy_h2d(m_ptr, p, n, nullptr), "HIPTensor::write");
+        }
+        void read(void* p, size_t n) const override
+        {
+            if (n != get_size_in_bytes())
+                throw out_of_range("partial tensor read access not supported");
+            if (n && !p)
+                throw runtime_error("HIPTensor::read: null destination");
+            check(hipq_memcpy_d2h(p, m_ptr, n, nullptr), "HIPTensor::read");
+        }
+        void copy_from(const runtime::Tensor& source) override
+        {
+            auto src = dynamic_cast<const HIPTensor*>(&source);
+            if (!src)
+                return runtime::Tensor::copy_from(source);
+            if (get_element_count() != source.get_element_count())
+                throw invalid_argument("runtime::Tensor::copy_from: element count does not match");
+            if (get_element_type() != source.get_element_type())
+                throw invalid_argument("runtime::Tensor::copy_from: element types do not match");
+            check(hipq_memcpy_d2d(m_ptr, src->m_ptr, get_size_in_bytes(), nullptr), "HIPTensor::copy_from");
+            check(hipq_stream_sync(nullptr), "HIPTensor::copy_from");
+        }
+        void* device_ptr() const { return m_ptr; }
+
+    private:
+        void* m_ptr;
+        bool m_owned;
+    };
+
+    // device allocation released with the executable
+    struct DeviceBlock
+    {
+        void* ptr = nullptr;
+        explicit DeviceBlock(size_t bytes) { check(hipq_malloc(&ptr, bytes), "device allocation"); }
+        ~DeviceBlock() { hipq_free(ptr); }
+        DeviceBlock(const DeviceBlock&) = delete;
+        DeviceBlock& operator=(const DeviceBlock&) = delete;
+    };
+
+    // ------------------------------------------------------------------ executable
+    struct Step
+    {
+        shared_ptr<Node> node;
+        vector<int> inputs; // value ids
+        int output = -1;    // value id
+        // launch(input pointers, output pointer, stream)
+        function<void(const vector<void*>&, void*, void*)> launch;
+    };
+
+    class HIPExecutable : public runtime::Executable
+    {
+    public:
+        HIPExecutable(const shared_ptr<Function>& func, int device, bool enable_performance_data);
+        ~HIPExecutable() override;
+        bool call(const vector<shared_ptr<runtime::Tensor>>& outputs, const vector<shared_ptr<runtime::Tensor>>& inputs) override;
+        vector<runtime::PerformanceCounter> get_performance_data() const override;
+        shared_ptr<runtime::Tensor> create_input_tensor(size_t i) override
+        {
+            return make_shared<HIPTensor>(m_parameters.at(i)->get_output_element_type(0), m_parameters.at(i)->get_output_shape(0));
+        }
+        shared_ptr<runtime::Tensor> create_output_tensor(size_t i) override
+        {
+            return make_shared<HIPTensor>(m_results.at(i)->get_output_element_type(0), m_results.at(i)->get_output_shape(0));
+        }
+        shared_ptr<runtime::Tensor> create_input_tensor(size_t i, void* p) override
+        {
+            return make_shared<HIPTensor>(m_parameters.at(i)->get_output_element_type(0), m_parameters.at(i)->get_output_shape(0), p);
+        }
+        shared_ptr<runtime::Tensor> create_output_tensor(size_t i, void* p) override
+        {
+            return make_shared<HIPTensor>(m_results.at(i)->get_output_element_type(0), m_results.at(i)->get_output_shape(0), p);
+        }
+
+    private:
+        int value_of(const Output<Node>& o) const { return m_value_of.at(o.get_node()); }
+        void* constant_ptr(const Output<Node>& o) const;
+        void lower(const shared_ptr<Node>& n);
+        void lower_conv(const shared_ptr<Node>& n, Step& st);
+        void lower_dot(const shared_ptr<Node>& n, Step& st);
+        shared_ptr<DeviceBlock> alloc(size_t bytes)
+        {
+            auto b = make_shared<DeviceBlock>(bytes ? bytes : 1);
+            m_blocks.push_back(b);
+            return b;
+        }
+
+        int m_device;
+        bool m_perf;
+        shared_ptr<Function> m_function;
+        unordered_map<const Node*, int> m_value_of; // node (output 0) -> value id
+        vector<void*> m_value_ptr;                  // persistent device pointer, or null when bound per call
+        vector<size_t> m_value_bytes;
+        vector<int> m_value_uses;
+        vector<int> m_param_value, m_result_value;
+        vector<Step> m_steps;
+        vector<shared_ptr<DeviceBlock>> m_blocks;
+        void* m_stream = nullptr;
+        mutex m_mutex;
+        // performance data
+        vector<void*> m_events;
+        vector<double> m_step_us;
+        size_t m_calls = 0;
+    };
+
+    void* HIPExecutable::constant_ptr(const Output<Node>& o) const { return m_value_ptr.at(value_of(o)); }
+
+    bool constant_is_zero(const Output<Node>& o)
+    {
+        auto c = as_type_ptr<op::v0::Constant>(o.get_node_shared_ptr());
+        if (!c)
+            return false;
+        for (double v : c->get_values_as_double())
+            if (v != 0.0)
+                return false;
+        return true;
+    }
+
+    void fill_conv_desc(hipq_conv_desc_t& d, const Node& n, const op::v0::ConvAttributes& a)
+    {
+        memset(&d, 0, sizeof(d));
+        const Shape& ds = n.get_input_shape(0);
+        const Shape& fs = n.get_input_shape(1);
+        const Shape& os = n.get_output_shape(0);
+        const size_t ns = ds.size() - 2;
+        if (ns < 1 || ns > HIPQ_MAX_SPATIAL)
+            throw unsupported_op("HIP backend: convolution with " + to_string(ns) + " spatial dimensions");
+        d.n_spatial = static_cast<int32_t>(ns);
+        d.data_t = dtype_of(n.get_input_element_type(0));
+        d.filter_t = dtype_of(n.get_input_element_type(1));
+        d.out_t = dtype_of(n.get_output_element_type(0));
+        d.data_layout = HIPQ_LAYOUT_NCX;
+        d.out_layout = HIPQ_LAYOUT_NCX;
+        d.N = static_cast<int64_t>(ds[0]);
+        d.C = static_cast<int64_t>(ds[1]);
+        d.K = static_cast<int64_t>(fs[0]);
+        for (size_t i = 0; i < HIPQ_MAX_SPATIAL; ++i)
+        {
+            d.in_sp[i] = d.f_sp[i] = d.out_sp[i] = d.stride[i] = d.dilation[i] = d.data_dilation[i] = 1;
+            d.pad_below[i] = d.pad_above[i] = 0;
+        }
+        for (size_t i = 0; i < ns; ++i)
+        {
+            d.in_sp[i] = static_cast<int64_t>(ds[2 + i]);
+            d.f_sp[i] = static_cast<int64_t>(fs[2 + i]);
+            d.out_sp[i] = static_cast<int64_t>(os[2 + i]);
+            d.stride[i] = static_cast<int64_t>(a.get_window_movement_strides()[i]);
+            d.dilation[i] = static_cast<int64_t>(a.get_window_dilation_strides()[i]);
+            d.data_dilation[i] = static_cast<int64_t>(a.get_data_dilation_strides()[i]);
+            d.pad_below[i] = a.get_padding_below()[i];
+            d.pad_above[i] = a.get_padding_above()[i];
+        }
+    }
+
+    void HIPExecutable::lower_conv(const shared_ptr<Node>& n, Step& st)
+    {
+        const op::v0::ConvAttributes* attrs = nullptr;
+        // input positions per op (src/ngraph/op/experimental/quantized_conv_bias.cpp, quantized_conv_relu.cpp)
+        int bias_i = -1, sum_i = -1, scale_i = -1, sum_scale_i = -1;
+        bool relu = false, plain = false;
+        int sum_t = HIPQ_U8;
+        if (auto q = as_type_ptr<op::v0::QuantizedConvolution>(n))
+        {
+            attrs = q.get();
+            plain = true;
+        }
+        else if (auto qb = as_type_ptr<op::v0::QuantizedConvolutionBias>(n))
+        {
+            attrs = qb.get();
+            bias_i = 2, scale_i = 3, relu = qb->with_relu();
+        }
+        else if (auto qr = as_type_ptr<op::v0::QuantizedConvolutionRelu>(n))
+        {
+            attrs = qr.get();
+            scale_i = 2, relu = true;
+        }
+        else if (auto qa = as_type_ptr<op::v0::QuantizedConvolutionBiasAdd>(n))
+        {
+            attrs = qa.get();
+            bias_i = 2, sum_i = 3, scale_i = 4, sum_scale_i = 5, relu = qa->with_relu();
+        }
+        else if (auto qs = as_type_ptr<op::v0::QuantizedConvolutionBiasSignedAdd>(n))
+        {
+            attrs = qs.get();
+            bias_i = 2, sum_i = 3, scale_i = 4, sum_scale_i = 5, relu = qs->with_relu();
+        }
+        hipq_conv_desc_t d;
+        fill_conv_desc(d, *n, *attrs);
+        if (sum_i >= 0)
+            sum_t = dtype_of(n->get_input_element_type(sum_i));
+
+        // A constant filter whose zero point is a constant 0 (the fused ops have none) is packed
+        // once here; the nGraph CPU backend makes the same demand of its fast path
+        // (src/ngraph/runtime/cpu/pass/cpu_assignment.cpp:801-825).
+        shared_ptr<DeviceBlock> packed;
+        const bool filter_const = n->get_argument(1)->is_constant();
+        const bool zp_zero = plain ? constant_is_zero(n->input_value(5)) : true;
+        size_t packed_bytes = hipq_conv_packed_filter_bytes(&d);
+        if (filter_const && zp_zero && packed_bytes)
+        {
+            packed = alloc(packed_bytes);
+            check(hipq_conv_pack_filter(&d, constant_ptr(n->input_value(1)), packed->ptr, m_stream), "filter packing");
+        }
+
+        if (plain)
+        {
+            st.launch = [d, packed](const vector<void*>& in, void* out, void* stream) {
+                check(hipq_quantized_convolution(&d, in[0], in[1], packed ? packed->ptr : nullptr, static_cast<const float*>(in[2]), in[3],
+                                                 static_cast<const float*>(in[4]), in[5], static_cast<const float*>(in[6]), in[7], out, stream),
+                      "QuantizedConvolution");
+            };
+            return;
+        }
+        hipq_fused_desc_t f;
+        memset(&f, 0, sizeof(f));
+        f.has_bias = bias_i >= 0;
+        f.has_sum = sum_i >= 0;
+        f.sum_t = sum_t;
+        f.with_relu = relu;
+        f.scale_count = static_cast<int64_t>(shape_size(n->get_input_shape(scale_i)));
+        if (f.scale_count != 1 && f.scale_count != d.K)
+            throw ngraph_error("HIP backend: requantization scale must be a scalar or have one entry per output channel");
+        if (sum_scale_i >= 0 && shape_size(n->get_input_shape(sum_scale_i)) != 1)
+            throw ngraph_error("HIP backend: sum scale must be a scalar");
+        const string name = n->get_type_name();
+        st.launch = [d, f, packed, bias_i, sum_i, scale_i, sum_scale_i, name](const vector<void*>& in, void* out, void* stream) {
+            check(hipq_quantized_convolution_fused(&d, &f, in[0], in[1], packed ? packed->ptr : nullptr,
+                                                   bias_i >= 0 ? static_cast<const int32_t*>(in[bias_i]) : nullptr,
+                                                   sum_i >= 0 ? in[sum_i] : nullptr, static_cast<const float*>(in[scale_i]),
+                                                   sum_scale_i >= 0 ? static_cast<const float*>(in[sum_scale_i]) : nullptr, out, stream),
+                  name.c_str());
+        };
+    }
+
+    void HIPExecutable::lower_dot(const shared_ptr<Node>& n, Step& st)
+    {
+        hipq_dot_desc_t d;
+        memset(&d, 0, sizeof(d));
+        const Shape& s0 = n->get_input_shape(0);
+        const Shape& s1 = n->get_input_shape(1);
+        d.a_t = dtype_of(n->get_input_element_type(0));
+        d.b_t = dtype_of(n->get_input_element_type(1));
+        d.out_t = dtype_of(n->get_output_element_type(0));
+        if (auto q = as_type_ptr<op::v0::QuantizedDot>(n))
+        {
+            // the INTERPRETER runs every QuantizedDot with one reduction axis (int_executable.hpp:1583)
+            if (q->get_reduction_axes_count() != 1)
+                throw unsupported_op("HIP backend: QuantizedDot with reduction_axes_count != 1");
+            d.b_layout = HIPQ_B_KN;
+            d.K = static_cast<int64_t>(s1.at(0));
+            d.M = static_cast<int64_t>(shape_size(s0) / (s0.empty() ? 1 : s0.back() ? s0.back() : 1));
+            d.N = static_cast<int64_t>(shape_size(s1) / (s1[0] ? s1[0] : 1));
+            shared_ptr<DeviceBlock> packed;
+            size_t pb = hipq_dot_packed_bytes(&d);
+            if (pb && n->get_argument(1)->is_constant() && constant_is_zero(n->input_value(5)))
+            {
+                packed = alloc(pb);
+                check(hipq_dot_pack(&d, constant_ptr(n->input_value(1)), packed->ptr, m_stream), "QuantizedDot operand packing");
+            }
+            st.launch = [d, packed](const vector<void*>& in, void* out, void* stream) {
+                // without a prepacked operand the direct kernel runs unless the zero point is known to be 0
+                check(hipq_quantized_dot(&d, in[0], in[1], packed ? packed->ptr : nullptr, static_cast<const float*>(in[2]), in[3],
+                                         static_cast<const float*>(in[4]), in[5], static_cast<const float*>(in[6]), in[7], out, stream),
+                      "QuantizedDot");
+            };
+            return;
+        }
+        auto qb = as_type_ptr<op::v0::QuantizedDotBias>(n);
+        d.b_layout = HIPQ_B_NK;
+        d.M = static_cast<int64_t>(s0.at(0));
+        d.K = static_cast<int64_t>(s0.at(1));
+        d.N = static_cast<int64_t>(s1.at(0));
+        hipq_fused_desc_t f;
+        memset(&f, 0, sizeof(f));
+        f.has_bias = 1;
+        f.with_relu = qb->with_relu();
+        f.scale_count = static_cast<int64_t>(shape_size(n->get_input_shape(3)));
+        if (f.scale_count != 1 && f.scale_count != d.N)
+            throw ngraph_error("HIP backend: QuantizedDotBias scale must be a scalar or have one entry per output column");
+        shared_ptr<DeviceBlock> packed;
+        size_t pb = hipq_dot_packed_bytes(&d);
+        if (pb && n->get_argument(1)->is_constant())
+        {
+            packed = alloc(pb);
+            check(hipq_dot_pack(&d, constant_ptr(n->input_value(1)), packed->ptr, m_stream), "QuantizedDotBias weight packing");
+        }
+        st.launch = [d, f, packed](const vector<void*>& in, void* out, void* stream) {
+            check(hipq_quantized_dot_bias(&d, &f, in[0], in[1], packed ? packed->ptr : nullptr, static_cast<const int32_t*>(in[2]),
+                                          static_cast<const float*>(in[3]), out, stream),
+                  "QuantizedDotBias");
+        };
+    }
+
+    int binary_code(const Node& n)
+    {
+        const auto& ti = n.get_type_info();
+        if (ti == op::v1::Add::type_info)
+            return HIPQ_OP_ADD;
+        if (ti == op::v1::Subtract::type_info)
+            return HIPQ_OP_SUBTRACT;
+        if (ti == op::v1::Multiply::type_info)
+            return HIPQ_OP_MULTIPLY;
+        if (ti == op::v1::Divide::type_info)
+            return HIPQ_OP_DIVIDE;
+        if (ti == op::v1::Maximum::type_info)
+            return HIPQ_OP_MAXIMUM;
+        if (ti == op::v1::Minimum::type_info)
+            return HIPQ_OP_MINIMUM;
+        return -1;
+    }
+
+    bool backend_supports(const Node& n)
+    {
+        static const vector<NodeTypeInfo> ops = {
+            op::v0::Parameter::type_info, op::v0::Constant::type_info, op::v0::Result::type_info, op::v0::Quantize::type_info,
+            op::v0::Dequantize::type_info, op::v0::QuantizedConvolution::type_info, op::v0::QuantizedConvolutionBias::type_info,
+            op::v0::QuantizedConvolutionRelu::type_info, op::v0::QuantizedConvolutionBiasAdd::type_info,
+            op::v0::QuantizedConvolutionBiasSignedAdd::type_info, op::v0::QuantizedDot::type_info, op::v0::QuantizedDotBias::type_info,
+            op::v0::Abs::type_info, op::v0::Relu::type_info, op::v0::Convert::type_info, op::v0::Broadcast::type_info,
+            op::v0::Reshape::type_info, op::v1::Add::type_info, op::v1::Subtract::type_info, op::v1::Multiply::type_info,
+            op::v1::Divide::type_info, op::v1::Maximum::type_info, op::v1::Minimum::type_info};
+        for (const auto& ti : ops)
+            if (n.get_type_info() == ti)
+                return true;
+        return false;
+    }
+
+    void HIPExecutable::lower(const shared_ptr<Node>& n)
+    {
+        if (!backend_supports(*n))
+            throw unsupported_op(string("Unsupported op '") + n->description() + "'");
+        if (n->get_output_size() != 1)
+            throw unsupported_op(string("HIP backend: op '") + n->description() + "' with " + to_string(n->get_output_size()) + " outputs");
+        const auto et = n->get_output_element_type(0);
+        const size_t bytes = shape_size(n->get_output_shape(0)) * et.size();
+        const int id = static_cast<int>(m_value_ptr.size());
+
+        if (n->is_output())
+        {
+            // a Result aliases the value it returns
+            m_value_of[n.get()] = value_of(n->input_value(0));
+            m_value_uses[value_of(n->input_value(0))] += 1;
+            return;
+        }
+        m_value_of[n.get()] = id;
+        m_value_ptr.push_back(nullptr);
+        m_value_bytes.push_back(bytes);
+        m_value_uses.push_back(0);
+        if (n->is_parameter())
+            return; // bound per call
+        if (auto c = as_type_ptr<op::v0::Constant>(n))
+        {
+            auto block = alloc(bytes);
+            check(hipq_memcpy_h2d(block->ptr, c->get_data_ptr(), bytes, m_stream), "constant upload");
+            m_value_ptr[id] = block->ptr;
+            return;
+        }
+        m_value_ptr[id] = alloc(bytes)->ptr;
+
+        Step st;
+        st.node = n;
+        st.output = id;
+        for (size_t i = 0; i < n->get_input_size(); ++i)
+        {
+            if (n->input_value(i).get_index() != 0)
+                throw unsupported_op("HIP backend: multi-output producers are not supported");
+            st.inputs.push_back(value_of(n->input_value(i)));
+            m_value_uses[st.inputs.back()] += 1;
+        }
+        const int64_t count = static_cast<int64_t>(shape_size(n->get_output_shape(0)));
+        const int dt = dtype_of(et);
+
+        if (auto q = as_type_ptr<op::v0::Quantize>(n))
+        {
+            hipq_quant_desc_t d;
+            memset(&d, 0, sizeof(d));
+            d.real_t = dtype_of(n->get_input_element_type(0));
+            d.quant_t = dt;
+            d.round_mode = static_cast<int32_t>(q->get_round_mode());
+            const Shape& s = n->get_input_shape(0);
+            if (s.size() > HIPQ_MAX_RANK)
+                throw unsupported_op("HIP backend: Quantize rank beyond 8");
+            d.rank = static_cast<int32_t>(s.size());
+            for (size_t i = 0; i < s.size(); ++i)
+                d.shape[i] = static_cast<int64_t>(s[i]);
+            for (size_t a : q->get_axes())
+                d.axes_mask |= 1u << a;
+            st.launch = [d](const vector<void*>& in, void* out, void* stream) { check(hipq_quantize(&d, in[0], in[1], in[2], out, stream), "Quantize"); };
+        }
+        else if (auto dq = as_type_ptr<op::v0::Dequantize>(n))
+        {
+            hipq_quant_desc_t d;
+            memset(&d, 0, sizeof(d));
+            d.real_t = dt;
+            d.quant_t = dtype_of(n->get_input_element_type(0));
+            const Shape& s = n->get_input_shape(0);
+            if (s.size() > HIPQ_MAX_RANK)
+                throw unsupported_op("HIP backend: Dequantize rank beyond 8");
+            d.rank = static_cast<int32_t>(s.size());
+            for (size_t i = 0; i < s.size(); ++i)
+                d.shape[i] = static_cast<int64_t>(s[i]);
+            for (size_t a : dq->get_axes())
+                d.axes_mask |= 1u << a;
+            st.launch = [d](const vector<void*>& in, void* out, void* stream) { check(hipq_dequantize(&d, in[0], in[1], in[2], out, stream), "Dequantize"); };
+        }
+        else if (is_type<op::v0::QuantizedConvolution>(n) || is_type<op::v0::QuantizedConvolutionBias>(n) ||
+                 is_type<op::v0::QuantizedConvolutionRelu>(n) || is_type<op::v0::QuantizedConvolutionBiasAdd>(n) ||
+                 is_type<op::v0::QuantizedConvolutionBiasSignedAdd>(n))
+        {
+            lower_conv(n, st);
+        }
+        else if (is_type<op::v0::QuantizedDot>(n) || is_type<op::v0::QuantizedDotBias>(n))
+        {
+            lower_dot(n, st);
+        }
+        else if (binary_code(*n) >= 0)
+        {
+            const int op = binary_code(*n);
+            const int64_t an = static_cast<int64_t>(shape_size(n->get_input_shape(0)));
+            const int64_t bn = static_cast<int64_t>(shape_size(n->get_input_shape(1)));
+            st.launch = [op, dt, an, bn, count](const vector<void*>& in, void* out, void* stream) {
+                check(hipq_binary(op, dt, in[0], an == count ? an : 1, in[1], bn == count ? bn : 1, out, count, stream), "elementwise");
+            };
+        }
+        else if (is_type<op::v0::Abs>(n) || is_type<op::v0::Relu>(n))
+        {
+            const int op = is_type<op::v0::Abs>(n) ? HIPQ_OP_ABS : HIPQ_OP_RELU;
+            st.launch = [op, dt, count](const vector<void*>& in, void* out, void* stream) { check(hipq_unary(op, dt, in[0], out, count, stream), "unary"); };
+        }
+        else if (is_type<op::v0::Convert>(n))
+        {
+            const int it = dtype_of(n->get_input_element_type(0));
+            st.launch = [it, dt, count](const vector<void*>& in, void* out, void* stream) { check(hipq_convert(it, dt, in[0], out, count, stream), "Convert"); };
+        }
+        else if (auto b = as_type_ptr<op::v0::Broadcast>(n))
+        {
+            const Shape& s = b->get_broadcast_shape();
+            if (s.size() > HIPQ_MAX_RANK)
+                throw unsupported_op("HIP backend: Broadcast rank beyond 8");
+            vector<int64_t> shape(s.begin(), s.end());
+            uint32_t mask = 0;
+            for (size_t a : b->get_broadcast_axes())
+                mask |= 1u << a;
+            const int eb = static_cast<int>(et.size());
+            st.launch = [shape, mask, eb](const vector<void*>& in, void* out, void* stream) {
+                check(hipq_broadcast(eb, in[0], out, static_cast<int32_t>(shape.size()), shape.data(), mask, stream), "Broadcast");
+            };
+        }
+        else if (auto r = as_type_ptr<op::v0::Reshape>(n))
+        {
+            const Shape& s = n->get_input_shape(0);
+            if (s.size() > HIPQ_MAX_RANK)
+                throw unsupported_op("HIP backend: Reshape rank beyond 8");
+            vector<int64_t> shape(s.begin(), s.end());
+            vector<int32_t> order(r->get_input_order().begin(), r->get_input_order().end());
+            const int eb = static_cast<int>(et.size());
+            st.launch = [shape, order, eb](const vector<void*>& in, void* out, void* stream) {
+                check(hipq_permute(eb, in[0], out, static_cast<int32_t>(shape.size()), shape.data(), order.data(), stream), "Reshape");
+            };
+        }
+        else
+        {
+            throw unsupported_op(string("Unsupported op '") + n->description() + "'");
+        }
+        m_steps.push_back(move(st));
+    }
+
+    HIPExecutable::HIPExecutable(const shared_ptr<Function>& func, int device, bool enable_performance_data)
+        : m_device(device), m_perf(enable_performance_data)
+    {
+        check(hipq_set_device(m_device), "HIP backend");
+        check(hipq_stream_create(&m_stream), "stream creation");
+        // work on a private copy: compile must not change the caller's graph
+        m_function = clone_function(*func);
+        pass::Manager pm;
+        pm.register_pass<pass::ConstantFolding>();
+        pm.run_passes(m_function);
+        for (const auto& n : m_function->get_ordered_ops())
+            lower(n);
+        for (const auto& p : m_function->get_parameters())
+            m_param_value.push_back(m_value_of.at(p.get()));
+        for (const auto& r : m_function->get_results())
+            m_result_value.push_back(m_value_of.at(r.get()));
+        check(hipq_stream_sync(m_stream), "compile-time uploads");
+        if (m_perf)
+        {
+            m_events.resize(m_steps.size() + 1, nullptr);
+            for (auto& e : m_events)
+                check(hipq_event_create(&e), "event creation");
+            m_step_us.assign(m_steps.size(), 0.0);
+        }
+        // validation is against the caller's function (same parameter / result signature)
+        set_parameters_and_results(*func);
+    }
+
+    HIPExecutable::~HIPExecutable()
+    {
+        for (auto e : m_events)
+            hipq_event_destroy(e);
+        if (m_stream)
+        {
+            hipq_stream_sync(m_stream);
+            hipq_stream_destroy(m_stream);
+        }
+    }
+
+    bool HIPExecutable::call(const vector<shared_ptr<runtime::Tensor>>& outputs, const vector<shared_ptr<runtime::Tensor>>& inputs)
+    {
+        lock_guard<mutex> lock(m_mutex);
+        check(hipq_set_device(m_device), "HIP backend");
+        if (inputs.size() != m_param_value.size() || outputs.size() != m_result_value.size())
+            throw runtime_error("HIP backend: wrong number of call arguments");
+        vector<void*> ptr = m_value_ptr;
+        for (size_t i = 0; i < inputs.size(); ++i)
+        {
+            auto t = dynamic_pointer_cast<HIPTensor>(inputs[i]);
+            if (!t)
+                throw runtime_error("HIP backend: input " + to_string(i) + " is not a tensor of this backend");
+            ptr[m_param_value[i]] = t->device_ptr();
+        }
+        // a value consumed only by one Result is produced straight into the caller's tensor
+        vector<void*> out_ptr(outputs.size());
+        vector<bool> direct(outputs.size(), false);
+        for (size_t i = 0; i < outputs.size(); ++i)
+        {
+            auto t = dynamic_pointer_cast<HIPTensor>(outputs[i]);
+            if (!t)
+                throw runtime_error("HIP backend: output " + to_string(i) + " is not a tensor of this backend");
+            out_ptr[i] = t->device_ptr();
+            const int v = m_result_value[i];
+            const Node* producer = m_function->get_results()[i]->input_value(0).get_node();
+            if (m_value_uses[v] == 1 && !producer->is_parameter() && !producer->is_constant())
+            {
+                ptr[v] = out_ptr[i];
+                direct[i] = true;
+            }
+        }
+        vector<void*> in;
+        for (size_t s = 0; s < m_steps.size(); ++s)
+        {
+            const Step& st = m_steps[s];
+            in.clear();
+            for (int v : st.inputs)
+                in.push_back(ptr[v]);
+            if (m_perf)
+                check(hipq_event_record(m_events[s], m_stream), "event record");
+            st.launch(in, ptr[st.output], m_stream);
+        }
+        if (m_perf)
+            check(hipq_event_record(m_events[m_steps.size()], m_stream), "event record");
+        for (size_t i = 0; i < outputs.size(); ++i)
+            if (!direct[i])
+                check(hipq_memcpy_d2d(out_ptr[i], ptr[m_result_value[i]], m_value_bytes[m_result_value[i]], m_stream), "result copy");
+        check(hipq_stream_sync(m_stream), "Executable::call");
+        if (m_perf)
+        {
+            for (size_t s = 0; s < m_steps.size(); ++s)
+            {
+                float ms = 0;
+                check(hipq_event_elapsed_ms(m_events[s], m_events[s + 1], &ms), "event timing");
+                m_step_us[s] += ms * 1e3;
+            }
+            ++m_calls;
+        }
+        for (auto& t : outputs)
+            t->set_stale(false);
+        return true;
+    }
+
+    vector<runtime::PerformanceCounter> HIPExecutable::get_performance_data() const
+    {
+        vector<runtime::PerformanceCounter> rc;
+        if (m_perf)
+            for (size_t s = 0; s < m_steps.size(); ++s)
+                rc.emplace_back(m_steps[s].node, static_cast<size_t>(m_step_us[s]), m_calls);
+        return rc;
+    }
+
+    // ------------------------------------------------------------------ backend
+    class HIPBackend : public runtime::Backend
+    {
+    public:
+        explicit HIPBackend(const string& config) : m_device(0)
+        {
+            // "HIP:<device ordinal>"
+            if (!config.empty())
+            {
+                size_t used = 0;
+                try
+                {
+                    m_device = stoi(config, &used);
+                }
+                catch (const exception&)
+                {
+                    used = 0;
+                }
+                if (used != config.size() || m_device < 0)
+                    throw runtime_error("HIP backend: cannot read device ordinal from '" + config + "'");
+            }
+            int rc = hipq_set_device(m_device);
+            if (rc != HIPQ_OK)
+                throw runtime_error(string("HIP backend: device ") + to_string(m_device) + " is not usable: " + hipq_last_error());
+        }
+        shared_ptr<runtime::Tensor> create_tensor() override { throw runtime_error("HIP backend does not support dynamic tensors"); }
+        shared_ptr<runtime::Tensor> create_tensor(const element::Type& et, const Shape& shape) override
+        {
+            use_device();
+            return make_shared<HIPTensor>(et, shape);
+        }
+        // memory_pointer is device memory owned by the caller
+        shared_ptr<runtime::Tensor> create_tensor(const element::Type& et, const Shape& shape, void* memory_pointer) override
+        {
+            use_device();
+            return make_shared<HIPTensor>(et, shape, memory_pointer);
+        }
+        shared_ptr<runtime::Executable> compile(shared_ptr<Function> func, bool enable_performance_data = false) override
+        {
+            lock_guard<mutex> lock(m_mutex);
+            auto it = m_cache.find(func);
+            if (it != m_cache.end() && !enable_performance_data)
+                return it->second;
+            auto exec = make_shared<HIPExecutable>(func, m_device, enable_performance_data);
+            if (!enable_performance_data)
+                m_cache[func] = exec;
+            return exec;
+        }
+        void remove_compiled_function(shared_ptr<runtime::Executable> exec) override
+        {
+            lock_guard<mutex> lock(m_mutex);
+            for (auto it = m_cache.begin(); it != m_cache.end(); ++it)
+                if (it->second == exec)
+                {
+                    m_cache.erase(it);
+                    break;
+                }
+        }
+        bool is_supported(const Node& node) const override { return backend_supports(node); }
+        bool is_supported_property(const Property prop) const override { return prop == Property::memory_attach; }
+        bool is_device_memory(void*) override { return true; }
+        string get_version() const override { return "hipq-" + to_string(hipq_version()); }
+
+    private:
+        void use_device() { check(hipq_set_device(m_device), "HIP backend"); }
+        int m_device;
+        mutex m_mutex;
+        map<shared_ptr<Function>, shared_ptr<runtime::Executable>> m_cache;
+    };
+}
+
+// Found by BackendManager through dlsym("ngraph_register_hip_backend")
+// (src/ngraph/runtime/backend_manager.cpp:106-113 of the nGraph tree).
+extern "C" HIP_BACKEND_API void ngraph_register_hip_backend()
+{
+    runtime::BackendManager::register_backend("HIP", [](const string& config) { return make_shared<HIPBackend>(config); });
+}

@@ -1,0 +1,43 @@
+// hip_backend_tests [--cpu | --gpu | --all] [substring]
+#include "mini_test.hpp"
+
+int main(int argc, char** argv)
+{
+    bool want_cpu = true, want_gpu = false;
+    std::string filter;
+    for (int i = 1; i < argc; ++i)
+    {
+        std::string a = argv[i];
+        if (a == "--cpu")
+            want_cpu = true, want_gpu = false;
+        else if (a == "--gpu")
+            want_cpu = false, want_gpu = true;
+        else if (a == "--all")
+            want_cpu = want_gpu = true;
+        else
+            filter = a;
+    }
+    int ran = 0;
+    for (const auto& c : mini_test::registry())
+    {
+        if ((c.needs_gpu && !want_gpu) || (!c.needs_gpu && !want_cpu))
+            continue;
+        std::string full = c.suite + "." + c.name;
+        if (!filter.empty() && full.find(filter) == std::string::npos)
+            continue;
+        std::cout << "[ RUN      ] " << full << std::endl;
+        int before = mini_test::failures();
+        try
+        {
+            c.fn();
+        }
+        catch (const std::exception& e)
+        {
+            mini_test::fail(__FILE__, __LINE__, full + " threw: " + e.what());
+        }
+        std::cout << (mini_test::failures() == before ? "[       OK ] " : "[  FAILED  ] ") << full << std::endl;
+        ++ran;
+    }
+    std::cout << ran << " tests ran, " << mini_test::failures() << " failures" << std::endl;
+    return mini_test::failures() == 0 && ran > 0 ? 0 : 1;
+}

@@ -215,7 +215,8 @@ namespace hipq
                          const void* packed,
                          const ZeroPoints& zp,
                          const Epilogue& epi,
-                         void* out_nxc,
+                         void* out,
+                         bool out_ncx, // false: out is channels-last; true: out is NCHW (written directly)
                          hipStream_t s);
     bool dot_mfma_eligible(const hipq_dot_desc_t& d);
     int launch_dot_mfma(const hipq_dot_desc_t& d,

@@ -1,0 +1,730 @@
+// int8 GEMM and implicit-GEMM convolution on the CDNA4 i8 matrix cores (v_mfma_i32_32x32x32_i8).
+//
+// out[m][n] = epilogue( sum_k (x[m][k] - x_zp) * w[n][k] )
+//   x : the activation operand.  GEMM: a row-major [M][K] matrix.  Convolution: gathered on the
+//       fly from channels-last data, m = (image, out_y, out_x), k = (filter_y, filter_x, channel).
+//   w : the weights as [N][K] int8, K contiguous (for convolution: K,spatial,C order).
+//
+// The matrix cores multiply signed by signed bytes only, so unsigned activations are biased:
+// x' = x ^ 0x80 = x - 128, and since  sum (x - zp) w = sum x' w + (128 - zp) * sum w  the
+// kernel adds (128 - zp) * wsum[n] to each accumulator.  Padding taps are materialised as the
+// byte `zp` (a real element equal to the zero point), which contributes (zp - zp) * w = 0 exactly
+// as the reference's skipped tap does.
+//
+// Work split: a workgroup of 4 wavefronts computes a BM (m) x BN (n) tile; each wavefront owns
+// WM x WN MFMA tiles of 32 x 32.  Large per-wave tiles keep LDS reads (the scarce resource next to
+// the matrix cores) low: a 128 x 64 wave tile reads 6 KiB of LDS per 8 MFMAs.  Operands are staged
+// through LDS in 64-byte K slices, double buffered: global loads of slice i+1 are in flight while
+// slice i feeds the MFMAs.  LDS rows are 64 bytes with the 16-byte chunk index XOR-swizzled by
+// (row >> 1) & 3, which makes both the 16-byte stores and the 16-byte fragment reads free of bank
+// conflicts.
+//
+// Which operand feeds MFMA source A decides what a lane's four consecutive accumulator registers
+// are: with the weights on A they are four consecutive output channels of one pixel (one 4-byte
+// store into a channels-last / row-major output); with the activations on A they are four
+// consecutive pixels of one channel (one 4-byte store into an NCHW output).
+//
+// Workgroup ids are remapped so that each of the 8 XCDs (which receive consecutive ids round-robin
+// and have private L2s) works on a contiguous range of m tiles.
+#pragma once
+#include "hipq_common.h"
+
+namespace hipq
+{
+    typedef int v4i __attribute__((ext_vector_type(4)));
+    typedef int v16i __attribute__((ext_vector_type(16)));
+
+    constexpr int BK = 64; // reduction bytes per LDS slice
+
+    __device__ __forceinline__ int lds_offset(int row, int chunk)
+    {
+        return row * BK + ((chunk ^ ((row >> 1) & 3)) << 4);
+    }
+
+    // ---- activation loaders ---------------------------------------------------------------------
+    // All tile loads are raw buffer loads: the hardware range check returns zeros for an offset
+    // beyond the buffer, so an out-of-range chunk (row beyond M, tap in the padding, K tail) is
+    // simply given the offset kOob -- no branch, and all loads of a slice issue back to back.
+    constexpr int32_t kOob = static_cast<int32_t>(0x80000000u);
+
+    __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes)
+    {
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, static_cast<int>(bytes), 0x00020000);
+    }
+
+    __device__ __forceinline__ v4i buffer_load16(__amdgpu_buffer_rsrc_t r, int32_t off)
+    {
+        return __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+    }
+
+    struct GemmX
+    {
+        const uint8_t* x;
+        int32_t K;
+        uint32_t bytes; // M * K
+
+        struct Row
+        {
+            int32_t off; // byte offset of the row, kOob when beyond M
+        };
+        struct Cursor
+        {
+            int32_t kbyte;
+        };
+        __device__ __forceinline__ void init_row(Row& r, int64_t m, int64_t M) const { r.off = m < M ? static_cast<int32_t>(m) * K : kOob; }
+        __device__ __forceinline__ void init_cursor(Cursor& c, int kbyte) const { c.kbyte = kbyte; }
+        __device__ __forceinline__ void advance(Cursor& c, int bytes_) const { c.kbyte += bytes_; }
+        __device__ __forceinline__ int32_t offset(const Row& r, const Cursor& c) const
+        {
+            return (r.off != kOob && c.kbyte < K) ? r.off + c.kbyte : kOob;
+        }
+        // slow path: exact accumulator of one output, any zero points
+        __device__ int32_t direct(int64_t m, const int8_t* wrow, int32_t xzp, int32_t wzp, bool x_unsigned) const
+        {
+            const uint8_t* p = x + m * static_cast<int64_t>(K);
+            int32_t acc = 0;
+            for (int32_t k = 0; k < K; ++k)
+            {
+                int32_t a = x_unsigned ? static_cast<int32_t>(p[k]) : static_cast<int32_t>(static_cast<int8_t>(p[k]));
+                acc += (a - xzp) * (static_cast<int32_t>(wrow[k]) - wzp);
+            }
+            return acc;
+        }
+    };
+
+    struct ConvX
+    {
+        const uint8_t* x; // [N][H][W][C]
+        int32_t H, W, C, Q, R, S, sh, sw, dh, dw, pbh, pbw;
+        int64_t PQ;
+        uint32_t bytes; // N * H * W * C
+
+        struct Row
+        {
+            int32_t base; // byte offset of the image, kOob when beyond M
+            int32_t yx;   // (top input row << 16) | (left input column & 0xffff) of the window
+        };
+        struct Cursor
+        {
+            int32_t r, s, c;
+        };
+        __device__ __forceinline__ void init_row(Row& rw, int64_t m, int64_t M) const
+        {
+            const bool valid = m < M;
+            const int64_t mm = valid ? m : 0;
+            const int64_t n = mm / PQ;
+            const int32_t rem = static_cast<int32_t>(mm - n * PQ);
+            const int32_t p = rem / Q;
+            const int32_t q = rem - p * Q;
+            rw.base = valid ? static_cast<int32_t>(n) * H * W * C : kOob;
+            rw.yx = ((p * sh - pbh) << 16) | ((q * sw - pbw) & 0xffff);
+        }
+        __device__ __forceinline__ void init_cursor(Cursor& c, int kbyte) const
+        {
+            const int tap = kbyte / C;
+            c.c = kbyte - tap * C;
+            c.r = tap / S;
+            c.s = tap - c.r * S;
+        }
+        __device__ __forceinline__ void advance(Cursor& c, int bytes_) const
+        {
+            c.c += bytes_;
+            while (c.c >= C)
+            {
+                c.c -= C;
+                if (++c.s == S)
+                {
+                    c.s = 0;
+                    ++c.r;
+                }
+            }
+        }
+        __device__ __forceinline__ int32_t offset(const Row& rw, const Cursor& c) const
+        {
+            const int32_t y = (rw.yx >> 16) + c.r * dh;
+            const int32_t xx = static_cast<int16_t>(rw.yx & 0xffff) + c.s * dw;
+            const bool ok = (rw.base != kOob) & (c.r < R) & (static_cast<uint32_t>(y) < static_cast<uint32_t>(H)) &
+                            (static_cast<uint32_t>(xx) < static_cast<uint32_t>(W));
+            return ok ? rw.base + (y * W + xx) * C + c.c : kOob;
+        }
+        __device__ int32_t direct(int64_t m, const int8_t* wrow, int32_t xzp, int32_t wzp, bool x_unsigned) const
+        {
+            Row rw;
+            init_row(rw, m, m + 1);
+            const int32_t iy0 = rw.yx >> 16, ix0 = static_cast<int16_t>(rw.yx & 0xffff);
+            int32_t acc = 0;
+            for (int32_t r = 0; r < R; ++r)
+                for (int32_t s = 0; s < S; ++s)
+                {
+                    int32_t y = iy0 + r * dh, xx = ix0 + s * dw;
+                    if (static_cast<uint32_t>(y) >= static_cast<uint32_t>(H) || static_cast<uint32_t>(xx) >= static_cast<uint32_t>(W))
+                        continue;
+                    const uint8_t* p = x + rw.base + (y * W + xx) * C;
+                    const int8_t* wp = wrow + (r * S + s) * C;
+                    for (int32_t c = 0; c < C; ++c)
+                    {
+                        int32_t a = x_unsigned ? static_cast<int32_t>(p[c]) : static_cast<int32_t>(static_cast<int8_t>(p[c]));
+                        acc += (a - xzp) * (static_cast<int32_t>(wp[c]) - wzp);
+                    }
+                }
+            return acc;
+        }
+    };
+
+    // Exact but slow tile for a non-zero weight zero point (w - wzp does not fit a signed byte).
+    struct OutMap
+    {
+        int32_t ncx;  // 1: out is [image][n][pixel], 0: out is [m][n]
+        int32_t N;
+        int64_t PQ;   // pixels per image (ncx only)
+        __device__ __forceinline__ int64_t index(int64_t m, int32_t n) const
+        {
+            if (!ncx)
+                return m * N + n;
+            int64_t img = m / PQ;
+            return (img * N + n) * PQ + (m - img * PQ);
+        }
+    };
+
+    template <class XL>
+    __device__ __noinline__ void slow_tile(const XL& xl,
+                                           const int8_t* __restrict__ w,
+                                           int64_t M,
+                                           int32_t Kred,
+                                           int32_t x_unsigned,
+                                           int32_t xzp,
+                                           int32_t wzp,
+                                           const Epilogue& epi,
+                                           const OutMap& om,
+                                           void* __restrict__ out,
+                                           int64_t m0,
+                                           int32_t n0,
+                                           int bm,
+                                           int bn)
+    {
+        const EpiRegs er = epi_load(epi);
+        for (int i = threadIdx.x; i < bm * bn; i += blockDim.x)
+        {
+            const int64_t m = m0 + i / bn;
+            const int32_t n = n0 + i % bn;
+            if (m < M && n < om.N)
+            {
+                int32_t a = xl.direct(m, w + static_cast<int64_t>(n) * Kred, xzp, wzp, x_unsigned != 0);
+                const int64_t o = om.index(m, n);
+                store_out(out, epi.out_t, o, epi_apply(epi, er, a, n, o));
+            }
+        }
+    }
+
+    // ---- lean, branch-free epilogues ------------------------------------------------------------
+    // MODE: EPI_INTERP / EPI_FUSED.  KIND: what an output element is.
+    enum
+    {
+        OUT_Q8 = 0, // u8 or i8, packed four to a dword by the caller
+        OUT_I32 = 1,
+        OUT_F32 = 2
+    };
+
+    struct EpiConst
+    {
+        float scale;      // interp scale, or the scalar fused scale
+        float sum_scale;  // fused
+        float lo, hi;     // fused saturation bounds
+        float relu_floor; // fused: 0 with relu, -inf without
+        int32_t ozp;      // interp
+        bool slow_cvt;    // interp: |round| may reach 2^31, take the x86 out-of-range rule
+    };
+
+    __device__ __forceinline__ EpiConst epi_const(const Epilogue& e)
+    {
+        EpiConst c;
+        const EpiRegs r = epi_load(e);
+        c.scale = r.scale;
+        c.sum_scale = r.sum_scale;
+        c.ozp = r.ozp;
+        c.lo = (e.out_t == HIPQ_U8) ? 0.0f : (e.out_t == HIPQ_I8 ? -128.0f : -2147483648.0f);
+        c.hi = (e.out_t == HIPQ_U8) ? 255.0f : (e.out_t == HIPQ_I8 ? 127.0f : 2147483520.0f);
+        c.relu_floor = e.relu ? 0.0f : -__builtin_huge_valf();
+        // |acc| <= 2^31, so |acc * scale| < 2^31 whenever |scale| < 1 (false for NaN)
+        c.slow_cvt = !(fabsf(r.scale) < 1.0f);
+        return c;
+    }
+
+    // INTERPRETER: (OUT) roundf(float(acc) * scale) + ozp; the caller keeps the low byte for 8-bit types
+    template <int KIND>
+    __device__ __forceinline__ int32_t epi_interp(const EpiConst& c, int32_t acc)
+    {
+        const float v = __fmul_rn(static_cast<float>(acc), c.scale);
+        // half away from zero from round-half-even: the two differ only at exact .5 ties that
+        // round-half-even took toward zero, i.e. where the residual d = v - r0 is +-0.5 with the
+        // sign of v; there the correction 2*d is exactly +-1 (d is exact: r0 is within 0.5 of v)
+        const float r0 = rintf(v);
+        const float d = __fsub_rn(v, r0);
+        const float r = (d == copysignf(0.5f, v)) ? __fadd_rn(r0, __fadd_rn(d, d)) : r0;
+        int32_t t = static_cast<int32_t>(r);
+        if (c.slow_cvt)
+            t = (!(fabsf(r) < 2147483648.0f)) ? INT32_MIN : t;
+        if (KIND == OUT_I32)
+            return static_cast<int32_t>(static_cast<uint32_t>(t) + static_cast<uint32_t>(c.ozp));
+        // narrowing first and adding the zero point afterwards is the same low byte
+        return t + c.ozp;
+    }
+
+    // oneDNN: sat(rne(relu(scale * (float(acc) + bias) (+ sum_scale * sum))))
+    template <int KIND>
+    __device__ __forceinline__ int32_t epi_fused(const EpiConst& c, int32_t acc, float bias, float scale, bool has_sum, float sum_v, bool relu)
+    {
+        float v = __fmul_rn(__fadd_rn(static_cast<float>(acc), bias), scale);
+        if (has_sum)
+            v = fmaf(c.sum_scale, sum_v, v);
+        if (KIND == OUT_F32)
+        {
+            if (relu)
+                v = (v > 0.0f) ? v : __fmul_rn(v, -0.0f);
+            return __float_as_int(v);
+        }
+        v = fmaxf(v, c.relu_floor);
+        v = fminf(fmaxf(v, c.lo), c.hi);
+        return static_cast<int32_t>(rintf(v));
+    }
+
+    __device__ __forceinline__ uint32_t pack4(const int32_t v[4])
+    {
+        return (v[0] & 0xFF) | ((v[1] & 0xFF) << 8) | ((v[2] & 0xFF) << 16) | (static_cast<uint32_t>(v[3]) << 24);
+    }
+
+    // sum input bytes of four consecutive elements -> floats
+    __device__ __forceinline__ void sum4(const void* sum_in, int sum_t, int64_t idx, bool aligned, float out[4])
+    {
+        uint32_t w;
+        if (aligned)
+            w = *reinterpret_cast<const uint32_t*>(static_cast<const uint8_t*>(sum_in) + idx);
+        else
+        {
+            const uint8_t* p = static_cast<const uint8_t*>(sum_in) + idx;
+            w = p[0] | (p[1] << 8) | (p[2] << 16) | (static_cast<uint32_t>(p[3]) << 24);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+        {
+            const uint32_t b = (w >> (8 * e)) & 0xFFu;
+            out[e] = sum_t == HIPQ_I8 ? static_cast<float>(static_cast<int8_t>(b)) : static_cast<float>(b);
+        }
+    }
+
+    // WM x WN MFMA tiles per wavefront, WAVES_M x WAVES_N wavefronts per workgroup (= 4).
+    // X_ON_A: activations feed MFMA source A (NCHW output) instead of the weights.
+    template <class XL, int WM, int WN, int WAVES_M, int WAVES_N, bool X_ON_A, int MODE, int KIND>
+    __global__ __launch_bounds__(256, 2) void igemm_i8_kernel(XL xl,
+                                                              const int8_t* __restrict__ w,
+                                                              const int32_t* __restrict__ wsum,
+                                                              int64_t M,
+                                                              int32_t Kred,
+                                                              int32_t x_unsigned,
+                                                              int32_t m_tiles,
+                                                              ZeroPoints zp,
+                                                              Epilogue epi,
+                                                              OutMap om,
+                                                              void* __restrict__ out)
+    {
+        static_assert(WAVES_M * WAVES_N == 4, "four wavefronts per workgroup");
+        constexpr int BM = WAVES_M * WM * 32;
+        constexpr int BN = WAVES_N * WN * 32;
+        constexpr int XLOADS = BM * 4 / 256; // 16-byte chunks per lane and slice
+        constexpr int WLOADS = (BN * 4 + 255) / 256;
+        constexpr int STAGE = (BM + BN) * BK;
+        extern __shared__ __attribute__((aligned(16))) uint8_t lds[]; // [2][x tile | w tile]
+
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = tid >> 6;
+        const int wn = wave % WAVES_N;
+        const int wm = wave / WAVES_N;
+        const int N = om.N;
+
+        // XCD-aware tile order: ids i, i+8, i+16, ... land on one XCD; give it consecutive m tiles
+        const int per_xcd = (m_tiles + 7) >> 3;
+        const int mt = static_cast<int>(blockIdx.x & 7) * per_xcd + static_cast<int>(blockIdx.x >> 3);
+        if (mt >= m_tiles)
+            return;
+        const int64_t m0 = static_cast<int64_t>(mt) * BM;
+        const int32_t n0 = static_cast<int32_t>(blockIdx.y) * BN;
+
+        const int32_t xzp = load_zp(zp.data_zp, zp.data_t);
+        const int32_t wzp = load_zp(zp.filter_zp, zp.filter_t);
+        if (wzp != 0) // uniform across the grid
+        {
+            slow_tile(xl, w, M, Kred, x_unsigned, xzp, wzp, epi, om, out, m0, n0, BM, BN);
+            return;
+        }
+
+        // Accumulators start at the sign-bias correction (128 - zp) * sum(w[n]) of their channel.
+        // MFMA result layout: lane holds column (source B index) lane % 32 and rows (source A
+        // index) 8*(r/4) + 4*(lane/32) + r%4 for accumulator register r.
+        const int32_t mult = (x_unsigned ? 128 : 0) - xzp;
+        v16i acc[WM][WN];
+#pragma unroll
+        for (int ni = 0; ni < WN; ++ni)
+        {
+            v16i init;
+            if (X_ON_A)
+            {
+                const int32_t n = n0 + (wn * WN + ni) * 32 + (lane & 31);
+                const int32_t c = n < N ? mult * wsum[n] : 0;
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    init[r] = c;
+            }
+            else
+            {
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                {
+                    const int32_t n = n0 + (wn * WN + ni) * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
+                    init[r] = n < N ? mult * wsum[n] : 0;
+                }
+            }
+#pragma unroll
+            for (int mi = 0; mi < WM; ++mi)
+                acc[mi][ni] = init;
+        }
+
+        {
+            const int lrow = tid >> 2;
+            const int lchunk = tid & 3;
+            const int xor_mask = x_unsigned ? static_cast<int>(0x80808080u) : 0;
+            const int fill = (xzp & 0xFF) * 0x01010101;
+
+            typename XL::Row xr[XLOADS];
+            typename XL::Cursor cur;
+#pragma unroll
+            for (int i = 0; i < XLOADS; ++i)
+                xl.init_row(xr[i], m0 + lrow + 64 * i, M);
+            xl.init_cursor(cur, lchunk * 16);
+            const __amdgpu_buffer_rsrc_t xrs = make_rsrc(xl.x, xl.bytes);
+            const __amdgpu_buffer_rsrc_t wrs = make_rsrc(w, static_cast<uint32_t>(N) * static_cast<uint32_t>(Kred));
+            int32_t woff[WLOADS]; // byte offset of this lane's weight row, kOob when beyond N
+#pragma unroll
+            for (int i = 0; i < WLOADS; ++i)
+            {
+                const int32_t r = lrow + 64 * i;
+                const int32_t n = n0 + r;
+                woff[i] = (n < N && r < BN) ? n * Kred : kOob;
+            }
+            int32_t kb = lchunk * 16;
+
+            v4i xreg[XLOADS], wreg[WLOADS];
+            uint32_t oob_mask = 0; // bit i: chunk i of the slice in flight was out of range
+            // nothing between the loads and the MFMAs may touch the loaded registers: the fix-ups
+            // (padding byte, sign bias) happen in lstore, one slice later
+            auto gload = [&]() {
+                oob_mask = 0;
+#pragma unroll
+                for (int i = 0; i < XLOADS; ++i)
+                {
+                    const int32_t off = xl.offset(xr[i], cur);
+                    oob_mask |= (off == kOob ? 1u : 0u) << i;
+                    xreg[i] = buffer_load16(xrs, off);
+                }
+#pragma unroll
+                for (int i = 0; i < WLOADS; ++i)
+                    wreg[i] = buffer_load16(wrs, (woff[i] != kOob && kb < Kred) ? woff[i] + kb : kOob);
+            };
+            auto lstore = [&](int buf) {
+                uint8_t* xs = lds + buf * STAGE;
+                uint8_t* ws = xs + BM * BK;
+#pragma unroll
+                for (int i = 0; i < XLOADS; ++i)
+                {
+                    v4i v = xreg[i];
+                    if (fill != 0) // uniform: a non-zero data zero point pads with that byte
+                    {
+                        const bool oob = (oob_mask >> i) & 1u;
+                        v = v4i{oob ? fill : v[0], oob ? fill : v[1], oob ? fill : v[2], oob ? fill : v[3]};
+                    }
+                    *reinterpret_cast<v4i*>(xs + lds_offset(lrow + 64 * i, lchunk)) =
+                        v4i{v[0] ^ xor_mask, v[1] ^ xor_mask, v[2] ^ xor_mask, v[3] ^ xor_mask};
+                }
+#pragma unroll
+                for (int i = 0; i < WLOADS; ++i)
+                    if (lrow + 64 * i < BN)
+                        *reinterpret_cast<v4i*>(ws + lds_offset(lrow + 64 * i, lchunk)) = wreg[i];
+            };
+
+            const int KT = (Kred + BK - 1) / BK;
+            gload();
+            lstore(0);
+            __syncthreads();
+            for (int kt = 0; kt < KT; ++kt)
+            {
+                const int buf = kt & 1;
+                const bool more = kt + 1 < KT;
+                if (more)
+                {
+                    xl.advance(cur, BK);
+                    kb += BK;
+                    gload();
+                }
+                const uint8_t* xs = lds + buf * STAGE;
+                const uint8_t* ws = xs + BM * BK;
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks)
+                {
+                    v4i wf[WN], xf[WM];
+                    const int chunk = ks * 2 + (lane >> 5);
+#pragma unroll
+                    for (int i = 0; i < WN; ++i)
+                        wf[i] = *reinterpret_cast<const v4i*>(ws + lds_offset((wn * WN + i) * 32 + (lane & 31), chunk));
+#pragma unroll
+                    for (int i = 0; i < WM; ++i)
+                        xf[i] = *reinterpret_cast<const v4i*>(xs + lds_offset((wm * WM + i) * 32 + (lane & 31), chunk));
+#pragma unroll
+                    for (int mi = 0; mi < WM; ++mi)
+#pragma unroll
+                        for (int ni = 0; ni < WN; ++ni)
+                        {
+                            if (X_ON_A)
+                                acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xf[mi], wf[ni], acc[mi][ni], 0, 0, 0);
+                            else
+                                acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ni], xf[mi], acc[mi][ni], 0, 0, 0);
+                        }
+                }
+                if (more)
+                    lstore(buf ^ 1);
+                __syncthreads();
+            }
+        }
+
+        // ---- epilogue on the accumulators in registers -----------------------------------------
+        const EpiConst ec = epi_const(epi);
+        const bool has_sum = MODE == EPI_FUSED && epi.sum_in != nullptr;
+        const bool relu = epi.relu != 0;
+        if (!X_ON_A)
+        {
+            // rows = output channels: 4 consecutive channels of one m -> out[m][n..n+3]
+            const bool vec_ok = (N & 3) == 0;
+#pragma unroll
+            for (int ni = 0; ni < WN; ++ni)
+            {
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                {
+                    const int32_t nb = n0 + (wn * WN + ni) * 32 + 8 * g + 4 * (lane >> 5);
+                    if (nb >= N)
+                        continue;
+                    // per-channel parameters of the four channels this lane holds
+                    float bias4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                    float scale4[4] = {ec.scale, ec.scale, ec.scale, ec.scale};
+                    if (MODE == EPI_FUSED)
+                    {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (nb + e < N)
+                            {
+                                if (epi.bias)
+                                    bias4[e] = static_cast<float>(epi.bias[nb + e]);
+                                if (epi.per_channel)
+                                    scale4[e] = epi.scale[nb + e];
+                            }
+                    }
+#pragma unroll
+                    for (int mi = 0; mi < WM; ++mi)
+                    {
+                        const int64_t m = m0 + (wm * WM + mi) * 32 + (lane & 31);
+                        if (m >= M)
+                            continue;
+                        const int64_t o = m * N + nb;
+                        float s4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                        if (has_sum)
+                        {
+                            if (vec_ok)
+                                sum4(epi.sum_in, epi.sum_t, o, true, s4);
+                            else
+                            {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e)
+                                    if (nb + e < N)
+                                        s4[e] = static_cast<float>(load_q(epi.sum_in, epi.sum_t, o + e));
+                            }
+                        }
+                        int32_t v[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                        {
+                            const int32_t a = acc[mi][ni][4 * g + e];
+                            v[e] = MODE == EPI_INTERP ? epi_interp<KIND>(ec, a) : epi_fused<KIND>(ec, a, bias4[e], scale4[e], has_sum, s4[e], relu);
+                        }
+                        if (vec_ok) // nb is a multiple of 4, so nb + 3 < N and the store is aligned
+                        {
+                            if (KIND == OUT_Q8)
+                                *reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(out) + o) = pack4(v);
+                            else
+                                *reinterpret_cast<v4i*>(static_cast<int32_t*>(out) + o) = v4i{v[0], v[1], v[2], v[3]};
+                        }
+                        else
+                        {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                if (nb + e < N)
+                                    store_out(out, KIND == OUT_Q8 ? HIPQ_U8 : HIPQ_I32, o + e, v[e]);
+                        }
+                    }
+                }
+            }
+        }
+        else
+        {
+            // rows = m: 4 consecutive pixels of one channel -> out[image][n][pixel..pixel+3]
+            const bool vec_ok = om.ncx && (om.PQ & 3) == 0;
+#pragma unroll
+            for (int ni = 0; ni < WN; ++ni)
+            {
+                const int32_t n = n0 + (wn * WN + ni) * 32 + (lane & 31);
+                if (n >= N)
+                    continue;
+                float bias = 0.0f, scale = ec.scale;
+                if (MODE == EPI_FUSED)
+                {
+                    if (epi.bias)
+                        bias = static_cast<float>(epi.bias[n]);
+                    if (epi.per_channel)
+                        scale = epi.scale[n];
+                }
+#pragma unroll
+                for (int mi = 0; mi < WM; ++mi)
+                {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                    {
+                        const int64_t mb = m0 + (wm * WM + mi) * 32 + 8 * g + 4 * (lane >> 5);
+                        if (mb >= M)
+                            continue;
+                        if (vec_ok) // mb % 4 == 0 and PQ % 4 == 0: same image, aligned, mb + 3 < M
+                        {
+                            const int64_t o = om.index(mb, n);
+                            float s4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                            if (has_sum)
+                                sum4(epi.sum_in, epi.sum_t, o, true, s4);
+                            int32_t v[4];
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                            {
+                                const int32_t a = acc[mi][ni][4 * g + e];
+                                v[e] = MODE == EPI_INTERP ? epi_interp<KIND>(ec, a) : epi_fused<KIND>(ec, a, bias, scale, has_sum, s4[e], relu);
+                            }
+                            if (KIND == OUT_Q8)
+                                *reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(out) + o) = pack4(v);
+                            else
+                                *reinterpret_cast<v4i*>(static_cast<int32_t*>(out) + o) = v4i{v[0], v[1], v[2], v[3]};
+                        }
+                        else
+                        {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                if (mb + e < M)
+                                {
+                                    const int64_t o = om.index(mb + e, n);
+                                    const int32_t a = acc[mi][ni][4 * g + e];
+                                    const float sv = has_sum ? static_cast<float>(load_q(epi.sum_in, epi.sum_t, o)) : 0.0f;
+                                    const int32_t v = MODE == EPI_INTERP ? epi_interp<KIND>(ec, a) : epi_fused<KIND>(ec, a, bias, scale, has_sum, sv, relu);
+                                    store_out(out, KIND == OUT_Q8 ? HIPQ_U8 : HIPQ_I32, o, v);
+                                }
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+    static inline bool fits_i32(int64_t v) { return v >= 0 && v < (1ll << 31); }
+
+    // one instantiation = one tile shape; sets the dynamic LDS limit on first use
+    template <class XL, int WM, int WN, int WAVES_M, int WAVES_N, bool X_ON_A, int MODE, int KIND>
+    static int launch_tile(const XL& xl,
+                           const int8_t* w,
+                           const int32_t* wsum,
+                           int64_t M,
+                           int32_t N,
+                           int32_t Kred,
+                           int x_unsigned,
+                           const ZeroPoints& zp,
+                           const Epilogue& epi,
+                           const OutMap& om,
+                           void* out,
+                           hipStream_t s,
+                           const char* name)
+    {
+        constexpr int BM = WAVES_M * WM * 32;
+        constexpr int BN = WAVES_N * WN * 32;
+        constexpr size_t lds_bytes = 2 * static_cast<size_t>(BM + BN) * BK;
+        auto kernel = igemm_i8_kernel<XL, WM, WN, WAVES_M, WAVES_N, X_ON_A, MODE, KIND>;
+        static bool configured[16] = {};
+        int dev = 0;
+        HIPQ_HIP(hipGetDevice(&dev));
+        if (dev >= 0 && dev < 16 && !configured[dev])
+        {
+            HIPQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+            configured[dev] = true;
+        }
+        const int64_t m_tiles = (M + BM - 1) / BM;
+        HIPQ_REQUIRE(fits_i32(m_tiles * 8), "too many row tiles");
+        dim3 grid(static_cast<unsigned>(((m_tiles + 7) / 8) * 8), static_cast<unsigned>((N + BN - 1) / BN));
+        kernel<<<grid, 256, lds_bytes, s>>>(xl, w, wsum, M, Kred, x_unsigned, static_cast<int32_t>(m_tiles), zp, epi, om, out);
+        return check_launch(name);
+    }
+
+    // tile choice: narrow outputs (N <= 64) take 512 x 64 so each wavefront still owns 128 x 64
+    template <class XL, bool X_ON_A, int MODE, int KIND>
+    static int launch_best(const XL& xl,
+                           const int8_t* w,
+                           const int32_t* wsum,
+                           int64_t M,
+                           int32_t N,
+                           int32_t Kred,
+                           int x_unsigned,
+                           const ZeroPoints& zp,
+                           const Epilogue& epi,
+                           const OutMap& om,
+                           void* out,
+                           hipStream_t s,
+                           const char* name)
+    {
+        if (N <= 64)
+            return launch_tile<XL, 4, 2, 4, 1, X_ON_A, MODE, KIND>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+        return launch_tile<XL, 4, 2, 2, 2, X_ON_A, MODE, KIND>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+    }
+
+    // epilogue policy x output kind -> instantiation
+    template <class XL, bool X_ON_A>
+    static int launch_epilogue(const XL& xl,
+                               const int8_t* w,
+                               const int32_t* wsum,
+                               int64_t M,
+                               int32_t N,
+                               int32_t Kred,
+                               int x_unsigned,
+                               const ZeroPoints& zp,
+                               const Epilogue& epi,
+                               const OutMap& om,
+                               void* out,
+                               hipStream_t s,
+                               const char* name)
+    {
+        const bool q8 = epi.out_t == HIPQ_U8 || epi.out_t == HIPQ_I8;
+        if (epi.mode == EPI_INTERP)
+        {
+            if (q8)
+                return launch_best<XL, X_ON_A, EPI_INTERP, OUT_Q8>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+            if (epi.out_t == HIPQ_I32)
+                return launch_best<XL, X_ON_A, EPI_INTERP, OUT_I32>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+        }
+        else
+        {
+            if (q8)
+                return launch_best<XL, X_ON_A, EPI_FUSED, OUT_Q8>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+            if (epi.out_t == HIPQ_F32)
+                return launch_best<XL, X_ON_A, EPI_FUSED, OUT_F32>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+        }
+        return fail(HIPQ_ERR_UNSUPPORTED, "no MFMA kernel for this epilogue / output type");
+    }
+}

@@ -29,57 +29,27 @@ namespace hipq
                         void* out,
                         hipStream_t s)
     {
-        if (!packed || !conv_mfma_eligible(g))
+        // the MFMA kernels have no fused-policy instantiation with int32 output (no nGraph op asks for one)
+        if (!packed || !conv_mfma_eligible(g) || (epi.mode == EPI_FUSED && g.out_t == HIPQ_I32))
             return launch_conv_direct(g, data, filter, zp, epi, out, s);
 
-        const size_t out_eb = dtype_size(g.out_t);
-        const int64_t in_sp = g.in[1] * g.in[2], out_sp = g.out[1] * g.out[2];
-        const size_t in_bytes = align_up(static_cast<size_t>(g.in_count()), 256);
-        const size_t out_bytes = align_up(static_cast<size_t>(g.out_count()) * out_eb, 256);
-        const size_t sum_bytes = epi.sum_in ? align_up(static_cast<size_t>(g.out_count()), 256) : 0;
+        // The kernel reads channels-last data; an NCHW input is transposed through the workspace.
+        // The output is written directly in either layout (sum_in is indexed like the output).
+        const int64_t in_sp = g.in[1] * g.in[2];
         const bool tr_in = g.data_layout == HIPQ_LAYOUT_NCX && g.C > 1;
-        const bool tr_out = g.out_layout == HIPQ_LAYOUT_NCX && g.K > 1;
         const void* x = data;
-        void* y = out;
-        if (tr_in || tr_out)
+        if (tr_in)
         {
-            uint8_t* ws = nullptr;
-            size_t need = (tr_in ? in_bytes : 0) + (tr_out ? out_bytes + sum_bytes : 0);
-            int rc = workspace(need, reinterpret_cast<void**>(&ws));
+            void* ws = nullptr;
+            int rc = workspace(align_up(static_cast<size_t>(g.in_count()), 256), &ws);
             if (rc)
                 return rc;
-            if (tr_in)
-            {
-                rc = launch_transpose(data, ws, g.N, g.C, in_sp, 1, s);
-                if (rc)
-                    return rc;
-                x = ws;
-                ws += in_bytes;
-            }
-            if (tr_out)
-            {
-                y = ws;
-                ws += out_bytes;
-                if (epi.sum_in)
-                {
-                    rc = launch_transpose(epi.sum_in, ws, g.N, g.K, out_sp, 1, s);
-                    if (rc)
-                        return rc;
-                    epi.sum_in = ws;
-                }
-            }
-        }
-        int rc = launch_conv_mfma(g, x, packed, zp, epi, y, s);
-        if (rc)
-            return rc;
-        if (tr_out)
-        {
-            rc = launch_transpose(y, out, g.N, out_sp, g.K, static_cast<int>(out_eb), s);
+            rc = launch_transpose(data, ws, g.N, g.C, in_sp, 1, s);
             if (rc)
                 return rc;
-            set_last_kernel("conv_mfma_i8_32x32x32");
+            x = ws;
         }
-        return HIPQ_OK;
+        return launch_conv_mfma(g, x, packed, zp, epi, out, g.out_layout == HIPQ_LAYOUT_NCX && g.K > 1, s);
     }
 
     static int fused_epilogue(const hipq_fused_desc_t* f,

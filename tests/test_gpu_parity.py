@@ -481,3 +481,30 @@ def test_transposes(gpu_lib, eb):
         back = H.DeviceBuffer(a.nbytes)
         H.check(gpu_lib.hipq_transpose_nxc_to_ncx(dst.ptr, back.ptr, N, Cc, X, eb, None))
         assert np.array_equal(back.to_numpy(dt, (N, Cc, X)), a)
+
+
+def test_mfma_requant_ties(gpu_lib):
+    """exact .5 ties of both signs and both parities on the MFMA path: half away from zero for the
+    INTERPRETER policy, half to even for the fused policy"""
+    say("requant ties")
+    K, N, M = 16, 64, 40
+    a = np.zeros((M, K), np.uint8)
+    a[:, 0] = 1  # acc[m, n] = w[n, 0]: every integer in [-32, 31]
+    w = np.zeros((N, K), np.int8)
+    w[:, 0] = np.arange(N) - 32
+    exp_acc = np.tile(w[:, 0].astype(np.int32), (M, 1))
+    d = H.make_dot_desc(M, K, N, out_t="i8", b_layout=H.B_NK)
+    got = H.quantized_dot(d, a, w, 0.5, 0, 1.0, 0, 1.0, 0)
+    assert H.last_kernel().startswith("dot_mfma")
+    half_away = np.sign(exp_acc) * np.floor(np.abs(exp_acc) / 2 + 0.5)
+    assert np.array_equal(got.astype(np.int64), half_away.astype(np.int64))
+    assert np.array_equal(got, O.quantized_dot(d, a, w, 0.5, 0, 1.0, 0, 1.0, 0))
+    f = H.make_fused_desc(has_bias=False)
+    got = H.quantized_dot_bias(d, f, a, w, None, 0.5)
+    assert np.array_equal(got.astype(np.int64), np.rint(exp_acc / 2).astype(np.int64))
+    assert np.array_equal(got, O.quantized_dot_bias(d, f, a, w, None, 0.5))
+    # a scale >= 1 takes the out-of-range-aware conversion; 2^31-sized products give INT32_MIN like x86
+    d32 = H.make_dot_desc(M, K, N, out_t="i32", b_layout=H.B_NK)
+    for s in (1.5, 3.0e8):
+        assert np.array_equal(H.quantized_dot(d32, a, w, s, 0, 1.0, 0, 1.0, 0), O.quantized_dot(d32, a, w, s, 0, 1.0, 0, 1.0, 0)), s
+        assert np.array_equal(H.quantized_dot(d, a, w, s, 0, 1.0, 0, 1.0, 5), O.quantized_dot(d, a, w, s, 0, 1.0, 0, 1.0, 5)), s

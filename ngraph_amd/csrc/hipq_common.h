@@ -210,6 +210,15 @@ namespace hipq
 
     // MFMA implicit-GEMM convolution on channels-last data (both data and out NXC).
     bool conv_mfma_eligible(const ConvGeom& g);
+    bool conv_band_eligible(const ConvGeom& g, bool out_ncx);
+    int launch_conv_band(const ConvGeom& g,
+                         const void* data_nxc,
+                         const void* packed,
+                         const ZeroPoints& zp,
+                         const Epilogue& epi,
+                         void* out,
+                         bool out_ncx,
+                         hipStream_t s);
     int launch_conv_mfma(const ConvGeom& g,
                          const void* data_nxc,
                          const void* packed,

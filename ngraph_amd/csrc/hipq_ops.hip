@@ -1,5 +1,7 @@
 // Entry points of the quantized convolution / dot family: argument checks, choice between the
 // MFMA kernels and the direct kernels, layout conversion through the device workspace.
+#include <cstdlib>
+
 #include "hipq_common.h"
 
 namespace hipq
@@ -49,7 +51,12 @@ namespace hipq
                 return rc;
             x = ws;
         }
-        return launch_conv_mfma(g, x, packed, zp, epi, out, g.out_layout == HIPQ_LAYOUT_NCX && g.K > 1, s);
+        const bool out_ncx = g.out_layout == HIPQ_LAYOUT_NCX && g.K > 1;
+        // layers whose filter fits in LDS take the band kernel (HIPQ_NO_BAND=1 forces the generic one)
+        const bool no_band = getenv("HIPQ_NO_BAND") != nullptr;
+        if (!no_band && conv_band_eligible(g, out_ncx))
+            return launch_conv_band(g, x, packed, zp, epi, out, out_ncx, s);
+        return launch_conv_mfma(g, x, packed, zp, epi, out, out_ncx, s);
     }
 
     static int fused_epilogue(const hipq_fused_desc_t* f,

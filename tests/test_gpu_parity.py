@@ -225,7 +225,7 @@ def test_conv_mfma_shapes(gpu_lib, i):
         exp = O.quantized_convolution(d, data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
         O.port().orc_set_threads(1)
         got = H.quantized_convolution(d, data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
-        assert H.last_kernel().startswith("conv_mfma"), H.last_kernel()
+        assert H.last_kernel().startswith(("conv_mfma", "conv_band")), H.last_kernel()
         assert np.array_equal(got, exp), (out_t, z)
     # reference layouts in and out (transposed through the workspace)
     d = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t="i8", **kw)
@@ -234,7 +234,7 @@ def test_conv_mfma_shapes(gpu_lib, i):
     exp = O.quantized_convolution(d, data, filt, 0.02, 0, 0.005, 0, 0.9, 0)
     O.port().orc_set_threads(1)
     got = H.quantized_convolution(d, data, filt, 0.02, 0, 0.005, 0, 0.9, 0)
-    assert H.last_kernel().startswith("conv_mfma"), H.last_kernel()
+    assert H.last_kernel().startswith(("conv_mfma", "conv_band")), H.last_kernel()
     assert np.array_equal(got, exp)
 
 
@@ -275,7 +275,7 @@ def test_conv_linearity_at_config1_batch(gpu_lib):
     a = H.quantized_convolution(d, data, f1, 1.0, 0, 1.0, 0, 1.0, 0).astype(np.int64)
     b = H.quantized_convolution(d, data, f2, 1.0, 0, 1.0, 0, 1.0, 0).astype(np.int64)
     c = H.quantized_convolution(d, data, (f1 + f2).astype(np.int8), 1.0, 0, 1.0, 0, 1.0, 0).astype(np.int64)
-    assert H.last_kernel().startswith("conv_mfma")
+    assert H.last_kernel().startswith(("conv_mfma", "conv_band"))
     assert np.array_equal(a + b, c)
     d1 = H.make_conv_desc(1, 64, 64, (56, 56), (3, 3), **kw)
     O.port().orc_set_threads(8)
@@ -356,6 +356,82 @@ def test_fused_conv_random(gpu_lib, relu, has_sum, layout):
     exp = O.quantized_convolution_fused(d, f, data, filt, None, summ, 1.5e-3, 0.8)
     got = H.quantized_convolution_fused(d, f, data, filt, None, summ, 1.5e-3, 0.8)
     assert np.array_equal(got, exp)
+
+
+BAND_SHAPES = [
+    # N, K, in_sp, f_sp, kw : 64 input channels, filter resident in LDS
+    (2, 64, (56, 56), (3, 3), dict(pad_below=(1, 1), pad_above=(1, 1))),  # 7 full bands an image
+    (1, 64, (20, 20), (3, 3), dict(pad_below=(1, 1), pad_above=(1, 1))),  # one band, ragged last tile
+    (3, 32, (30, 24), (3, 3), dict(pad_below=(1, 1), pad_above=(1, 1))),  # short last band, K < 64
+    (2, 48, (14, 14), (1, 1), dict()),                                    # 1x1, K not a multiple of 32
+    (1, 16, (12, 16), (3, 2), dict(pad_below=(1, 0), pad_above=(1, 1))),  # asymmetric filter and padding
+    (1, 64, (9, 40), (3, 3), dict()),                                     # no padding
+]
+
+
+@pytest.mark.parametrize("i", range(len(BAND_SHAPES)))
+def test_conv_band(gpu_lib, i):
+    """the LDS-resident-filter kernel against the oracle: both requantization policies, both output
+    layouts, both fixed-point and float requantization branches, i32 output, zero points"""
+    N, K, in_sp, f_sp, kw = BAND_SHAPES[i]
+    say("band conv", BAND_SHAPES[i])
+    O.port().orc_set_threads(8)
+    kernels = set()
+    for dl, ol in ((H.NXC, H.NXC), (H.NXC, H.NCX), (H.NCX, H.NCX)):
+        for out_t, data_t, s, z in (
+            ("i8", "u8", (0.02, 0.005, 0.9), (0, 0, -3)),     # fixed-point requantization
+            ("u8", "u8", (0.02, 0.005, 0.7), (131, 0, 7)),    # padding materialised as the zero point
+            ("i8", "u8", (1.0, 1.0, 1.0), (0, 0, 0)),         # |scale| too large for fixed point; wraps
+            ("i32", "u8", (1.0, 1.0, 1.0), (3, 0, 11)),
+            ("i8", "i8", (0.02, 0.005, 0.9), (-5, 0, 0)),
+            ("u8", "u8", (0.02, 0.005, 0.9), (9, -7, 1)),     # filter zero point: exact slow path
+        ):
+            d = H.make_conv_desc(N, 64, K, in_sp, f_sp, data_t=data_t, out_t=out_t, data_layout=dl, out_layout=ol, **kw)
+            dn = H.make_conv_desc(N, 64, K, in_sp, f_sp, data_t=data_t, out_t=out_t, **kw)
+            lo, hi = (0, 255) if data_t == "u8" else (-128, 127)
+            data = synth.uniform_int(300 + i, dn.data_shape(), lo, hi, H.NP_OF[H.dtype_code(data_t)])
+            filt = synth.uniform_int(400 + i, d.filter_shape(), -128, 127, np.int8)
+            exp = O.quantized_convolution(dn, data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
+            got = H.quantized_convolution(d, cases.to_nxc(data) if dl == H.NXC else data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
+            kernels.add(H.last_kernel())
+            got = cases.to_ncx(got) if ol == H.NXC else got
+            assert np.array_equal(got, exp), (dl, ol, out_t, data_t, z, H.last_kernel())
+        # fused policy: bias, per-channel scales, residual sum, relu
+        for relu, has_sum, per_channel in ((True, True, True), (False, False, False), (True, False, True), (False, True, False)):
+            out_t = "u8" if relu else "i8"
+            d = H.make_conv_desc(N, 64, K, in_sp, f_sp, out_t=out_t, data_layout=dl, out_layout=ol, **kw)
+            dn = H.make_conv_desc(N, 64, K, in_sp, f_sp, out_t=out_t, **kw)
+            data = synth.uniform_int(500 + i, dn.data_shape(), 0, 255, np.uint8)
+            filt = synth.uniform_int(600 + i, d.filter_shape(), -127, 127, np.int8)
+            bias = synth.uniform_int(63, (K,), -20000, 20000, np.int32)
+            scales = synth.uniform_f32(64, (K,), 2e-4, 9e-4) if per_channel else np.float32(5e-4)
+            summ = synth.uniform_int(65, dn.out_shape(), -128, 127, np.int8) if has_sum else None
+            f = H.make_fused_desc(has_bias=True, has_sum=has_sum, sum_t="i8", with_relu=relu, scale_count=K if per_channel else 1)
+            ss = 0.37 if has_sum else None
+            exp = O.quantized_convolution_fused(dn, H.make_fused_desc(has_bias=True, has_sum=has_sum, sum_t="i8", with_relu=relu, scale_count=K if per_channel else 1), data, filt, bias, summ, scales, ss)
+            got = H.quantized_convolution_fused(
+                d, f, cases.to_nxc(data) if dl == H.NXC else data, filt, bias, (cases.to_nxc(summ) if ol == H.NXC else summ) if has_sum else None, scales, ss
+            )
+            kernels.add(H.last_kernel())
+            got = cases.to_ncx(got) if ol == H.NXC else got
+            assert np.array_equal(got, exp), (dl, ol, relu, has_sum, per_channel, H.last_kernel())
+    O.port().orc_set_threads(1)
+    assert any(k.startswith("conv_band") for k in kernels), kernels
+
+
+def test_conv_band_matches_generic_kernel(gpu_lib, monkeypatch):
+    """the band kernel and the generic implicit-GEMM kernel agree byte for byte at a size the oracle
+    does not reach (BASELINE config 1 at batch 16, wrapping requantization included)"""
+    say("band vs generic")
+    d = H.make_conv_desc(16, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1))
+    data = synth.uniform_int(701, d.data_shape(), 0, 255, np.uint8)
+    filt = synth.uniform_int(702, d.filter_shape(), -127, 127, np.int8)
+    a = H.quantized_convolution(d, data, filt, 0.02, 0, 0.005, 0, 0.1, 0)
+    assert H.last_kernel().startswith("conv_band"), H.last_kernel()
+    monkeypatch.setenv("HIPQ_NO_BAND", "1")
+    b = H.quantized_convolution(d, data, filt, 0.02, 0, 0.005, 0, 0.1, 0)
+    assert H.last_kernel().startswith("conv_mfma"), H.last_kernel()
+    assert np.array_equal(a, b)
 
 
 # ------------------------------------------------------------------ QuantizedDot

@@ -36,9 +36,13 @@ namespace hipq
 
     constexpr int BK = 64; // reduction bytes per LDS slice
 
+    // A ds_read_b128 is served 16 lanes at a time from 64 banks: full rate needs 16 consecutive rows
+    // at one chunk index in 16 different 16-byte columns of a 256-byte line.  Rows r, r+4, r+8, r+12
+    // share a 64-byte column group, hence the rotation by (r / 4) % 4 (measured 190 B/clk/CU; a
+    // rotation by (r / 2) % 4 gives 128, none 64).
     __device__ __forceinline__ int lds_offset(int row, int chunk)
     {
-        return row * BK + ((chunk ^ ((row >> 1) & 3)) << 4);
+        return row * BK + ((chunk ^ ((row >> 2) & 3)) << 4);
     }
 
     // ---- activation loaders ---------------------------------------------------------------------

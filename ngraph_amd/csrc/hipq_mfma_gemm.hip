@@ -1,8 +1,146 @@
 // int8 GEMM on the i8 matrix cores: eligibility and launch (kernel in hipq_igemm.h).
+#include <cstdlib>
+
 #include "hipq_igemm.h"
 
 namespace hipq
 {
+    // ---- skinny GEMM: M <= 64 ------------------------------------------------------------------
+    // With a handful of rows the product is a stream over the weights: every weight byte must come
+    // from HBM once and is used for at most 64 MACs.  One workgroup owns 16 output columns and the
+    // whole reduction, so no partial sums leave the CU; its four wavefronts split K four ways, each
+    // lane loads its v_mfma_i32_16x16x64_i8 fragments straight from global memory (16 bytes a lane,
+    // sixteen 64-byte steps in flight before the first MFMA), and the four partial 16x16 tiles meet in
+    // LDS.  N / 16 workgroups: 256 for N = 4096, one per CU.
+    typedef int v4acc __attribute__((ext_vector_type(4)));
+
+    template <int MT, int STEPS>
+    __global__ __launch_bounds__(256) void dot_skinny_kernel(const uint8_t* __restrict__ a,
+                                                             const int8_t* __restrict__ w,
+                                                             const int32_t* __restrict__ wsum,
+                                                             int32_t M,
+                                                             int32_t N,
+                                                             int32_t K,
+                                                             int32_t x_unsigned,
+                                                             ZeroPoints zp,
+                                                             Epilogue epi,
+                                                             void* __restrict__ out)
+    {
+        __shared__ int32_t red[3][MT][4][64];
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = tid >> 6;
+        const int r16 = lane & 15; // A: row within the m-tile, B: column within the n-tile
+        const int kc = lane >> 4;  // 16-byte chunk of a 64-byte step
+        const int n0 = blockIdx.x * 16;
+        const int32_t xzp = load_zp(zp.data_zp, zp.data_t);
+        const int32_t wzp = load_zp(zp.filter_zp, zp.filter_t);
+        const EpiRegs er = epi_load(epi);
+        if (wzp != 0) // uniform; w - wzp does not fit a signed byte: exact, slow
+        {
+            for (int i = tid; i < 16 * M; i += 256)
+            {
+                const int m = i >> 4, n = n0 + (i & 15);
+                if (n < N)
+                {
+                    int32_t acc = 0;
+                    for (int k = 0; k < K; ++k)
+                    {
+                        const int32_t xv = x_unsigned ? static_cast<int32_t>(a[static_cast<int64_t>(m) * K + k])
+                                                      : static_cast<int32_t>(static_cast<int8_t>(a[static_cast<int64_t>(m) * K + k]));
+                        acc += (xv - xzp) * (static_cast<int32_t>(w[static_cast<int64_t>(n) * K + k]) - wzp);
+                    }
+                    const int64_t o = static_cast<int64_t>(m) * N + n;
+                    store_out(out, epi.out_t, o, epi_apply(epi, er, acc, n, o));
+                }
+            }
+            return;
+        }
+        const int xor_mask = x_unsigned ? static_cast<int>(0x80808080u) : 0;
+        const __amdgpu_buffer_rsrc_t ars = make_rsrc(a, static_cast<uint32_t>(M) * static_cast<uint32_t>(K));
+        const __amdgpu_buffer_rsrc_t wrs = make_rsrc(w, static_cast<uint32_t>(N) * static_cast<uint32_t>(K));
+        const int kq = ((K / 64 + 3) / 4) * 64; // bytes of K per wavefront, whole 64-byte steps
+        const int k_begin = wave * kq;
+        const int k_end = min(K, k_begin + kq);
+        const int32_t wrow = n0 + r16 < N ? (n0 + r16) * K + kc * 16 : kOob;
+        int32_t arow[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            arow[mt] = mt * 16 + r16 < M ? (mt * 16 + r16) * K + kc * 16 : kOob;
+
+        v4acc acc[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            acc[mt] = v4acc{0, 0, 0, 0};
+        for (int kb = k_begin; kb < k_end; kb += 64 * STEPS)
+        {
+            v4i bf[STEPS], af[MT][STEPS];
+#pragma unroll
+            for (int st = 0; st < STEPS; ++st)
+            {
+                const int k = kb + st * 64;
+                bf[st] = buffer_load16(wrs, (wrow != kOob && k < k_end) ? wrow + k : kOob);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    af[mt][st] = buffer_load16(ars, (arow[mt] != kOob && k < k_end) ? arow[mt] + k : kOob);
+            }
+#pragma unroll
+            for (int st = 0; st < STEPS; ++st)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                {
+                    // out-of-range fragments read zeros; a zero weight fragment cancels whatever the
+                    // sign bias makes of a zero activation fragment
+                    const v4i x = v4i{af[mt][st][0] ^ xor_mask, af[mt][st][1] ^ xor_mask, af[mt][st][2] ^ xor_mask, af[mt][st][3] ^ xor_mask};
+                    acc[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(x, bf[st], acc[mt], 0, 0, 0);
+                }
+        }
+        // ---- the four partial tiles meet in LDS; wavefront 0 requantizes ----------------------------
+        if (wave > 0)
+        {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    red[wave - 1][mt][r][lane] = acc[mt][r];
+        }
+        __syncthreads();
+        if (wave > 0)
+            return;
+        const int n = n0 + r16;
+        if (n >= N)
+            return;
+        const int32_t corr = ((x_unsigned ? 128 : 0) - xzp) * wsum[n];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+            {
+                // lane: column lane % 16; accumulator register r is row 4 * (lane / 16) + r of the tile
+                const int m = mt * 16 + 4 * kc + r;
+                if (m < M)
+                {
+                    const int32_t v = acc[mt][r] + red[0][mt][r][lane] + red[1][mt][r][lane] + red[2][mt][r][lane] + corr;
+                    const int64_t o = static_cast<int64_t>(m) * N + n;
+                    store_out(out, epi.out_t, o, epi_apply(epi, er, v, n, o));
+                }
+            }
+    }
+
+    static bool dot_skinny_eligible(const hipq_dot_desc_t& d)
+    {
+        return d.M <= 64 && d.K % 64 == 0 && d.K >= 256;
+    }
+
+    template <int MT, int STEPS>
+    static int launch_skinny(const hipq_dot_desc_t& d, const void* a, const void* w_nk, const int32_t* wsum, const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s)
+    {
+        const unsigned grid = static_cast<unsigned>((d.N + 15) / 16);
+        dot_skinny_kernel<MT, STEPS><<<grid, 256, 0, s>>>(static_cast<const uint8_t*>(a), static_cast<const int8_t*>(w_nk), wsum, static_cast<int32_t>(d.M),
+                                                      static_cast<int32_t>(d.N), static_cast<int32_t>(d.K), d.a_t == HIPQ_U8 ? 1 : 0, zp, epi, out);
+        return check_launch("dot_skinny_i8_16x16x64");
+    }
+
     bool dot_mfma_eligible(const hipq_dot_desc_t& d)
     {
         if (d.b_t != HIPQ_I8 || (d.a_t != HIPQ_U8 && d.a_t != HIPQ_I8))
@@ -27,6 +165,14 @@ namespace hipq
         HIPQ_REQUIRE((reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_nk) & 15) == 0 &&
                          (reinterpret_cast<uintptr_t>(out) & 15) == 0,
                      "MFMA dot needs 16-byte aligned tensors");
+        if (dot_skinny_eligible(d) && getenv("HIPQ_NO_SKINNY") == nullptr)
+        {
+            if (d.M <= 16)
+                return launch_skinny<1, 16>(d, a, w_nk, wsum, zp, epi, out, s);
+            if (d.M <= 32)
+                return launch_skinny<2, 16>(d, a, w_nk, wsum, zp, epi, out, s);
+            return launch_skinny<4, 8>(d, a, w_nk, wsum, zp, epi, out, s);
+        }
         GemmX xl;
         xl.x = static_cast<const uint8_t*>(a);
         xl.K = static_cast<int32_t>(d.K);

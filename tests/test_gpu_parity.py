@@ -462,7 +462,7 @@ def test_dot_reference_vectors(gpu_lib, ref_vectors):
             got = H.quantized_dot(d, a, b, s[0], z[0], s[1], z[1], s[2], z[2], prepare=prepare)
             used.add(H.last_kernel())
             assert np.array_equal(got, arrays[m["name"]]), (m["name"], prepare, H.last_kernel())
-    assert "dot_direct" in used and any(k.startswith("dot_mfma") for k in used), used
+    assert "dot_direct" in used and any(k.startswith(("dot_mfma", "dot_skinny")) for k in used), used
 
 
 @pytest.mark.parametrize("M", [1, 32, 256, 130])
@@ -476,7 +476,7 @@ def test_dot_mfma_vs_oracle(gpu_lib, M):
         d = H.make_dot_desc(M, K, N, out_t=out_t)
         exp = O.quantized_dot(d, a, b, s[0], z[0], s[1], z[1], s[2], z[2])
         got = H.quantized_dot(d, a, b, s[0], z[0], s[1], z[1], s[2], z[2])
-        assert H.last_kernel().startswith("dot_mfma")
+        assert H.last_kernel().startswith(("dot_mfma", "dot_skinny")), H.last_kernel()
         assert np.array_equal(got, exp), (out_t, z)
     O.port().orc_set_threads(1)
 
@@ -514,7 +514,7 @@ def test_dot_bias_config2_shape(gpu_lib, M):
         f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
         exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
         got = H.quantized_dot_bias(d, f, a, w, bias, scales)
-        assert H.last_kernel().startswith("dot_mfma")
+        assert H.last_kernel().startswith(("dot_mfma", "dot_skinny")), H.last_kernel()
         assert np.array_equal(got, exp), (out_t, relu)
         assert len(np.unique(exp)) > 20  # the case is not degenerate (all saturated)
     O.port().orc_set_threads(1)
@@ -530,7 +530,7 @@ def test_dot_config2_full_size_properties(gpu_lib):
     w = synth.uniform_int(96, (N, K), -127, 127, np.int8)
     d = H.make_dot_desc(256, K, N, out_t="i32", b_layout=H.B_NK)
     got = H.quantized_dot(d, a, w, 1.0, 0, 1.0, 0, 1.0, 0)
-    assert H.last_kernel().startswith("dot_mfma")
+    assert H.last_kernel().startswith(("dot_mfma", "dot_skinny")), H.last_kernel()
     rows = [0, 1, 31, 32, 127, 128, 255]
     exp = a[rows].astype(np.int64) @ w.astype(np.int64).T
     assert np.array_equal(got[rows].astype(np.int64), exp)
@@ -538,6 +538,35 @@ def test_dot_config2_full_size_properties(gpu_lib):
         dm = H.make_dot_desc(M, K, N, out_t="i32", b_layout=H.B_NK)
         gm = H.quantized_dot(dm, a[:M], w, 1.0, 0, 1.0, 0, 1.0, 0)
         assert np.array_equal(gm, got[:M])
+
+
+@pytest.mark.parametrize("M", [1, 7, 16, 17, 33, 64])
+def test_dot_skinny(gpu_lib, M):
+    """the weight-streaming kernel for a handful of rows: ragged row and column tiles, a reduction
+    that does not split evenly over the four wavefronts, signed and unsigned data, zero points,
+    both requantization policies, f32 output, and the exact path for a non-zero weight zero point"""
+    say("dot skinny M", M)
+    O.port().orc_set_threads(8)
+    for K, N in ((320, 40), (1024, 100), (256, 16)):
+        w = synth.uniform_int(802, (N, K), -128, 127, np.int8)
+        for a_t, lo, hi in (("u8", 0, 255), ("i8", -128, 127)):
+            a = synth.uniform_int(801, (M, K), lo, hi, H.NP_OF[H.dtype_code(a_t)])
+            for out_t, s, z in (("i32", (1.0, 1.0, 1.0), (0, 0, 0)), ("i8", (0.01, 0.01, 2.5), (5 if a_t == "u8" else -5, 0, 4)), ("u8", (0.01, 0.01, 2.5), (0, 3, 9))):
+                d = H.make_dot_desc(M, K, N, a_t=a_t, out_t=out_t, b_layout=H.B_NK)
+                exp = O.quantized_dot(d, a, w, s[0], z[0], s[1], z[1], s[2], z[2])
+                got = H.quantized_dot(d, a, w, s[0], z[0], s[1], z[1], s[2], z[2])
+                assert H.last_kernel().startswith("dot_skinny"), H.last_kernel()
+                assert np.array_equal(got, exp), (K, N, a_t, out_t, z)
+            bias = synth.uniform_int(803, (N,), -(2**15), 2**15, np.int32)
+            scales = synth.uniform_f32(804, (N,), 0.001, 0.01) * np.float32(0.05)
+            for out_t, relu in (("i8", False), ("u8", True), ("f32", True)):
+                d = H.make_dot_desc(M, K, N, a_t=a_t, out_t=out_t, b_layout=H.B_NK)
+                f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
+                exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
+                got = H.quantized_dot_bias(d, f, a, w, bias, scales)
+                assert H.last_kernel().startswith("dot_skinny"), H.last_kernel()
+                assert np.array_equal(got, exp), (K, N, a_t, out_t, relu)
+    O.port().orc_set_threads(1)
 
 
 # ------------------------------------------------------------------ layout helpers
@@ -571,7 +600,7 @@ def test_mfma_requant_ties(gpu_lib):
     exp_acc = np.tile(w[:, 0].astype(np.int32), (M, 1))
     d = H.make_dot_desc(M, K, N, out_t="i8", b_layout=H.B_NK)
     got = H.quantized_dot(d, a, w, 0.5, 0, 1.0, 0, 1.0, 0)
-    assert H.last_kernel().startswith("dot_mfma")
+    assert H.last_kernel().startswith(("dot_mfma", "dot_skinny")), H.last_kernel()
     half_away = np.sign(exp_acc) * np.floor(np.abs(exp_acc) / 2 + 0.5)
     assert np.array_equal(got.astype(np.int64), half_away.astype(np.int64))
     assert np.array_equal(got, O.quantized_dot(d, a, w, 0.5, 0, 1.0, 0, 1.0, 0))

@@ -30,12 +30,93 @@ namespace hipq
         }
     }
 
+    // Byte transpose at memory speed: in [B][R][Cc] -> out [B][Cc][R], R and Cc multiples of 16.
+    // A wavefront owns a 64 x 64 byte tile: every lane loads 16 bytes from each of 4 consecutive
+    // rows, transposes its four 4x4 byte blocks in registers (8 v_perm_b32 a block), writes the 16
+    // resulting dwords -- 4 rows of one column each -- into a [64 columns][17 dwords] LDS tile, and
+    // reads back 16 consecutive rows of one column as the 16-byte piece it stores.  Loads and stores
+    // are buffer accesses: tile parts beyond the tensor read zeros and are not written.
+    __device__ __forceinline__ void transpose4x4(const uint32_t d[4], uint32_t o[4])
+    {
+        const uint32_t t0 = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u); // d0.b0 d1.b0 d0.b1 d1.b1
+        const uint32_t t1 = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u); // d0.b2 d1.b2 d0.b3 d1.b3
+        const uint32_t t2 = __builtin_amdgcn_perm(d[3], d[2], 0x05010400u);
+        const uint32_t t3 = __builtin_amdgcn_perm(d[3], d[2], 0x07030602u);
+        o[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+        o[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+        o[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+        o[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+    }
+
+    typedef int v4t __attribute__((ext_vector_type(4)));
+
+    // tiles_c wavefront tiles side by side along the columns, 4 / tiles_c along the rows
+    __global__ __launch_bounds__(256) void transpose_bytes_kernel(const uint8_t* __restrict__ in, uint8_t* __restrict__ out, int32_t R, int32_t Cc, int32_t tiles_c, uint32_t bytes)
+    {
+        __shared__ uint32_t tile[4][64][17];
+        const int wave = threadIdx.x >> 6;
+        const int t = threadIdx.x & 63;
+        const int tc = wave % tiles_c, tr = wave / tiles_c;
+        const int r0 = (static_cast<int>(blockIdx.y) * (4 / tiles_c) + tr) * 64;
+        const int c0 = (static_cast<int>(blockIdx.x) * tiles_c + tc) * 64;
+        const uint32_t plane = static_cast<uint32_t>(R) * static_cast<uint32_t>(Cc);
+        const __amdgpu_buffer_rsrc_t irs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(in) + static_cast<size_t>(blockIdx.z) * plane, 0, plane, 0x00020000);
+        const __amdgpu_buffer_rsrc_t ors = __builtin_amdgcn_make_buffer_rsrc(out + static_cast<size_t>(blockIdx.z) * plane, 0, plane, 0x00020000);
+        constexpr int32_t oob = static_cast<int32_t>(0x80000000u);
+        (void)bytes;
+        {
+            const int rg = t >> 2, cb = t & 3; // rows 4rg..4rg+3, columns 16cb..16cb+15 of the tile
+            v4t l[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                const int r = r0 + 4 * rg + i, c = c0 + 16 * cb;
+                l[i] = __builtin_amdgcn_raw_buffer_load_b128(irs, (r < R && c < Cc) ? r * Cc + c : oob, 0, 0);
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                const uint32_t d[4] = {static_cast<uint32_t>(l[0][q]), static_cast<uint32_t>(l[1][q]), static_cast<uint32_t>(l[2][q]), static_cast<uint32_t>(l[3][q])};
+                uint32_t o[4];
+                transpose4x4(d, o);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    tile[wave][16 * cb + 4 * q + j][rg] = o[j];
+            }
+        }
+        // the tile is private to the wavefront and its LDS accesses complete in order: no barrier
+        {
+#pragma unroll
+            for (int it = 0; it < 4; ++it)
+            {
+                const int col = it * 16 + (t >> 2), q = t & 3;
+                const v4t v = v4t{static_cast<int>(tile[wave][col][4 * q]), static_cast<int>(tile[wave][col][4 * q + 1]), static_cast<int>(tile[wave][col][4 * q + 2]),
+                                  static_cast<int>(tile[wave][col][4 * q + 3])};
+                const int c = c0 + col, r = r0 + 16 * q;
+                __builtin_amdgcn_raw_buffer_store_b128(v, ors, (c < Cc && r < R) ? c * R + r : oob, 0, 0);
+            }
+        }
+    }
+
     int launch_transpose(const void* in, void* out, int64_t B, int64_t R, int64_t Cc, int elem_bytes, hipStream_t s)
     {
         if (B == 0 || R == 0 || Cc == 0)
             return HIPQ_OK;
         HIPQ_REQUIRE(in && out, "null tensor pointer");
         HIPQ_REQUIRE(B <= 65535, "batch %lld beyond 65535", (long long)B);
+        if (elem_bytes == 1 && R % 16 == 0 && Cc % 16 == 0 && R * Cc < (1ll << 31) && (reinterpret_cast<uintptr_t>(in) & 15) == 0 &&
+            (reinterpret_cast<uintptr_t>(out) & 15) == 0)
+        {
+            const int tiles_c = Cc > 128 ? 4 : (Cc > 64 ? 2 : 1);
+            const int64_t gx = (Cc + 64 * tiles_c - 1) / (64 * tiles_c), gy = (R + 64 * (4 / tiles_c) - 1) / (64 * (4 / tiles_c));
+            if (gy <= 65535)
+            {
+                dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(gy), static_cast<unsigned>(B));
+                transpose_bytes_kernel<<<grid, 256, 0, s>>>(static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), static_cast<int32_t>(R), static_cast<int32_t>(Cc),
+                                                           tiles_c, 0u);
+                return check_launch("transpose_bytes");
+            }
+        }
         dim3 grid(static_cast<unsigned>((Cc + 63) / 64), static_cast<unsigned>((R + 63) / 64), static_cast<unsigned>(B));
         HIPQ_REQUIRE((R + 63) / 64 <= 65535, "extent too large for the transpose grid");
         if (elem_bytes == 1)

@@ -576,7 +576,7 @@ def test_dot_skinny(gpu_lib, M):
 def test_transposes(gpu_lib, eb):
     say("transpose", eb)
     dt = np.uint8 if eb == 1 else np.int32
-    for (N, Cc, X) in ((2, 64, 3136), (3, 5, 7), (1, 130, 67)):
+    for (N, Cc, X) in ((2, 64, 3136), (3, 5, 7), (1, 130, 67), (3, 48, 80), (1, 256, 208), (2, 16, 16), (1, 144, 400)):
         a = synth.uniform_int(5, (N, Cc, X), 0, 255, np.uint8).astype(dt)
         src = H.DeviceBuffer.from_numpy(a)
         dst = H.DeviceBuffer(a.nbytes)

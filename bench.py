@@ -64,9 +64,10 @@ def scalar(v, dt):
     return dev(np.asarray(v, dtype=dt))
 
 
-def bench_conv(lib, stream, timer, N, steps, warmup, layout):
-    d = H.make_conv_desc(N, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1), data_layout=layout, out_layout=layout)
-    one = H.make_conv_desc(1, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1), data_layout=layout, out_layout=layout)
+def bench_conv(lib, stream, timer, N, steps, warmup, layout, out_layout=None):
+    out_layout = layout if out_layout is None else out_layout
+    d = H.make_conv_desc(N, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1), data_layout=layout, out_layout=out_layout)
+    one = H.make_conv_desc(1, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1), data_layout=layout, out_layout=out_layout)
     img = synth.uniform_int(1001, one.data_shape(), 0, 255, np.uint8)
     data = dev(np.ascontiguousarray(np.broadcast_to(img, d.data_shape())))
     filt = dev(synth.uniform_int(1002, d.filter_shape(), -127, 127, np.int8))
@@ -84,7 +85,8 @@ def bench_conv(lib, stream, timer, N, steps, warmup, layout):
     wall, ev = timer.run(step, steps, warmup)
     kern = H.last_kernel()
     ops = d.ops()
-    return dict(N=N, layout="NCHW" if layout == H.NCX else "NHWC", ops=ops, ms_wall=wall, ms_event=ev, tops=ops / (wall * 1e-3) / 1e12, tops_event=ops / (ev * 1e-3) / 1e12, kernel=kern)
+    name = lambda l: "NCHW" if l == H.NCX else "NHWC"
+    return dict(N=N, layout=name(layout), out_layout=name(out_layout), ops=ops, ms_wall=wall, ms_event=ev, tops=ops / (wall * 1e-3) / 1e12, tops_event=ops / (ev * 1e-3) / 1e12, kernel=kern)
 
 
 def bench_gemm(lib, stream, timer, M, steps, warmup):
@@ -194,10 +196,26 @@ def main():
 
     # headline: the reference's NCHW tensors in, NCHW out
     head = bench_conv(lib, stream, timer, args.batch, args.steps, args.warmup, H.NCX)
-    # dominant kernel alone (channels-last in and out: the call launches only the MFMA kernel)
-    kern = bench_conv(lib, stream, timer, args.batch, args.steps, args.warmup, H.NXC)
+    # the dominant kernel of that call alone: channels-last data in (what the call's transpose
+    # hands it), NCHW out -- such a call launches only the MFMA kernel
+    kern = bench_conv(lib, stream, timer, args.batch, args.steps, args.warmup, H.NXC, H.NCX)
+    # channels-last in and out, the layout a backend keeps between layers
+    nhwc = bench_conv(lib, stream, timer, args.batch, args.steps, args.warmup, H.NXC)
 
-    results = {"conv_nchw": [head], "conv_nhwc_kernel": [kern]}
+    results = {"conv_nchw": [head], "conv_kernel_nhwc_in_nchw_out": [kern], "conv_nhwc_kernel": [nhwc]}
+    # a plain device-to-device copy of known size: the yardstick for the FETCH_SIZE / WRITE_SIZE
+    # counters of a profiler run over this same command
+    cal_bytes = 64 << 20
+    ca, cb = H.DeviceBuffer(cal_bytes), H.DeviceBuffer(cal_bytes)
+    H.check(lib.hipq_fill_bytes(ca.ptr, 1, cal_bytes, stream))
+
+    def copy():
+        rc = lib.hipq_memcpy_d2d(cb.ptr, ca.ptr, cal_bytes, stream)
+        if rc:
+            H.check(rc)
+
+    _, cev = timer.run(copy, 10, 2)
+    results["copy_calibration"] = dict(bytes=cal_bytes, ms_event=cev, gbs=2 * cal_bytes / (cev * 1e-3) / 1e9)
     cpu = None
     if not args.quick:
         small = max(20, args.steps // 4)

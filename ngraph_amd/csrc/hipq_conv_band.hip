@@ -124,14 +124,19 @@ namespace hipq
             const bool ok = col_ok & (sy < band_rows) & (static_cast<uint32_t>(iy) < static_cast<uint32_t>(p.H));
             if (STORE)
             {
+                // padding is the data zero point (out-of-range loads gave zeros); a select per dword is
+                // cheaper than a branch around it, taken or not
                 v4i t = b.v[u];
-                if (fill != 0) // uniform: a non-zero data zero point pads with that byte
-                    t = v4i{ok ? t[0] : fill, ok ? t[1] : fill, ok ? t[2] : fill, ok ? t[3] : fill};
+                t = v4i{ok ? t[0] : fill, ok ? t[1] : fill, ok ? t[2] : fill, ok ? t[3] : fill};
                 *reinterpret_cast<v4i*>(lds + (in ? xs_off + band_slot_offset(sy * p.BW + sx, c4) : p.sink)) =
                     v4i{t[0] ^ xor_mask, t[1] ^ xor_mask, t[2] ^ xor_mask, t[3] ^ xor_mask};
             }
             else
+#ifdef BAND_EXP_NOBANDLOAD
+                b.v[u] = v4i{iy, ix, c4, u};
+#else
                 b.v[u] = buffer_load16(xrs, ok ? img_base + (iy * p.W + ix) * kBandC + c4 * 16 : kOob);
+#endif
         }
     }
 
@@ -139,9 +144,10 @@ namespace hipq
     // tap 2 weight fragments, T pixel fragments, 2T MFMAs; no barrier, no global access.  Two
     // fragment sets alternate (statically indexed) so that the reads of one half overlap the MFMAs
     // of the other.  woff: LDS offset of this lane's weight row at tap 0, chunk lane/32.
-    // One loop trip per tap (unrolling the taps of a 3x3 filter made the register allocator spill
-    // accumulators, which costs far more than the nine taken branches).
-    template <int T>
+    // U taps per loop trip; the tap count must be a multiple of U.  (A taken branch costs about as
+    // much as four MFMAs here, but unrolling all nine taps of a 3x3 filter made the register
+    // allocator spill accumulators, which costs far more.)
+    template <int T, int U>
     __device__ __forceinline__ void band_reduce(v16i (&acc)[4][2], const uint8_t* lds, int xs_off, int woff, const int (&slot0)[4], int half, int R, int S, int BW)
     {
         v4i xa[T], xb[T], wa[2], wb[2];
@@ -202,39 +208,43 @@ namespace hipq
             int r = 0, s = 0;
             const int taps = R * S;
 #pragma unroll 1
-            for (int tap = 0; tap < taps; ++tap)
+            for (int tap = 0; tap < taps; tap += U)
             {
-                load(wp, xoff, 32, xb, wb);
-                // the next tap; after the last one this wraps to tap 0, a harmless re-read that keeps
-                // the loop free of conditional loads
-                wp += 64 * kBandC;
-                ++s;
-                if (s == S)
-                {
-                    s = 0;
-                    ++r;
-                }
-                if (r == R)
-                {
-                    r = 0;
-                    wp = woff;
-                }
-                addr(r * BW + s, xnext);
-                mac(xa, wa);
-                interleave();
 #pragma unroll
-                for (int ti = 0; ti < T; ++ti)
-                    xoff[ti] = xnext[ti];
-                load(wp, xoff, 0, xa, wa);
-                mac(xb, wb);
-                interleave();
+                for (int u = 0; u < U; ++u)
+                {
+                    load(wp, xoff, 32, xb, wb);
+                    // the next tap; after the last one this wraps to tap 0, a harmless re-read that
+                    // keeps the loop free of conditional loads
+                    wp += 64 * kBandC;
+                    ++s;
+                    if (s == S)
+                    {
+                        s = 0;
+                        ++r;
+                    }
+                    if (r == R)
+                    {
+                        r = 0;
+                        wp = woff;
+                    }
+                    addr(r * BW + s, xnext);
+                    mac(xa, wa);
+                    interleave();
+#pragma unroll
+                    for (int ti = 0; ti < T; ++ti)
+                        xoff[ti] = xnext[ti];
+                    load(wp, xoff, 0, xa, wa);
+                    mac(xb, wb);
+                    interleave();
+                }
             }
         }
     }
 
-    template <int MODE, int KIND, bool OUT_NCX>
+    // U: filter taps per trip of the reduction loop (the tap count is a multiple of it)
+    template <int MODE, int KIND, bool OUT_NCX, int U>
     __global__ __launch_bounds__(kBandThreads) void conv_band_kernel(BandParams p,
-                                                                    ConvX xl,
                                                                     const int8_t* __restrict__ w,
                                                                     const int32_t* __restrict__ wsum,
                                                                     int32_t x_unsigned,
@@ -245,8 +255,11 @@ namespace hipq
         extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
         const int tid = threadIdx.x;
         const int lane = tid & 63;
-        const int grp = tid >> 8;       // group of four wavefronts
-        const int gw = (tid >> 6) & 3;  // wavefront within the group (= its SIMD)
+        // wavefront-uniform values, told so to the compiler: item geometry and loop control then run
+        // on the scalar unit instead of in vector registers under exec masks
+        const int wave_id = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int grp = wave_id >> 2; // group of four wavefronts
+        const int gw = wave_id & 3;   // wavefront within the group (= its SIMD)
         const int half = lane >> 5;
         const int l32 = lane & 31;
         const int xs_off = p.x_lds + grp * p.band_bytes;
@@ -297,14 +310,35 @@ namespace hipq
             band_x_copy<false>(xb0, xrs, lds, p, xs_off, 0, 0, rows + p.R - 1, img * p.H * p.W * kBandC, p0, 0, 0);
         }
 
-        if (wzp != 0) // uniform; w - wzp does not fit a signed byte: exact, slow
+        if (wzp != 0) // uniform; w - wzp does not fit a signed byte: exact, slow, one output a lane
         {
-            const OutMap om{OUT_NCX ? 1 : 0, p.K, p.PQ};
+            const EpiRegs er = epi_load(epi);
             for (int j = 0; j < my_items; ++j)
             {
                 item_geom(j, img, p0, rows);
-                slow_tile(xl, w, static_cast<int64_t>(p.items) * p.PQ, kred, x_unsigned, xzp, wzp, epi, om, out,
-                          static_cast<int64_t>(img) * p.PQ + static_cast<int64_t>(p0) * p.Q, 0, rows * p.Q, p.K);
+                for (int i = tid; i < rows * p.Q * p.K; i += kBandThreads)
+                {
+                    const int n = i % p.K, pix = i / p.K;
+                    const int py = p0 + pix / p.Q, px = pix % p.Q;
+                    int32_t a = 0;
+                    for (int r = 0; r < p.R; ++r)
+                        for (int sx = 0; sx < p.S; ++sx)
+                        {
+                            const int iy = py + r - p.pbh, ix = px + sx - p.pbw;
+                            if (static_cast<uint32_t>(iy) >= static_cast<uint32_t>(p.H) || static_cast<uint32_t>(ix) >= static_cast<uint32_t>(p.W))
+                                continue; // padding is the data zero point: contributes nothing
+                            const uint8_t* xp = p.x + (static_cast<int64_t>(img) * p.H * p.W + iy * p.W + ix) * kBandC;
+                            const int8_t* wp = w + static_cast<int64_t>(n) * kred + (r * p.S + sx) * kBandC;
+                            for (int c = 0; c < kBandC; ++c)
+                            {
+                                const int32_t xv = x_unsigned ? static_cast<int32_t>(xp[c]) : static_cast<int32_t>(static_cast<int8_t>(xp[c]));
+                                a += (xv - xzp) * (static_cast<int32_t>(wp[c]) - wzp);
+                            }
+                        }
+                    const int64_t gp = static_cast<int64_t>(img) * p.PQ + static_cast<int64_t>(p0) * p.Q + pix;
+                    const int64_t o = OUT_NCX ? (static_cast<int64_t>(img) * p.K + n) * p.PQ + static_cast<int64_t>(p0) * p.Q + pix : gp * p.K + n;
+                    store_out(out, epi.out_t, o, epi_apply(epi, er, a, n, o));
+                }
             }
             return;
         }
@@ -390,7 +424,7 @@ namespace hipq
                         }
                         const int woff = band_slot_offset(l32, half);
                         if (sp <= 1) HIPQ_PHASE(11);
-                        band_reduce<4>(acc, lds, xs_off, woff, slot0, half, p.R, p.S, p.BW);
+                        band_reduce<4, U>(acc, lds, xs_off, woff, slot0, half, p.R, p.S, p.BW);
                         if (sp <= 1) HIPQ_PHASE(12);
                     }
                 }
@@ -655,10 +689,10 @@ namespace hipq
         return band_plan(g, out_ncx, &bp, &lds_bytes);
     }
 
-    template <int MODE, int KIND, bool OUT_NCX>
-    static int launch_band(const BandParams& bp, const ConvX& xl, size_t lds_bytes, const int8_t* w, const int32_t* wsum, int xu, const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s)
+    template <int MODE, int KIND, bool OUT_NCX, int U>
+    static int launch_band(const BandParams& bp, size_t lds_bytes, const int8_t* w, const int32_t* wsum, int xu, const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s)
     {
-        auto kernel = conv_band_kernel<MODE, KIND, OUT_NCX>;
+        auto kernel = conv_band_kernel<MODE, KIND, OUT_NCX, U>;
         static bool configured[16] = {};
         int dev = 0;
         HIPQ_HIP(hipGetDevice(&dev));
@@ -676,7 +710,7 @@ namespace hipq
         }
         const int slots = dev >= 0 && dev < 16 && cus[dev] > 0 ? cus[dev] : 256; // one persistent workgroup per CU
         const unsigned grid = static_cast<unsigned>(bp.items < slots ? bp.items : slots);
-        kernel<<<grid, kBandThreads, lds_bytes, s>>>(bp, xl, w, wsum, xu, zp, epi, out);
+        kernel<<<grid, kBandThreads, lds_bytes, s>>>(bp, w, wsum, xu, zp, epi, out);
         return check_launch("conv_band_i8_32x32x32");
     }
 
@@ -696,27 +730,17 @@ namespace hipq
                          (reinterpret_cast<uintptr_t>(out) & 15) == 0,
                      "band convolution needs 16-byte aligned tensors");
         bp.x = static_cast<const uint8_t*>(data_nxc);
-        ConvX xl;
-        xl.x = bp.x;
-        xl.H = bp.H;
-        xl.W = bp.W;
-        xl.C = kBandC;
-        xl.Q = bp.Q;
-        xl.R = bp.R;
-        xl.S = bp.S;
-        xl.sh = xl.sw = xl.dh = xl.dw = 1;
-        xl.pbh = bp.pbh;
-        xl.pbw = bp.pbw;
-        xl.PQ = bp.PQ;
-        xl.bytes = bp.x_bytes;
         const int kred = bp.R * bp.S * kBandC;
         const int8_t* w = static_cast<const int8_t*>(packed);
         const int32_t* wsum = reinterpret_cast<const int32_t*>(static_cast<const uint8_t*>(packed) + align_up(static_cast<size_t>(g.K) * kred, 256));
         const int xu = g.data_t == HIPQ_U8 ? 1 : 0;
         const bool q8 = g.out_t == HIPQ_U8 || g.out_t == HIPQ_I8;
+        const bool u3 = (bp.R * bp.S) % 3 == 0;
 #define BAND(MODE, KIND)                                                                           \
-    (out_ncx ? launch_band<MODE, KIND, true>(bp, xl, lds_bytes, w, wsum, xu, zp, epi, out, s)      \
-             : launch_band<MODE, KIND, false>(bp, xl, lds_bytes, w, wsum, xu, zp, epi, out, s))
+    (out_ncx ? (u3 ? launch_band<MODE, KIND, true, 3>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)     \
+                   : launch_band<MODE, KIND, true, 1>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s))    \
+             : (u3 ? launch_band<MODE, KIND, false, 3>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)    \
+                   : launch_band<MODE, KIND, false, 1>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)))
         if (epi.mode == EPI_INTERP)
             return q8 ? BAND(EPI_INTERP, OUT_Q8) : BAND(EPI_INTERP, OUT_I32);
         if (q8)

@@ -83,7 +83,7 @@ namespace hipq
             return (r.off != kOob && c.kbyte < K) ? r.off + c.kbyte : kOob;
         }
         // slow path: exact accumulator of one output, any zero points
-        __device__ int32_t direct(int64_t m, const int8_t* wrow, int32_t xzp, int32_t wzp, bool x_unsigned) const
+        __device__ __forceinline__ int32_t direct(int64_t m, const int8_t* wrow, int32_t xzp, int32_t wzp, bool x_unsigned) const
         {
             const uint8_t* p = x + m * static_cast<int64_t>(K);
             int32_t acc = 0;
@@ -151,7 +151,7 @@ namespace hipq
                             (static_cast<uint32_t>(xx) < static_cast<uint32_t>(W));
             return ok ? rw.base + (y * W + xx) * C + c.c : kOob;
         }
-        __device__ int32_t direct(int64_t m, const int8_t* wrow, int32_t xzp, int32_t wzp, bool x_unsigned) const
+        __device__ __forceinline__ int32_t direct(int64_t m, const int8_t* wrow, int32_t xzp, int32_t wzp, bool x_unsigned) const
         {
             Row rw;
             init_row(rw, m, m + 1);
@@ -190,16 +190,19 @@ namespace hipq
         }
     };
 
+    // Out of line, so that its registers do not weigh on the MFMA path, with the descriptors passed
+    // by value: passed by reference the kernel's own arguments would have to live in scratch
+    // memory, and every lane of every launch would store them there on entry.
     template <class XL>
-    __device__ __noinline__ void slow_tile(const XL& xl,
+    __device__ __noinline__ void slow_tile(const XL xl,
                                            const int8_t* __restrict__ w,
                                            int64_t M,
                                            int32_t Kred,
                                            int32_t x_unsigned,
                                            int32_t xzp,
                                            int32_t wzp,
-                                           const Epilogue& epi,
-                                           const OutMap& om,
+                                           const Epilogue epi,
+                                           const OutMap om,
                                            void* __restrict__ out,
                                            int64_t m0,
                                            int32_t n0,

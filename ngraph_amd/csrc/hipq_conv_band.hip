@@ -20,6 +20,7 @@
 // sign-bias correction are per-lane constants) and four consecutive pixels per accumulator group.
 // 8-bit results are staged through LDS so that every global store is a full 16-byte piece of a
 // line in either output layout.
+#include <cstdlib>
 #include <type_traits>
 
 #include "hipq_igemm.h"
@@ -34,12 +35,32 @@ static __device__ long long g_phase_clock[32];
         if (blockIdx.x == 0 && (threadIdx.x & 255) == 0 && (i) < 16)                               \
             g_phase_clock[(threadIdx.x >> 8) * 16 + (i)] = clock64();                              \
     } while (0)
+static __device__ long long g_block_times[256][4];
+#define HIPQ_BLOCK_BEGIN()                                                                         \
+    long long blk_w0 = wall_clock64(), blk_c0 = clock64()
+#define HIPQ_BLOCK_END()                                                                           \
+    do                                                                                             \
+    {                                                                                              \
+        if (threadIdx.x == 0 && blockIdx.x < 256)                                                  \
+        {                                                                                          \
+            g_block_times[blockIdx.x][0] = blk_w0;                                                 \
+            g_block_times[blockIdx.x][1] = wall_clock64();                                         \
+            g_block_times[blockIdx.x][2] = clock64() - blk_c0;                                     \
+            g_block_times[blockIdx.x][3] = __builtin_amdgcn_s_getreg(((32 - 1) << 11) | 4);        \
+        }                                                                                          \
+    } while (0)
+extern "C" HIPQ_API int hipq_debug_band_blocks(long long* out1024)
+{
+    return hipMemcpyFromSymbol(out1024, HIP_SYMBOL(g_block_times), sizeof(long long) * 1024) == hipSuccess ? 0 : 1;
+}
 extern "C" HIPQ_API int hipq_debug_band_phases(long long* out32)
 {
     return hipMemcpyFromSymbol(out32, HIP_SYMBOL(g_phase_clock), sizeof(long long) * 32) == hipSuccess ? 0 : 1;
 }
 #else
 #define HIPQ_PHASE(i) ((void)0)
+#define HIPQ_BLOCK_BEGIN() ((void)0)
+#define HIPQ_BLOCK_END() ((void)0)
 #endif
 
 namespace hipq
@@ -59,7 +80,10 @@ namespace hipq
         int32_t TP;         // output rows per band
         int32_t bands;      // bands per image
         int32_t items;      // N * bands
-        int32_t BW;         // band width in pixel slots: Q + S - 1
+        int32_t BW;         // slots per band row in LDS: Q + S - 1 rounded up to a multiple of 16, so that
+                            // the chunk rotation of a slot does not depend on its row
+        int32_t BWr;        // slots per band row that hold data: Q + S - 1
+        int32_t q_magic;    // ceil(2^20 / Q): pix / Q = (pix * q_magic) >> 20 for pix < 2048
         int32_t x_lds;      // LDS byte offset of band buffer 0 (the filter sits in front of it)
         int32_t band_bytes; // bytes of one band buffer
         int32_t stage_lds;  // LDS byte offset of the output staging area (4 x kBandStageWave)
@@ -67,15 +91,19 @@ namespace hipq
         int64_t PQ;
     };
 
-    // LDS offset of 16-byte chunk `chunk` of 64-byte row `slot`.  A ds_read_b128 is served 16 lanes
-    // at a time from 64 banks: it runs at full rate when 16 consecutive rows at one chunk index land
-    // in 16 different 16-byte columns of a 256-byte line; rows s, s+4, s+8, s+12 share a 64-byte
-    // column group, so the chunk is rotated by (s / 4) % 4 (measured: 190 B/clk/CU against 128 for
-    // a rotation by (s / 2) % 4 and 64 for none).
-    __device__ __forceinline__ int band_slot_offset(int slot, int chunk)
+    // LDS layout of a row of 64-byte cells (the pixel slots of a band row, the 64 filter rows of a
+    // tap): two planes of 32-byte half cells, plane h holding the 16-byte chunks 2h and 2h+1 of
+    // every cell.  An MFMA fragment read takes chunk 2h + lane/32 of 32 consecutive cells, so both
+    // halves of a 64-byte step are one per-lane address plus a constant.  A ds_read_b128 is served
+    // 16 lanes at a time from 64 banks: 16 consecutive cells at one chunk index must land in 16
+    // different 16-byte columns of a 256-byte line; cells x and x+8 share a column pair, so the
+    // chunk within the half cell is flipped by (x / 8) % 2.  (Measured on 64-byte cells: 190
+    // B/clk/CU conflict-free against 128 with two-way and 64 with four-way conflicts.)
+    __device__ __forceinline__ int band_cell(int x, int chunk, int plane_bytes)
     {
-        return slot * kBandC + ((chunk ^ ((slot >> 2) & 3)) << 4);
+        return (chunk >> 1) * plane_bytes + x * 32 + (((chunk & 1) ^ ((x >> 3) & 1)) << 4);
     }
+    constexpr int kTapBytes = 64 * kBandC; // a filter tap in LDS: two planes of 64 x 32 bytes
 
     // Copies into LDS go in batches: all loads of a batch are issued before any is stored, and
     // issue and store recompute the addresses so that only the data stays in registers between.
@@ -85,8 +113,7 @@ namespace hipq
     };
 
     // Filter (all 512 lanes): 8 lanes per row n = tid / 8, lane tid % 8 takes every eighth 16-byte
-    // chunk of the row; batch element u is chunk tid % 8 + 8 * (u0 + u).  LDS: [tap][64 rows][64
-    // bytes], chunks swizzled like the band's.
+    // chunk of the row; batch element u is chunk tid % 8 + 8 * (u0 + u).  LDS: [tap][plane][64 rows].
     template <bool STORE>
     __device__ __forceinline__ void band_w_copy(BandBatch& b, __amdgpu_buffer_rsrc_t wrs, uint8_t* lds, int u0, int taps, int kred, int K, int sink)
     {
@@ -98,7 +125,7 @@ namespace hipq
             const int c = sub + 8 * (u0 + u);
             const bool in = c < taps * 4;
             if (STORE)
-                *reinterpret_cast<v4i*>(lds + (in ? (c >> 2) * (64 * kBandC) + band_slot_offset(n, c & 3) : sink)) = b.v[u];
+                *reinterpret_cast<v4i*>(lds + (in ? (c >> 2) * kTapBytes + band_cell(n, c & 3, kTapBytes / 2) : sink)) = b.v[u];
             else
                 b.v[u] = buffer_load16(wrs, (in && n < K) ? n * kred + c * 16 : kOob); // rows beyond K read as zeros
         }
@@ -106,14 +133,15 @@ namespace hipq
 
     // Band (the 256 lanes of a group): lane takes chunk cx = cx0 + gtid of a row of BW pixel slots
     // (4 chunks a slot); batch element u is band row sy0 + u.  xs_off: LDS offset of the group's buffer.
-    template <bool STORE>
+    // FILL: padding is a non-zero byte (out-of-range loads give zeros, which is the padding otherwise)
+    template <bool STORE, bool FILL = false>
     __device__ __forceinline__ void band_x_copy(BandBatch& b, __amdgpu_buffer_rsrc_t xrs, uint8_t* lds, const BandParams& p, int xs_off, int cx0, int sy0, int band_rows, int img_base, int p0, int fill, int xor_mask)
     {
         const int cx = cx0 + (static_cast<int>(threadIdx.x) & 255);
         const int sx = cx >> 2;
         const int c4 = cx & 3;
         const int ix = sx - p.pbw;
-        const bool col_in = sx < p.BW;
+        const bool col_in = sx < p.BWr;
         const bool col_ok = col_in & (static_cast<uint32_t>(ix) < static_cast<uint32_t>(p.W));
 #pragma unroll
         for (int u = 0; u < kBandBatch; ++u)
@@ -124,11 +152,10 @@ namespace hipq
             const bool ok = col_ok & (sy < band_rows) & (static_cast<uint32_t>(iy) < static_cast<uint32_t>(p.H));
             if (STORE)
             {
-                // padding is the data zero point (out-of-range loads gave zeros); a select per dword is
-                // cheaper than a branch around it, taken or not
                 v4i t = b.v[u];
-                t = v4i{ok ? t[0] : fill, ok ? t[1] : fill, ok ? t[2] : fill, ok ? t[3] : fill};
-                *reinterpret_cast<v4i*>(lds + (in ? xs_off + band_slot_offset(sy * p.BW + sx, c4) : p.sink)) =
+                if (FILL)
+                    t = v4i{ok ? t[0] : fill, ok ? t[1] : fill, ok ? t[2] : fill, ok ? t[3] : fill};
+                *reinterpret_cast<v4i*>(lds + (in ? xs_off + sy * (p.BW * kBandC) + band_cell(sx, c4, p.BW * 32) : p.sink)) =
                     v4i{t[0] ^ xor_mask, t[1] ^ xor_mask, t[2] ^ xor_mask, t[3] ^ xor_mask};
             }
             else
@@ -143,47 +170,34 @@ namespace hipq
     // Reduction of T pixel tiles x 2 channel tiles over all taps, out of LDS: per 32-byte half of a
     // tap 2 weight fragments, T pixel fragments, 2T MFMAs; no barrier, no global access.  Two
     // fragment sets alternate (statically indexed) so that the reads of one half overlap the MFMAs
-    // of the other.  woff: LDS offset of this lane's weight row at tap 0, chunk lane/32.
-    // U taps per loop trip; the tap count must be a multiple of U.  (A taken branch costs about as
-    // much as four MFMAs here, but unrolling all nine taps of a 3x3 filter made the register
-    // allocator spill accumulators, which costs far more.)
+    // of the other.  woff: LDS offset of this lane's filter row in plane 0 of tap 0; xrow0 / xcol0:
+    // LDS offset of the band row and the slot in it of each tile's pixel (tap 0,0).
+    // U taps per loop trip; the tap count must be a multiple of U.
     template <int T, int U>
-    __device__ __forceinline__ void band_reduce(v16i (&acc)[4][2], const uint8_t* lds, int xs_off, int woff, const int (&slot0)[4], int half, int R, int S, int BW)
+    __device__ __forceinline__ void band_reduce(v16i (&acc)[4][2], const uint8_t* lds, int woff, const int (&xrow0)[4], const int (&xcol0)[4], int half, int R, int S, int BW)
     {
+        const int plane = BW * 32, rowp = BW * kBandC;
         v4i xa[T], xb[T], wa[2], wb[2];
         int xoff[T], xnext[T];
-        auto addr = [&](int tap_slot, int(&xo)[T]) {
+        auto addr = [&](int r, int sx, int(&xo)[T]) {
 #pragma unroll
             for (int ti = 0; ti < T; ++ti)
-                xo[ti] = xs_off + band_slot_offset(slot0[ti] + tap_slot, half);
+                xo[ti] = xrow0[ti] + r * rowp + band_cell(xcol0[ti] + sx, half, 0);
         };
-        // chunks 2,3 of a 64-byte row are chunks 0,1 with offset bit 5 flipped
-        auto load = [&](int wp, const int(&xo)[T], int flip, v4i(&xf)[T], v4i(&wf)[2]) {
+        auto load = [&](int wp, const int(&xo)[T], int h, v4i(&xf)[T], v4i(&wf)[2]) {
 #pragma unroll
             for (int ni = 0; ni < 2; ++ni)
-#ifdef BAND_EXP_NOLDS
-                wf[ni] = v4i{wp, flip, ni, wp};
-#else
-                wf[ni] = *reinterpret_cast<const v4i*>(lds + (wp ^ flip) + ni * 32 * kBandC);
-#endif
+                wf[ni] = *reinterpret_cast<const v4i*>(lds + wp + h * (kTapBytes / 2) + ni * 32 * 32);
 #pragma unroll
             for (int ti = 0; ti < T; ++ti)
-#ifdef BAND_EXP_NOLDS
-                xf[ti] = v4i{xo[ti], flip, ti, wp};
-#else
-                xf[ti] = *reinterpret_cast<const v4i*>(lds + (xo[ti] ^ flip));
-#endif
+                xf[ti] = *reinterpret_cast<const v4i*>(lds + xo[ti] + h * plane);
         };
         auto mac = [&](const v4i(&xf)[T], const v4i(&wf)[2]) {
 #pragma unroll
             for (int ti = 0; ti < T; ++ti)
 #pragma unroll
                 for (int ni = 0; ni < 2; ++ni)
-#ifdef BAND_EXP_NOMFMA
-                    acc[ti][ni][0] += xf[ti][0] ^ wf[ni][0] ^ xf[ti][3] ^ wf[ni][3];
-#else
                     acc[ti][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xf[ti], wf[ni], acc[ti][ni], 0, 0, 0);
-#endif
         };
         // One wavefront issues in order: an MFMA occupies the matrix core for 32 cycles and anything
         // issued behind it runs in its shadow, but 2T MFMAs back to back leave no shadow for the
@@ -200,49 +214,114 @@ namespace hipq
         };
         // The pipeline, per tap: while half 0 multiplies, half 1 is read and the next tap's LDS
         // offsets are computed; while half 1 multiplies, the next tap's half 0 is read.
-        addr(0, xoff);
+        addr(0, 0, xoff);
         load(woff, xoff, 0, xa, wa);
         __builtin_amdgcn_sched_barrier(0);
-        {
-            int wp = woff;
-            int r = 0, s = 0;
-            const int taps = R * S;
+        int wp = woff;
+        int r = 0, sx = 0;
+        const int taps = R * S;
 #pragma unroll 1
-            for (int tap = 0; tap < taps; tap += U)
+        for (int tap = 0; tap < taps; tap += U)
+        {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
             {
-#pragma unroll
-                for (int u = 0; u < U; ++u)
+                load(wp, xoff, 1, xb, wb);
+                // the next tap; after the last one this wraps to tap 0, a harmless re-read that
+                // keeps the loop free of conditional loads
+                wp += kTapBytes;
+                ++sx;
+                if (sx == S)
                 {
-                    load(wp, xoff, 32, xb, wb);
-                    // the next tap; after the last one this wraps to tap 0, a harmless re-read that
-                    // keeps the loop free of conditional loads
-                    wp += 64 * kBandC;
-                    ++s;
-                    if (s == S)
-                    {
-                        s = 0;
-                        ++r;
-                    }
-                    if (r == R)
-                    {
-                        r = 0;
-                        wp = woff;
-                    }
-                    addr(r * BW + s, xnext);
-                    mac(xa, wa);
-                    interleave();
-#pragma unroll
-                    for (int ti = 0; ti < T; ++ti)
-                        xoff[ti] = xnext[ti];
-                    load(wp, xoff, 0, xa, wa);
-                    mac(xb, wb);
-                    interleave();
+                    sx = 0;
+                    ++r;
                 }
+                if (r == R)
+                {
+                    r = 0;
+                    wp = woff;
+                }
+                addr(r, sx, xnext);
+                mac(xa, wa);
+                interleave();
+#pragma unroll
+                for (int ti = 0; ti < T; ++ti)
+                    xoff[ti] = xnext[ti];
+                load(wp, xoff, 0, xa, wa);
+                mac(xb, wb);
+                interleave();
             }
         }
     }
 
-    // U: filter taps per trip of the reduction loop (the tap count is a multiple of it)
+    // The same reduction for a 3x3 filter over band rows of 64 slots: every LDS address is a
+    // per-lane base (one per pixel tile and filter column, computed once per band) plus a
+    // compile-time offset (filter row, half, tap, channel tile), so the 144 MFMAs and 108 reads run
+    // as straight-line code without address arithmetic, loop branches or register shuffles.
+    template <int T>
+    __device__ __forceinline__ void band_reduce_33(v16i (&acc)[4][2], const uint8_t* lds, int woff, const int (&xrow0)[4], const int (&xcol0)[4], int half, const int32_t (&corr)[2])
+    {
+        constexpr int kRow = 64 * kBandC; // bytes of a band row of 64 slots (two planes of 2048)
+        int xbase[T][3];
+#pragma unroll
+        for (int ti = 0; ti < T; ++ti)
+#pragma unroll
+            for (int sx = 0; sx < 3; ++sx)
+                xbase[ti][sx] = xrow0[ti] + band_cell(xcol0[ti] + sx, half, 0);
+        v4i xa[T], xb[T], wa[2], wb[2];
+        auto load = [&](int k, v4i(&xf)[T], v4i(&wf)[2]) {
+            const int tap = k >> 1, h = k & 1, r = tap / 3, sx = tap % 3;
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+                wf[ni] = *reinterpret_cast<const v4i*>(lds + woff + tap * kTapBytes + h * (kTapBytes / 2) + ni * 32 * 32);
+#pragma unroll
+            for (int ti = 0; ti < T; ++ti)
+                xf[ti] = *reinterpret_cast<const v4i*>(lds + xbase[ti][sx] + r * kRow + h * (kRow / 2));
+        };
+        // the first step starts the accumulators from the constant 0 (no initialisation moves; tuples
+        // preloaded with the correction made the register allocator spill); the sign-bias correction
+        // is added after the last MFMA, still in the multiply phase, which is the shorter one
+        auto mac = [&](const v4i(&xf)[T], const v4i(&wf)[2], bool first) {
+            const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int ti = 0; ti < T; ++ti)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+                    acc[ti][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xf[ti], wf[ni], first ? zero : acc[ti][ni], 0, 0, 0);
+        };
+        auto interleave = [&]() {
+#pragma unroll
+            for (int i = 0; i < 2 * T; ++i)
+            {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        load(0, xa, wa);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < 18; k += 2)
+        {
+            load(k + 1, xb, wb);
+            mac(xa, wa, k == 0);
+            interleave();
+            if (k + 2 < 18)
+                load(k + 2, xa, wa);
+            mac(xb, wb, false);
+            interleave();
+        }
+#pragma unroll
+        for (int ti = 0; ti < T; ++ti)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    acc[ti][ni][r] += corr[ni];
+    }
+
+    // U: filter taps per trip of the reduction loop (the tap count is a multiple of it); 0: the
+    // straight-line 3x3 reduction over 64-slot band rows
     template <int MODE, int KIND, bool OUT_NCX, int U>
     __global__ __launch_bounds__(kBandThreads) void conv_band_kernel(BandParams p,
                                                                     const int8_t* __restrict__ w,
@@ -264,6 +343,7 @@ namespace hipq
         const int l32 = lane & 31;
         const int xs_off = p.x_lds + grp * p.band_bytes;
 
+        HIPQ_BLOCK_BEGIN();
         HIPQ_PHASE(0);
         // ---- small loads first: they must not queue behind the bulk loads ------------------------
         const int32_t xzp = load_zp(zp.data_zp, zp.data_t);
@@ -355,13 +435,18 @@ namespace hipq
             item_geom(j, img, p0, rows);
             const int band_rows = rows + p.R - 1;
             const int img_base = img * p.H * p.W * kBandC;
-            for (int cx0 = 0; cx0 < p.BW * 4; cx0 += 256)
-                for (int sy0 = 0; sy0 < band_rows; sy0 += kBandBatch)
-                {
-                    if (cx0 | sy0)
-                        band_x_copy<false>(xb0, xrs, lds, p, xs_off, cx0, sy0, band_rows, img_base, p0, fill, xor_mask);
-                    band_x_copy<true>(xb0, xrs, lds, p, xs_off, cx0, sy0, band_rows, img_base, p0, fill, xor_mask);
-                }
+            if (fill == 0)
+                band_x_copy<true, false>(xb0, xrs, lds, p, xs_off, 0, 0, band_rows, img_base, p0, fill, xor_mask);
+            else
+                band_x_copy<true, true>(xb0, xrs, lds, p, xs_off, 0, 0, band_rows, img_base, p0, fill, xor_mask);
+            if (p.BWr * 4 > 256 || band_rows > kBandBatch) // wide or tall bands: the rest, batch by batch
+                for (int cx0 = 0; cx0 < p.BWr * 4; cx0 += 256)
+                    for (int sy0 = 0; sy0 < band_rows; sy0 += kBandBatch)
+                        if (cx0 | sy0)
+                        {
+                            band_x_copy<false>(xb0, xrs, lds, p, xs_off, cx0, sy0, band_rows, img_base, p0, fill, xor_mask);
+                            band_x_copy<true, true>(xb0, xrs, lds, p, xs_off, cx0, sy0, band_rows, img_base, p0, fill, xor_mask);
+                        }
         };
 
         HIPQ_PHASE(1);
@@ -404,27 +489,34 @@ namespace hipq
                     const int npix = rows * p.Q;
                     const int ntiles = (npix + 31) >> 5;
                     // wavefront gw owns tiles 4*gw .. 4*gw+3
+                    if (U != 0) // the straight-line reduction brings the correction in with its first MFMAs
+                    {
 #pragma unroll
-                    for (int ti = 0; ti < 4; ++ti)
+                        for (int ti = 0; ti < 4; ++ti)
 #pragma unroll
-                        for (int ni = 0; ni < 2; ++ni)
+                            for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-                            for (int r = 0; r < 16; ++r)
-                                acc[ti][ni][r] = corr[ni];
+                                for (int r = 0; r < 16; ++r)
+                                    acc[ti][ni][r] = corr[ni];
+                    }
                     if (4 * gw < ntiles)
                     {
-                        int slot0[4];
+                        int xrow0[4], xcol0[4];
 #pragma unroll
                         for (int ti = 0; ti < 4; ++ti)
                         {
                             // tiles past the end re-read the last pixel; their results are never stored
                             const int pix = min((4 * gw + ti) * 32 + l32, npix - 1);
-                            const int py = pix / p.Q;
-                            slot0[ti] = py * p.BW + (pix - py * p.Q);
+                            const int py = (pix * p.q_magic) >> 20;
+                            xrow0[ti] = xs_off + py * (p.BW * kBandC);
+                            xcol0[ti] = pix - py * p.Q;
                         }
-                        const int woff = band_slot_offset(l32, half);
+                        const int woff = band_cell(l32, half, 0);
                         if (sp <= 1) HIPQ_PHASE(11);
-                        band_reduce<4, U>(acc, lds, xs_off, woff, slot0, half, p.R, p.S, p.BW);
+                        if (U == 0)
+                            band_reduce_33<4>(acc, lds, woff, xrow0, xcol0, half, corr);
+                        else
+                            band_reduce<4, U == 0 ? 1 : U>(acc, lds, woff, xrow0, xcol0, half, p.R, p.S, p.BW);
                         if (sp <= 1) HIPQ_PHASE(12);
                     }
                 }
@@ -615,6 +707,7 @@ namespace hipq
         }
         for (; phases_done < my_items + 1; ++phases_done)
             __syncthreads();
+        HIPQ_BLOCK_END();
     }
 
     // rows per band and LDS bytes; false when the layer does not fit this kernel
@@ -637,7 +730,8 @@ namespace hipq
         if (g.in_count() >= (1ll << 31) || g.out_count() >= (1ll << 31) || g.N * P >= (1ll << 30))
             return false;
         const int64_t wbytes = R * S * 64 * kBandC; // [tap][64][64]
-        const int64_t BW = Q + S - 1;
+        const int64_t BWr = Q + S - 1;
+        const int64_t BW = (BWr + 15) / 16 * 16;
         const int64_t budget = 160 * 1024; // one workgroup per CU: filter, two band buffers, staging
         int64_t best = 0;
         for (int64_t tp = 1; tp <= P && tp * Q <= 512; ++tp)
@@ -671,6 +765,8 @@ namespace hipq
         bp->bands = static_cast<int32_t>((P + best - 1) / best);
         bp->items = static_cast<int32_t>(g.N * bp->bands);
         bp->BW = static_cast<int32_t>(BW);
+        bp->BWr = static_cast<int32_t>(BWr);
+        bp->q_magic = static_cast<int32_t>(((1 << 20) + Q - 1) / Q);
         bp->x_lds = static_cast<int32_t>(wbytes);
         bp->band_bytes = static_cast<int32_t>(band_bytes);
         bp->stage_lds = static_cast<int32_t>(wbytes + 2 * band_bytes);
@@ -735,17 +831,19 @@ namespace hipq
         const int32_t* wsum = reinterpret_cast<const int32_t*>(static_cast<const uint8_t*>(packed) + align_up(static_cast<size_t>(g.K) * kred, 256));
         const int xu = g.data_t == HIPQ_U8 ? 1 : 0;
         const bool q8 = g.out_t == HIPQ_U8 || g.out_t == HIPQ_I8;
-        const bool u3 = (bp.R * bp.S) % 3 == 0;
-#define BAND(MODE, KIND)                                                                           \
-    (out_ncx ? (u3 ? launch_band<MODE, KIND, true, 3>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)     \
-                   : launch_band<MODE, KIND, true, 1>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s))    \
-             : (u3 ? launch_band<MODE, KIND, false, 3>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)    \
-                   : launch_band<MODE, KIND, false, 1>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)))
+        // straight-line reduction for 3x3 filters over 64-slot band rows, else a loop of 3 or 1 taps a trip
+        const int u = (bp.R == 3 && bp.S == 3 && bp.BW == 64 && getenv("HIPQ_BAND_LOOP") == nullptr) ? 0 : ((bp.R * bp.S) % 3 == 0 ? 3 : 1);
+#define BAND_U(MODE, KIND, NCX)                                                                    \
+    (u == 0 ? launch_band<MODE, KIND, NCX, 0>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)          \
+            : (u == 3 ? launch_band<MODE, KIND, NCX, 3>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s) \
+                      : launch_band<MODE, KIND, NCX, 1>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)))
+#define BAND(MODE, KIND) (out_ncx ? BAND_U(MODE, KIND, true) : BAND_U(MODE, KIND, false))
         if (epi.mode == EPI_INTERP)
             return q8 ? BAND(EPI_INTERP, OUT_Q8) : BAND(EPI_INTERP, OUT_I32);
         if (q8)
             return BAND(EPI_FUSED, OUT_Q8);
 #undef BAND
+#undef BAND_U
         return fail(HIPQ_ERR_UNSUPPORTED, "no band kernel for this epilogue / output type");
     }
 }

@@ -36,6 +36,17 @@ static __device__ long long g_phase_clock[32];
             g_phase_clock[(threadIdx.x >> 8) * 16 + (i)] = clock64();                              \
     } while (0)
 static __device__ long long g_block_times[256][4];
+static __device__ long long g_wave_clock[8][8][2]; // [phase][wave][arrive at barrier, leave barrier]
+#define HIPQ_WAVE_MARK(phase, which)                                                               \
+    do                                                                                             \
+    {                                                                                              \
+        if (blockIdx.x == 0 && (threadIdx.x & 63) == 0 && (phase) < 8)                             \
+            g_wave_clock[phase][threadIdx.x >> 6][which] = clock64();                              \
+    } while (0)
+extern "C" HIPQ_API int hipq_debug_band_waves(long long* out128)
+{
+    return hipMemcpyFromSymbol(out128, HIP_SYMBOL(g_wave_clock), sizeof(long long) * 128) == hipSuccess ? 0 : 1;
+}
 #define HIPQ_BLOCK_BEGIN()                                                                         \
     long long blk_w0 = wall_clock64(), blk_c0 = clock64()
 #define HIPQ_BLOCK_END()                                                                           \
@@ -61,6 +72,7 @@ extern "C" HIPQ_API int hipq_debug_band_phases(long long* out32)
 #define HIPQ_PHASE(i) ((void)0)
 #define HIPQ_BLOCK_BEGIN() ((void)0)
 #define HIPQ_BLOCK_END() ((void)0)
+#define HIPQ_WAVE_MARK(phase, which) ((void)0)
 #endif
 
 namespace hipq
@@ -159,11 +171,7 @@ namespace hipq
                     v4i{t[0] ^ xor_mask, t[1] ^ xor_mask, t[2] ^ xor_mask, t[3] ^ xor_mask};
             }
             else
-#ifdef BAND_EXP_NOBANDLOAD
-                b.v[u] = v4i{iy, ix, c4, u};
-#else
                 b.v[u] = buffer_load16(xrs, ok ? img_base + (iy * p.W + ix) * kBandC + c4 * 16 : kOob);
-#endif
         }
     }
 
@@ -483,6 +491,10 @@ namespace hipq
             v16i acc[4][2];
             {
                 // ================= multiply: item sp =================
+                // The SIMD's arbiter favours its older wavefront; without a hint group 1 starves in
+                // either role.  The multiply phase has few, long instructions: it gets priority and the
+                // requantizing wavefront fills the gaps.
+                __builtin_amdgcn_s_setprio(3);
                 {
                     if (sp <= 1) HIPQ_PHASE(10);
                     item_geom(sp, img, p0, rows);
@@ -521,6 +533,7 @@ namespace hipq
                     }
                 }
             }
+            __builtin_amdgcn_s_setprio(0);
             // the group's next band starts its way into registers now (the fragment registers are
             // free), flies through the barrier and the requantization, and moves into the band buffer
             // at the end of the next phase
@@ -530,7 +543,9 @@ namespace hipq
                 item_geom(sp + 2, img, p0, rows);
                 band_x_copy<false>(nb, xrs, lds, p, xs_off, 0, 0, rows + p.R - 1, img * p.H * p.W * kBandC, p0, 0, 0);
             }
+            HIPQ_WAVE_MARK(phases_done, 0);
             __syncthreads();
+            HIPQ_WAVE_MARK(phases_done, 1);
             ++phases_done;
             HIPQ_PHASE(2 + phases_done);
             {
@@ -701,7 +716,9 @@ namespace hipq
                     band_store(nb, sp + 2);
                 if (sp <= 1) HIPQ_PHASE(8);
             }
+            HIPQ_WAVE_MARK(phases_done, 0);
             __syncthreads();
+            HIPQ_WAVE_MARK(phases_done, 1);
             ++phases_done;
             HIPQ_PHASE(2 + phases_done);
         }

@@ -1,11 +1,12 @@
 // int8 GEMM on the i8 matrix cores: eligibility and launch (kernel in hipq_igemm.h).
 #include <cstdlib>
+#include <type_traits>
 
 #include "hipq_igemm.h"
 
 namespace hipq
 {
-    // ---- skinny GEMM: M <= 64 ------------------------------------------------------------------
+    // ---- skinny GEMM: M <= 256 ------------------------------------------------------------------
     // With a handful of rows the product is a stream over the weights: every weight byte must come
     // from HBM once and is used for at most 64 MACs.  One workgroup owns 16 output columns and the
     // whole reduction, so no partial sums leave the CU; its four wavefronts split K four ways, each
@@ -13,6 +14,51 @@ namespace hipq
     // sixteen 64-byte steps in flight before the first MFMA), and the four partial 16x16 tiles meet in
     // LDS.  N / 16 workgroups: 256 for N = 4096, one per CU.
     typedef int v4acc __attribute__((ext_vector_type(4)));
+
+    // Requantization and store of one lane's finished outputs (column n, rows m[i]), with the
+    // policy and output kind resolved once instead of per element.
+    template <int COUNT, class RowOf, class AccOf>
+    __device__ __forceinline__ void skinny_finish(const Epilogue& epi, int32_t M, int32_t N, int n, RowOf row_of, AccOf acc_of, void* __restrict__ out)
+    {
+        const EpiConst ec = epi_const(epi);
+        const float bias = (epi.mode == EPI_FUSED && epi.bias) ? static_cast<float>(epi.bias[n]) : 0.0f;
+        const float scale = (epi.mode == EPI_FUSED && epi.per_channel) ? epi.scale[n] : ec.scale;
+        const bool relu = epi.relu != 0;
+        auto run = [&](auto mode_c, auto kind_c) {
+            constexpr int MODE = decltype(mode_c)::value;
+            constexpr int KIND = decltype(kind_c)::value;
+#pragma unroll
+            for (int i = 0; i < COUNT; ++i)
+            {
+                const int m = row_of(i);
+                if (m < M)
+                {
+                    const int32_t a = acc_of(i);
+                    const int32_t v = MODE == EPI_INTERP ? epi_interp<KIND>(ec, a) : epi_fused<KIND>(ec, a, bias, scale, false, 0.0f, relu);
+                    const int64_t o = static_cast<int64_t>(m) * N + n;
+                    if (KIND == OUT_Q8)
+                        static_cast<uint8_t*>(out)[o] = static_cast<uint8_t>(v);
+                    else
+                        static_cast<int32_t*>(out)[o] = v;
+                }
+            }
+        };
+        using std::integral_constant;
+        const bool q8 = epi.out_t == HIPQ_U8 || epi.out_t == HIPQ_I8;
+        if (epi.mode == EPI_INTERP)
+        {
+            if (q8)
+                run(integral_constant<int, EPI_INTERP>{}, integral_constant<int, OUT_Q8>{});
+            else
+                run(integral_constant<int, EPI_INTERP>{}, integral_constant<int, OUT_I32>{});
+        }
+        else if (q8)
+            run(integral_constant<int, EPI_FUSED>{}, integral_constant<int, OUT_Q8>{});
+        else if (epi.out_t == HIPQ_F32)
+            run(integral_constant<int, EPI_FUSED>{}, integral_constant<int, OUT_F32>{});
+        else
+            run(integral_constant<int, EPI_FUSED>{}, integral_constant<int, OUT_I32>{});
+    }
 
     template <int MT, int STEPS>
     __global__ __launch_bounds__(256) void dot_skinny_kernel(const uint8_t* __restrict__ a,
@@ -60,7 +106,8 @@ namespace hipq
         const __amdgpu_buffer_rsrc_t ars = make_rsrc(a, static_cast<uint32_t>(M) * static_cast<uint32_t>(K));
         const __amdgpu_buffer_rsrc_t wrs = make_rsrc(w, static_cast<uint32_t>(N) * static_cast<uint32_t>(K));
         const int kq = ((K / 64 + 3) / 4) * 64; // bytes of K per wavefront, whole 64-byte steps
-        const int k_begin = wave * kq;
+        // (rotated by workgroup: in lockstep all workgroups would queue on the same activation lines in L2)
+        const int k_begin = ((wave + static_cast<int>(blockIdx.x)) & 3) * kq;
         const int k_end = min(K, k_begin + kq);
         const int32_t wrow = n0 + r16 < N ? (n0 + r16) * K + kc * 16 : kOob;
         int32_t arow[MT];
@@ -111,25 +158,153 @@ namespace hipq
         if (n >= N)
             return;
         const int32_t corr = ((x_unsigned ? 128 : 0) - xzp) * wsum[n];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
+        // lane: column lane % 16; accumulator register r is row 4 * (lane / 16) + r of the tile
+        skinny_finish<MT * 4>(
+            epi, M, N, n, [&](int i) { return (i >> 2) * 16 + 4 * kc + (i & 3); },
+            [&](int i) { return acc[i >> 2][i & 3] + red[0][i >> 2][i & 3][lane] + red[1][i >> 2][i & 3][lane] + red[2][i >> 2][i & 3][lane] + corr; }, out);
+    }
+
+    // The same idea for up to 256 rows: the weight fragments of a 256-byte piece of K stay in
+    // registers while the row tiles stream past them (activations come from L2, where all
+    // workgroups share them); the activation fragments run four row tiles ahead of the MFMAs.
+    template <int MT>
+    __global__ __launch_bounds__(256) void dot_skinny_wide_kernel(const uint8_t* __restrict__ a,
+                                                                  const int8_t* __restrict__ w,
+                                                                  const int32_t* __restrict__ wsum,
+                                                                  int32_t M,
+                                                                  int32_t N,
+                                                                  int32_t K,
+                                                                  int32_t x_unsigned,
+                                                                  ZeroPoints zp,
+                                                                  Epilogue epi,
+                                                                  void* __restrict__ out)
+    {
+        constexpr int D = 4;     // row tiles in flight
+        constexpr int STEPS = 4; // 64-byte steps per piece of K
+        __shared__ int32_t red[3][MT][4][64];
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = tid >> 6;
+        const int r16 = lane & 15;
+        const int kc = lane >> 4;
+        const int n0 = blockIdx.x * 16;
+        const int32_t xzp = load_zp(zp.data_zp, zp.data_t);
+        const int32_t wzp = load_zp(zp.filter_zp, zp.filter_t);
+        const EpiRegs er = epi_load(epi);
+        if (wzp != 0) // uniform; exact, slow
+        {
+            for (int i = tid; i < 16 * M; i += 256)
             {
-                // lane: column lane % 16; accumulator register r is row 4 * (lane / 16) + r of the tile
-                const int m = mt * 16 + 4 * kc + r;
-                if (m < M)
+                const int m = i >> 4, n = n0 + (i & 15);
+                if (n < N)
                 {
-                    const int32_t v = acc[mt][r] + red[0][mt][r][lane] + red[1][mt][r][lane] + red[2][mt][r][lane] + corr;
+                    int32_t acc = 0;
+                    for (int k = 0; k < K; ++k)
+                    {
+                        const int32_t xv = x_unsigned ? static_cast<int32_t>(a[static_cast<int64_t>(m) * K + k])
+                                                      : static_cast<int32_t>(static_cast<int8_t>(a[static_cast<int64_t>(m) * K + k]));
+                        acc += (xv - xzp) * (static_cast<int32_t>(w[static_cast<int64_t>(n) * K + k]) - wzp);
+                    }
                     const int64_t o = static_cast<int64_t>(m) * N + n;
-                    store_out(out, epi.out_t, o, epi_apply(epi, er, v, n, o));
+                    store_out(out, epi.out_t, o, epi_apply(epi, er, acc, n, o));
                 }
             }
+            return;
+        }
+        const int xor_mask = x_unsigned ? static_cast<int>(0x80808080u) : 0;
+        const __amdgpu_buffer_rsrc_t ars = make_rsrc(a, static_cast<uint32_t>(M) * static_cast<uint32_t>(K));
+        const __amdgpu_buffer_rsrc_t wrs = make_rsrc(w, static_cast<uint32_t>(N) * static_cast<uint32_t>(K));
+        // All workgroups read the same activations: in lockstep they would queue on the same L2
+        // lines.  Each workgroup therefore gives its wavefronts another quarter of K and walks the
+        // quarter's pieces from another starting piece.
+        const int kq = ((K / 64 + 3) / 4) * 64;
+        const int k_begin = ((wave + static_cast<int>(blockIdx.x)) & 3) * kq;
+        const int k_end = min(K, k_begin + kq);
+        const int pieces = (max(k_end - k_begin, 0) + 64 * STEPS - 1) / (64 * STEPS);
+        const int rot = pieces > 0 ? (static_cast<int>(blockIdx.x) >> 2) % pieces : 0;
+        auto piece_k = [&](int c) { // byte offset of the c-th piece in this workgroup's order
+            int q = c + rot;
+            q = q >= pieces ? q - pieces : q;
+            return c < pieces ? k_begin + q * 64 * STEPS : k_end; // past the end: everything out of range
+        };
+        const int32_t wrow = n0 + r16 < N ? (n0 + r16) * K + kc * 16 : kOob;
+        const int32_t arow0 = r16 * K + kc * 16; // row r16 of row tile 0
+
+        auto load_b = [&](int kb, v4i(&bf)[STEPS]) {
+#pragma unroll
+            for (int st = 0; st < STEPS; ++st)
+            {
+                const int k = kb + st * 64;
+                bf[st] = buffer_load16(wrs, (wrow != kOob && k < k_end) ? wrow + k : kOob);
+            }
+        };
+        auto load_a = [&](int kb, int mt, v4i(&af)[STEPS]) {
+#pragma unroll
+            for (int st = 0; st < STEPS; ++st)
+            {
+                const int k = kb + st * 64;
+                af[st] = buffer_load16(ars, (mt * 16 + r16 < M && k < k_end) ? arow0 + mt * 16 * K + k : kOob);
+            }
+        };
+
+        v4acc acc[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            acc[mt] = v4acc{0, 0, 0, 0};
+        v4i bf[STEPS], bfn[STEPS], af[D][STEPS];
+        load_b(piece_k(0), bf);
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+            load_a(piece_k(0), d, af[d]);
+        for (int c = 0; c < pieces; ++c)
+        {
+            const int kb = piece_k(c), kb_next = piece_k(c + 1);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+            {
+                v4i x[STEPS];
+#pragma unroll
+                for (int st = 0; st < STEPS; ++st)
+                    x[st] = v4i{af[mt % D][st][0] ^ xor_mask, af[mt % D][st][1] ^ xor_mask, af[mt % D][st][2] ^ xor_mask, af[mt % D][st][3] ^ xor_mask};
+                // refill the slot with the row tile D ahead (of the next piece of K past the last tile)
+                if (mt + D < MT)
+                    load_a(kb, mt + D, af[mt % D]);
+                else
+                    load_a(kb_next, mt + D - MT, af[mt % D]);
+                if (mt == MT - D)
+                    load_b(kb_next, bfn);
+#pragma unroll
+                for (int st = 0; st < STEPS; ++st)
+                    acc[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(x[st], bf[st], acc[mt], 0, 0, 0);
+            }
+#pragma unroll
+            for (int st = 0; st < STEPS; ++st)
+                bf[st] = bfn[st];
+        }
+        if (wave > 0)
+        {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    red[wave - 1][mt][r][lane] = acc[mt][r];
+        }
+        __syncthreads();
+        if (wave > 0)
+            return;
+        const int n = n0 + r16;
+        if (n >= N)
+            return;
+        const int32_t corr = ((x_unsigned ? 128 : 0) - xzp) * wsum[n];
+        // lane: column lane % 16; accumulator register r is row 4 * (lane / 16) + r of the tile
+        skinny_finish<MT * 4>(
+            epi, M, N, n, [&](int i) { return (i >> 2) * 16 + 4 * kc + (i & 3); },
+            [&](int i) { return acc[i >> 2][i & 3] + red[0][i >> 2][i & 3][lane] + red[1][i >> 2][i & 3][lane] + red[2][i >> 2][i & 3][lane] + corr; }, out);
     }
 
     static bool dot_skinny_eligible(const hipq_dot_desc_t& d)
     {
-        return d.M <= 64 && d.K % 64 == 0 && d.K >= 256;
+        return d.M <= 256 && d.K % 64 == 0 && d.K >= 256 && d.M * d.K < (1ll << 31);
     }
 
     template <int MT, int STEPS>
@@ -139,6 +314,15 @@ namespace hipq
         dot_skinny_kernel<MT, STEPS><<<grid, 256, 0, s>>>(static_cast<const uint8_t*>(a), static_cast<const int8_t*>(w_nk), wsum, static_cast<int32_t>(d.M),
                                                       static_cast<int32_t>(d.N), static_cast<int32_t>(d.K), d.a_t == HIPQ_U8 ? 1 : 0, zp, epi, out);
         return check_launch("dot_skinny_i8_16x16x64");
+    }
+
+    template <int MT>
+    static int launch_skinny_wide(const hipq_dot_desc_t& d, const void* a, const void* w_nk, const int32_t* wsum, const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s)
+    {
+        const unsigned grid = static_cast<unsigned>((d.N + 15) / 16);
+        dot_skinny_wide_kernel<MT><<<grid, 256, 0, s>>>(static_cast<const uint8_t*>(a), static_cast<const int8_t*>(w_nk), wsum, static_cast<int32_t>(d.M),
+                                                   static_cast<int32_t>(d.N), static_cast<int32_t>(d.K), d.a_t == HIPQ_U8 ? 1 : 0, zp, epi, out);
+        return check_launch("dot_skinny_wide_i8_16x16x64");
     }
 
     bool dot_mfma_eligible(const hipq_dot_desc_t& d)
@@ -171,7 +355,11 @@ namespace hipq
                 return launch_skinny<1, 16>(d, a, w_nk, wsum, zp, epi, out, s);
             if (d.M <= 32)
                 return launch_skinny<2, 16>(d, a, w_nk, wsum, zp, epi, out, s);
-            return launch_skinny<4, 8>(d, a, w_nk, wsum, zp, epi, out, s);
+            if (d.M <= 64)
+                return launch_skinny<4, 8>(d, a, w_nk, wsum, zp, epi, out, s);
+            if (d.M <= 128)
+                return launch_skinny_wide<8>(d, a, w_nk, wsum, zp, epi, out, s);
+            return launch_skinny_wide<16>(d, a, w_nk, wsum, zp, epi, out, s);
         }
         GemmX xl;
         xl.x = static_cast<const uint8_t*>(a);

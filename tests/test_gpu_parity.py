@@ -540,7 +540,7 @@ def test_dot_config2_full_size_properties(gpu_lib):
         assert np.array_equal(gm, got[:M])
 
 
-@pytest.mark.parametrize("M", [1, 7, 16, 17, 33, 64])
+@pytest.mark.parametrize("M", [1, 7, 16, 17, 33, 64, 100, 129, 256])
 def test_dot_skinny(gpu_lib, M):
     """the weight-streaming kernel for a handful of rows: ragged row and column tiles, a reduction
     that does not split evenly over the four wavefronts, signed and unsigned data, zero points,

@@ -28,6 +28,9 @@ from ngraph_amd import synth  # noqa: E402
 
 PEAK_I8_TOPS = 5000.0  # MI355X dense int8 MFMA, published
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published
+# HBM bytes per launch of the headline kernel at batch 128, from the FETCH_SIZE / WRITE_SIZE
+# counter runs summarised in profiles/conv_band_config1_hbm_traffic.md (scaled by a 64 MiB copy)
+MEASURED_TRAFFIC_BYTES = {("conv_band_i8_32x32x32", 128): 57.6e6}
 
 
 class Timer:
@@ -256,7 +259,8 @@ def main():
             "peak": PEAK_I8_TOPS,
             "unit": "TOP/s",
             "frac": kern["tops_event"] / PEAK_I8_TOPS,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((kern["kernel"], args.batch)),
+            "algorithmic_bytes": 2 * args.batch * 64 * 56 * 56 + 64 * 64 * 9,
             "kernel_ms": kern["ms_event"],
         },
         "cpu_baseline": cpu,

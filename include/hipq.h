@@ -371,6 +371,52 @@ HIPQ_API int hipq_permute(int32_t elem_bytes,
                           const int32_t* order,    /* host */
                           void* stream);
 
+/* ---- pooling and concatenation: the integer glue between the quantized convolutions of a network ----
+ * MaxPool / AvgPool replace runtime::reference::max_pool<T> (src/ngraph/runtime/reference/
+ * max_pool.hpp:127-222) and avg_pool<T> (src/ngraph/runtime/reference/avg_pool.hpp:128-250):
+ * padding never wins a maximum (a window wholly in the padding gives the type's lowest value); the
+ * average sums in the element type -- an 8-bit sum wraps -- and for 8-bit types is
+ * nearbyint(float(sum) / count), ties to even; padding enters sum and count only when
+ * include_padding is set.  Types: u8, i8, f32, and i32 for MaxPool. */
+typedef enum
+{
+    HIPQ_POOL_MAX = 0,
+    HIPQ_POOL_AVG = 1
+} hipq_pool_op_t;
+
+typedef struct
+{
+    int32_t op;              /* hipq_pool_op_t */
+    int32_t dtype;           /* hipq_dtype_t */
+    int32_t layout;          /* hipq_layout_t of input and output */
+    int32_t n_spatial;       /* 1..HIPQ_MAX_SPATIAL */
+    int32_t include_padding; /* AvgPool's include_padding_in_avg_computation */
+    int64_t N, C;
+    int64_t in_sp[HIPQ_MAX_SPATIAL];
+    int64_t window[HIPQ_MAX_SPATIAL];
+    int64_t stride[HIPQ_MAX_SPATIAL];
+    int64_t pad_below[HIPQ_MAX_SPATIAL];
+    int64_t pad_above[HIPQ_MAX_SPATIAL];
+    int64_t out_sp[HIPQ_MAX_SPATIAL]; /* filled by hipq_pool_infer_output */
+} hipq_pool_desc_t;
+
+/* out_sp[i] = (in + pad_below + pad_above - window) / stride + 1, the rule of
+ * infer_batched_pooling_forward (src/ngraph/validation_util.cpp) */
+HIPQ_API int hipq_pool_infer_output(hipq_pool_desc_t* desc);
+HIPQ_API int hipq_pool(const hipq_pool_desc_t* desc, const void* in, void* out, void* stream);
+
+/* op::v0::Concat (src/ngraph/runtime/reference/concat.hpp): piece i is [outer][extent[i]][inner]
+ * elements, the result [outer][sum extent][inner]; `inputs` and `extents` are host arrays of
+ * device pointers / axis extents. */
+HIPQ_API int hipq_concat(int32_t elem_bytes,
+                         int32_t n_inputs,
+                         const void* const* inputs,
+                         const int64_t* extents,
+                         int64_t outer,
+                         int64_t inner,
+                         void* out,
+                         void* stream);
+
 /* Which kernel the last hipq_quantized_* call on this thread used: "mfma", "direct", ... (host
  * string, never NULL).  For tests and profiles. */
 HIPQ_API const char* hipq_last_kernel(void);

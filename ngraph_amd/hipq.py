@@ -122,6 +122,35 @@ class DotDesc(C.Structure):
     ]
 
 
+class PoolDesc(C.Structure):
+    _fields_ = [
+        ("op", C.c_int32),
+        ("dtype", C.c_int32),
+        ("layout", C.c_int32),
+        ("n_spatial", C.c_int32),
+        ("include_padding", C.c_int32),
+        ("N", C.c_int64),
+        ("C", C.c_int64),
+        ("in_sp", C.c_int64 * 3),
+        ("window", C.c_int64 * 3),
+        ("stride", C.c_int64 * 3),
+        ("pad_below", C.c_int64 * 3),
+        ("pad_above", C.c_int64 * 3),
+        ("out_sp", C.c_int64 * 3),
+    ]
+
+    def in_shape(self):
+        sp = list(self.in_sp)[: self.n_spatial]
+        return (self.N, self.C, *sp) if self.layout == NCX else (self.N, *sp, self.C)
+
+    def out_shape(self):
+        sp = list(self.out_sp)[: self.n_spatial]
+        return (self.N, self.C, *sp) if self.layout == NCX else (self.N, *sp, self.C)
+
+
+POOL_MAX, POOL_AVG = 0, 1
+
+
 class DeviceInfo(C.Structure):
     _fields_ = [
         ("name", C.c_char * 64),
@@ -196,6 +225,22 @@ def make_fused_desc(has_bias=True, has_sum=False, sum_t=U8, with_relu=False, sca
     return f
 
 
+def make_pool_desc(op, dtype, N, Cc, in_sp, window, stride=None, pad_below=None, pad_above=None, include_padding=False, layout=NCX) -> PoolDesc:
+    """out_sp follows the reference's rule (src/ngraph/validation_util.cpp, infer_batched_pooling_forward)"""
+    ns = len(in_sp)
+    d = PoolDesc()
+    d.op = POOL_AVG if op in (POOL_AVG, "avg") else POOL_MAX
+    d.dtype, d.layout, d.n_spatial, d.include_padding = dtype_code(dtype), layout, ns, int(include_padding)
+    d.N, d.C = N, Cc
+    stride = stride or [1] * ns
+    pad_below = pad_below or [0] * ns
+    pad_above = pad_above or [0] * ns
+    for i in range(ns):
+        d.in_sp[i], d.window[i], d.stride[i], d.pad_below[i], d.pad_above[i] = in_sp[i], window[i], stride[i], pad_below[i], pad_above[i]
+        d.out_sp[i] = (in_sp[i] + pad_below[i] + pad_above[i] - window[i]) // stride[i] + 1
+    return d
+
+
 def make_dot_desc(M, K, N, a_t=U8, b_t=I8, out_t=I8, b_layout=B_KN) -> DotDesc:
     d = DotDesc()
     d.a_t, d.b_t, d.out_t, d.b_layout = dtype_code(a_t), dtype_code(b_t), dtype_code(out_t), b_layout
@@ -241,6 +286,9 @@ EXPORTS = [
     "hipq_convert",
     "hipq_broadcast",
     "hipq_permute",
+    "hipq_pool_infer_output",
+    "hipq_pool",
+    "hipq_concat",
     "hipq_last_kernel",
 ]
 
@@ -302,6 +350,9 @@ def load():
     lib.hipq_convert.argtypes = [i32, i32, vp, vp, i64, vp]
     lib.hipq_broadcast.argtypes = [i32, vp, vp, i32, C.POINTER(C.c_int64), C.c_uint32, vp]
     lib.hipq_permute.argtypes = [i32, vp, vp, i32, C.POINTER(C.c_int64), C.POINTER(C.c_int32), vp]
+    lib.hipq_pool_infer_output.argtypes = [C.POINTER(PoolDesc)]
+    lib.hipq_pool.argtypes = [C.POINTER(PoolDesc), vp, vp, vp]
+    lib.hipq_concat.argtypes = [i32, i32, C.POINTER(vp), C.POINTER(C.c_int64), i64, i64, vp, vp]
     _lib = lib
     return lib
 
@@ -446,6 +497,33 @@ def quantized_convolution_fused(desc, fused, data, filt, bias, sum_in, scale, su
     )
     check(lib.hipq_stream_sync(None))
     return out.to_numpy(NP_OF[desc.out_t], oshape)
+
+
+def pool(desc, x):
+    lib = load()
+    bx = _dev(np.ascontiguousarray(x))
+    oshape = desc.out_shape()
+    out = DeviceBuffer(int(np.prod(oshape)) * x.dtype.itemsize)
+    check(lib.hipq_pool(C.byref(desc), bx.ptr, out.ptr, None))
+    check(lib.hipq_stream_sync(None))
+    return out.to_numpy(x.dtype, oshape)
+
+
+def concat(arrays, axis):
+    lib = load()
+    arrays = [np.ascontiguousarray(a) for a in arrays]
+    bufs = [_dev(a) for a in arrays]
+    shape = list(arrays[0].shape)
+    outer = int(np.prod(shape[:axis]))
+    inner = int(np.prod(shape[axis + 1 :]))
+    extents = [a.shape[axis] for a in arrays]
+    shape[axis] = sum(extents)
+    out = DeviceBuffer(int(np.prod(shape)) * arrays[0].dtype.itemsize)
+    ptrs = (C.c_void_p * len(bufs))(*[b.ptr for b in bufs])
+    ext = (C.c_int64 * len(bufs))(*extents)
+    check(lib.hipq_concat(arrays[0].dtype.itemsize, len(bufs), ptrs, ext, outer, inner, out.ptr, None))
+    check(lib.hipq_stream_sync(None))
+    return out.to_numpy(arrays[0].dtype, shape)
 
 
 def quantized_dot(desc, a, b, a_scale, a_zp, b_scale, b_zp, out_scale, out_zp, prepare=True):

@@ -33,6 +33,7 @@
  */
 #include "../include/hipq.h"
 
+#include <float.h>
 #include <math.h>
 #include <stdint.h>
 #include <stdlib.h>
@@ -740,6 +741,90 @@ ORC_API float orc_get_conv_requant_scale(
     float fs = orc_get_scale(min_f, max_f, filter_t, 0);
     float os = orc_get_scale(min_out, max_out, out_t, 0);
     return is * fs / os;
+}
+
+/* ---- MaxPool / AvgPool (src/ngraph/runtime/reference/max_pool.hpp:127-222, avg_pool.hpp:128-250) ----
+ * NCX or NXC tensors; padding never wins a maximum; the average sums in the element type (8-bit
+ * sums wrap), divides by the count of in-bounds (or, with include_padding, all) window positions,
+ * and for 8-bit types rounds the float quotient with nearbyint (ties to even). */
+#define ORC_POOL_BODY(T, LOWEST, IS8)                                                              \
+    for (int64_t n = 0; n < d->N; ++n)                                                             \
+        for (int64_t c = 0; c < d->C; ++c)                                                         \
+            for (int64_t o0 = 0; o0 < out[0]; ++o0)                                                \
+                for (int64_t o1 = 0; o1 < out[1]; ++o1)                                            \
+                    for (int64_t o2 = 0; o2 < out[2]; ++o2)                                        \
+                    {                                                                              \
+                        T best = LOWEST, sum = 0;                                                  \
+                        uint64_t cnt = 0;                                                          \
+                        for (int64_t w0 = 0; w0 < win[0]; ++w0)                                    \
+                            for (int64_t w1 = 0; w1 < win[1]; ++w1)                                \
+                                for (int64_t w2 = 0; w2 < win[2]; ++w2)                            \
+                                {                                                                  \
+                                    int64_t y0 = o0 * st[0] + w0 - pb[0], y1 = o1 * st[1] + w1 - pb[1], y2 = o2 * st[2] + w2 - pb[2]; \
+                                    int inb = y0 >= 0 && y0 < in[0] && y1 >= 0 && y1 < in[1] && y2 >= 0 && y2 < in[2]; \
+                                    if (inb)                                                       \
+                                    {                                                              \
+                                        int64_t sp = (y0 * in[1] + y1) * in[2] + y2;               \
+                                        T v = nxc ? ((const T*)src)[(n * in_sp + sp) * d->C + c] : ((const T*)src)[(n * d->C + c) * in_sp + sp]; \
+                                        sum = (T)(sum + v);                                        \
+                                        ++cnt;                                                     \
+                                        best = v > best ? v : best;                                \
+                                    }                                                              \
+                                    else if (d->include_padding)                                   \
+                                        ++cnt;                                                     \
+                                }                                                                  \
+                        int64_t osp = (o0 * out[1] + o1) * out[2] + o2;                            \
+                        int64_t oi = nxc ? (n * out_sp + osp) * d->C + c : (n * d->C + c) * out_sp + osp; \
+                        if (d->op == HIPQ_POOL_MAX)                                                \
+                            ((T*)dst)[oi] = best;                                                  \
+                        else if (cnt == 0)                                                         \
+                            return -2;                                                             \
+                        else if (IS8)                                                              \
+                            ((T*)dst)[oi] = (T)nearbyintf((float)sum / (float)cnt);                \
+                        else                                                                       \
+                            ((T*)dst)[oi] = (T)(sum / (T)cnt);                                     \
+                    }
+
+ORC_API int orc_pool(const hipq_pool_desc_t* d, const void* src, void* dst)
+{
+    int64_t in[3], win[3], st[3], pb[3], out[3];
+    const int lead = 3 - d->n_spatial;
+    for (int i = 0; i < 3; ++i)
+    {
+        const int real = i >= lead;
+        in[i] = real ? d->in_sp[i - lead] : 1;
+        win[i] = real ? d->window[i - lead] : 1;
+        st[i] = real ? d->stride[i - lead] : 1;
+        pb[i] = real ? d->pad_below[i - lead] : 0;
+        out[i] = real ? (d->in_sp[i - lead] + d->pad_below[i - lead] + d->pad_above[i - lead] - d->window[i - lead]) / d->stride[i - lead] + 1 : 1;
+    }
+    const int64_t in_sp = in[0] * in[1] * in[2], out_sp = out[0] * out[1] * out[2];
+    const int nxc = d->layout == HIPQ_LAYOUT_NXC;
+    switch (d->dtype)
+    {
+    case HIPQ_U8: ORC_POOL_BODY(uint8_t, 0, 1) break;
+    case HIPQ_I8: ORC_POOL_BODY(int8_t, -128, 1) break;
+    case HIPQ_I32: ORC_POOL_BODY(int32_t, INT32_MIN, 0) break;
+    case HIPQ_F32: ORC_POOL_BODY(float, -FLT_MAX, 0) break;
+    default: return -1;
+    }
+    return 0;
+}
+
+/* op::v0::Concat along one axis: piece i is [outer][extent[i]][inner] elements */
+ORC_API int orc_concat(int elem_bytes, int n_inputs, const void* const* inputs, const int64_t* extents, int64_t outer, int64_t inner, void* out)
+{
+    int64_t total = 0, offset = 0;
+    for (int i = 0; i < n_inputs; ++i)
+        total += extents[i];
+    for (int i = 0; i < n_inputs; ++i)
+    {
+        for (int64_t o = 0; o < outer; ++o)
+            memcpy((char*)out + ((o * total + offset) * inner) * elem_bytes, (const char*)inputs[i] + (o * extents[i] * inner) * elem_bytes,
+                   (size_t)(extents[i] * inner) * elem_bytes);
+        offset += extents[i];
+    }
+    return 0;
 }
 
 ORC_API size_t orc_dtype_size(int t)

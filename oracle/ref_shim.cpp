@@ -10,9 +10,11 @@
 
 #include "ngraph/axis_set.hpp"
 #include "ngraph/coordinate_diff.hpp"
+#include "ngraph/runtime/reference/avg_pool.hpp"
 #include "ngraph/runtime/reference/convolution.hpp"
 #include "ngraph/runtime/reference/dequantize.hpp"
 #include "ngraph/runtime/reference/dot.hpp"
+#include "ngraph/runtime/reference/max_pool.hpp"
 #include "ngraph/runtime/reference/quantize.hpp"
 #include "ngraph/shape.hpp"
 #include "ngraph/strides.hpp"
@@ -290,6 +292,49 @@ __attribute__((visibility("default"))) int ref_dequantize(int rank,
     else
         return 2;
 #undef DQ
+    return 0;
+}
+
+// runtime::reference::max_pool<T> / avg_pool<T> on NCX tensors; dtype codes as in hipq.h; op 0 = max, 1 = avg
+__attribute__((visibility("default"))) int ref_pool(int op,
+                                                      int dtype,
+                                                      int n_spatial,
+                                                      const int64_t* arg_shape,
+                                                      const int64_t* out_shape,
+                                                      const int64_t* window,
+                                                      const int64_t* stride,
+                                                      const int64_t* pad_below,
+                                                      const int64_t* pad_above,
+                                                      int include_padding,
+                                                      const void* in,
+                                                      void* out)
+{
+    Shape as = make_shape(arg_shape, n_spatial + 2), os = make_shape(out_shape, n_spatial + 2);
+    Shape w = make_shape(window, n_spatial), pb = make_shape(pad_below, n_spatial), pa = make_shape(pad_above, n_spatial);
+    Strides st;
+    for (int i = 0; i < n_spatial; ++i)
+        st.push_back(static_cast<size_t>(stride[i]));
+    try
+    {
+#define P(T)                                                                                       \
+    if (op == 0)                                                                                   \
+        runtime::reference::max_pool<T>(static_cast<const T*>(in), static_cast<T*>(out), as, os, w, st, pb, pa); \
+    else                                                                                           \
+        runtime::reference::avg_pool<T>(static_cast<const T*>(in), static_cast<T*>(out), as, os, w, st, pb, pa, include_padding != 0)
+        switch (dtype)
+        {
+        case 0: P(uint8_t); break;
+        case 1: P(int8_t); break;
+        case 2: P(int32_t); break;
+        case 3: P(float); break;
+        default: return -1;
+        }
+#undef P
+    }
+    catch (const std::exception&)
+    {
+        return -2;
+    }
     return 0;
 }
 }

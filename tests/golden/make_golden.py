@@ -7,6 +7,8 @@ oracle/_ref has been built (`make -C oracle ref`).  The committed outputs are da
   quantize_dequantize_kats.json   inputs / attributes / expected outputs of the 28 tests of
                                   test/backend/quantize_dequantize.in.cpp, read from its literals
   qlinearconv{2d,3d}_{x,y}.bin    the byte fixtures of test/files/onnx/qlinearconv{2d,3d}/
+  pool_vectors.npz + .json        outputs of the compiled reference max_pool / avg_pool (oracle/_ref)
+                                  on seeded synthetic inputs (`--pool-only` writes just these)
   ref_vectors.npz + .json         outputs of the compiled reference kernels (oracle/_ref) on seeded
                                   synthetic inputs; inputs are regenerated from the seed by
                                   ngraph_amd.synth (or stored, where they are floating point)
@@ -215,7 +217,53 @@ def ref_vectors():
     print("ref_vectors:", len(manifest), "cases,", os.path.getsize(os.path.join(HERE, "ref_vectors.npz")), "bytes")
 
 
+POOL_CASES = [
+    # name, seed, op, dtype, N, C, in_sp, window, stride, pad_below, pad_above, include_padding
+    ("max_u8_resnet_stem", 4001, "max", "u8", 1, 16, (28, 28), (3, 3), (2, 2), (1, 1), (1, 1), False),
+    ("max_i8_pad", 4002, "max", "i8", 2, 5, (9, 7), (3, 2), (2, 1), (1, 0), (0, 1), False),
+    ("max_i8_window_in_padding", 4003, "max", "i8", 1, 3, (4, 4), (2, 2), (3, 3), (2, 2), (2, 2), False),
+    ("max_f32_3d", 4004, "max", "f32", 1, 2, (5, 6, 4), (2, 3, 2), (1, 2, 1), (1, 0, 1), (0, 1, 1), False),
+    ("max_i32_1d", 4005, "max", "i32", 2, 3, (17,), (4,), (3,), (2,), (1,), False),
+    ("avg_u8_global7x7_wraps", 4010, "avg", "u8", 2, 8, (7, 7), (7, 7), (1, 1), (0, 0), (0, 0), False),
+    ("avg_i8_global7x7_wraps", 4011, "avg", "i8", 2, 8, (7, 7), (7, 7), (1, 1), (0, 0), (0, 0), False),
+    ("avg_u8_pad_excluded", 4012, "avg", "u8", 1, 4, (6, 5), (3, 3), (2, 2), (1, 1), (1, 1), False),
+    ("avg_u8_pad_included", 4013, "avg", "u8", 1, 4, (6, 5), (3, 3), (2, 2), (1, 1), (1, 1), True),
+    ("avg_i8_ties", 4014, "avg", "i8", 1, 6, (8, 8), (2, 1), (2, 1), (0, 0), (0, 0), False),
+    ("avg_f32", 4015, "avg", "f32", 1, 3, (6, 6), (3, 3), (1, 1), (1, 1), (1, 1), True),
+]
+
+
+def pool_input(seed, dtype, shape):
+    from ngraph_amd import synth
+
+    if dtype == "f32":
+        return synth.normal_f32(seed, shape)
+    lo, hi = {"u8": (0, 255), "i8": (-128, 127), "i32": (-(2**20), 2**20)}[dtype]
+    return synth.uniform_int(seed, shape, lo, hi, {"u8": np.uint8, "i8": np.int8, "i32": np.int32}[dtype])
+
+
+def pool_vectors():
+    """outputs of runtime::reference::max_pool / avg_pool (oracle/_ref) on seeded inputs"""
+    import oracle_lib as O
+    from ngraph_amd import hipq as H
+
+    if not O.have_ref():
+        raise SystemExit("oracle/_ref is not built: make -C oracle ref")
+    arrays, manifest = {}, []
+    for name, seed, op, dtype, N, Cc, in_sp, win, st, pb, pa, incl in POOL_CASES:
+        d = H.make_pool_desc(op, dtype, N, Cc, list(in_sp), list(win), list(st), list(pb), list(pa), incl)
+        x = pool_input(seed, dtype, d.in_shape())
+        arrays[name] = O.ref_pool(d, x)
+        manifest.append(dict(name=name, seed=seed, op=op, dtype=dtype, N=N, C=Cc, in_sp=list(in_sp), window=list(win), stride=list(st), pad_below=list(pb), pad_above=list(pa), include_padding=incl))
+    np.savez_compressed(os.path.join(HERE, "pool_vectors.npz"), **arrays)
+    with open(os.path.join(HERE, "pool_vectors.json"), "w") as f:
+        json.dump(manifest, f, indent=1)
+    print("pool_vectors:", len(manifest), "cases")
+
+
 if __name__ == "__main__":
-    parse_quantize_dequantize()
-    copy_onnx_bins()
-    ref_vectors()
+    if "--pool-only" not in sys.argv:
+        parse_quantize_dequantize()
+        copy_onnx_bins()
+        ref_vectors()
+    pool_vectors()

@@ -36,6 +36,8 @@ def port():
         lib.orc_dot_accumulate.argtypes = [C.POINTER(H.DotDesc), vp, vp, C.c_int32, C.c_int32, vp]
         lib.orc_quantized_dot.argtypes = [C.POINTER(H.DotDesc)] + [vp] * 9
         lib.orc_quantized_dot_bias.argtypes = [C.POINTER(H.DotDesc), C.POINTER(H.FusedDesc)] + [vp] * 5
+        lib.orc_pool.argtypes = [C.POINTER(H.PoolDesc), vp, vp]
+        lib.orc_concat.argtypes = [C.c_int, C.c_int, C.POINTER(vp), C.POINTER(C.c_int64), C.c_int64, C.c_int64, vp]
         f = C.c_float
         lib.orc_get_scale.restype = f
         lib.orc_get_scale.argtypes = [f, f, C.c_int, C.c_int]
@@ -64,6 +66,7 @@ def ref():
         lib.ref_quantized_dot.argtypes = [C.c_int64] * 3 + [C.c_int] * 3 + [vp] * 9
         lib.ref_quantize.argtypes = [C.c_int, i64p, C.c_uint32, C.c_int, C.c_int, C.c_int] + [vp] * 4
         lib.ref_dequantize.argtypes = [C.c_int, i64p, C.c_uint32, C.c_int, C.c_int] + [vp] * 4
+        lib.ref_pool.argtypes = [C.c_int] * 3 + [i64p] * 6 + [C.c_int, vp, vp]
         _ref = lib
     return _ref
 
@@ -241,4 +244,44 @@ def ref_dequantize(q, scale, zp, real_t=H.F32, axes=()):
     out = np.empty(q.shape, dtype=H.NP_OF[rt])
     mask = sum(1 << int(a) for a in axes)
     _ok(ref().ref_dequantize(q.ndim, _i64(q.shape), mask, rt, H.dtype_code(q.dtype), _ptr(q), _ptr(s), _ptr(z), _ptr(out)))
+    return out
+
+
+def pool(desc, x):
+    """C restatement of MaxPool / AvgPool in either layout"""
+    x = np.ascontiguousarray(x)
+    out = np.empty(desc.out_shape(), dtype=x.dtype)
+    rc = port().orc_pool(C.byref(desc), _ptr(x), _ptr(out))
+    if rc == -2:
+        raise RuntimeError("AvgPool elements == 0, must be non-zero")
+    _ok(rc)
+    return out
+
+
+def ref_pool(desc, x):
+    """runtime::reference::max_pool / avg_pool themselves (NCX tensors only)"""
+    assert desc.layout == H.NCX
+    ns = desc.n_spatial
+    x = np.ascontiguousarray(x)
+    out = np.empty(desc.out_shape(), dtype=x.dtype)
+    rc = ref().ref_pool(
+        desc.op, desc.dtype, ns, _i64(desc.in_shape()), _i64(desc.out_shape()), _i64(list(desc.window)[:ns]), _i64(list(desc.stride)[:ns]),
+        _i64(list(desc.pad_below)[:ns]), _i64(list(desc.pad_above)[:ns]), desc.include_padding, _ptr(x), _ptr(out)
+    )
+    if rc == -2:
+        raise RuntimeError("AvgPool elements == 0, must be non-zero")
+    _ok(rc)
+    return out
+
+
+def concat(arrays, axis):
+    arrays = [np.ascontiguousarray(a) for a in arrays]
+    shape = list(arrays[0].shape)
+    outer, inner = int(np.prod(shape[:axis])), int(np.prod(shape[axis + 1 :]))
+    extents = [a.shape[axis] for a in arrays]
+    shape[axis] = sum(extents)
+    out = np.empty(shape, dtype=arrays[0].dtype)
+    ptrs = (C.c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
+    ext = (C.c_int64 * len(arrays))(*extents)
+    _ok(port().orc_concat(arrays[0].dtype.itemsize, len(arrays), ptrs, ext, outer, inner, _ptr(out)))
     return out

@@ -146,6 +146,7 @@ namespace
         void lower(const shared_ptr<Node>& n);
         void lower_conv(const shared_ptr<Node>& n, Step& st);
         void lower_dot(const shared_ptr<Node>& n, Step& st);
+        void lower_pool(const shared_ptr<Node>& n, Step& st);
         shared_ptr<DeviceBlock> alloc(size_t bytes)
         {
             auto b = make_shared<DeviceBlock>(bytes ? bytes : 1);
@@ -377,6 +378,55 @@ namespace
         return -1;
     }
 
+    // MaxPool / AvgPool over [N, C, spatial...] (src/ngraph/runtime/reference/max_pool.hpp:127-222, avg_pool.hpp:128-250)
+    void HIPExecutable::lower_pool(const shared_ptr<Node>& n, Step& st)
+    {
+        hipq_pool_desc_t d;
+        memset(&d, 0, sizeof(d));
+        const Shape& in = n->get_input_shape(0);
+        if (in.size() < 3 || in.size() > 5)
+            throw unsupported_op("HIP backend: pooling with " + to_string(in.size() < 2 ? 0 : in.size() - 2) + " spatial dimensions");
+        const Shape *window, *pb, *pa;
+        const Strides* strides;
+        if (auto mp = as_type_ptr<op::v0::MaxPool>(n))
+        {
+            d.op = HIPQ_POOL_MAX;
+            window = &mp->get_window_shape();
+            strides = &mp->get_window_movement_strides();
+            pb = &mp->get_padding_below();
+            pa = &mp->get_padding_above();
+        }
+        else
+        {
+            auto ap = as_type_ptr<op::v0::AvgPool>(n);
+            d.op = HIPQ_POOL_AVG;
+            d.include_padding = ap->get_include_padding_in_avg_computation() ? 1 : 0;
+            window = &ap->get_window_shape();
+            strides = &ap->get_window_movement_strides();
+            pb = &ap->get_padding_below();
+            pa = &ap->get_padding_above();
+        }
+        d.dtype = dtype_of(n->get_output_element_type(0));
+        d.layout = HIPQ_LAYOUT_NCX;
+        d.n_spatial = static_cast<int32_t>(in.size() - 2);
+        d.N = static_cast<int64_t>(in[0]);
+        d.C = static_cast<int64_t>(in[1]);
+        for (int i = 0; i < d.n_spatial; ++i)
+        {
+            d.in_sp[i] = static_cast<int64_t>(in[2 + i]);
+            d.window[i] = static_cast<int64_t>((*window)[i]);
+            d.stride[i] = static_cast<int64_t>((*strides)[i]);
+            d.pad_below[i] = static_cast<int64_t>((*pb)[i]);
+            d.pad_above[i] = static_cast<int64_t>((*pa)[i]);
+        }
+        check(hipq_pool_infer_output(&d), n->description().c_str());
+        const Shape& out = n->get_output_shape(0);
+        for (int i = 0; i < d.n_spatial; ++i)
+            if (d.out_sp[i] != static_cast<int64_t>(out[2 + i]))
+                throw runtime_error("HIP backend: pooling output shape disagrees with the node's");
+        st.launch = [d](const vector<void*>& in, void* out, void* stream) { check(hipq_pool(&d, in[0], out, stream), "pooling"); };
+    }
+
     bool backend_supports(const Node& n)
     {
         static const vector<NodeTypeInfo> ops = {
@@ -386,7 +436,8 @@ namespace
             op::v0::QuantizedConvolutionBiasSignedAdd::type_info, op::v0::QuantizedDot::type_info, op::v0::QuantizedDotBias::type_info,
             op::v0::Abs::type_info, op::v0::Relu::type_info, op::v0::Convert::type_info, op::v0::Broadcast::type_info,
             op::v0::Reshape::type_info, op::v1::Add::type_info, op::v1::Subtract::type_info, op::v1::Multiply::type_info,
-            op::v1::Divide::type_info, op::v1::Maximum::type_info, op::v1::Minimum::type_info};
+            op::v1::Divide::type_info, op::v1::Maximum::type_info, op::v1::Minimum::type_info, op::v0::MaxPool::type_info,
+            op::v0::AvgPool::type_info, op::v0::Concat::type_info};
         for (const auto& ti : ops)
             if (n.get_type_info() == ti)
                 return true;
@@ -524,6 +575,25 @@ namespace
             const int eb = static_cast<int>(et.size());
             st.launch = [shape, order, eb](const vector<void*>& in, void* out, void* stream) {
                 check(hipq_permute(eb, in[0], out, static_cast<int32_t>(shape.size()), shape.data(), order.data(), stream), "Reshape");
+            };
+        }
+        else if (is_type<op::v0::MaxPool>(n) || is_type<op::v0::AvgPool>(n))
+        {
+            lower_pool(n, st);
+        }
+        else if (auto cc = as_type_ptr<op::v0::Concat>(n))
+        {
+            const size_t axis = static_cast<size_t>(cc->get_concatenation_axis());
+            const Shape& os = n->get_output_shape(0);
+            int64_t outer = 1, inner = 1;
+            for (size_t a = 0; a < os.size(); ++a)
+                (a < axis ? outer : inner) *= a == axis ? 1 : static_cast<int64_t>(os[a]);
+            vector<int64_t> extents;
+            for (size_t i = 0; i < n->get_input_size(); ++i)
+                extents.push_back(static_cast<int64_t>(n->get_input_shape(i)[axis]));
+            const int eb = static_cast<int>(et.size());
+            st.launch = [extents, outer, inner, eb](const vector<void*>& in, void* out, void* stream) {
+                check(hipq_concat(eb, static_cast<int32_t>(extents.size()), const_cast<const void* const*>(in.data()), extents.data(), outer, inner, out, stream), "Concat");
             };
         }
         else

@@ -450,6 +450,23 @@ namespace ngraph
                 Shape m_padding_below, m_padding_above;
                 bool m_include_padding;
             };
+
+            // joins tensors that agree on every axis but `axis` (src/ngraph/op/concat.hpp:30-68);
+            // a negative axis counts from the back
+            class NGRAPH_API Concat : public Op
+            {
+            public:
+                NGRAPH_OP_DECL("Concat", 0)
+                Concat(const OutputVector& args, int64_t axis);
+                void validate_and_infer_types() override;
+                int64_t get_concatenation_axis() const { return m_concat_axis; }
+                int64_t get_axis() const { return m_axis; }
+                std::shared_ptr<Node> clone_with_new_inputs(const OutputVector& new_args) const override;
+
+            private:
+                int64_t m_axis;
+                int64_t m_concat_axis = -1;
+            };
         }
 
         namespace v1
@@ -493,6 +510,7 @@ namespace ngraph
         using v0::Abs;
         using v0::AvgPool;
         using v0::Broadcast;
+        using v0::Concat;
         using v0::Constant;
         using v0::Convert;
         using v0::Dequantize;

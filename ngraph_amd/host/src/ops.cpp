@@ -779,6 +779,46 @@ namespace ngraph
                 check_new_args_count(this, a);
                 return make_shared<AvgPool>(a.at(0), m_window_shape, m_strides, m_padding_below, m_padding_above, m_include_padding);
             }
+
+            constexpr NodeTypeInfo Concat::type_info;
+            Concat::Concat(const OutputVector& args, int64_t axis) : Op(args), m_axis(axis) { constructor_validate_and_infer_types(); }
+            void Concat::validate_and_infer_types()
+            {
+                // src/ngraph/op/concat.cpp:42-100, static shapes only
+                NODE_VALIDATION_CHECK(this, get_input_size() >= 1, "At least one argument required.");
+                const int64_t rank = static_cast<int64_t>(get_input_shape(0).size());
+                if (m_concat_axis < 0)
+                    m_concat_axis = m_axis < 0 ? m_axis + rank : m_axis;
+                Shape out = get_input_shape(0);
+                size_t joined = 0;
+                for (size_t i = 0; i < get_input_size(); ++i)
+                {
+                    NODE_VALIDATION_CHECK(this, get_input_element_type(i) == get_input_element_type(0), "Argument element types are inconsistent.");
+                    const Shape& s = get_input_shape(i);
+                    NODE_VALIDATION_CHECK(this,
+                                          m_concat_axis >= 0 && m_concat_axis < static_cast<int64_t>(s.size()),
+                                          "Concatenation axis (",
+                                          m_concat_axis,
+                                          ") is out of bounds for argument ",
+                                          i,
+                                          ", which has shape ",
+                                          s,
+                                          ".");
+                    bool same = s.size() == out.size();
+                    for (size_t a = 0; same && a < s.size(); ++a)
+                        same = static_cast<int64_t>(a) == m_concat_axis || s[a] == out[a];
+                    NODE_VALIDATION_CHECK(this,
+                                          same,
+                                          "Argument shapes are inconsistent; they must have the same rank, and must have equal dimension "
+                                          "everywhere except on the concatenation axis (axis ",
+                                          m_concat_axis,
+                                          ").");
+                    joined += s[m_concat_axis];
+                }
+                out[m_concat_axis] = joined;
+                set_output_type(0, get_input_element_type(0), out);
+            }
+            shared_ptr<Node> Concat::clone_with_new_inputs(const OutputVector& a) const { return make_shared<Concat>(a, m_axis); }
         }
 
         namespace v1

@@ -67,6 +67,20 @@ def _numpy_pool(d, x):
     return out
 
 
+def _known_answers():
+    with open(os.path.join(GOLDEN, "pool_known_answers.json")) as f:
+        return json.load(f)["cases"]
+
+
+def test_oracle_pool_against_reference_test_values():
+    """the values the reference's own backend tests expect (test/backend/pool.in.cpp)"""
+    for m in _known_answers():
+        d = _desc(m)
+        x = np.array(m["x"], dtype=NP[m["dtype"]]).reshape(d.in_shape())
+        y = np.array(m["y"], dtype=NP[m["dtype"]]).reshape(d.out_shape())
+        assert np.array_equal(O.pool(d, x), y), m["name"]
+
+
 def test_oracle_pool_against_reference_vectors():
     manifest, arrays = _manifest()
     assert len(manifest) >= 11
@@ -160,6 +174,16 @@ def test_gpu_pool_vectors(gpu_lib):
         assert H.last_kernel() in ("max_pool", "avg_pool")
         dl = _desc(m, H.NXC)
         assert np.array_equal(cases.to_ncx(H.pool(dl, cases.to_nxc(x))), arrays[m["name"]]), (m["name"], "nxc")
+
+
+@pytest.mark.gpu
+def test_gpu_pool_reference_test_values(gpu_lib):
+    for m in _known_answers():
+        print("[case]", m["name"], flush=True)
+        d = _desc(m)
+        x = np.array(m["x"], dtype=NP[m["dtype"]]).reshape(d.in_shape())
+        y = np.array(m["y"], dtype=NP[m["dtype"]]).reshape(d.out_shape())
+        assert np.array_equal(H.pool(d, x), y), m["name"]
 
 
 @pytest.mark.gpu

@@ -148,6 +148,28 @@ def bench_qdq(lib, stream, timer, steps, warmup):
     )
 
 
+def bench_pool(lib, stream, timer, steps, warmup, batch=128):
+    """ResNet-50's two pools on u8 activations: 3x3/2 max pool after the stem, 7x7 global average"""
+    out = []
+    for op, Cc, sp, win, st, pad in (("max", 64, 112, 3, 2, 1), ("avg", 2048, 7, 7, 1, 0)):
+        for layout, lname in ((H.NCX, "nchw"), (H.NXC, "nhwc")):
+            d = H.make_pool_desc(op, "u8", batch, Cc, [sp, sp], [win, win], [st, st], [pad, pad], [pad, pad], False, layout)
+            nin = batch * Cc * sp * sp
+            nout = int(np.prod(d.out_shape()))
+            bx, by = H.DeviceBuffer(nin), H.DeviceBuffer(nout)
+            H.check(lib.hipq_fill_bytes(bx.ptr, 7, nin, stream))
+
+            def step():
+                rc = lib.hipq_pool(C.byref(d), bx.ptr, by.ptr, stream)
+                if rc:
+                    H.check(rc)
+
+            _, ev = timer.run(step, steps, warmup)
+            gbs = (nin + nout) / (ev * 1e-3) / 1e9
+            out.append(dict(op=op + "_pool", layout=lname, shape=[batch, Cc, sp, sp], window=win, stride=st, ms_event=ev, gbs=gbs, frac_hbm=gbs / PEAK_HBM_GBS, kernel=H.last_kernel()))
+    return out
+
+
 def cpu_baseline(seconds=12.0):
     """The reference's own convolution kernel (oracle/_ref, compiled from the nGraph tree) when it
     was built, else the C restatement; BASELINE config 1 at N=1 on one host core."""
@@ -227,6 +249,7 @@ def main():
             results["conv_nhwc_kernel"].append(bench_conv(lib, stream, timer, n, args.steps, args.warmup, H.NXC))
         results["gemm_config2"] = [bench_gemm(lib, stream, timer, m, small, 5) for m in (1, 32, 256)]
         results["quantize_dequantize_config3"] = bench_qdq(lib, stream, timer, small, 5)
+        results["pool_resnet50_u8"] = bench_pool(lib, stream, timer, small, 5, args.batch)
         cpu = cpu_baseline()
 
     derived_peak = info.compute_units * info.clock_mhz * 1e6 * 8192 / 1e12

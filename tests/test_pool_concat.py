@@ -171,7 +171,7 @@ def test_gpu_pool_vectors(gpu_lib):
         d = _desc(m)
         x = _input(m["seed"], m["dtype"], d.in_shape())
         assert np.array_equal(H.pool(d, x), arrays[m["name"]]), m["name"]
-        assert H.last_kernel() in ("max_pool", "avg_pool")
+        assert H.last_kernel().startswith(("max_pool", "avg_pool"))
         dl = _desc(m, H.NXC)
         assert np.array_equal(cases.to_ncx(H.pool(dl, cases.to_nxc(x))), arrays[m["name"]]), (m["name"], "nxc")
 
@@ -201,6 +201,58 @@ def test_gpu_pool_resnet_shapes(gpu_lib):
             assert np.array_equal(cases.to_ncx(got) if layout == H.NXC else got, exp), (op, layout)
 
 
+# (N, C, in_sp, window, stride, pad_below, pad_above): chosen to reach every variant of the 8-bit
+# kernels -- widths that are / are not multiples of 4 on either side, planes small enough to share a
+# workgroup (with a ragged last group), channel counts that are multiples of 16, of 4 only, and of
+# neither, one and three spatial axes, windows that hang into the padding on every side
+POOL8_SHAPES = [
+    (2, 16, (12, 16), (3, 3), (2, 2), (1, 1), (1, 1)),
+    (3, 5, (7, 7), (7, 7), (1, 1), (0, 0), (0, 0)),
+    (1, 67, (7, 7), (7, 7), (1, 1), (0, 0), (0, 0)),
+    (2, 4, (9, 10), (2, 3), (1, 2), (0, 2), (1, 0)),
+    (1, 32, (8, 8), (2, 2), (2, 2), (0, 0), (0, 0)),
+    (2, 20, (6, 12), (3, 2), (1, 1), (2, 1), (2, 1)),
+    (1, 3, (70, 72), (3, 3), (2, 2), (1, 1), (1, 1)),
+    (1, 2, (200, 200), (3, 3), (2, 2), (1, 1), (0, 0)),
+    (2, 8, (33,), (4,), (3,), (2,), (3,)),
+    (2, 16, (4, 5, 6), (2, 3, 2), (1, 2, 2), (1, 1, 0), (0, 1, 1)),
+    (1, 48, (5, 5), (3, 3), (1, 1), (2, 2), (2, 2)),
+    (2, 6, (7, 7), (7, 7), (1, 1), (0, 0), (0, 0)),
+    (1, 100, (7, 7), (3, 3), (2, 2), (1, 1), (1, 1)),
+    (4, 25, (5, 6), (2, 2), (1, 1), (0, 0), (0, 0)),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape_id", range(len(POOL8_SHAPES)))
+def test_gpu_pool_8bit_kernels(gpu_lib, monkeypatch, shape_id):
+    N, Cc, in_sp, win, st, pb, pa = POOL8_SHAPES[shape_id]
+    seen = set()
+    for dtype in ("u8", "i8"):
+        for op, incl in (("max", False), ("avg", False), ("avg", True)):
+            if op == "avg" and not incl and any(b >= w for b, w in zip(pb, win)):
+                continue
+            print("[case] pool8", shape_id, dtype, op, incl, flush=True)
+            dn = H.make_pool_desc(op, dtype, N, Cc, list(in_sp), list(win), list(st), list(pb), list(pa), incl)
+            x = _input(500 + shape_id, dtype, dn.in_shape())
+            try:
+                exp = O.pool(dn, x)
+            except RuntimeError:
+                continue
+            for layout in (H.NCX, H.NXC):
+                d = H.make_pool_desc(op, dtype, N, Cc, list(in_sp), list(win), list(st), list(pb), list(pa), incl, layout)
+                xin = cases.to_nxc(x) if layout == H.NXC else x
+                got = H.pool(d, xin)
+                seen.add(H.last_kernel())
+                assert np.array_equal(cases.to_ncx(got) if layout == H.NXC else got, exp), (dtype, op, incl, layout, H.last_kernel())
+                monkeypatch.setenv("HIPQ_NO_FAST_POOL", "1")
+                slow = H.pool(d, xin)
+                assert H.last_kernel() in ("max_pool", "avg_pool")
+                monkeypatch.delenv("HIPQ_NO_FAST_POOL")
+                assert np.array_equal(slow, got)
+    print("kernels", sorted(seen), flush=True)
+
+
 @pytest.mark.gpu
 def test_gpu_pool_errors_and_empty(gpu_lib):
     lib = gpu_lib
@@ -220,6 +272,10 @@ def test_gpu_concat(gpu_lib):
     parts = [synth.uniform_int(10 + i, (3, c, 6, 5), 0, 255, np.uint8) for i, c in enumerate((64, 32, 1, 96))]
     assert np.array_equal(H.concat(parts, 1), np.concatenate(parts, axis=1))
     assert H.last_kernel() == "concat"
+    wide = [parts[0], parts[1], parts[3]]  # every piece a multiple of 16 bytes: the 16-byte copy
+    assert np.array_equal(H.concat(wide, 1), np.concatenate(wide, axis=1))
+    odd = [synth.uniform_int(30 + i, (5, c, 3), -128, 127, np.int8) for i, c in enumerate((3, 1, 7))]
+    assert np.array_equal(H.concat(odd, 1), np.concatenate(odd, axis=1))
     nh = [cases.to_nxc(p) for p in parts]
     assert np.array_equal(H.concat(nh, 3), np.concatenate(nh, axis=3))
     f = [synth.normal_f32(20 + i, (4, 2 + i, 3)) for i in range(3)]

@@ -170,6 +170,33 @@ def bench_pool(lib, stream, timer, steps, warmup, batch=128):
     return out
 
 
+def bench_glue(lib, stream, timer, steps, warmup, batch=128):
+    """the elementwise / layout glue of an int8 ResNet-50 stage on u8[batch,256,56,56]"""
+    n = batch * 256 * 56 * 56
+    ba, bb, bo = H.DeviceBuffer(n), H.DeviceBuffer(n), H.DeviceBuffer(n)
+    H.check(lib.hipq_fill_bytes(ba.ptr, 3, n, stream))
+    H.check(lib.hipq_fill_bytes(bb.ptr, 5, n, stream))
+    shape = (C.c_int64 * 4)(batch, 256, 56, 56)
+    order = (C.c_int32 * 4)(0, 2, 3, 1)
+    ops = {
+        "add_u8": (lambda: lib.hipq_binary(0, H.U8, ba.ptr, n, bb.ptr, n, bo.ptr, n, stream), 3 * n),
+        "relu_i8": (lambda: lib.hipq_unary(1, H.I8, ba.ptr, bo.ptr, n, stream), 2 * n),
+        "convert_i8_u8": (lambda: lib.hipq_convert(H.I8, H.U8, ba.ptr, bo.ptr, n, stream), 2 * n),
+        "reshape_nchw_to_nhwc_u8": (lambda: lib.hipq_permute(1, ba.ptr, bo.ptr, 4, shape, order, stream), 2 * n),
+    }
+    out = []
+    for name, (fn, nbytes) in ops.items():
+        def step():
+            rc = fn()
+            if rc:
+                H.check(rc)
+
+        _, ev = timer.run(step, steps, warmup)
+        gbs = nbytes / (ev * 1e-3) / 1e9
+        out.append(dict(op=name, elements=n, ms_event=ev, gbs=gbs, frac_hbm=gbs / PEAK_HBM_GBS, kernel=H.last_kernel()))
+    return out
+
+
 def cpu_baseline(seconds=12.0):
     """The reference's own convolution kernel (oracle/_ref, compiled from the nGraph tree) when it
     was built, else the C restatement; BASELINE config 1 at N=1 on one host core."""
@@ -250,6 +277,7 @@ def main():
         results["gemm_config2"] = [bench_gemm(lib, stream, timer, m, small, 5) for m in (1, 32, 256)]
         results["quantize_dequantize_config3"] = bench_qdq(lib, stream, timer, small, 5)
         results["pool_resnet50_u8"] = bench_pool(lib, stream, timer, small, 5, args.batch)
+        results["glue_resnet50_u8"] = bench_glue(lib, stream, timer, small, 5, args.batch)
         cpu = cpu_baseline()
 
     derived_peak = info.compute_units * info.clock_mhz * 1e6 * 8192 / 1e12

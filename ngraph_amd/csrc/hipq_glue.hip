@@ -154,6 +154,64 @@ namespace hipq
         }
     }
 
+    // 16 bytes per lane for the element types networks move in bulk: the same scalar expression per
+    // element, on registers
+    template <typename T, int OP>
+    __global__ __launch_bounds__(256) void binary_vec_kernel(const uint4* __restrict__ a, const uint4* __restrict__ b, uint4* __restrict__ out, int64_t vecs)
+    {
+        constexpr int V = 16 / sizeof(T);
+        union Pack
+        {
+            uint4 q;
+            T e[V];
+        };
+        int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+        const int64_t step = static_cast<int64_t>(gridDim.x) * 256;
+        for (; i < vecs; i += step)
+        {
+            Pack x, y, r;
+            x.q = a[i];
+            y.q = b[i];
+#pragma unroll
+            for (int j = 0; j < V; ++j)
+            {
+                if (sizeof(T) == 1 && OP == HIPQ_OP_DIVIDE && y.e[j] == 0)
+                    r.e[j] = 0;
+                else
+                    r.e[j] = binary_apply<T>(OP, x.e[j], y.e[j]);
+            }
+            out[i] = r.q;
+        }
+    }
+
+    template <typename T, int OP>
+    __global__ __launch_bounds__(256) void unary_vec_kernel(const uint4* __restrict__ in, uint4* __restrict__ out, int64_t vecs)
+    {
+        constexpr int V = 16 / sizeof(T);
+        union Pack
+        {
+            uint4 q;
+            T e[V];
+        };
+        int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+        const int64_t step = static_cast<int64_t>(gridDim.x) * 256;
+        for (; i < vecs; i += step)
+        {
+            Pack x;
+            x.q = in[i];
+            if (OP != HIPQ_OP_COPY)
+            {
+#pragma unroll
+                for (int j = 0; j < V; ++j)
+                {
+                    const T v = x.e[j];
+                    x.e[j] = OP == HIPQ_OP_ABS ? (v < T(0) ? static_cast<T>(-v) : v) : (v > T(0) ? v : T(0));
+                }
+            }
+            out[i] = x.q;
+        }
+    }
+
     static unsigned blocks_for(int64_t n)
     {
         int64_t b = (n + 255) / 256;
@@ -173,6 +231,40 @@ int hipq_binary(int32_t op, int32_t dtype, const void* a, int64_t an, const void
         return HIPQ_OK;
     HIPQ_REQUIRE(a && b && out, "null tensor pointer");
     hipStream_t s = as_stream(stream);
+    // bulk tensors: whole 16-byte groups through the vector kernel, the remainder through the scalar one
+    const size_t esz = dtype_size(dtype);
+    if (an == n && bn == n && dtype != HIPQ_F64 && n * static_cast<int64_t>(esz) >= 4096 &&
+        (reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(out)) % 16 == 0)
+    {
+        const int64_t per = 16 / static_cast<int64_t>(esz), vecs = n / per;
+        const unsigned grid = blocks_for(vecs);
+#define VEC_B(T, OP)                                                                               \
+    case OP:                                                                                       \
+        binary_vec_kernel<T, OP><<<grid, 256, 0, s>>>(static_cast<const uint4*>(a), static_cast<const uint4*>(b), static_cast<uint4*>(out), vecs); \
+        break;
+#define VEC_B_ALL(T)                                                                               \
+    switch (op)                                                                                    \
+    {                                                                                              \
+        VEC_B(T, HIPQ_OP_ADD) VEC_B(T, HIPQ_OP_SUBTRACT) VEC_B(T, HIPQ_OP_MULTIPLY) VEC_B(T, HIPQ_OP_DIVIDE) VEC_B(T, HIPQ_OP_MAXIMUM)          \
+            VEC_B(T, HIPQ_OP_MINIMUM)                                                              \
+    }
+        switch (dtype)
+        {
+        case HIPQ_U8: VEC_B_ALL(uint8_t) break;
+        case HIPQ_I8: VEC_B_ALL(int8_t) break;
+        case HIPQ_I32: VEC_B_ALL(int32_t) break;
+        case HIPQ_F32: VEC_B_ALL(float) break;
+        default: return fail(HIPQ_ERR_UNSUPPORTED, "element type %d", dtype);
+        }
+#undef VEC_B_ALL
+#undef VEC_B
+        int rc = check_launch("binary_vec");
+        const int64_t done = vecs * per;
+        if (rc || done == n)
+            return rc;
+        return hipq_binary(op, dtype, static_cast<const char*>(a) + done * esz, n - done, static_cast<const char*>(b) + done * esz, n - done,
+                           static_cast<char*>(out) + done * esz, n - done, stream);
+    }
 #define LAUNCH_B(T) binary_kernel<T><<<blocks_for(n), 256, 0, s>>>(op, static_cast<const T*>(a), an, static_cast<const T*>(b), bn, static_cast<T*>(out), n)
     switch (dtype)
     {
@@ -195,6 +287,34 @@ int hipq_unary(int32_t op, int32_t dtype, const void* in, void* out, int64_t n, 
         return HIPQ_OK;
     HIPQ_REQUIRE(in && out, "null tensor pointer");
     hipStream_t s = as_stream(stream);
+    const size_t esz = dtype_size(dtype);
+    if (dtype != HIPQ_F64 && n * static_cast<int64_t>(esz) >= 4096 && (reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) % 16 == 0)
+    {
+        const int64_t per = 16 / static_cast<int64_t>(esz), vecs = n / per;
+        const unsigned grid = blocks_for(vecs);
+#define VEC_U(T, OP)                                                                               \
+    case OP: unary_vec_kernel<T, OP><<<grid, 256, 0, s>>>(static_cast<const uint4*>(in), static_cast<uint4*>(out), vecs); break;
+#define VEC_U_ALL(T)                                                                               \
+    switch (op)                                                                                    \
+    {                                                                                              \
+        VEC_U(T, HIPQ_OP_ABS) VEC_U(T, HIPQ_OP_RELU) VEC_U(T, HIPQ_OP_COPY)                        \
+    }
+        switch (dtype)
+        {
+        case HIPQ_U8: VEC_U_ALL(uint8_t) break;
+        case HIPQ_I8: VEC_U_ALL(int8_t) break;
+        case HIPQ_I32: VEC_U_ALL(int32_t) break;
+        case HIPQ_F32: VEC_U_ALL(float) break;
+        default: return fail(HIPQ_ERR_UNSUPPORTED, "element type %d", dtype);
+        }
+#undef VEC_U_ALL
+#undef VEC_U
+        int rc = check_launch("unary_vec");
+        const int64_t done = vecs * per;
+        if (rc || done == n)
+            return rc;
+        return hipq_unary(op, dtype, static_cast<const char*>(in) + done * esz, static_cast<char*>(out) + done * esz, n - done, stream);
+    }
 #define LAUNCH_U(T) unary_kernel<T><<<blocks_for(n), 256, 0, s>>>(op, static_cast<const T*>(in), static_cast<T*>(out), n)
     switch (dtype)
     {
@@ -215,6 +335,10 @@ int hipq_convert(int32_t in_t, int32_t out_t, const void* in, void* out, int64_t
     if (n == 0)
         return HIPQ_OK;
     HIPQ_REQUIRE(in && out, "null tensor pointer");
+    // between the two 8-bit types, and within one type, static_cast keeps the bits (the reference's CPU
+    // backend aliases the buffers for it, src/ngraph/runtime/cpu/pass/cpu_assignment.cpp:983-997)
+    if (in_t == out_t || ((in_t == HIPQ_U8 || in_t == HIPQ_I8) && (out_t == HIPQ_U8 || out_t == HIPQ_I8)))
+        return hipq_unary(HIPQ_OP_COPY, out_t, in, out, n, stream);
     hipStream_t s = as_stream(stream);
 #define LAUNCH_C(TI, TO) convert_kernel<TI, TO><<<blocks_for(n), 256, 0, s>>>(static_cast<const TI*>(in), static_cast<TO*>(out), n)
 #define CONVERT_TO(TI)                                                                             \
@@ -300,6 +424,32 @@ int hipq_permute(int32_t elem_bytes, const void* in, void* out, int32_t rank, co
         return HIPQ_OK;
     HIPQ_REQUIRE(in && out, "null tensor pointer");
     hipStream_t s = as_stream(stream);
+    if (elem_bytes == 1 || elem_bytes == 4)
+    {
+        // order = (0..b-1 | m..rank-1 | b..m-1) is a batched 2-D transpose [B][R][C] -> [B][C][R]: the
+        // NCHW <-> NHWC changes are of this kind
+        int lead = 0;
+        while (lead < rank && order[lead] == lead)
+            ++lead;
+        if (lead == rank)
+            return hipq_memcpy_d2d(out, in, static_cast<size_t>(n) * elem_bytes, stream);
+        const int m = order[lead];
+        bool two_blocks = m > lead;
+        for (int i = lead; two_blocks && i < rank; ++i)
+            two_blocks = order[i] == (i - lead < rank - m ? m + (i - lead) : lead + (i - lead - (rank - m)));
+        if (two_blocks)
+        {
+            int64_t B = 1, R = 1, Cc = 1;
+            for (int i = 0; i < lead; ++i)
+                B *= in_shape[i];
+            for (int i = lead; i < m; ++i)
+                R *= in_shape[i];
+            for (int i = m; i < rank; ++i)
+                Cc *= in_shape[i];
+            if (R < 65535 * 64 && Cc < (1ll << 31) && B < 65536)
+                return launch_transpose(in, out, B, R, Cc, elem_bytes, s);
+        }
+    }
     switch (elem_bytes)
     {
     case 1: permute_kernel<uint8_t><<<blocks_for(n), 256, 0, s>>>(static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), n, pi); break;

@@ -526,6 +526,56 @@ def concat(arrays, axis):
     return out.to_numpy(arrays[0].dtype, shape)
 
 
+BINARY_OPS = {"add": 0, "subtract": 1, "multiply": 2, "divide": 3, "maximum": 4, "minimum": 5}
+UNARY_OPS = {"abs": 0, "relu": 1, "copy": 2}
+
+
+def binary(op, a, b):
+    """elementwise a (op) b; either side may be a single element"""
+    lib = load()
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    big = a if a.size >= b.size else b
+    ba, bb = _dev(a), _dev(b)
+    out = DeviceBuffer(big.nbytes)
+    check(lib.hipq_binary(BINARY_OPS[op], dtype_code(a.dtype), ba.ptr, a.size, bb.ptr, b.size, out.ptr, big.size, None))
+    check(lib.hipq_stream_sync(None))
+    return out.to_numpy(a.dtype, big.shape)
+
+
+def unary(op, x):
+    lib = load()
+    x = np.ascontiguousarray(x)
+    bx = _dev(x)
+    out = DeviceBuffer(x.nbytes)
+    check(lib.hipq_unary(UNARY_OPS[op], dtype_code(x.dtype), bx.ptr, out.ptr, x.size, None))
+    check(lib.hipq_stream_sync(None))
+    return out.to_numpy(x.dtype, x.shape)
+
+
+def convert(x, out_dtype):
+    lib = load()
+    x = np.ascontiguousarray(x)
+    out_dtype = np.dtype(out_dtype)
+    bx = _dev(x)
+    out = DeviceBuffer(x.size * out_dtype.itemsize)
+    check(lib.hipq_convert(dtype_code(x.dtype), dtype_code(out_dtype), bx.ptr, out.ptr, x.size, None))
+    check(lib.hipq_stream_sync(None))
+    return out.to_numpy(out_dtype, x.shape)
+
+
+def permute(x, order):
+    """out = x with axes read in `order` (numpy's transpose(order), made contiguous)"""
+    lib = load()
+    x = np.ascontiguousarray(x)
+    bx = _dev(x)
+    out = DeviceBuffer(x.nbytes)
+    shape = (C.c_int64 * x.ndim)(*x.shape)
+    ordr = (C.c_int32 * x.ndim)(*order)
+    check(lib.hipq_permute(x.dtype.itemsize, bx.ptr, out.ptr, x.ndim, shape, ordr, None))
+    check(lib.hipq_stream_sync(None))
+    return out.to_numpy(x.dtype, [x.shape[i] for i in order])
+
+
 def quantized_dot(desc, a, b, a_scale, a_zp, b_scale, b_zp, out_scale, out_zp, prepare=True):
     lib = load()
     ba, bb = _dev(a), _dev(b)

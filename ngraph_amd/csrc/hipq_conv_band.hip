@@ -96,6 +96,7 @@ namespace hipq
                             // the chunk rotation of a slot does not depend on its row
         int32_t BWr;        // slots per band row that hold data: Q + S - 1
         int32_t q_magic;    // ceil(2^20 / Q): pix / Q = (pix * q_magic) >> 20 for pix < 2048
+        uint32_t bands_magic; // 2^32 / bands + 1: item / bands = hi32(item * bands_magic), exact while items * bands < 2^32 (0: one band)
         int32_t x_lds;      // LDS byte offset of band buffer 0 (the filter sits in front of it)
         int32_t band_bytes; // bytes of one band buffer
         int32_t stage_lds;  // LDS byte offset of the output staging area (4 x kBandStageWave)
@@ -144,9 +145,18 @@ namespace hipq
     }
 
     // Band (the 256 lanes of a group): lane takes chunk cx = cx0 + gtid of a row of BW pixel slots
-    // (4 chunks a slot); batch element u is band row sy0 + u.  xs_off: LDS offset of the group's buffer.
+    // (4 chunks a slot); batch element u < NB is band row sy0 + u.  xs_off: LDS offset of the group's
+    // buffer.  A lane's column and a batch element's row are each valid or not on their own (the row
+    // uniformly), so an address is the sum of a per-lane and a per-row part, and either part being
+    // half of the out-of-range offset puts the sum out of range: one scalar select and one add per
+    // load.  (The tensor is at most 2^30 bytes, checked by the launcher.)
     // FILL: padding is a non-zero byte (out-of-range loads give zeros, which is the padding otherwise)
-    template <bool STORE, bool FILL = false>
+    // PLAIN: the batch is the whole band and every row of it lies inside the image (all bands but an
+    // image's first and last): row offsets ride in the scalar offset of the load (which the range
+    // check ignores -- the rows are known to be valid), no per-row tests.  PITCH: bytes per band row
+    // in LDS when known at compile time (row offsets become immediates), else 0.
+    constexpr int kHalfOob = 0x40000000;
+    template <bool STORE, bool FILL, int NB, bool PLAIN, int PITCH>
     __device__ __forceinline__ void band_x_copy(BandBatch& b, __amdgpu_buffer_rsrc_t xrs, uint8_t* lds, const BandParams& p, int xs_off, int cx0, int sy0, int band_rows, int img_base, int p0, int fill, int xor_mask)
     {
         const int cx = cx0 + (static_cast<int>(threadIdx.x) & 255);
@@ -155,23 +165,44 @@ namespace hipq
         const int ix = sx - p.pbw;
         const bool col_in = sx < p.BWr;
         const bool col_ok = col_in & (static_cast<uint32_t>(ix) < static_cast<uint32_t>(p.W));
-#pragma unroll
-        for (int u = 0; u < kBandBatch; ++u)
+        const int pitch = PITCH ? PITCH : p.BW * kBandC;
+        if (!STORE)
         {
-            const int sy = sy0 + u;
-            const int iy = p0 + sy - p.pbh;
-            const bool in = col_in & (sy < band_rows);
-            const bool ok = col_ok & (sy < band_rows) & (static_cast<uint32_t>(iy) < static_cast<uint32_t>(p.H));
-            if (STORE)
+            const int v_col = col_ok ? img_base + ix * kBandC + c4 * 16 : kHalfOob;
+#pragma unroll
+            for (int u = 0; u < NB; ++u)
             {
-                v4i t = b.v[u];
-                if (FILL)
-                    t = v4i{ok ? t[0] : fill, ok ? t[1] : fill, ok ? t[2] : fill, ok ? t[3] : fill};
-                *reinterpret_cast<v4i*>(lds + (in ? xs_off + sy * (p.BW * kBandC) + band_cell(sx, c4, p.BW * 32) : p.sink)) =
-                    v4i{t[0] ^ xor_mask, t[1] ^ xor_mask, t[2] ^ xor_mask, t[3] ^ xor_mask};
+                const int sy = sy0 + u;
+                const int iy = p0 + sy - p.pbh;
+                if (PLAIN)
+                    b.v[u] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(xrs, v_col, iy * p.W * kBandC, 0));
+                else
+                {
+                    const bool row_ok = (sy < band_rows) & (static_cast<uint32_t>(iy) < static_cast<uint32_t>(p.H));
+                    const int s_row = row_ok ? iy * p.W * kBandC : kHalfOob;
+                    b.v[u] = buffer_load16(xrs, v_col + s_row);
+                }
             }
-            else
-                b.v[u] = buffer_load16(xrs, ok ? img_base + (iy * p.W + ix) * kBandC + c4 * 16 : kOob);
+        }
+        else if (col_in)
+        {
+            const int v_cell = xs_off + band_cell(sx, c4, pitch / 2);
+#pragma unroll
+            for (int u = 0; u < NB; ++u)
+            {
+                const int sy = sy0 + u;
+                if (PLAIN || sy < band_rows) // uniform
+                {
+                    v4i t = b.v[u];
+                    if (FILL)
+                    {
+                        const int iy = p0 + sy - p.pbh;
+                        const bool ok = col_ok & (static_cast<uint32_t>(iy) < static_cast<uint32_t>(p.H));
+                        t = v4i{ok ? t[0] : fill, ok ? t[1] : fill, ok ? t[2] : fill, ok ? t[3] : fill};
+                    }
+                    *reinterpret_cast<v4i*>(lds + v_cell + sy * pitch) = v4i{t[0] ^ xor_mask, t[1] ^ xor_mask, t[2] ^ xor_mask, t[3] ^ xor_mask};
+                }
+            }
         }
     }
 
@@ -182,7 +213,7 @@ namespace hipq
     // LDS offset of the band row and the slot in it of each tile's pixel (tap 0,0).
     // U taps per loop trip; the tap count must be a multiple of U.
     template <int T, int U>
-    __device__ __forceinline__ void band_reduce(v16i (&acc)[4][2], const uint8_t* lds, int woff, const int (&xrow0)[4], const int (&xcol0)[4], int half, int R, int S, int BW)
+    __device__ __forceinline__ void band_reduce(v16i (&acc)[T][2], const uint8_t* lds, int woff, const int (&xrow0)[T], const int (&xcol0)[T], int half, int R, int S, int BW)
     {
         const int plane = BW * 32, rowp = BW * kBandC;
         v4i xa[T], xb[T], wa[2], wb[2];
@@ -267,7 +298,7 @@ namespace hipq
     // compile-time offset (filter row, half, tap, channel tile), so the 144 MFMAs and 108 reads run
     // as straight-line code without address arithmetic, loop branches or register shuffles.
     template <int T>
-    __device__ __forceinline__ void band_reduce_33(v16i (&acc)[4][2], const uint8_t* lds, int woff, const int (&xrow0)[4], const int (&xcol0)[4], int half, const int32_t (&corr)[2])
+    __device__ __forceinline__ void band_reduce_33(v16i (&acc)[T][2], const uint8_t* lds, int woff, const int (&xrow0)[T], const int (&xcol0)[T], int half, const int32_t (&corr)[2])
     {
         constexpr int kRow = 64 * kBandC; // bytes of a band row of 64 slots (two planes of 2048)
         int xbase[T][3];
@@ -330,7 +361,9 @@ namespace hipq
 
     // U: filter taps per trip of the reduction loop (the tap count is a multiple of it); 0: the
     // straight-line 3x3 reduction over 64-slot band rows
-    template <int MODE, int KIND, bool OUT_NCX, int U>
+    // T: 32-pixel tiles per wavefront (4: items of up to 512 pixels; 2: items of up to 256 pixels,
+    // which fill and drain the two-group pipeline in half the time and split a layer more evenly)
+    template <int MODE, int KIND, bool OUT_NCX, int U, int T>
     __global__ __launch_bounds__(kBandThreads) void conv_band_kernel(BandParams p,
                                                                     const int8_t* __restrict__ w,
                                                                     const int32_t* __restrict__ wsum,
@@ -381,21 +414,21 @@ namespace hipq
 
         auto item_geom = [&](int j, int& img, int& p0, int& rows) {
             const int item = static_cast<int>(blockIdx.x) + j * grid;
-            img = item / p.bands;
+            img = p.bands_magic ? static_cast<int>(__umulhi(static_cast<uint32_t>(item), p.bands_magic)) : item;
             p0 = (item - img * p.bands) * p.TP;
             rows = min(p.TP, p.P - p0);
         };
 
         // ---- the filter and each group's first band ---------------------------------------------
-        // Group 0's first band is needed first: it goes out together with the filter.  Group 1
-        // multiplies one phase later and fetches its first band while group 0 multiplies.
+        // Both groups fetch their first band together with the filter: group 1 multiplies one phase
+        // later, but a fetch started then would not be back before group 0 is done.
         BandBatch wb0, xb0;
         int img, p0, rows;
         band_w_copy<false>(wb0, wrs, lds, 0, taps, kred, p.K, p.sink);
-        if (grp == 0)
+        if (grp < my_items)
         {
-            item_geom(0, img, p0, rows);
-            band_x_copy<false>(xb0, xrs, lds, p, xs_off, 0, 0, rows + p.R - 1, img * p.H * p.W * kBandC, p0, 0, 0);
+            item_geom(grp, img, p0, rows);
+            band_x_copy<false, false, (T == 2 ? 6 : kBandBatch), false, 0>(xb0, xrs, lds, p, xs_off, 0, 0, rows + p.R - 1, img * p.H * p.W * kBandC, p0, 0, 0);
         }
 
         if (wzp != 0) // uniform; w - wzp does not fit a signed byte: exact, slow, one output a lane
@@ -439,21 +472,38 @@ namespace hipq
         const bool fast_interp = fabsf(ec.scale) * acc_max < 4194304.0f;
 
         // moves a band into the group's buffer; the first batch is already in xb0
+        // rows of a band a lane fetches in one go: the bands of two-tile items are short
+        constexpr int NB = T == 2 ? 6 : kBandBatch;
+        constexpr int PITCH = U == 0 ? 64 * kBandC : 0; // the straight-line kernel runs on 64-slot band rows
+        // every row of item j's band inside the image, and the band exactly one batch: no per-row tests
+        auto band_plain = [&]() { return p.BWr * 4 <= 256 && rows + p.R - 1 == NB && p0 >= p.pbh && p0 - p.pbh + NB <= p.H; };
+        auto band_fetch = [&](BandBatch& xb, int j) {
+            item_geom(j, img, p0, rows);
+            if (band_plain())
+                band_x_copy<false, false, NB, true, PITCH>(xb, xrs, lds, p, xs_off, 0, 0, NB, img * p.H * p.W * kBandC, p0, 0, 0);
+            else
+                band_x_copy<false, false, NB, false, PITCH>(xb, xrs, lds, p, xs_off, 0, 0, rows + p.R - 1, img * p.H * p.W * kBandC, p0, 0, 0);
+        };
         auto band_store = [&](BandBatch& xb0, int j) {
             item_geom(j, img, p0, rows);
             const int band_rows = rows + p.R - 1;
             const int img_base = img * p.H * p.W * kBandC;
+            if (fill == 0 && band_plain())
+            {
+                band_x_copy<true, false, NB, true, PITCH>(xb0, xrs, lds, p, xs_off, 0, 0, NB, img_base, p0, fill, xor_mask);
+                return;
+            }
             if (fill == 0)
-                band_x_copy<true, false>(xb0, xrs, lds, p, xs_off, 0, 0, band_rows, img_base, p0, fill, xor_mask);
+                band_x_copy<true, false, NB, false, PITCH>(xb0, xrs, lds, p, xs_off, 0, 0, band_rows, img_base, p0, fill, xor_mask);
             else
-                band_x_copy<true, true>(xb0, xrs, lds, p, xs_off, 0, 0, band_rows, img_base, p0, fill, xor_mask);
-            if (p.BWr * 4 > 256 || band_rows > kBandBatch) // wide or tall bands: the rest, batch by batch
+                band_x_copy<true, true, NB, false, PITCH>(xb0, xrs, lds, p, xs_off, 0, 0, band_rows, img_base, p0, fill, xor_mask);
+            if (p.BWr * 4 > 256 || band_rows > NB) // wide or tall bands: the rest, batch by batch
                 for (int cx0 = 0; cx0 < p.BWr * 4; cx0 += 256)
-                    for (int sy0 = 0; sy0 < band_rows; sy0 += kBandBatch)
+                    for (int sy0 = 0; sy0 < band_rows; sy0 += NB)
                         if (cx0 | sy0)
                         {
-                            band_x_copy<false>(xb0, xrs, lds, p, xs_off, cx0, sy0, band_rows, img_base, p0, fill, xor_mask);
-                            band_x_copy<true, true>(xb0, xrs, lds, p, xs_off, cx0, sy0, band_rows, img_base, p0, fill, xor_mask);
+                            band_x_copy<false, false, NB, false, PITCH>(xb0, xrs, lds, p, xs_off, cx0, sy0, band_rows, img_base, p0, fill, xor_mask);
+                            band_x_copy<true, true, NB, false, PITCH>(xb0, xrs, lds, p, xs_off, cx0, sy0, band_rows, img_base, p0, fill, xor_mask);
                         }
         };
 
@@ -464,8 +514,8 @@ namespace hipq
                 band_w_copy<false>(wb0, wrs, lds, u0, taps, kred, p.K, p.sink);
             band_w_copy<true>(wb0, wrs, lds, u0, taps, kred, p.K, p.sink);
         }
-        if (grp == 0)
-            band_store(xb0, 0);
+        if (grp < my_items)
+            band_store(xb0, grp);
         __syncthreads();
         HIPQ_PHASE(2);
 
@@ -476,19 +526,22 @@ namespace hipq
         int phases_done = 0;
         if (grp == 1)
         {
-            if (1 < my_items)
-            {
-                item_geom(1, img, p0, rows);
-                band_x_copy<false>(xb0, xrs, lds, p, xs_off, 0, 0, rows + p.R - 1, img * p.H * p.W * kBandC, p0, 0, 0);
-                band_store(xb0, 1);
-            }
             __syncthreads();
             HIPQ_PHASE(3);
             phases_done = 1;
         }
         for (int sp = grp; sp < my_items; sp += 2)
         {
-            v16i acc[4][2];
+            v16i acc[T][2];
+            // The group's next band travels through registers: fetched during this multiply phase,
+            // moved into the band buffer in the requantize phase that follows (when nobody reads the
+            // buffer).  With two tiles a wavefront the registers are free from the start of the
+            // phase and the data is back before the barrier; with four the fetch starts once the
+            // fragment registers are free and is awaited at the end of the requantize phase.
+            constexpr bool kEarlyFetch = T == 2;
+            BandBatch nb;
+            if (kEarlyFetch && sp + 2 < my_items)
+                band_fetch(nb, sp + 2);
             {
                 // ================= multiply: item sp =================
                 // The SIMD's arbiter favours its older wavefront; without a hint group 1 starves in
@@ -500,25 +553,25 @@ namespace hipq
                     item_geom(sp, img, p0, rows);
                     const int npix = rows * p.Q;
                     const int ntiles = (npix + 31) >> 5;
-                    // wavefront gw owns tiles 4*gw .. 4*gw+3
+                    // wavefront gw owns tiles T*gw .. T*gw+T-1
                     if (U != 0) // the straight-line reduction brings the correction in with its first MFMAs
                     {
 #pragma unroll
-                        for (int ti = 0; ti < 4; ++ti)
+                        for (int ti = 0; ti < T; ++ti)
 #pragma unroll
                             for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
                                 for (int r = 0; r < 16; ++r)
                                     acc[ti][ni][r] = corr[ni];
                     }
-                    if (4 * gw < ntiles)
+                    if (T * gw < ntiles)
                     {
-                        int xrow0[4], xcol0[4];
+                        int xrow0[T], xcol0[T];
 #pragma unroll
-                        for (int ti = 0; ti < 4; ++ti)
+                        for (int ti = 0; ti < T; ++ti)
                         {
                             // tiles past the end re-read the last pixel; their results are never stored
-                            const int pix = min((4 * gw + ti) * 32 + l32, npix - 1);
+                            const int pix = min((T * gw + ti) * 32 + l32, npix - 1);
                             const int py = (pix * p.q_magic) >> 20;
                             xrow0[ti] = xs_off + py * (p.BW * kBandC);
                             xcol0[ti] = pix - py * p.Q;
@@ -526,28 +579,21 @@ namespace hipq
                         const int woff = band_cell(l32, half, 0);
                         if (sp <= 1) HIPQ_PHASE(11);
                         if (U == 0)
-                            band_reduce_33<4>(acc, lds, woff, xrow0, xcol0, half, corr);
+                            band_reduce_33<T>(acc, lds, woff, xrow0, xcol0, half, corr);
                         else
-                            band_reduce<4, U == 0 ? 1 : U>(acc, lds, woff, xrow0, xcol0, half, p.R, p.S, p.BW);
+                            band_reduce<T, U == 0 ? 1 : U>(acc, lds, woff, xrow0, xcol0, half, p.R, p.S, p.BW);
                         if (sp <= 1) HIPQ_PHASE(12);
                     }
                 }
             }
             __builtin_amdgcn_s_setprio(0);
-            // the group's next band starts its way into registers now (the fragment registers are
-            // free), flies through the barrier and the requantization, and moves into the band buffer
-            // at the end of the next phase
-            BandBatch nb;
-            if (sp + 2 < my_items)
-            {
-                item_geom(sp + 2, img, p0, rows);
-                band_x_copy<false>(nb, xrs, lds, p, xs_off, 0, 0, rows + p.R - 1, img * p.H * p.W * kBandC, p0, 0, 0);
-            }
+            if (!kEarlyFetch && sp + 2 < my_items)
+                band_fetch(nb, sp + 2);
             HIPQ_WAVE_MARK(phases_done, 0);
             __syncthreads();
             HIPQ_WAVE_MARK(phases_done, 1);
             ++phases_done;
-            HIPQ_PHASE(2 + phases_done);
+            if (phases_done < 6) HIPQ_PHASE(2 + phases_done);
             {
                 // ================= requantize and write out: item sp =================
                 if (sp <= 1) HIPQ_PHASE(13);
@@ -563,8 +609,14 @@ namespace hipq
                 // lane: channel ni*32 + lane%32; accumulator register 4g+e of tile ti is pixel
                 // (4*gw + ti)*32 + 8g + 4*(lane/32) + e of the band
                 const int64_t img_pix0 = static_cast<int64_t>(img) * p.PQ + static_cast<int64_t>(p0) * p.Q; // first pixel of the band, image-major
+                if (kEarlyFetch && sp + 2 < my_items)
+                {
+                    band_store(nb, sp + 2);
+                    item_geom(sp, img, p0, rows);
+                }
 
-                auto epilogue = [&](auto fast_c, auto sum_c) {
+                auto epilogue = [&](auto fast_c, auto sum_c, auto ti0_c, auto ti1_c) {
+                    constexpr int ti0 = decltype(ti0_c)::value, ti1 = decltype(ti1_c)::value;
                     constexpr bool FAST = decltype(fast_c)::value;
                     constexpr bool SUM = decltype(sum_c)::value;
                     const float s256 = __fmul_rn(ec.scale, 256.0f);
@@ -575,13 +627,13 @@ namespace hipq
                     {
                         const int n = ni * 32 + l32;
 #pragma unroll
-                        for (int ti = 0; ti < 4; ++ti)
+                        for (int ti = ti0; ti < ti1; ++ti)
                         {
 #pragma unroll
                             for (int g = 0; g < 4; ++g)
                             {
-                                const int lpix = ti * 32 + 8 * g + 4 * half; // pixel within the wavefront's 128
-                                const int bpix = gw * 128 + lpix;           // pixel within the band
+                                const int lpix = ti * 32 + 8 * g + 4 * half; // pixel within the wavefront's 32 * T
+                                const int bpix = gw * (32 * T) + lpix;      // pixel within the band
                                 float s4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
                                 if (SUM && n < p.K && bpix < npix)
                                 {
@@ -660,59 +712,81 @@ namespace hipq
                 if (sp <= 1) HIPQ_PHASE(14);
                 using std::false_type;
                 using std::true_type;
-                if (MODE == EPI_FUSED)
-                {
-                    if (has_sum)
-                        epilogue(true_type{}, true_type{});
+                auto requantize = [&](auto ti0, auto ti1) {
+                    if (MODE == EPI_FUSED)
+                    {
+                        if (has_sum)
+                            epilogue(true_type{}, true_type{}, ti0, ti1);
+                        else
+                            epilogue(true_type{}, false_type{}, ti0, ti1);
+                    }
+                    else if (KIND == OUT_Q8 && fast_interp)
+                        epilogue(true_type{}, false_type{}, ti0, ti1);
                     else
-                        epilogue(true_type{}, false_type{});
-                }
-                else if (KIND == OUT_Q8 && fast_interp)
-                    epilogue(true_type{}, false_type{});
-                else
-                    epilogue(false_type{}, false_type{});
-
-                if (sp <= 1) HIPQ_PHASE(15);
+                        epilogue(false_type{}, false_type{}, ti0, ti1);
+                };
+                // Staging regions are wavefront-private and a wavefront's LDS accesses complete in order:
+                // no barrier.  Lanes with nothing to store get an out-of-range offset, which the buffer
+                // store drops: no branches.  The tile is written out in two halves of 16 * T pixels; the
+                // staging reads of the first half are in flight while the second half is requantized.
+                const __amdgpu_buffer_rsrc_t ors = make_rsrc(out, p.out_bytes);
+                v4i piece[T];
+                auto stage_read = [&](int h) {
+#pragma unroll
+                    for (int j = 0; j < T; ++j)
+                    {
+                        const int id = j * 64 + lane_v;
+                        if (OUT_NCX) // 64 channel rows: a lane moves 16 consecutive pixels of one channel
+                            piece[j] = *reinterpret_cast<const v4i*>(stage + (id / T) * kBandStagePitch + (h * T + id % T) * 16);
+                        else // 16 * T pixel rows of 64 channels: a lane moves 16 consecutive channels of one pixel
+                            piece[j] = *reinterpret_cast<const v4i*>(stage + (16 * T * h + (id >> 2)) * 64 + (id & 3) * 16);
+                    }
+                };
+                auto stage_write_out = [&](int h) {
+#pragma unroll
+                    for (int j = 0; j < T; ++j)
+                    {
+                        const int id = j * 64 + lane_v;
+                        if (OUT_NCX)
+                        {
+                            // bands and images hold multiples of 16 pixels (checked by the launcher)
+                            const int ch = id / T;
+                            const int part = h * T + id % T;
+                            const int band0 = (img * p.K) * static_cast<int>(p.PQ) + p0 * p.Q + gw * (32 * T);
+                            const bool ok = (ch < p.K) & (gw * (32 * T) + part * 16 < npix);
+                            __builtin_amdgcn_raw_buffer_store_b128(piece[j], ors, ok ? band0 + ch * static_cast<int>(p.PQ) + part * 16 : kOob, 0, 0);
+                        }
+                        else
+                        {
+                            const int px = 16 * T * h + (id >> 2);
+                            const int part = id & 3;
+                            const int band0 = (img * static_cast<int>(p.PQ) + p0 * p.Q + gw * (32 * T)) * p.K;
+                            const bool ok = (gw * (32 * T) + px < npix) & (part * 16 < p.K);
+                            __builtin_amdgcn_raw_buffer_store_b128(piece[j], ors, ok ? band0 + px * p.K + part * 16 : kOob, 0, 0);
+                        }
+                    }
+                };
                 if (KIND == OUT_Q8)
                 {
-                    // staging regions are wavefront-private and a wavefront's LDS accesses complete in
-                    // order: no barrier.  Lanes with nothing to store get an out-of-range offset, which
-                    // the buffer store drops: no branches.
-                    const __amdgpu_buffer_rsrc_t ors = make_rsrc(out, p.out_bytes);
-                    if (OUT_NCX)
-                    {
-                        // 64 channel rows of 128 pixels: a lane moves 16 consecutive pixels of one channel
-                        // (bands and images hold multiples of 16 pixels, checked by the launcher)
-                        const int band0 = (img * p.K) * static_cast<int>(p.PQ) + p0 * p.Q + gw * 128;
-#pragma unroll
-                        for (int j = 0; j < 8; ++j)
-                        {
-                            const int id = j * 64 + lane_v;
-                            const int ch = id >> 3;
-                            const int part = id & 7;
-                            const bool ok = (ch < p.K) & (gw * 128 + part * 16 < npix);
-                            const v4i val = *reinterpret_cast<const v4i*>(stage + ch * kBandStagePitch + part * 16);
-                            __builtin_amdgcn_raw_buffer_store_b128(val, ors, ok ? band0 + ch * static_cast<int>(p.PQ) + part * 16 : kOob, 0, 0);
-                        }
-                    }
-                    else
-                    {
-                        // 128 pixel rows of 64 channels: a lane moves 16 consecutive channels of one pixel
-                        const int band0 = (img * static_cast<int>(p.PQ) + p0 * p.Q + gw * 128) * p.K;
-#pragma unroll
-                        for (int j = 0; j < 8; ++j)
-                        {
-                            const int id = j * 64 + lane_v;
-                            const int px = id >> 2;
-                            const int part = id & 3;
-                            const bool ok = (gw * 128 + px < npix) & (part * 16 < p.K);
-                            const v4i val = *reinterpret_cast<const v4i*>(stage + px * 64 + part * 16);
-                            __builtin_amdgcn_raw_buffer_store_b128(val, ors, ok ? band0 + px * p.K + part * 16 : kOob, 0, 0);
-                        }
-                    }
+                    requantize(std::integral_constant<int, 0>{}, std::integral_constant<int, T / 2>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                    stage_read(0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    requantize(std::integral_constant<int, T / 2>{}, std::integral_constant<int, T>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (sp <= 1) HIPQ_PHASE(15);
+                    stage_write_out(0);
+                    stage_read(1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    stage_write_out(1);
+                }
+                else
+                {
+                    requantize(std::integral_constant<int, 0>{}, std::integral_constant<int, T>{});
+                    if (sp <= 1) HIPQ_PHASE(15);
                 }
                 if (sp <= 1) HIPQ_PHASE(9);
-                if (sp + 2 < my_items)
+                if (!kEarlyFetch && sp + 2 < my_items)
                     band_store(nb, sp + 2);
                 if (sp <= 1) HIPQ_PHASE(8);
             }
@@ -720,7 +794,7 @@ namespace hipq
             __syncthreads();
             HIPQ_WAVE_MARK(phases_done, 1);
             ++phases_done;
-            HIPQ_PHASE(2 + phases_done);
+            if (phases_done < 6) HIPQ_PHASE(2 + phases_done);
         }
         for (; phases_done < my_items + 1; ++phases_done)
             __syncthreads();
@@ -728,7 +802,7 @@ namespace hipq
     }
 
     // rows per band and LDS bytes; false when the layer does not fit this kernel
-    static bool band_plan(const ConvGeom& g, bool out_ncx, BandParams* bp, size_t* lds_bytes)
+    static bool band_plan(const ConvGeom& g, bool out_ncx, int tiles, BandParams* bp, size_t* lds_bytes)
     {
         if (g.in[0] != 1 || g.f[0] != 1 || g.out[0] != 1)
             return false;
@@ -744,14 +818,14 @@ namespace hipq
         const int64_t R = g.f[1], S = g.f[2], P = g.out[1], Q = g.out[2];
         if (R * S > 25 || Q > 512 || Q < 1)
             return false;
-        if (g.in_count() >= (1ll << 31) || g.out_count() >= (1ll << 31) || g.N * P >= (1ll << 30))
+        if (g.in_count() > (1ll << 30) || g.out_count() >= (1ll << 31) || g.N * P >= (1ll << 30))
             return false;
         const int64_t wbytes = R * S * 64 * kBandC; // [tap][64][64]
         const int64_t BWr = Q + S - 1;
         const int64_t BW = (BWr + 15) / 16 * 16;
         const int64_t budget = 160 * 1024; // one workgroup per CU: filter, two band buffers, staging
         int64_t best = 0;
-        for (int64_t tp = 1; tp <= P && tp * Q <= 512; ++tp)
+        for (int64_t tp = 1; tp <= P && tp * Q <= 4 * 32 * tiles; ++tp)
         {
             const int64_t band_bytes = (tp + R - 1) * BW * kBandC;
             const int64_t need = wbytes + 2 * band_bytes + 4 * kBandStageWave + 16;
@@ -784,6 +858,9 @@ namespace hipq
         bp->BW = static_cast<int32_t>(BW);
         bp->BWr = static_cast<int32_t>(BWr);
         bp->q_magic = static_cast<int32_t>(((1 << 20) + Q - 1) / Q);
+        bp->bands_magic = bp->bands > 1 ? static_cast<uint32_t>((1ull << 32) / static_cast<uint64_t>(bp->bands) + 1) : 0u;
+        if (static_cast<int64_t>(bp->items) * bp->bands >= (1ll << 32))
+            return false;
         bp->x_lds = static_cast<int32_t>(wbytes);
         bp->band_bytes = static_cast<int32_t>(band_bytes);
         bp->stage_lds = static_cast<int32_t>(wbytes + 2 * band_bytes);
@@ -799,13 +876,27 @@ namespace hipq
     {
         BandParams bp;
         size_t lds_bytes;
-        return band_plan(g, out_ncx, &bp, &lds_bytes);
+        return band_plan(g, out_ncx, 4, &bp, &lds_bytes);
     }
 
-    template <int MODE, int KIND, bool OUT_NCX, int U>
+    static int band_slots()
+    {
+        static int cus[16] = {};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16)
+            return 256;
+        if (cus[dev] == 0)
+        {
+            hipDeviceProp_t prop;
+            cus[dev] = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        }
+        return cus[dev]; // one persistent workgroup per CU
+    }
+
+    template <int MODE, int KIND, bool OUT_NCX, int U, int T>
     static int launch_band(const BandParams& bp, size_t lds_bytes, const int8_t* w, const int32_t* wsum, int xu, const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s)
     {
-        auto kernel = conv_band_kernel<MODE, KIND, OUT_NCX, U>;
+        auto kernel = conv_band_kernel<MODE, KIND, OUT_NCX, U, T>;
         static bool configured[16] = {};
         int dev = 0;
         HIPQ_HIP(hipGetDevice(&dev));
@@ -814,14 +905,7 @@ namespace hipq
             HIPQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
             configured[dev] = true;
         }
-        hipDeviceProp_t prop;
-        static int cus[16] = {};
-        if (dev >= 0 && dev < 16 && cus[dev] == 0)
-        {
-            HIPQ_HIP(hipGetDeviceProperties(&prop, dev));
-            cus[dev] = prop.multiProcessorCount;
-        }
-        const int slots = dev >= 0 && dev < 16 && cus[dev] > 0 ? cus[dev] : 256; // one persistent workgroup per CU
+        const int slots = band_slots();
         const unsigned grid = static_cast<unsigned>(bp.items < slots ? bp.items : slots);
         kernel<<<grid, kBandThreads, lds_bytes, s>>>(bp, w, wsum, xu, zp, epi, out);
         return check_launch("conv_band_i8_32x32x32");
@@ -838,7 +922,31 @@ namespace hipq
     {
         BandParams bp;
         size_t lds_bytes = 0;
-        HIPQ_REQUIRE(band_plan(g, out_ncx, &bp, &lds_bytes), "layer does not fit the band convolution");
+        HIPQ_REQUIRE(band_plan(g, out_ncx, 4, &bp, &lds_bytes), "layer does not fit the band convolution");
+        // Items of half the size (two tiles a wavefront) for the straight-line 3x3 kernel when that is
+        // estimated faster: time ~ (phases + fill and drain) x tiles, a phase being one item per group
+        // and the small items paying about a tenth more per pixel (filter fragments reused half as often)
+        int tiles = 4;
+        {
+            BandParams b2;
+            size_t l2 = 0;
+            const char* force = getenv("HIPQ_BAND_TILES");
+            if (bp.R == 3 && bp.S == 3 && bp.BW == 64 && getenv("HIPQ_BAND_LOOP") == nullptr && band_plan(g, out_ncx, 2, &b2, &l2))
+            {
+                const int slots = band_slots();
+                auto cost = [slots](const BandParams& b, double per_tile) {
+                    const int grid = b.items < slots ? b.items : slots;
+                    return ((b.items + grid - 1) / grid + 1.6) * per_tile;
+                };
+                const bool small = force ? atoi(force) == 2 : cost(b2, 2 * 1.1) < cost(bp, 4);
+                if (small)
+                {
+                    bp = b2;
+                    lds_bytes = l2;
+                    tiles = 2;
+                }
+            }
+        }
         HIPQ_REQUIRE((reinterpret_cast<uintptr_t>(data_nxc) & 15) == 0 && (reinterpret_cast<uintptr_t>(packed) & 15) == 0 &&
                          (reinterpret_cast<uintptr_t>(out) & 15) == 0,
                      "band convolution needs 16-byte aligned tensors");
@@ -851,9 +959,10 @@ namespace hipq
         // straight-line reduction for 3x3 filters over 64-slot band rows, else a loop of 3 or 1 taps a trip
         const int u = (bp.R == 3 && bp.S == 3 && bp.BW == 64 && getenv("HIPQ_BAND_LOOP") == nullptr) ? 0 : ((bp.R * bp.S) % 3 == 0 ? 3 : 1);
 #define BAND_U(MODE, KIND, NCX)                                                                    \
-    (u == 0 ? launch_band<MODE, KIND, NCX, 0>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)          \
-            : (u == 3 ? launch_band<MODE, KIND, NCX, 3>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s) \
-                      : launch_band<MODE, KIND, NCX, 1>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)))
+    (u == 0 ? (tiles == 2 ? launch_band<MODE, KIND, NCX, 0, 2>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)                      \
+                          : launch_band<MODE, KIND, NCX, 0, 4>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s))                     \
+            : (u == 3 ? launch_band<MODE, KIND, NCX, 3, 4>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)                          \
+                      : launch_band<MODE, KIND, NCX, 1, 4>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)))
 #define BAND(MODE, KIND) (out_ncx ? BAND_U(MODE, KIND, true) : BAND_U(MODE, KIND, false))
         if (epi.mode == EPI_INTERP)
             return q8 ? BAND(EPI_INTERP, OUT_Q8) : BAND(EPI_INTERP, OUT_I32);

@@ -32,20 +32,20 @@ static __device__ long long g_phase_clock[32];
 #define HIPQ_PHASE(i)                                                                              \
     do                                                                                             \
     {                                                                                              \
-        if (blockIdx.x == 0 && (threadIdx.x & 255) == 0 && (i) < 16)                               \
+        if (blockIdx.x == 0 && (threadIdx.x & 255) == 0 && (i) < 16 && threadIdx.x < 512)                               \
             g_phase_clock[(threadIdx.x >> 8) * 16 + (i)] = clock64();                              \
     } while (0)
 static __device__ long long g_block_times[256][4];
-static __device__ long long g_wave_clock[8][8][2]; // [phase][wave][arrive at barrier, leave barrier]
+static __device__ long long g_wave_clock[12][12][2]; // [phase][wave][arrive at barrier, leave barrier]
 #define HIPQ_WAVE_MARK(phase, which)                                                               \
     do                                                                                             \
     {                                                                                              \
-        if (blockIdx.x == 0 && (threadIdx.x & 63) == 0 && (phase) < 8)                             \
+        if (blockIdx.x == 0 && (threadIdx.x & 63) == 0 && (phase) < 12)                             \
             g_wave_clock[phase][threadIdx.x >> 6][which] = clock64();                              \
     } while (0)
-extern "C" HIPQ_API int hipq_debug_band_waves(long long* out128)
+extern "C" HIPQ_API int hipq_debug_band_waves(long long* out288)
 {
-    return hipMemcpyFromSymbol(out128, HIP_SYMBOL(g_wave_clock), sizeof(long long) * 128) == hipSuccess ? 0 : 1;
+    return hipMemcpyFromSymbol(out288, HIP_SYMBOL(g_wave_clock), sizeof(long long) * 288) == hipSuccess ? 0 : 1;
 }
 #define HIPQ_BLOCK_BEGIN()                                                                         \
     long long blk_w0 = wall_clock64(), blk_c0 = clock64()
@@ -78,7 +78,7 @@ extern "C" HIPQ_API int hipq_debug_band_phases(long long* out32)
 namespace hipq
 {
     constexpr int kBandC = 64;           // input channels (bytes per pixel slot)
-    constexpr int kBandThreads = 512;    // two groups of four wavefronts
+    constexpr int kBandGroupThreads = 256; // a group: four wavefronts, one per SIMD
     constexpr int kBandStagePitch = 144; // NCHW staging: bytes per channel row (128 pixels + pad, 16-byte multiple)
     constexpr int kBandStageWave = 64 * kBandStagePitch; // 9216 bytes per wavefront
     constexpr int kBandBatch = 10;       // 16-byte loads a lane keeps in flight while filling LDS
@@ -96,10 +96,11 @@ namespace hipq
                             // the chunk rotation of a slot does not depend on its row
         int32_t BWr;        // slots per band row that hold data: Q + S - 1
         int32_t q_magic;    // ceil(2^20 / Q): pix / Q = (pix * q_magic) >> 20 for pix < 2048
+        int32_t xcd_map;     // renumber workgroups so that each XCD gets a contiguous run of items
         uint32_t bands_magic; // 2^32 / bands + 1: item / bands = hi32(item * bands_magic), exact while items * bands < 2^32 (0: one band)
         int32_t x_lds;      // LDS byte offset of band buffer 0 (the filter sits in front of it)
         int32_t band_bytes; // bytes of one band buffer
-        int32_t stage_lds;  // LDS byte offset of the output staging area (4 x kBandStageWave)
+        int32_t stage_lds;  // LDS byte offset of the output staging area (one region per wavefront)
         int32_t sink;       // LDS byte offset of 16 spare bytes that absorb the copies' out-of-range lanes
         int64_t PQ;
     };
@@ -130,6 +131,8 @@ namespace hipq
     template <bool STORE>
     __device__ __forceinline__ void band_w_copy(BandBatch& b, __amdgpu_buffer_rsrc_t wrs, uint8_t* lds, int u0, int taps, int kred, int K, int sink)
     {
+        if (threadIdx.x >= 512) // 64 rows x 8 lanes; a third group has no part in it
+            return;
         const int n = static_cast<int>(threadIdx.x) >> 3;
         const int sub = static_cast<int>(threadIdx.x) & 7;
 #pragma unroll
@@ -297,7 +300,7 @@ namespace hipq
     // per-lane base (one per pixel tile and filter column, computed once per band) plus a
     // compile-time offset (filter row, half, tap, channel tile), so the 144 MFMAs and 108 reads run
     // as straight-line code without address arithmetic, loop branches or register shuffles.
-    template <int T>
+    template <int T, bool ADD_CORR>
     __device__ __forceinline__ void band_reduce_33(v16i (&acc)[T][2], const uint8_t* lds, int woff, const int (&xrow0)[T], const int (&xcol0)[T], int half, const int32_t (&corr)[2])
     {
         constexpr int kRow = 64 * kBandC; // bytes of a band row of 64 slots (two planes of 2048)
@@ -350,21 +353,28 @@ namespace hipq
             mac(xb, wb, false);
             interleave();
         }
+        if (ADD_CORR)
+        {
 #pragma unroll
-        for (int ti = 0; ti < T; ++ti)
+            for (int ti = 0; ti < T; ++ti)
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni)
+                for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-                for (int r = 0; r < 16; ++r)
-                    acc[ti][ni][r] += corr[ni];
+                    for (int r = 0; r < 16; ++r)
+                        acc[ti][ni][r] += corr[ni];
+        }
     }
 
     // U: filter taps per trip of the reduction loop (the tap count is a multiple of it); 0: the
     // straight-line 3x3 reduction over 64-slot band rows
     // T: 32-pixel tiles per wavefront (4: items of up to 512 pixels; 2: items of up to 256 pixels,
     // which fill and drain the two-group pipeline in half the time and split a layer more evenly)
-    template <int MODE, int KIND, bool OUT_NCX, int U, int T>
-    __global__ __launch_bounds__(kBandThreads) void conv_band_kernel(BandParams p,
+    // G: groups of four wavefronts.  Two groups alternate between multiplying and requantizing; three
+    // groups (two-tile items only: the registers allow three wavefronts a SIMD) rotate through
+    // multiply / requantize first half / requantize second half, which keeps a third wavefront on
+    // every SIMD to fill the gaps the other two leave.
+    template <int MODE, int KIND, bool OUT_NCX, int U, int T, int G>
+    __global__ __launch_bounds__(kBandGroupThreads * G) void conv_band_kernel(BandParams p,
                                                                     const int8_t* __restrict__ w,
                                                                     const int32_t* __restrict__ wsum,
                                                                     int32_t x_unsigned,
@@ -410,10 +420,15 @@ namespace hipq
         const int grid = static_cast<int>(gridDim.x);
         // this workgroup's items are blockIdx.x + j * grid, j = 0 .. my_items-1; item j belongs to
         // group j % 2, is reduced in phase j and requantized in phase j + 1
-        const int my_items = (p.items - static_cast<int>(blockIdx.x) + grid - 1) / grid;
+        // Workgroups are dealt round-robin to the 8 XCDs, each with an L2 of its own: workgroup b works as
+        // number vb, which gives every XCD a contiguous run of items in each round, so that the halo
+        // rows neighbouring bands share are fetched into one L2 (grids that are not a multiple of 8 keep
+        // the plain numbering).
+        const int vb = ((grid & 7) == 0 && p.xcd_map) ? (static_cast<int>(blockIdx.x) & 7) * (grid >> 3) + (static_cast<int>(blockIdx.x) >> 3) : static_cast<int>(blockIdx.x);
+        const int my_items = (p.items - vb + grid - 1) / grid;
 
         auto item_geom = [&](int j, int& img, int& p0, int& rows) {
-            const int item = static_cast<int>(blockIdx.x) + j * grid;
+            const int item = vb + j * grid;
             img = p.bands_magic ? static_cast<int>(__umulhi(static_cast<uint32_t>(item), p.bands_magic)) : item;
             p0 = (item - img * p.bands) * p.TP;
             rows = min(p.TP, p.P - p0);
@@ -437,7 +452,7 @@ namespace hipq
             for (int j = 0; j < my_items; ++j)
             {
                 item_geom(j, img, p0, rows);
-                for (int i = tid; i < rows * p.Q * p.K; i += kBandThreads)
+                for (int i = tid; i < rows * p.Q * p.K; i += kBandGroupThreads * G)
                 {
                     const int n = i % p.K, pix = i / p.K;
                     const int py = p0 + pix / p.Q, px = pix % p.Q;
@@ -514,8 +529,10 @@ namespace hipq
                 band_w_copy<false>(wb0, wrs, lds, u0, taps, kred, p.K, p.sink);
             band_w_copy<true>(wb0, wrs, lds, u0, taps, kred, p.K, p.sink);
         }
-        if (grp < my_items)
-            band_store(xb0, grp);
+        // group 0's first band is awaited here; the later groups move theirs into LDS just before the
+        // barrier that precedes their first multiply phase, so that the first phase does not wait for them
+        if (grp == 0 && 0 < my_items)
+            band_store(xb0, 0);
         __syncthreads();
         HIPQ_PHASE(2);
 
@@ -524,13 +541,26 @@ namespace hipq
         // group 1 one barrier behind group 0, and whichever finishes first keeps arriving at the
         // barrier until my_items + 1 phases have passed.  The accumulators never cross a loop trip.
         int phases_done = 0;
-        if (grp == 1)
+        for (; phases_done < grp; ++phases_done)
         {
+            if (phases_done == grp - 1 && grp < my_items)
+                band_store(xb0, grp);
+            HIPQ_WAVE_MARK(phases_done, 0);
             __syncthreads();
-            HIPQ_PHASE(3);
-            phases_done = 1;
+            HIPQ_WAVE_MARK(phases_done, 1);
         }
-        for (int sp = grp; sp < my_items; sp += 2)
+        // staging holds a whole wavefront tile (two groups) or half of one (three groups: LDS is short)
+        constexpr bool kStageHalf = G == 3;
+        constexpr int kStagePitch = kStageHalf ? 16 * T + 16 : kBandStagePitch;
+        constexpr int kStageWave = kStageHalf ? 64 * kStagePitch : kBandStageWave;
+        // Three groups: the group's next band is fetched at the start of its second phase and enters the
+        // band buffer at the end of its third (nobody reads the buffer in between, and two phases
+        // cover the round trip to memory); the multiply phase carries no fetch registers.
+        constexpr bool kCarryFetch = G == 3;
+        // three groups: the multiply phase is the long one, the sign-bias correction moves to the requantization
+        constexpr bool kCorrLate = G == 3 && U == 0;
+        BandBatch nb;
+        for (int sp = grp; sp < my_items; sp += G)
         {
             v16i acc[T][2];
             // The group's next band travels through registers: fetched during this multiply phase,
@@ -539,9 +569,8 @@ namespace hipq
             // phase and the data is back before the barrier; with four the fetch starts once the
             // fragment registers are free and is awaited at the end of the requantize phase.
             constexpr bool kEarlyFetch = T == 2;
-            BandBatch nb;
-            if (kEarlyFetch && sp + 2 < my_items)
-                band_fetch(nb, sp + 2);
+            if (kEarlyFetch && !kCarryFetch && sp + G < my_items)
+                band_fetch(nb, sp + G);
             {
                 // ================= multiply: item sp =================
                 // The SIMD's arbiter favours its older wavefront; without a hint group 1 starves in
@@ -579,7 +608,7 @@ namespace hipq
                         const int woff = band_cell(l32, half, 0);
                         if (sp <= 1) HIPQ_PHASE(11);
                         if (U == 0)
-                            band_reduce_33<T>(acc, lds, woff, xrow0, xcol0, half, corr);
+                            band_reduce_33<T, !kCorrLate>(acc, lds, woff, xrow0, xcol0, half, corr);
                         else
                             band_reduce<T, U == 0 ? 1 : U>(acc, lds, woff, xrow0, xcol0, half, p.R, p.S, p.BW);
                         if (sp <= 1) HIPQ_PHASE(12);
@@ -587,8 +616,8 @@ namespace hipq
                 }
             }
             __builtin_amdgcn_s_setprio(0);
-            if (!kEarlyFetch && sp + 2 < my_items)
-                band_fetch(nb, sp + 2);
+            if (!kEarlyFetch && sp + G < my_items)
+                band_fetch(nb, sp + G);
             HIPQ_WAVE_MARK(phases_done, 0);
             __syncthreads();
             HIPQ_WAVE_MARK(phases_done, 1);
@@ -603,17 +632,18 @@ namespace hipq
                 asm volatile("" : "+v"(lane_v));
                 const int half = lane_v >> 5;
                 const int l32 = lane_v & 31;
-                uint8_t* const stage = lds + p.stage_lds + gw * kBandStageWave;
+                uint8_t* const stage = lds + p.stage_lds + (G == 3 ? wave_id : gw) * kStageWave;
                 item_geom(sp, img, p0, rows);
                 const int npix = rows * p.Q;
                 // lane: channel ni*32 + lane%32; accumulator register 4g+e of tile ti is pixel
                 // (4*gw + ti)*32 + 8g + 4*(lane/32) + e of the band
                 const int64_t img_pix0 = static_cast<int64_t>(img) * p.PQ + static_cast<int64_t>(p0) * p.Q; // first pixel of the band, image-major
-                if (kEarlyFetch && sp + 2 < my_items)
-                {
-                    band_store(nb, sp + 2);
+                if (kEarlyFetch && !kCarryFetch && sp + G < my_items)
+                    band_store(nb, sp + G);
+                if (kCarryFetch && sp + G < my_items)
+                    band_fetch(nb, sp + G);
+                if (kEarlyFetch)
                     item_geom(sp, img, p0, rows);
-                }
 
                 auto epilogue = [&](auto fast_c, auto sum_c, auto ti0_c, auto ti1_c) {
                     constexpr int ti0 = decltype(ti0_c)::value, ti1 = decltype(ti1_c)::value;
@@ -653,7 +683,7 @@ namespace hipq
 #pragma unroll
                                 for (int e = 0; e < 4; ++e)
                                 {
-                                    const int32_t a = acc[ti][ni][4 * g + e];
+                                    const int32_t a = acc[ti][ni][4 * g + e] + (kCorrLate ? corr[ni] : 0);
                                     if (KIND != OUT_Q8)
                                         x[e] = epi_interp<KIND>(ec, a);
                                     else if (MODE == EPI_INTERP && FAST)
@@ -682,13 +712,13 @@ namespace hipq
                                         constexpr uint32_t sel = BYTE ? 0x0c0c0501u : 0x0c0c0400u;
                                         const uint32_t lo2 = __builtin_amdgcn_perm(x[1], x[0], sel);
                                         const uint32_t hi2 = __builtin_amdgcn_perm(x[3], x[2], sel);
-                                        *reinterpret_cast<uint32_t*>(stage + n * kBandStagePitch + lpix) = (hi2 << 16) | lo2;
+                                        *reinterpret_cast<uint32_t*>(stage + n * kStagePitch + lpix - (kStageHalf ? ti0 * 32 : 0)) = (hi2 << 16) | lo2;
                                     }
                                     else
                                     {
 #pragma unroll
                                         for (int e = 0; e < 4; ++e)
-                                            stage[(lpix + e) * 64 + n] = static_cast<uint8_t>(BYTE ? (x[e] >> 8) : x[e]);
+                                            stage[(lpix - (kStageHalf ? ti0 * 32 : 0) + e) * 64 + n] = static_cast<uint8_t>(BYTE ? (x[e] >> 8) : x[e]);
                                     }
                                 }
                                 else if (n < p.K && bpix < npix)
@@ -737,9 +767,9 @@ namespace hipq
                     {
                         const int id = j * 64 + lane_v;
                         if (OUT_NCX) // 64 channel rows: a lane moves 16 consecutive pixels of one channel
-                            piece[j] = *reinterpret_cast<const v4i*>(stage + (id / T) * kBandStagePitch + (h * T + id % T) * 16);
+                            piece[j] = *reinterpret_cast<const v4i*>(stage + (id / T) * kStagePitch + ((kStageHalf ? 0 : h * T) + id % T) * 16);
                         else // 16 * T pixel rows of 64 channels: a lane moves 16 consecutive channels of one pixel
-                            piece[j] = *reinterpret_cast<const v4i*>(stage + (16 * T * h + (id >> 2)) * 64 + (id & 3) * 16);
+                            piece[j] = *reinterpret_cast<const v4i*>(stage + ((kStageHalf ? 0 : 16 * T * h) + (id >> 2)) * 64 + (id & 3) * 16);
                     }
                 };
                 auto stage_write_out = [&](int h) {
@@ -772,22 +802,43 @@ namespace hipq
                     __builtin_amdgcn_sched_barrier(0);
                     stage_read(0);
                     __builtin_amdgcn_sched_barrier(0);
+                    if (G == 3) // the second half of the tile is the group's third phase
+                    {
+                        HIPQ_WAVE_MARK(phases_done, 0);
+                        __syncthreads();
+                        HIPQ_WAVE_MARK(phases_done, 1);
+                        ++phases_done;
+                    }
+                    if (kStageHalf) // the first half leaves the staging area before the second half enters
+                    {
+                        stage_write_out(0);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                     requantize(std::integral_constant<int, T / 2>{}, std::integral_constant<int, T>{});
                     __builtin_amdgcn_sched_barrier(0);
                     if (sp <= 1) HIPQ_PHASE(15);
-                    stage_write_out(0);
+                    if (!kStageHalf)
+                        stage_write_out(0);
                     stage_read(1);
                     __builtin_amdgcn_sched_barrier(0);
                     stage_write_out(1);
                 }
                 else
                 {
-                    requantize(std::integral_constant<int, 0>{}, std::integral_constant<int, T>{});
+                    requantize(std::integral_constant<int, 0>{}, std::integral_constant<int, T / 2>{});
+                    if (G == 3)
+                    {
+                        __syncthreads();
+                        ++phases_done;
+                    }
+                    requantize(std::integral_constant<int, T / 2>{}, std::integral_constant<int, T>{});
                     if (sp <= 1) HIPQ_PHASE(15);
                 }
                 if (sp <= 1) HIPQ_PHASE(9);
-                if (!kEarlyFetch && sp + 2 < my_items)
-                    band_store(nb, sp + 2);
+                if (!kEarlyFetch && sp + G < my_items)
+                    band_store(nb, sp + G);
+                if (kCarryFetch && sp + G < my_items)
+                    band_store(nb, sp + G);
                 if (sp <= 1) HIPQ_PHASE(8);
             }
             HIPQ_WAVE_MARK(phases_done, 0);
@@ -796,14 +847,21 @@ namespace hipq
             ++phases_done;
             if (phases_done < 6) HIPQ_PHASE(2 + phases_done);
         }
-        for (; phases_done < my_items + 1; ++phases_done)
+        for (; phases_done < my_items + G - 1; ++phases_done)
+        {
+            HIPQ_WAVE_MARK(phases_done, 0);
             __syncthreads();
+            HIPQ_WAVE_MARK(phases_done, 1);
+        }
         HIPQ_BLOCK_END();
     }
 
     // rows per band and LDS bytes; false when the layer does not fit this kernel
-    static bool band_plan(const ConvGeom& g, bool out_ncx, int tiles, BandParams* bp, size_t* lds_bytes)
+    static bool band_plan(const ConvGeom& g, bool out_ncx, int tiles, int groups, BandParams* bp, size_t* lds_bytes)
     {
+        const int64_t stage_wave = groups == 3 ? 64 * (16 * tiles + 16) : kBandStageWave;
+        // two groups: only one requantizes at a time, a region per SIMD; three: two do, a region per wavefront
+        const int64_t stage_regions = groups == 3 ? 12 : 4;
         if (g.in[0] != 1 || g.f[0] != 1 || g.out[0] != 1)
             return false;
         if (g.C != kBandC || g.K > 64 || g.K % 16 != 0)
@@ -828,7 +886,7 @@ namespace hipq
         for (int64_t tp = 1; tp <= P && tp * Q <= 4 * 32 * tiles; ++tp)
         {
             const int64_t band_bytes = (tp + R - 1) * BW * kBandC;
-            const int64_t need = wbytes + 2 * band_bytes + 4 * kBandStageWave + 16;
+            const int64_t need = wbytes + groups * band_bytes + stage_regions * stage_wave + 16;
             if (need > budget)
                 break;
             // full 32-pixel tiles and (for NCHW output) 16-byte aligned band starts
@@ -861,10 +919,11 @@ namespace hipq
         bp->bands_magic = bp->bands > 1 ? static_cast<uint32_t>((1ull << 32) / static_cast<uint64_t>(bp->bands) + 1) : 0u;
         if (static_cast<int64_t>(bp->items) * bp->bands >= (1ll << 32))
             return false;
+        bp->xcd_map = tiles == 2 ? 1 : 0; // short bands share more halo rows; measured neutral to harmful for tall ones
         bp->x_lds = static_cast<int32_t>(wbytes);
         bp->band_bytes = static_cast<int32_t>(band_bytes);
-        bp->stage_lds = static_cast<int32_t>(wbytes + 2 * band_bytes);
-        bp->sink = bp->stage_lds + 4 * kBandStageWave;
+        bp->stage_lds = static_cast<int32_t>(wbytes + groups * band_bytes);
+        bp->sink = bp->stage_lds + static_cast<int32_t>(stage_regions * stage_wave);
         bp->PQ = P * Q;
         bp->x_bytes = static_cast<uint32_t>(g.in_count());
         bp->out_bytes = static_cast<uint32_t>(g.out_count() * static_cast<int64_t>(dtype_size(g.out_t)));
@@ -876,7 +935,7 @@ namespace hipq
     {
         BandParams bp;
         size_t lds_bytes;
-        return band_plan(g, out_ncx, 4, &bp, &lds_bytes);
+        return band_plan(g, out_ncx, 4, 2, &bp, &lds_bytes);
     }
 
     static int band_slots()
@@ -893,10 +952,10 @@ namespace hipq
         return cus[dev]; // one persistent workgroup per CU
     }
 
-    template <int MODE, int KIND, bool OUT_NCX, int U, int T>
+    template <int MODE, int KIND, bool OUT_NCX, int U, int T, int G>
     static int launch_band(const BandParams& bp, size_t lds_bytes, const int8_t* w, const int32_t* wsum, int xu, const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s)
     {
-        auto kernel = conv_band_kernel<MODE, KIND, OUT_NCX, U, T>;
+        auto kernel = conv_band_kernel<MODE, KIND, OUT_NCX, U, T, G>;
         static bool configured[16] = {};
         int dev = 0;
         HIPQ_HIP(hipGetDevice(&dev));
@@ -907,7 +966,7 @@ namespace hipq
         }
         const int slots = band_slots();
         const unsigned grid = static_cast<unsigned>(bp.items < slots ? bp.items : slots);
-        kernel<<<grid, kBandThreads, lds_bytes, s>>>(bp, w, wsum, xu, zp, epi, out);
+        kernel<<<grid, kBandGroupThreads * G, lds_bytes, s>>>(bp, w, wsum, xu, zp, epi, out);
         return check_launch("conv_band_i8_32x32x32");
     }
 
@@ -922,7 +981,7 @@ namespace hipq
     {
         BandParams bp;
         size_t lds_bytes = 0;
-        HIPQ_REQUIRE(band_plan(g, out_ncx, 4, &bp, &lds_bytes), "layer does not fit the band convolution");
+        HIPQ_REQUIRE(band_plan(g, out_ncx, 4, 2, &bp, &lds_bytes), "layer does not fit the band convolution");
         // Items of half the size (two tiles a wavefront) for the straight-line 3x3 kernel when that is
         // estimated faster: time ~ (phases + fill and drain) x tiles, a phase being one item per group
         // and the small items paying about a tenth more per pixel (filter fragments reused half as often)
@@ -931,14 +990,15 @@ namespace hipq
             BandParams b2;
             size_t l2 = 0;
             const char* force = getenv("HIPQ_BAND_TILES");
-            if (bp.R == 3 && bp.S == 3 && bp.BW == 64 && getenv("HIPQ_BAND_LOOP") == nullptr && band_plan(g, out_ncx, 2, &b2, &l2))
+            if (bp.R == 3 && bp.S == 3 && bp.BW == 64 && getenv("HIPQ_BAND_LOOP") == nullptr && band_plan(g, out_ncx, 2, 3, &b2, &l2))
             {
                 const int slots = band_slots();
-                auto cost = [slots](const BandParams& b, double per_tile) {
+                auto cost = [slots](const BandParams& b, double fill, double per_phase) {
                     const int grid = b.items < slots ? b.items : slots;
-                    return ((b.items + grid - 1) / grid + 1.6) * per_tile;
+                    return ((b.items + grid - 1) / grid + fill) * per_phase;
                 };
-                const bool small = force ? atoi(force) == 2 : cost(b2, 2 * 1.1) < cost(bp, 4);
+                // measured: a phase of the three-group kernel takes about 0.4 of a four-tile phase
+                const bool small = force ? atoi(force) == 2 : cost(b2, 3.0, 0.4) < cost(bp, 1.6, 1.0);
                 if (small)
                 {
                     bp = b2;
@@ -959,10 +1019,10 @@ namespace hipq
         // straight-line reduction for 3x3 filters over 64-slot band rows, else a loop of 3 or 1 taps a trip
         const int u = (bp.R == 3 && bp.S == 3 && bp.BW == 64 && getenv("HIPQ_BAND_LOOP") == nullptr) ? 0 : ((bp.R * bp.S) % 3 == 0 ? 3 : 1);
 #define BAND_U(MODE, KIND, NCX)                                                                    \
-    (u == 0 ? (tiles == 2 ? launch_band<MODE, KIND, NCX, 0, 2>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)                      \
-                          : launch_band<MODE, KIND, NCX, 0, 4>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s))                     \
-            : (u == 3 ? launch_band<MODE, KIND, NCX, 3, 4>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)                          \
-                      : launch_band<MODE, KIND, NCX, 1, 4>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)))
+    (u == 0 ? (tiles == 2 ? launch_band<MODE, KIND, NCX, 0, 2, 3>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)                   \
+                          : launch_band<MODE, KIND, NCX, 0, 4, 2>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s))                  \
+            : (u == 3 ? launch_band<MODE, KIND, NCX, 3, 4, 2>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)                       \
+                      : launch_band<MODE, KIND, NCX, 1, 4, 2>(bp, lds_bytes, w, wsum, xu, zp, epi, out, s)))
 #define BAND(MODE, KIND) (out_ncx ? BAND_U(MODE, KIND, true) : BAND_U(MODE, KIND, false))
         if (epi.mode == EPI_INTERP)
             return q8 ? BAND(EPI_INTERP, OUT_Q8) : BAND(EPI_INTERP, OUT_I32);

@@ -366,6 +366,8 @@ BAND_SHAPES = [
     (2, 48, (14, 14), (1, 1), dict()),                                    # 1x1, K not a multiple of 32
     (1, 16, (12, 16), (3, 2), dict(pad_below=(1, 0), pad_above=(1, 1))),  # asymmetric filter and padding
     (1, 64, (9, 40), (3, 3), dict()),                                     # no padding
+    (2, 32, (5, 60), (3, 3), dict(pad_below=(1, 1), pad_above=(1, 1))),   # 64-slot rows, one-row items with ragged tiles, K < 64
+    (3, 48, (10, 48), (3, 3), dict(pad_below=(1, 1), pad_above=(1, 1))),  # 64-slot rows, short last band, idle wavefronts
 ]
 
 

@@ -30,7 +30,7 @@ PEAK_I8_TOPS = 5000.0  # MI355X dense int8 MFMA, published
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the headline kernel at batch 128, from the FETCH_SIZE / WRITE_SIZE
 # counter runs summarised in profiles/conv_band_config1_hbm_traffic.md (scaled by a 64 MiB copy)
-MEASURED_TRAFFIC_BYTES = {("conv_band_i8_32x32x32", 128): 57.6e6}
+MEASURED_TRAFFIC_BYTES = {("conv_band_i8_32x32x32", 128): 52.3e6}
 
 
 class Timer:

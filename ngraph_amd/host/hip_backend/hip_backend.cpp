@@ -13,6 +13,7 @@
 
 #include "hipq.h"
 #include "ngraph/ngraph.hpp"
+#include "ngraph/runtime/hip/pass/hip_quant_fusion.hpp"
 
 using namespace std;
 using namespace ngraph;
@@ -611,6 +612,7 @@ namespace
         // work on a private copy: compile must not change the caller's graph
         m_function = clone_function(*func);
         pass::Manager pm;
+        pm.register_pass<runtime::hip::pass::HIPQuantFusion>();
         pm.register_pass<pass::ConstantFolding>();
         pm.run_passes(m_function);
         for (const auto& n : m_function->get_ordered_ops())

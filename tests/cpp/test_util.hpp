@@ -26,3 +26,13 @@ inline void constant_fold(const std::shared_ptr<ngraph::Function>& f)
     pm.register_pass<ngraph::pass::ConstantFolding>();
     pm.run_passes(f);
 }
+
+template <typename T>
+size_t count_ops_of_type(const std::shared_ptr<ngraph::Function>& f)
+{
+    size_t n = 0;
+    for (const auto& op : f->get_ordered_ops())
+        if (ngraph::is_type<T>(op))
+            ++n;
+    return n;
+}

@@ -7,6 +7,7 @@
 // a flat list of launches over device buffers; call() binds parameter / result tensors and replays
 // the list on one stream.
 #include <cstring>
+#include <functional>
 #include <map>
 #include <mutex>
 #include <unordered_map>
@@ -148,6 +149,8 @@ namespace
         void lower_conv(const shared_ptr<Node>& n, Step& st);
         void lower_dot(const shared_ptr<Node>& n, Step& st);
         void lower_pool(const shared_ptr<Node>& n, Step& st);
+        void assign_layouts();
+        bool nxc(const Node* n) const { return m_nxc.count(n) != 0; }
         shared_ptr<DeviceBlock> alloc(size_t bytes)
         {
             auto b = make_shared<DeviceBlock>(bytes ? bytes : 1);
@@ -159,6 +162,7 @@ namespace
         bool m_perf;
         shared_ptr<Function> m_function;
         unordered_map<const Node*, int> m_value_of; // node (output 0) -> value id
+        unordered_map<const Node*, bool> m_nxc;     // nodes whose output tensor is kept channels-last
         vector<void*> m_value_ptr;                  // persistent device pointer, or null when bound per call
         vector<size_t> m_value_bytes;
         vector<int> m_value_uses;
@@ -222,6 +226,108 @@ namespace
         }
     }
 
+
+    // ------------------------------------------------------------------ HIPLayout
+    // Keeps the interior of a quantized network channels-last, the layout the convolution kernels
+    // read and write without a transposition -- the job CPULayout does for the reference's CPU
+    // backend with its blocked formats (src/ngraph/runtime/cpu/pass/cpu_layout.cpp:80-160), minus
+    // the inserted ConvertLayout nodes: a convolution converts on the way in or out for free, so
+    // tensors only ever change layout inside one.  Tensors joined by layout-agnostic ops (Relu,
+    // Convert, elementwise binaries, per-tensor Quantize / Dequantize, pools, Concat) form a class
+    // that shares a layout; a class becomes channels-last unless some member is produced or read by
+    // an op that only knows nGraph's [N, C, spatial...] (Parameters, Results, Reshape, Dot, ...).
+    // NGRAPH_PASS_ENABLES "HIPLayout:0" keeps every tensor in nGraph's layout.
+    int binary_code(const Node& n);
+    static bool is_conv(const Node* n)
+    {
+        return is_type<op::v0::QuantizedConvolution>(n) || is_type<op::v0::QuantizedConvolutionBias>(n) || is_type<op::v0::QuantizedConvolutionRelu>(n) ||
+               is_type<op::v0::QuantizedConvolutionBiasAdd>(n) || is_type<op::v0::QuantizedConvolutionBiasSignedAdd>(n);
+    }
+    static int conv_sum_input(const Node* n)
+    {
+        return (is_type<op::v0::QuantizedConvolutionBiasAdd>(n) || is_type<op::v0::QuantizedConvolutionBiasSignedAdd>(n)) ? 3 : -1;
+    }
+    // inputs of a layout-agnostic op that must share its output's layout (empty: not such an op)
+    static vector<size_t> tied_inputs(const Node* n)
+    {
+        vector<size_t> r;
+        const size_t rank = n->get_output_size() == 1 ? n->get_output_shape(0).size() : 0;
+        if (rank < 3)
+            return r;
+        if (is_type<op::v0::Relu>(n) || is_type<op::v0::Abs>(n) || is_type<op::v0::Convert>(n) || is_type<op::v0::MaxPool>(n) || is_type<op::v0::AvgPool>(n))
+            r.push_back(0);
+        else if (auto q = as_type<op::v0::Quantize>(n))
+        {
+            if (q->get_axes().empty())
+                r.push_back(0);
+        }
+        else if (auto dq = as_type<op::v0::Dequantize>(n))
+        {
+            if (dq->get_axes().empty())
+                r.push_back(0);
+        }
+        else if (is_type<op::v0::Concat>(n))
+            for (size_t i = 0; i < n->get_input_size(); ++i)
+                r.push_back(i);
+        else if (binary_code(*n) >= 0)
+            for (size_t i = 0; i < 2; ++i)
+                if (n->get_input_shape(i) == n->get_output_shape(0))
+                    r.push_back(i);
+        return r;
+    }
+
+    void HIPExecutable::assign_layouts()
+    {
+        pass::PassConfig config;
+        auto en = config.get_enables().find("HIPLayout");
+        if (en != config.get_enables().end() && !en->second)
+            return;
+        const auto ops = m_function->get_ordered_ops();
+        unordered_map<const Node*, const Node*> parent;
+        for (const auto& n : ops)
+            parent[n.get()] = n.get();
+        function<const Node*(const Node*)> find = [&](const Node* x) {
+            while (parent[x] != x)
+                x = parent[x] = parent[parent[x]];
+            return x;
+        };
+        auto unite = [&](const Node* a, const Node* b) { parent[find(a)] = find(b); };
+        // classes
+        for (const auto& n : ops)
+        {
+            for (size_t i : tied_inputs(n.get()))
+                unite(n->input_value(i).get_node(), n.get());
+            const int si = conv_sum_input(n.get());
+            if (si >= 0)
+                unite(n->input_value(si).get_node(), n.get());
+        }
+        // pins
+        unordered_map<const Node*, bool> pinned;
+        auto pin = [&](const Node* x) { pinned[find(x)] = true; };
+        for (const auto& n : ops)
+        {
+            const Node* p = n.get();
+            const bool conv = is_conv(p);
+            const vector<size_t> tied = tied_inputs(p);
+            if (!conv && tied.empty())
+                pin(p); // produces nGraph's layout (or has none)
+            if (p->get_output_size() != 1 || p->get_output_shape(0).size() < 3)
+                pin(p);
+            for (size_t i = 0; i < p->get_input_size(); ++i)
+            {
+                const bool free_read = conv && (i == 0 || static_cast<int>(i) == conv_sum_input(p));
+                const bool tied_read = find(p->input_value(i).get_node()) == find(p) && !tied.empty();
+                if (!free_read && !tied_read)
+                    pin(p->input_value(i).get_node());
+                if (p->input_value(i).get_index() != 0)
+                    pin(p->input_value(i).get_node());
+            }
+        }
+        for (const auto& n : ops)
+            if (!pinned.count(find(n.get())))
+                m_nxc[n.get()] = true;
+    }
+
     void HIPExecutable::lower_conv(const shared_ptr<Node>& n, Step& st)
     {
         const op::v0::ConvAttributes* attrs = nullptr;
@@ -256,6 +362,8 @@ namespace
         }
         hipq_conv_desc_t d;
         fill_conv_desc(d, *n, *attrs);
+        d.data_layout = nxc(n->input_value(0).get_node()) ? HIPQ_LAYOUT_NXC : HIPQ_LAYOUT_NCX;
+        d.out_layout = nxc(n.get()) ? HIPQ_LAYOUT_NXC : HIPQ_LAYOUT_NCX; // the sum input is in the output's class
         if (sum_i >= 0)
             sum_t = dtype_of(n->get_input_element_type(sum_i));
 
@@ -408,7 +516,7 @@ namespace
             pa = &ap->get_padding_above();
         }
         d.dtype = dtype_of(n->get_output_element_type(0));
-        d.layout = HIPQ_LAYOUT_NCX;
+        d.layout = nxc(n.get()) ? HIPQ_LAYOUT_NXC : HIPQ_LAYOUT_NCX; // input and output share a class
         d.n_spatial = static_cast<int32_t>(in.size() - 2);
         d.N = static_cast<int64_t>(in[0]);
         d.C = static_cast<int64_t>(in[1]);
@@ -586,9 +694,22 @@ namespace
         {
             const size_t axis = static_cast<size_t>(cc->get_concatenation_axis());
             const Shape& os = n->get_output_shape(0);
-            int64_t outer = 1, inner = 1;
+            // the order the axes have in memory: nGraph's, or batch, spatial..., channels
+            vector<size_t> order;
             for (size_t a = 0; a < os.size(); ++a)
-                (a < axis ? outer : inner) *= a == axis ? 1 : static_cast<int64_t>(os[a]);
+                if (!(nxc(n.get()) && a == 1))
+                    order.push_back(a);
+            if (nxc(n.get()))
+                order.push_back(1);
+            int64_t outer = 1, inner = 1;
+            bool before = true;
+            for (size_t a : order)
+            {
+                if (a == axis)
+                    before = false;
+                else
+                    (before ? outer : inner) *= static_cast<int64_t>(os[a]);
+            }
             vector<int64_t> extents;
             for (size_t i = 0; i < n->get_input_size(); ++i)
                 extents.push_back(static_cast<int64_t>(n->get_input_shape(i)[axis]));
@@ -615,6 +736,7 @@ namespace
         pm.register_pass<runtime::hip::pass::HIPQuantFusion>();
         pm.register_pass<pass::ConstantFolding>();
         pm.run_passes(m_function);
+        assign_layouts();
         for (const auto& n : m_function->get_ordered_ops())
             lower(n);
         for (const auto& p : m_function->get_parameters())

@@ -1,0 +1,101 @@
+// The backend's layout assignment (channels-last interiors): a quantized residual block --
+// 1x1 convolution, 3x3 convolution, max pool, 1x1 convolution with a residual sum, concat, 1x1
+// convolution -- gives byte-identical results with NGRAPH_PASS_ENABLES "HIPLayout:0" (every tensor in
+// nGraph's [N, C, H, W]) and with the pass on (only the block's input and output are).  The test
+// also reports the time of a call either way.
+#include <chrono>
+#include <cstdlib>
+
+#include "test_util.hpp"
+
+using namespace std;
+using namespace ngraph;
+
+namespace
+{
+    struct Lcg
+    {
+        uint32_t s;
+        int next(int lo, int hi)
+        {
+            s = s * 1664525u + 1013904223u;
+            return lo + static_cast<int>((s >> 8) % static_cast<uint32_t>(hi - lo + 1));
+        }
+    };
+
+    template <typename T>
+    shared_ptr<Node> random_constant(const element::Type& et, const Shape& shape, Lcg& rng, int lo, int hi)
+    {
+        vector<T> v(shape_size(shape));
+        for (auto& x : v)
+            x = static_cast<T>(rng.next(lo, hi));
+        return make_shared<op::v0::Constant>(et, shape, v);
+    }
+
+    shared_ptr<Function> residual_block(size_t N, size_t HW)
+    {
+        Lcg rng{12345u};
+        auto x = make_shared<op::v0::Parameter>(element::u8, Shape{N, 64, HW, HW});
+        auto scale = [](float v) { return op::v0::Constant::create(element::f32, Shape{}, {v}); };
+        auto conv = [&](const Output<Node>& data, size_t K, size_t C, size_t R, bool relu) {
+            auto w = random_constant<int8_t>(element::i8, Shape{K, C, R, R}, rng, -20, 20);
+            auto b = random_constant<int32_t>(element::i32, Shape{K}, rng, -2000, 2000);
+            const ptrdiff_t pad = static_cast<ptrdiff_t>(R / 2);
+            return make_shared<op::v0::QuantizedConvolutionBias>(data, w, b, Strides{1, 1}, Strides{1, 1}, CoordinateDiff{pad, pad}, CoordinateDiff{pad, pad}, Strides{1, 1},
+                                                                 scale(R == 1 ? 1.0f / 900 : 1.0f / 2500), relu);
+        };
+        auto c1 = conv(x, 64, 64, 1, true);
+        auto c2 = conv(c1, 64, 64, 3, true);
+        auto mp = make_shared<op::v0::MaxPool>(c2, Shape{3, 3}, Strides{1, 1}, Shape{1, 1}, Shape{1, 1});
+        auto w3 = random_constant<int8_t>(element::i8, Shape{64, 64, 1, 1}, rng, -20, 20);
+        auto b3 = random_constant<int32_t>(element::i32, Shape{64}, rng, -2000, 2000);
+        auto c3 = make_shared<op::v0::QuantizedConvolutionBiasAdd>(mp, w3, b3, c1, Strides{1, 1}, Strides{1, 1}, CoordinateDiff{0, 0}, CoordinateDiff{0, 0}, Strides{1, 1}, scale(1.0f / 1100),
+                                                                   scale(0.5f), true);
+        auto cat = make_shared<op::v0::Concat>(OutputVector{c3, mp}, 1);
+        auto c4 = conv(cat, 32, 128, 1, false);
+        return make_shared<Function>(OutputVector{c4}, ParameterVector{x});
+    }
+
+    vector<int8_t> run_block(size_t N, size_t HW, bool layout_pass, double* us_per_call)
+    {
+        setenv("NGRAPH_PASS_ENABLES", layout_pass ? "HIPLayout:1" : "HIPLayout:0", 1);
+        auto f = residual_block(N, HW);
+        auto backend = runtime::Backend::create("HIP");
+        auto a = backend->create_tensor(element::u8, f->get_parameters()[0]->get_output_shape(0));
+        Lcg rng{777u};
+        vector<uint8_t> data(a->get_element_count());
+        for (auto& v : data)
+            v = static_cast<uint8_t>(rng.next(0, 255));
+        copy_data(a, data);
+        auto r = backend->create_tensor(element::i8, f->get_output_shape(0));
+        auto exec = backend->compile(f);
+        unsetenv("NGRAPH_PASS_ENABLES");
+        exec->call_with_validate({r}, {a});
+        if (us_per_call)
+        {
+            const int reps = 30;
+            auto t0 = chrono::steady_clock::now();
+            for (int i = 0; i < reps; ++i)
+                exec->call({r}, {a});
+            *us_per_call = chrono::duration<double, micro>(chrono::steady_clock::now() - t0).count() / reps;
+        }
+        return read_vector<int8_t>(r);
+    }
+}
+
+GPU_TEST(HIP, layout_pass_residual_block)
+{
+    // 14x14 maps: generic convolution kernels; 56x56 maps at 64 channels: the band kernel
+    for (size_t hw : {14u, 56u})
+    {
+        double us_off = 0, us_on = 0;
+        auto off = run_block(4, hw, false, &us_off);
+        auto on = run_block(4, hw, true, &us_on);
+        EXPECT_TRUE(off == on);
+        size_t nonzero = 0;
+        for (int8_t v : on)
+            nonzero += v != 0;
+        EXPECT_TRUE(nonzero > on.size() / 4); // the block computes something
+        std::cout << "[   INFO   ] residual block N=4 " << hw << "x" << hw << ": " << us_off << " us per call in nGraph's layout, " << us_on << " us channels-last inside" << std::endl;
+    }
+}

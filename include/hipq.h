@@ -100,6 +100,18 @@ HIPQ_API int hipq_fill_bytes(void* dst_dev, int value, size_t bytes, void* strea
 HIPQ_API int hipq_stream_create(void** stream);
 HIPQ_API int hipq_stream_destroy(void* stream);
 HIPQ_API int hipq_stream_sync(void* stream);
+/* Stream capture into a HIP graph, for callers that replay one fixed launch sequence (what
+ * runtime::Executable::call does, src/ngraph/runtime/executable.hpp:44-52): begin, issue the launches
+ * on `stream` as usual (nothing runs), end -> an executable graph; hipq_graph_launch replays it on a
+ * stream.  The launches between begin and end must not grow the per-device workspace: run the
+ * sequence once uncaptured first.  hipq_workspace_epoch changes whenever the workspace of the
+ * current device is reallocated; a graph captured under an older epoch may point into freed memory
+ * and must be captured again. */
+HIPQ_API int hipq_capture_begin(void* stream);
+HIPQ_API int hipq_capture_end(void* stream, void** graph_exec);
+HIPQ_API int hipq_graph_launch(void* graph_exec, void* stream);
+HIPQ_API int hipq_graph_destroy(void* graph_exec);
+HIPQ_API uint64_t hipq_workspace_epoch(void);
 HIPQ_API int hipq_event_create(void** event);
 HIPQ_API int hipq_event_destroy(void* event);
 HIPQ_API int hipq_event_record(void* event, void* stream);

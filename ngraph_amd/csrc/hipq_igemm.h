@@ -322,7 +322,7 @@ namespace hipq
     // WM x WN MFMA tiles per wavefront, WAVES_M x WAVES_N wavefronts per workgroup (= 4).
     // X_ON_A: activations feed MFMA source A (NCHW output) instead of the weights.
     template <class XL, int WM, int WN, int WAVES_M, int WAVES_N, bool X_ON_A, int MODE, int KIND>
-    __global__ __launch_bounds__(256, 2) void igemm_i8_kernel(XL xl,
+    __global__ __launch_bounds__(256, (WM * WN <= 4 ? 4 : 2)) void igemm_i8_kernel(XL xl,
                                                               const int8_t* __restrict__ w,
                                                               const int32_t* __restrict__ wsum,
                                                               int64_t M,
@@ -510,6 +510,13 @@ namespace hipq
         {
             // rows = output channels: 4 consecutive channels of one m -> out[m][n..n+3]
             const bool vec_ok = (N & 3) == 0;
+            // 8-bit outputs whose rows are whole 16-byte pieces leave through LDS (the operand buffers
+            // are free now): a lane's dword of four channels goes into a [BM][BN + 16] byte tile, and
+            // the tile is written out 16 bytes a lane with neighbouring lanes on neighbouring pieces
+            // of a row -- full lines instead of 64 scattered dwords per store instruction
+            constexpr int SP = BN + 16; // staging pitch: 16-byte aligned rows, two-way bank conflicts at worst
+            constexpr bool kCanStage = KIND == OUT_Q8 && BM * SP <= 2 * STAGE;
+            const bool staged = kCanStage && (N & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
 #pragma unroll
             for (int ni = 0; ni < WN; ++ni)
             {
@@ -561,7 +568,9 @@ namespace hipq
                             const int32_t a = acc[mi][ni][4 * g + e];
                             v[e] = MODE == EPI_INTERP ? epi_interp<KIND>(ec, a) : epi_fused<KIND>(ec, a, bias4[e], scale4[e], has_sum, s4[e], relu);
                         }
-                        if (vec_ok) // nb is a multiple of 4, so nb + 3 < N and the store is aligned
+                        if (kCanStage && staged)
+                            *reinterpret_cast<uint32_t*>(lds + ((wm * WM + mi) * 32 + (lane & 31)) * SP + (nb - n0)) = pack4(v);
+                        else if (vec_ok) // nb is a multiple of 4, so nb + 3 < N and the store is aligned
                         {
                             if (KIND == OUT_Q8)
                                 *reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(out) + o) = pack4(v);
@@ -576,6 +585,23 @@ namespace hipq
                                     store_out(out, KIND == OUT_Q8 ? HIPQ_U8 : HIPQ_I32, o + e, v[e]);
                         }
                     }
+                }
+            }
+            if (kCanStage && staged) // uniform
+            {
+                __syncthreads();
+                constexpr int PIECES = BN / 16; // per row
+                uint8_t* o8 = static_cast<uint8_t*>(out);
+#pragma unroll
+                for (int i = 0; i < BM * PIECES / 256; ++i)
+                {
+                    const int id = i * 256 + tid;
+                    const int row = id / PIECES;
+                    const int piece = id % PIECES;
+                    const int64_t m = m0 + row;
+                    const int32_t n = n0 + piece * 16;
+                    if (m < M && n < N)
+                        *reinterpret_cast<v4i*>(o8 + m * N + n) = *reinterpret_cast<const v4i*>(lds + row * SP + piece * 16);
                 }
             }
         }
@@ -696,6 +722,10 @@ namespace hipq
                            hipStream_t s,
                            const char* name)
     {
+        // short reductions are bound by latency, not by LDS traffic: small wavefront tiles (64 x 64)
+        // take half the registers, so twice as many workgroups are resident to hide it
+        if (Kred <= 512 && N > 64 && getenv("HIPQ_NO_SMALL_TILE") == nullptr)
+            return launch_tile<XL, 2, 2, 2, 2, X_ON_A, MODE, KIND>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
         if (N <= 64)
             return launch_tile<XL, 4, 2, 4, 1, X_ON_A, MODE, KIND>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
         return launch_tile<XL, 4, 2, 2, 2, X_ON_A, MODE, KIND>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);

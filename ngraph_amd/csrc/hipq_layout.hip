@@ -153,20 +153,70 @@ namespace hipq
         return check_launch("row_sums_i8");
     }
 
-    // filter [K][C][taps] -> packed [K][taps][C]
+    // filter [K][C][taps] -> packed [K][taps][Cp], channels C .. Cp-1 zero
     __global__ __launch_bounds__(256) void pack_filter_kernel(
-        const int8_t* __restrict__ f, int8_t* __restrict__ p, int64_t K, int64_t Cc, int64_t taps)
+        const int8_t* __restrict__ f, int8_t* __restrict__ p, int64_t K, int64_t Cc, int64_t Cp, int64_t taps)
     {
-        int64_t total = K * Cc * taps;
+        int64_t total = K * Cp * taps;
         int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
         int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
         for (; i < total; i += step)
         {
-            int64_t c = i % Cc;
-            int64_t t = (i / Cc) % taps;
-            int64_t k = i / (Cc * taps);
-            p[i] = f[(k * Cc + c) * taps + t];
+            int64_t c = i % Cp;
+            int64_t t = (i / Cp) % taps;
+            int64_t k = i / (Cp * taps);
+            p[i] = c < Cc ? f[(k * Cc + c) * taps + t] : static_cast<int8_t>(0);
         }
+    }
+
+    // [N][C][X] or [N][X][C] bytes -> [N][X][16] with the channels C .. 15 holding the data zero point
+    // (they meet zero weights; as the zero point they also vanish on the exact path for a non-zero
+    // filter zero point); one pixel a lane, one 16-byte store
+    __global__ __launch_bounds__(256) void pad_channels_kernel(const uint8_t* __restrict__ in, uint8_t* __restrict__ out, int64_t pixels, int64_t X, int32_t Cc, int32_t in_ncx,
+                                                               const void* zp, int32_t zp_t)
+    {
+        const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+        if (i >= pixels)
+            return;
+        const int64_t n = i / X, x = i - n * X;
+        const uint32_t fill = (static_cast<uint32_t>(load_zp(zp, zp_t)) & 0xffu) * 0x01010101u;
+        uint32_t w[4] = {fill, fill, fill, fill};
+        for (int c = 0; c < Cc; ++c)
+            w[c >> 2] &= ~(0xffu << (8 * (c & 3)));
+        for (int c = 0; c < Cc; ++c)
+        {
+            const uint32_t b = in_ncx ? in[(n * Cc + c) * X + x] : in[i * Cc + c];
+            w[c >> 2] |= b << (8 * (c & 3));
+        }
+        reinterpret_cast<uint4*>(out)[i] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+
+    int launch_pad_channels(const void* in, void* out, int64_t N, int64_t X, int64_t Cc, bool in_ncx, const void* zp, int zp_t, hipStream_t s)
+    {
+        const int64_t pixels = N * X;
+        if (pixels == 0)
+            return HIPQ_OK;
+        HIPQ_REQUIRE(Cc >= 1 && Cc < 16, "channel padding takes fewer than 16 channels");
+        HIPQ_REQUIRE((pixels + 255) / 256 < (1ll << 31), "tensor too large for one launch");
+        pad_channels_kernel<<<static_cast<unsigned>((pixels + 255) / 256), 256, 0, s>>>(static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), pixels, X, static_cast<int32_t>(Cc),
+                                                                                       in_ncx ? 1 : 0, zp, zp_t);
+        return check_launch("pad_channels");
+    }
+
+    // Fewer than 16 input channels (a network's first layer): the MFMA kernels take the layer with the
+    // channels padded to 16 -- zero weights in the packed filter, a padded copy of the data
+    bool conv_pad_eligible(const ConvGeom& g, ConvGeom* padded)
+    {
+        if (g.C >= 16 || g.C < 1)
+            return false;
+        ConvGeom p = g;
+        p.C = 16;
+        p.data_layout = HIPQ_LAYOUT_NXC;
+        if (!conv_mfma_eligible(p))
+            return false;
+        if (padded)
+            *padded = p;
+        return true;
     }
 }
 
@@ -189,7 +239,9 @@ int hipq_transpose_nxc_to_ncx(const void* in, void* out, int64_t N, int64_t C, i
 size_t hipq_conv_packed_filter_bytes(const hipq_conv_desc_t* desc)
 {
     ConvGeom g;
-    if (make_geom(desc, &g) != HIPQ_OK || !conv_mfma_eligible(g))
+    if (make_geom(desc, &g) != HIPQ_OK)
+        return 0;
+    if (!conv_mfma_eligible(g) && !conv_pad_eligible(g, &g))
         return 0;
     size_t w = align_up(static_cast<size_t>(g.K * g.C * g.taps()), 256);
     return w + static_cast<size_t>(g.K) * sizeof(int32_t);
@@ -201,7 +253,8 @@ int hipq_conv_pack_filter(const hipq_conv_desc_t* desc, const void* filter, void
     int rc = make_geom(desc, &g);
     if (rc)
         return rc;
-    if (!conv_mfma_eligible(g))
+    const int64_t src_c = g.C;
+    if (!conv_mfma_eligible(g) && !conv_pad_eligible(g, &g))
         return fail(HIPQ_ERR_UNSUPPORTED, "shape is not eligible for the MFMA path (hipq_conv_packed_filter_bytes is 0)");
     HIPQ_REQUIRE(filter && packed, "null pointer");
     hipStream_t s = as_stream(stream);
@@ -210,7 +263,7 @@ int hipq_conv_pack_filter(const hipq_conv_desc_t* desc, const void* filter, void
     if (blocks > 65536)
         blocks = 65536;
     pack_filter_kernel<<<static_cast<unsigned>(blocks), 256, 0, s>>>(
-        static_cast<const int8_t*>(filter), static_cast<int8_t*>(packed), g.K, g.C, g.taps());
+        static_cast<const int8_t*>(filter), static_cast<int8_t*>(packed), g.K, src_c, g.C, g.taps());
     rc = check_launch("pack_filter");
     if (rc)
         return rc;

@@ -32,6 +32,20 @@ namespace hipq
                         hipStream_t s)
     {
         // the MFMA kernels have no fused-policy instantiation with int32 output (no nGraph op asks for one)
+        ConvGeom padded;
+        if (packed && !conv_mfma_eligible(g) && conv_pad_eligible(g, &padded) && !(epi.mode == EPI_FUSED && g.out_t == HIPQ_I32))
+        {
+            // a first layer's few channels: a 16-channel channels-last copy, then the MFMA kernel
+            void* ws = nullptr;
+            const int64_t in_sp = g.in[1] * g.in[2];
+            int rc = workspace(align_up(static_cast<size_t>(g.N * in_sp * 16), 256), &ws);
+            if (rc)
+                return rc;
+            rc = launch_pad_channels(data, ws, g.N, in_sp, g.C, g.data_layout == HIPQ_LAYOUT_NCX, zp.data_zp, zp.data_t, s);
+            if (rc)
+                return rc;
+            return launch_conv_mfma(padded, ws, packed, zp, epi, out, g.out_layout == HIPQ_LAYOUT_NCX && g.K > 1, s);
+        }
         if (!packed || !conv_mfma_eligible(g) || (epi.mode == EPI_FUSED && g.out_t == HIPQ_I32))
             return launch_conv_direct(g, data, filter, zp, epi, out, s);
 

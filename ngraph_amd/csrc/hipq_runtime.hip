@@ -32,6 +32,7 @@ namespace hipq
     static std::mutex g_ws_mutex;
     static void* g_ws_ptr[kMaxDevices] = {};
     static size_t g_ws_bytes[kMaxDevices] = {};
+    static uint64_t g_ws_epoch[kMaxDevices] = {};
 
     int workspace(size_t bytes, void** ptr)
     {
@@ -53,6 +54,7 @@ namespace hipq
             size_t want = align_up(bytes + bytes / 4, 1 << 20);
             HIPQ_HIP(hipMalloc(&g_ws_ptr[dev], want));
             g_ws_bytes[dev] = want;
+            ++g_ws_epoch[dev];
         }
         *ptr = g_ws_ptr[dev];
         return HIPQ_OK;
@@ -210,6 +212,51 @@ int hipq_stream_sync(void* stream)
 {
     HIPQ_HIP(hipStreamSynchronize(as_stream(stream)));
     return HIPQ_OK;
+}
+
+int hipq_capture_begin(void* stream)
+{
+    HIPQ_REQUIRE(stream, "capture needs a stream of its own, not the null stream");
+    HIPQ_HIP(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeRelaxed));
+    return HIPQ_OK;
+}
+
+int hipq_capture_end(void* stream, void** graph_exec)
+{
+    HIPQ_REQUIRE(stream && graph_exec, "null argument");
+    *graph_exec = nullptr;
+    hipGraph_t graph = nullptr;
+    HIPQ_HIP(hipStreamEndCapture(as_stream(stream), &graph));
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    hipGraphDestroy(graph);
+    if (e != hipSuccess)
+        return fail(HIPQ_ERR_HIP, "hipGraphInstantiate: %s", hipGetErrorString(e));
+    *graph_exec = exec;
+    return HIPQ_OK;
+}
+
+int hipq_graph_launch(void* graph_exec, void* stream)
+{
+    HIPQ_REQUIRE(graph_exec, "graph is null");
+    HIPQ_HIP(hipGraphLaunch(reinterpret_cast<hipGraphExec_t>(graph_exec), as_stream(stream)));
+    return HIPQ_OK;
+}
+
+int hipq_graph_destroy(void* graph_exec)
+{
+    if (graph_exec)
+        HIPQ_HIP(hipGraphExecDestroy(reinterpret_cast<hipGraphExec_t>(graph_exec)));
+    return HIPQ_OK;
+}
+
+uint64_t hipq_workspace_epoch(void)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return 0;
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    return g_ws_epoch[dev];
 }
 
 int hipq_event_create(void** event)

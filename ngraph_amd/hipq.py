@@ -263,6 +263,11 @@ EXPORTS = [
     "hipq_stream_create",
     "hipq_stream_destroy",
     "hipq_stream_sync",
+    "hipq_capture_begin",
+    "hipq_capture_end",
+    "hipq_graph_launch",
+    "hipq_graph_destroy",
+    "hipq_workspace_epoch",
     "hipq_event_create",
     "hipq_event_destroy",
     "hipq_event_record",
@@ -345,6 +350,12 @@ def load():
     lib.hipq_quantized_dot_bias.argtypes = [C.POINTER(DotDesc), C.POINTER(FusedDesc)] + [vp] * 7
     for n in ("hipq_transpose_ncx_to_nxc", "hipq_transpose_nxc_to_ncx"):
         getattr(lib, n).argtypes = [vp, vp, i64, i64, i64, i32, vp]
+    lib.hipq_capture_begin.argtypes = [vp]
+    lib.hipq_capture_end.argtypes = [vp, C.POINTER(vp)]
+    lib.hipq_graph_launch.argtypes = [vp, vp]
+    lib.hipq_graph_destroy.argtypes = [vp]
+    lib.hipq_workspace_epoch.argtypes = []
+    lib.hipq_workspace_epoch.restype = C.c_uint64
     lib.hipq_binary.argtypes = [i32, i32, vp, i64, vp, i64, vp, i64, vp]
     lib.hipq_unary.argtypes = [i32, i32, vp, vp, i64, vp]
     lib.hipq_convert.argtypes = [i32, i32, vp, vp, i64, vp]

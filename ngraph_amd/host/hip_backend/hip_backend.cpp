@@ -171,6 +171,12 @@ namespace
         vector<shared_ptr<DeviceBlock>> m_blocks;
         void* m_stream = nullptr;
         mutex m_mutex;
+        // HIP graph of the call's launch sequence: captured on the second call with a given set of
+        // tensor addresses, replayed while the addresses (and the library's workspace) stay the same
+        bool m_use_graph = true;
+        void* m_graph = nullptr;
+        vector<void*> m_graph_key, m_last_key;
+        uint64_t m_graph_epoch = 0;
         // performance data
         vector<void*> m_events;
         vector<double> m_step_us;
@@ -751,6 +757,11 @@ namespace
                 check(hipq_event_create(&e), "event creation");
             m_step_us.assign(m_steps.size(), 0.0);
         }
+        {
+            pass::PassConfig config;
+            auto en = config.get_enables().find("HIPGraph");
+            m_use_graph = !m_perf && !(en != config.get_enables().end() && !en->second);
+        }
         // validation is against the caller's function (same parameter / result signature)
         set_parameters_and_results(*func);
     }
@@ -759,6 +770,8 @@ namespace
     {
         for (auto e : m_events)
             hipq_event_destroy(e);
+        if (m_graph)
+            hipq_graph_destroy(m_graph);
         if (m_stream)
         {
             hipq_stream_sync(m_stream);
@@ -797,22 +810,60 @@ namespace
                 direct[i] = true;
             }
         }
-        vector<void*> in;
-        for (size_t s = 0; s < m_steps.size(); ++s)
-        {
-            const Step& st = m_steps[s];
-            in.clear();
-            for (int v : st.inputs)
-                in.push_back(ptr[v]);
+        auto issue = [&]() {
+            vector<void*> in;
+            for (size_t s = 0; s < m_steps.size(); ++s)
+            {
+                const Step& st = m_steps[s];
+                in.clear();
+                for (int v : st.inputs)
+                    in.push_back(ptr[v]);
+                if (m_perf)
+                    check(hipq_event_record(m_events[s], m_stream), "event record");
+                st.launch(in, ptr[st.output], m_stream);
+            }
             if (m_perf)
-                check(hipq_event_record(m_events[s], m_stream), "event record");
-            st.launch(in, ptr[st.output], m_stream);
+                check(hipq_event_record(m_events[m_steps.size()], m_stream), "event record");
+            for (size_t i = 0; i < outputs.size(); ++i)
+                if (!direct[i])
+                    check(hipq_memcpy_d2d(out_ptr[i], ptr[m_result_value[i]], m_value_bytes[m_result_value[i]], m_stream), "result copy");
+        };
+        // The launch sequence of a call depends only on the tensor addresses: the first call with a
+        // set of addresses runs eagerly (and lets the library size its workspace), the second is
+        // captured into a HIP graph, later ones replay it -- one launch instead of one per op.
+        vector<void*> key;
+        for (size_t i = 0; i < inputs.size(); ++i)
+            key.push_back(ptr[m_param_value[i]]);
+        key.insert(key.end(), out_ptr.begin(), out_ptr.end());
+        if (m_use_graph && m_graph && key == m_graph_key && hipq_workspace_epoch() == m_graph_epoch)
+            check(hipq_graph_launch(m_graph, m_stream), "graph launch");
+        else if (m_use_graph && !m_steps.empty() && key == m_last_key)
+        {
+            if (m_graph)
+            {
+                hipq_graph_destroy(m_graph);
+                m_graph = nullptr;
+            }
+            check(hipq_capture_begin(m_stream), "stream capture");
+            try
+            {
+                issue();
+            }
+            catch (...)
+            {
+                void* dropped = nullptr;
+                hipq_capture_end(m_stream, &dropped);
+                hipq_graph_destroy(dropped);
+                throw;
+            }
+            check(hipq_capture_end(m_stream, &m_graph), "stream capture");
+            m_graph_key = key;
+            m_graph_epoch = hipq_workspace_epoch();
+            check(hipq_graph_launch(m_graph, m_stream), "graph launch");
         }
-        if (m_perf)
-            check(hipq_event_record(m_events[m_steps.size()], m_stream), "event record");
-        for (size_t i = 0; i < outputs.size(); ++i)
-            if (!direct[i])
-                check(hipq_memcpy_d2d(out_ptr[i], ptr[m_result_value[i]], m_value_bytes[m_result_value[i]], m_stream), "result copy");
+        else
+            issue();
+        m_last_key = key;
         check(hipq_stream_sync(m_stream), "Executable::call");
         if (m_perf)
         {

@@ -96,6 +96,53 @@ GPU_TEST(HIP, layout_pass_residual_block)
         for (int8_t v : on)
             nonzero += v != 0;
         EXPECT_TRUE(nonzero > on.size() / 4); // the block computes something
+        {
+            // device time per op (events around every launch)
+            auto f = residual_block(4, hw);
+            auto backend = runtime::Backend::create("HIP");
+            auto a = backend->create_tensor(element::u8, f->get_parameters()[0]->get_output_shape(0));
+            auto r = backend->create_tensor(element::i8, f->get_output_shape(0));
+            auto exec = backend->compile(f, true);
+            for (int i = 0; i < 10; ++i)
+                exec->call({r}, {a});
+            for (const auto& pc : exec->get_performance_data())
+                std::cout << "[   INFO   ]   " << pc.get_node()->description() << " " << pc.microseconds() << " us" << std::endl;
+        }
         std::cout << "[   INFO   ] residual block N=4 " << hw << "x" << hw << ": " << us_off << " us per call in nGraph's layout, " << us_on << " us channels-last inside" << std::endl;
+    }
+}
+
+// Executable::call replays a HIP graph from its third call with the same tensors on.  Every replay is
+// checked against an executable that never captures (NGRAPH_PASS_ENABLES "HIPGraph:0"), with new input
+// data before each call and the other executable's eager launches and synchronizations in between.
+GPU_TEST(HIP, call_replays_hip_graph)
+{
+    for (bool layout_pass : {true, false}) // without the layout pass the calls go through the library's workspace
+    {
+        const size_t N = 2, HW = 56;
+        auto backend = runtime::Backend::create("HIP");
+        setenv("NGRAPH_PASS_ENABLES", layout_pass ? "HIPGraph:1;HIPLayout:1" : "HIPGraph:1;HIPLayout:0", 1);
+        auto with_graph = backend->compile(residual_block(N, HW));
+        setenv("NGRAPH_PASS_ENABLES", layout_pass ? "HIPGraph:0;HIPLayout:1" : "HIPGraph:0;HIPLayout:0", 1);
+        auto eager = backend->compile(residual_block(N, HW));
+        unsetenv("NGRAPH_PASS_ENABLES");
+        const Shape in_shape{N, 64, HW, HW}, out_shape{N, 32, HW, HW};
+        auto a = backend->create_tensor(element::u8, in_shape);
+        auto r1 = backend->create_tensor(element::i8, out_shape);
+        auto r2 = backend->create_tensor(element::i8, out_shape);
+        auto other = backend->create_tensor(element::i8, out_shape);
+        Lcg rng{99u};
+        vector<uint8_t> data(shape_size(in_shape));
+        for (int call = 0; call < 7; ++call)
+        {
+            for (auto& v : data)
+                v = static_cast<uint8_t>(rng.next(0, 255));
+            copy_data(a, data);
+            // call 5 writes to another tensor (a new set of addresses: eager again), call 6 returns to the first set
+            auto& target = call == 5 ? other : r1;
+            with_graph->call_with_validate({target}, {a});
+            eager->call_with_validate({r2}, {a});
+            EXPECT_TRUE(read_vector<int8_t>(target) == read_vector<int8_t>(r2));
+        }
     }
 }

@@ -197,6 +197,26 @@ def bench_glue(lib, stream, timer, steps, warmup, batch=128):
     return out
 
 
+def bench_resnet50(lib, stream, timer, batches=(1, 32, 128)):
+    """synthetic int8 ResNet-50 (ngraph_amd/resnet50.py), every tensor resident in HBM, channels-last,
+    one forward pass = 53 convolutions, 2 pools, 1 GEMM; replayed as one HIP graph"""
+    from ngraph_amd import resnet50 as R
+
+    out = []
+    for n in batches:
+        plan = R.DevicePlan(lib, stream, n)
+        plan.set_images_nchw(R.synthetic_images(min(n, 4)).repeat((n + 3) // 4, axis=0)[:n])
+        steps = 30 if n <= 32 else 10
+        _, eager = timer.run(plan.launch, steps, 2)
+        plan.capture()
+        _, graph = timer.run(plan.replay, steps, 2)
+        H.check(lib.hipq_graph_destroy(plan.graph))
+        best = min(eager, graph)
+        out.append(dict(batch=n, ms_eager=eager, ms_graph=graph, images_per_s=n / (best * 1e-3), tops=plan.ops_per_image * n / (best * 1e-3) / 1e12, launches=len(plan.calls)))
+        del plan
+    return out
+
+
 def cpu_baseline(seconds=12.0):
     """The reference's own convolution kernel (oracle/_ref, compiled from the nGraph tree) when it
     was built, else the C restatement; BASELINE config 1 at N=1 on one host core."""
@@ -278,6 +298,7 @@ def main():
         results["quantize_dequantize_config3"] = bench_qdq(lib, stream, timer, small, 5)
         results["pool_resnet50_u8"] = bench_pool(lib, stream, timer, small, 5, args.batch)
         results["glue_resnet50_u8"] = bench_glue(lib, stream, timer, small, 5, args.batch)
+        results["resnet50_int8"] = bench_resnet50(lib, stream, timer)
         cpu = cpu_baseline()
 
     derived_peak = info.compute_units * info.clock_mhz * 1e6 * 8192 / 1e12

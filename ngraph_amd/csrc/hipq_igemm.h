@@ -32,6 +32,7 @@
 namespace hipq
 {
     typedef int v4i __attribute__((ext_vector_type(4)));
+    typedef float v4f __attribute__((ext_vector_type(4)));
     typedef int v16i __attribute__((ext_vector_type(16)));
 
     constexpr int BK = 64; // reduction bytes per LDS slice
@@ -669,6 +670,297 @@ namespace hipq
         }
     }
 
+
+    // ---- persistent, software-pipelined variant ---------------------------------------------------
+    // For 8-bit channels-last / row-major outputs whose rows are whole 16-byte pieces.  A workgroup
+    // walks its tiles (tile = vb + j * grid) and treats all their 64-byte reduction slices as one
+    // sequence: while slice s feeds the MFMAs out of LDS, slice s+1 waits in registers and the loads
+    // of slice s+2 -- possibly the next tile's -- are in flight, so short reductions (1x1
+    // convolutions over 64 channels are a single slice) overlap their loads with the neighbouring
+    // tiles' arithmetic and epilogues, and long ones have two slices of latency cover.  Each
+    // wavefront requantizes its own 64 x 64 sub-tile into a private swizzled LDS region and writes it
+    // out 16 bytes a lane; per-channel constants of the current column tile sit in LDS.
+    template <class XL, int WM, int WN, int WAVES_M, int WAVES_N, int MODE>
+    __global__ __launch_bounds__(256, 2) void igemm_pipe_kernel(XL xl,
+                                                                const int8_t* __restrict__ w,
+                                                                const int32_t* __restrict__ wsum,
+                                                                int64_t M,
+                                                                int32_t Kred,
+                                                                int32_t x_unsigned,
+                                                                int32_t m_tiles,
+                                                                int32_t n_tiles,
+                                                                ZeroPoints zp,
+                                                                Epilogue epi,
+                                                                OutMap om,
+                                                                void* __restrict__ out)
+    {
+        static_assert(WAVES_M * WAVES_N == 4, "four wavefronts per workgroup");
+        constexpr int BM = WAVES_M * WM * 32;
+        constexpr int BN = WAVES_N * WN * 32;
+        constexpr int TM = WM * 32, TN = WN * 32; // a wavefront's sub-tile
+        constexpr int XLOADS = BM * 4 / 256;
+        constexpr int WLOADS = (BN * 4 + 255) / 256;
+        constexpr int STAGE = (BM + BN) * BK;
+        constexpr int OUT_STAGE = TM * TN; // per wavefront
+        static_assert(TN == 64, "the output staging swizzle is written for 64-byte rows");
+        extern __shared__ __attribute__((aligned(16))) uint8_t lds[]; // [2][x | w] operands, 4 output regions, per-channel constants
+        uint8_t* const ostage = lds + 2 * STAGE + (threadIdx.x >> 6) * OUT_STAGE;
+        float* const params = reinterpret_cast<float*>(lds + 2 * STAGE + 4 * OUT_STAGE); // [3][BN]: correction (as int), bias, scale
+
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = tid >> 6;
+        const int wn = wave % WAVES_N;
+        const int wm = wave / WAVES_N;
+        const int N = om.N;
+        const int grid = static_cast<int>(gridDim.x);
+        const int total_tiles = m_tiles * n_tiles;
+        const int vb = (grid & 7) == 0 ? (static_cast<int>(blockIdx.x) & 7) * (grid >> 3) + (static_cast<int>(blockIdx.x) >> 3) : static_cast<int>(blockIdx.x);
+        if (vb >= total_tiles)
+            return;
+        const int my_tiles = (total_tiles - vb + grid - 1) / grid;
+        // tiles of one column block are consecutive, so a workgroup rarely changes its column block
+        auto tile_origin = [&](int j, int64_t& m0, int32_t& n0) {
+            const int t = vb + j * grid;
+            const int nt = t / m_tiles;
+            m0 = static_cast<int64_t>(t - nt * m_tiles) * BM;
+            n0 = nt * BN;
+        };
+
+        const int32_t xzp = load_zp(zp.data_zp, zp.data_t);
+        const int32_t wzp = load_zp(zp.filter_zp, zp.filter_t);
+        if (wzp != 0) // uniform across the grid
+        {
+            for (int j = 0; j < my_tiles; ++j)
+            {
+                int64_t m0;
+                int32_t n0;
+                tile_origin(j, m0, n0);
+                slow_tile(xl, w, M, Kred, x_unsigned, xzp, wzp, epi, om, out, m0, n0, BM, BN);
+            }
+            return;
+        }
+        const int32_t mult = (x_unsigned ? 128 : 0) - xzp;
+        const EpiConst ec = epi_const(epi);
+        const bool has_sum = MODE == EPI_FUSED && epi.sum_in != nullptr;
+        const bool relu = epi.relu != 0;
+
+        // ---- loader --------------------------------------------------------------------------
+        const int lrow = tid >> 2;
+        const int lchunk = tid & 3;
+        const int xor_mask = x_unsigned ? static_cast<int>(0x80808080u) : 0;
+        const int fill = (xzp & 0xFF) * 0x01010101;
+        const __amdgpu_buffer_rsrc_t xrs = make_rsrc(xl.x, xl.bytes);
+        const __amdgpu_buffer_rsrc_t wrs = make_rsrc(w, static_cast<uint32_t>(N) * static_cast<uint32_t>(Kred));
+        const int KT = (Kred + BK - 1) / BK;
+        const int total = my_tiles * KT;
+        typename XL::Row xr[XLOADS];
+        typename XL::Cursor cur;
+        int32_t woff[WLOADS];
+        int32_t kb = 0;
+        int lj = 0, lkt = 0;
+        auto loader_tile = [&](int j) {
+            int64_t m0;
+            int32_t n0;
+            tile_origin(j, m0, n0);
+#pragma unroll
+            for (int i = 0; i < XLOADS; ++i)
+                xl.init_row(xr[i], m0 + lrow + 64 * i, M);
+            xl.init_cursor(cur, lchunk * 16);
+#pragma unroll
+            for (int i = 0; i < WLOADS; ++i)
+            {
+                const int32_t r = lrow + 64 * i;
+                woff[i] = (n0 + r < N && r < BN) ? (n0 + r) * Kred : kOob;
+            }
+            kb = lchunk * 16;
+        };
+        struct Regs
+        {
+            v4i x[XLOADS];
+            v4i w[WLOADS];
+            uint32_t oob;
+        };
+        auto gload = [&](Regs& r) {
+            r.oob = 0;
+#pragma unroll
+            for (int i = 0; i < XLOADS; ++i)
+            {
+                const int32_t off = xl.offset(xr[i], cur);
+                r.oob |= (off == kOob ? 1u : 0u) << i;
+                r.x[i] = buffer_load16(xrs, off);
+            }
+#pragma unroll
+            for (int i = 0; i < WLOADS; ++i)
+                r.w[i] = buffer_load16(wrs, (woff[i] != kOob && kb < Kred) ? woff[i] + kb : kOob);
+            if (++lkt == KT)
+            {
+                lkt = 0;
+                if (++lj < my_tiles)
+                    loader_tile(lj);
+            }
+            else
+            {
+                xl.advance(cur, BK);
+                kb += BK;
+            }
+        };
+        auto lstore = [&](const Regs& r, int buf) {
+            uint8_t* xs = lds + buf * STAGE;
+            uint8_t* ws = xs + BM * BK;
+#pragma unroll
+            for (int i = 0; i < XLOADS; ++i)
+            {
+                v4i v = r.x[i];
+                if (fill != 0) // uniform: a non-zero data zero point pads with that byte
+                {
+                    const bool oob = (r.oob >> i) & 1u;
+                    v = v4i{oob ? fill : v[0], oob ? fill : v[1], oob ? fill : v[2], oob ? fill : v[3]};
+                }
+                *reinterpret_cast<v4i*>(xs + lds_offset(lrow + 64 * i, lchunk)) = v4i{v[0] ^ xor_mask, v[1] ^ xor_mask, v[2] ^ xor_mask, v[3] ^ xor_mask};
+            }
+#pragma unroll
+            for (int i = 0; i < WLOADS; ++i)
+                if (lrow + 64 * i < BN)
+                    *reinterpret_cast<v4i*>(ws + lds_offset(lrow + 64 * i, lchunk)) = r.w[i];
+        };
+
+        // ---- consumer ------------------------------------------------------------------------
+        v16i acc[WM][WN];
+        auto clear = [&]() {
+#pragma unroll
+            for (int mi = 0; mi < WM; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < WN; ++ni)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        acc[mi][ni][r] = 0;
+        };
+        auto compute = [&](int buf) {
+            const uint8_t* xs = lds + buf * STAGE;
+            const uint8_t* ws = xs + BM * BK;
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+            {
+                v4i wf[WN], xf[WM];
+                const int chunk = ks * 2 + (lane >> 5);
+#pragma unroll
+                for (int i = 0; i < WN; ++i)
+                    wf[i] = *reinterpret_cast<const v4i*>(ws + lds_offset((wn * WN + i) * 32 + (lane & 31), chunk));
+#pragma unroll
+                for (int i = 0; i < WM; ++i)
+                    xf[i] = *reinterpret_cast<const v4i*>(xs + lds_offset((wm * WM + i) * 32 + (lane & 31), chunk));
+#pragma unroll
+                for (int mi = 0; mi < WM; ++mi)
+#pragma unroll
+                    for (int ni = 0; ni < WN; ++ni)
+                        acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ni], xf[mi], acc[mi][ni], 0, 0, 0);
+            }
+        };
+        int cj = 0, ckt = 0;
+        int64_t cm0;
+        int32_t cn0, params_n0 = -1;
+        tile_origin(0, cm0, cn0);
+        // per-channel constants of column block n0 -> LDS; callers put a barrier behind it
+        auto load_params = [&](int32_t n0) {
+            if (tid < BN)
+            {
+                const int32_t n = n0 + tid;
+                const bool ok = n < N;
+                reinterpret_cast<int32_t*>(params)[tid] = ok ? mult * wsum[n] : 0;
+                params[BN + tid] = (MODE == EPI_FUSED && epi.bias && ok) ? static_cast<float>(epi.bias[n]) : 0.0f;
+                params[2 * BN + tid] = (MODE == EPI_FUSED && epi.per_channel && ok) ? epi.scale[n] : ec.scale;
+            }
+            params_n0 = n0;
+        };
+        // requantizes the wavefront's sub-tile into its staging region and writes it out
+        auto epilogue = [&]() {
+            uint8_t* o8 = static_cast<uint8_t*>(out);
+#pragma unroll
+            for (int ni = 0; ni < WN; ++ni)
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                {
+                    const int nl = ni * 32 + 8 * g + 4 * (lane >> 5); // channel within the wavefront's 64
+                    const int nt = wn * TN + nl;                     // within the column block
+                    const v4i corr4 = *reinterpret_cast<const v4i*>(reinterpret_cast<const int32_t*>(params) + nt);
+                    const v4f bias4 = *reinterpret_cast<const v4f*>(params + BN + nt);
+                    const v4f scale4 = *reinterpret_cast<const v4f*>(params + 2 * BN + nt);
+#pragma unroll
+                    for (int mi = 0; mi < WM; ++mi)
+                    {
+                        const int row = mi * 32 + (lane & 31);
+                        float s4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                        if (has_sum)
+                        {
+                            const int64_t m = cm0 + wm * TM + row;
+                            if (m < M && cn0 + nt < N)
+                                sum4(epi.sum_in, epi.sum_t, m * N + cn0 + nt, true, s4);
+                        }
+                        int32_t v[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                        {
+                            const int32_t a = acc[mi][ni][4 * g + e] + corr4[e];
+                            v[e] = MODE == EPI_INTERP ? epi_interp<OUT_Q8>(ec, a) : epi_fused<OUT_Q8>(ec, a, bias4[e], scale4[e], has_sum, s4[e], relu);
+                        }
+                        *reinterpret_cast<uint32_t*>(ostage + row * TN + ((((nl >> 4) ^ ((row >> 2) & 3))) << 4) + (nl & 15)) = pack4(v);
+                    }
+                }
+#pragma unroll
+            for (int i = 0; i < TM * TN / 16 / 64; ++i)
+            {
+                const int id = i * 64 + lane;
+                const int row = id >> 2;
+                const int piece = id & 3;
+                const int64_t m = cm0 + wm * TM + row;
+                const int32_t n = cn0 + wn * TN + piece * 16;
+                if (m < M && n < N)
+                    *reinterpret_cast<v4i*>(o8 + m * N + n) = *reinterpret_cast<const v4i*>(ostage + row * TN + ((piece ^ ((row >> 2) & 3)) << 4));
+            }
+        };
+        // one slice: LDS buffer `buf` feeds the MFMAs, `next` (slice s+1) moves into the other
+        // buffer, `free_regs` takes the loads of slice s+2
+        auto step = [&](int s, int buf, const Regs& next, Regs& free_regs) {
+            if (s + 2 < total)
+                gload(free_regs);
+            compute(buf);
+            const bool tile_done = ++ckt == KT;
+            if (tile_done)
+            {
+                epilogue();
+                clear();
+                ckt = 0;
+                if (++cj < my_tiles)
+                    tile_origin(cj, cm0, cn0);
+            }
+            if (s + 1 < total)
+                lstore(next, buf ^ 1);
+            __syncthreads();
+            if (tile_done && cj < my_tiles && cn0 != params_n0) // uniform
+            {
+                load_params(cn0);
+                __syncthreads();
+            }
+        };
+
+        Regs r0, r1;
+        loader_tile(0);
+        gload(r0);
+        if (total > 1)
+            gload(r1);
+        load_params(cn0);
+        clear();
+        lstore(r0, 0);
+        __syncthreads();
+        for (int s = 0; s < total; s += 2)
+        {
+            step(s, 0, r1, r0);
+            if (s + 1 < total)
+                step(s + 1, 1, r0, r1);
+        }
+    }
+
     static inline bool fits_i32(int64_t v) { return v >= 0 && v < (1ll << 31); }
 
     // one instantiation = one tile shape; sets the dynamic LDS limit on first use
@@ -706,6 +998,46 @@ namespace hipq
         return check_launch(name);
     }
 
+    template <class XL, int WAVES_M, int WAVES_N, int MODE>
+    static int launch_pipe(const XL& xl,
+                           const int8_t* w,
+                           const int32_t* wsum,
+                           int64_t M,
+                           int32_t N,
+                           int32_t Kred,
+                           int x_unsigned,
+                           const ZeroPoints& zp,
+                           const Epilogue& epi,
+                           const OutMap& om,
+                           void* out,
+                           hipStream_t s,
+                           const char* name)
+    {
+        constexpr int BM = WAVES_M * 64, BN = WAVES_N * 64;
+        constexpr size_t lds_bytes = 2 * static_cast<size_t>(BM + BN) * BK + 4 * 64 * 64 + 3 * BN * sizeof(float);
+        auto kernel = igemm_pipe_kernel<XL, 2, 2, WAVES_M, WAVES_N, MODE>;
+        static bool configured[16] = {};
+        static int cus[16] = {};
+        int dev = 0;
+        HIPQ_HIP(hipGetDevice(&dev));
+        if (dev >= 0 && dev < 16 && !configured[dev])
+        {
+            HIPQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+            hipDeviceProp_t prop;
+            HIPQ_HIP(hipGetDeviceProperties(&prop, dev));
+            cus[dev] = prop.multiProcessorCount;
+            configured[dev] = true;
+        }
+        const int64_t m_tiles = (M + BM - 1) / BM;
+        const int64_t n_tiles = (N + BN - 1) / BN;
+        HIPQ_REQUIRE(fits_i32(m_tiles * n_tiles), "too many tiles");
+        const int64_t resident = static_cast<int64_t>(dev >= 0 && dev < 16 && cus[dev] > 0 ? cus[dev] : 256) * (160 * 1024 / lds_bytes);
+        const int64_t tiles = m_tiles * n_tiles;
+        const unsigned grid = static_cast<unsigned>(tiles < resident ? tiles : resident);
+        kernel<<<grid, 256, lds_bytes, s>>>(xl, w, wsum, M, Kred, x_unsigned, static_cast<int32_t>(m_tiles), static_cast<int32_t>(n_tiles), zp, epi, om, out);
+        return check_launch(name);
+    }
+
     // tile choice: narrow outputs (N <= 64) take 512 x 64 so each wavefront still owns 128 x 64
     template <class XL, bool X_ON_A, int MODE, int KIND>
     static int launch_best(const XL& xl,
@@ -722,6 +1054,13 @@ namespace hipq
                            hipStream_t s,
                            const char* name)
     {
+        // 8-bit channels-last outputs in whole 16-byte pieces: the persistent pipelined kernel
+        if (!X_ON_A && KIND == OUT_Q8 && (N & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 && getenv("HIPQ_NO_PIPE") == nullptr)
+        {
+            if (N <= 64)
+                return launch_pipe<XL, 4, 1, MODE>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+            return launch_pipe<XL, 2, 2, MODE>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+        }
         // short reductions are bound by latency, not by LDS traffic: small wavefront tiles (64 x 64)
         // take half the registers, so twice as many workgroups are resident to hide it
         if (Kred <= 512 && N > 64 && getenv("HIPQ_NO_SMALL_TILE") == nullptr)

@@ -1,0 +1,95 @@
+"""The synthetic int8 ResNet-50 (ngraph_amd/resnet50.py): every one of its 60 ops on the GPU against the
+CPU oracle on a full-size image, bit for bit, and the device-resident channels-last plan (with and
+without HIP-graph replay) against the op-by-op run."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from ngraph_amd import hipq as H
+from ngraph_amd import resnet50 as R
+
+
+class OracleProvider:
+    @staticmethod
+    def conv(d, f, x, filt, bias, sum_in, scales, sum_scale):
+        return O.quantized_convolution_fused(d, f, x, filt, bias, sum_in, scales, sum_scale)
+
+    @staticmethod
+    def pool(d, x):
+        return O.pool(d, x)
+
+    @staticmethod
+    def dot_bias(d, f, a, w, bias, scales):
+        return O.quantized_dot_bias(d, f, a, w, bias, scales)
+
+
+def test_layer_list_is_resnet50():
+    ops = R.layers()
+    convs = [o for o in ops if o["op"] == "conv"]
+    assert len(convs) == 53 and sum(o["op"] == "fc" for o in ops) == 1
+    assert sum(o["R"] == 3 for o in convs) == 16 and sum(o["R"] == 7 for o in convs) == 1
+    names = {"input"}
+    for o in ops:  # every op reads tensors that exist by then
+        assert o["src"] in names and (o.get("sum_src") is None or o["sum_src"] in names)
+        names.add(o["name"])
+    # multiply-accumulates of the convolutions at 224 x 224: the well-known ~4.1 G
+    hw, shape, macs = 224, {"input": (3, 224)}, 0
+    for o in ops:
+        c, h = shape[o["src"]]
+        if o["op"] == "conv":
+            ho = R.out_hw(h, o["R"], o["stride"], o["pad"])
+            macs += o["K"] * o["C"] * o["R"] ** 2 * ho * ho
+            shape[o["name"]] = (o["K"], ho)
+        elif o["op"] in ("maxpool", "avgpool"):
+            shape[o["name"]] = (c, R.out_hw(h, o["window"], o["stride"], o["pad"]))
+        else:
+            shape[o["name"]] = (c, h)
+    assert shape["pool5"] == (2048, 1)
+    assert 4.0e9 < macs < 4.2e9
+
+
+@pytest.mark.gpu
+def test_resnet50_every_op_against_oracle(gpu_lib):
+    images = R.synthetic_images(1)
+    O.port().orc_set_threads(8)
+    print("[case] resnet50 oracle", flush=True)
+    exp = R.run(OracleProvider, images)
+    O.port().orc_set_threads(1)
+    print("[case] resnet50 gpu", flush=True)
+    got = R.run(R.HipProvider, images)
+    for op in R.layers():
+        a, b = got[op["name"]], exp[op["name"]]
+        assert a.dtype == b.dtype and a.shape == b.shape, op["name"]
+        assert np.array_equal(a, b), op["name"]
+    # the network is alive to the end: the last block still uses the 8-bit range, the logits differ
+    last = exp["s5_b2_out"]
+    assert 0.2 < np.count_nonzero(last) / last.size and (last == 255).mean() < 0.2
+    assert np.unique(exp["logits"]).size > 900
+
+
+@pytest.mark.gpu
+def test_resnet50_device_plan_and_graph_replay(gpu_lib):
+    lib = gpu_lib
+    N = 2
+    images = R.synthetic_images(N, seed=7)
+    ref = R.run(R.HipProvider, images)  # op by op, NCHW
+    sp = C.c_void_p()
+    H.check(lib.hipq_stream_create(C.byref(sp)))
+    plan = R.DevicePlan(lib, sp.value, N)
+    plan.set_images_nchw(images)
+    print("[case] resnet50 plan launch", flush=True)
+    plan.launch()
+    assert np.array_equal(plan.read_logits(), ref["logits"])
+    assert np.array_equal(plan.read("s3_b0_out", 512, 28), ref["s3_b0_out"])
+    print("[case] resnet50 plan capture", flush=True)
+    plan.capture()
+    for seed in (8, 9, 10):  # new images before every replay, an eager op-by-op run in between
+        images = R.synthetic_images(N, seed=seed)
+        ref = R.run(R.HipProvider, images)
+        plan.set_images_nchw(images)
+        plan.replay()
+        assert np.array_equal(plan.read_logits(), ref["logits"]), seed
+    H.check(lib.hipq_graph_destroy(plan.graph))
+    H.check(lib.hipq_stream_destroy(sp.value))

@@ -240,5 +240,6 @@ namespace hipq
     int launch_transpose(const void* in, void* out, int64_t N, int64_t R, int64_t Cc, int elem_bytes, hipStream_t s);
     int launch_pad_channels(const void* in, void* out, int64_t N, int64_t X, int64_t Cc, bool in_ncx, const void* zp, int zp_t, hipStream_t s);
     bool conv_pad_eligible(const ConvGeom& g, ConvGeom* padded);
+    int launch_im2col_nxc(const ConvGeom& g, const void* x_nxc, void* a, const void* zp, int zp_t, hipStream_t s);
     int launch_row_sums_i8(const void* w, int64_t rows, int64_t cols, int32_t* sums, hipStream_t s);
 }

@@ -203,6 +203,49 @@ namespace hipq
         return check_launch("pad_channels");
     }
 
+    // Channels-last data -> the [M][taps * C] matrix of a convolution's receptive fields (M = images x
+    // output pixels), 16 bytes a lane; taps in the padding hold the data zero point, which
+    // contributes nothing.  Only for the few-row case (M <= 256), where the matrix is small and the
+    // weight-streaming GEMM kernels beat the tiled ones by far.
+    __global__ __launch_bounds__(256) void im2col_nxc_kernel(const uint8_t* __restrict__ x, uint8_t* __restrict__ a, ConvGeom g, int32_t M, int32_t chunks_per_row, const void* zp, int32_t zp_t)
+    {
+        const int32_t i = static_cast<int32_t>(blockIdx.x) * 256 + threadIdx.x;
+        if (i >= M * chunks_per_row)
+            return;
+        const int32_t m = i / chunks_per_row;
+        const int32_t kbyte = (i - m * chunks_per_row) * 16;
+        const int32_t Cc = static_cast<int32_t>(g.C), S = static_cast<int32_t>(g.f[2]);
+        const int32_t tap = kbyte / Cc, c = kbyte - tap * Cc;
+        const int32_t r = tap / S, s = tap - r * S;
+        const int32_t PQ = static_cast<int32_t>(g.out[1] * g.out[2]), Q = static_cast<int32_t>(g.out[2]);
+        const int32_t n = m / PQ, rem = m - n * PQ;
+        const int32_t p = rem / Q, q = rem - p * Q;
+        const int32_t iy = p * static_cast<int32_t>(g.st[1]) - static_cast<int32_t>(g.pb[1]) + r * static_cast<int32_t>(g.dl[1]);
+        const int32_t ix = q * static_cast<int32_t>(g.st[2]) - static_cast<int32_t>(g.pb[2]) + s * static_cast<int32_t>(g.dl[2]);
+        uint4 v;
+        if (static_cast<uint32_t>(iy) < static_cast<uint32_t>(g.in[1]) && static_cast<uint32_t>(ix) < static_cast<uint32_t>(g.in[2]))
+            v = *reinterpret_cast<const uint4*>(x + ((static_cast<int64_t>(n) * g.in[1] + iy) * g.in[2] + ix) * Cc + c);
+        else
+        {
+            const uint32_t fill = (static_cast<uint32_t>(load_zp(zp, zp_t)) & 0xffu) * 0x01010101u;
+            v = make_uint4(fill, fill, fill, fill);
+        }
+        reinterpret_cast<uint4*>(a)[i] = v;
+    }
+
+    int launch_im2col_nxc(const ConvGeom& g, const void* x_nxc, void* a, const void* zp, int zp_t, hipStream_t s)
+    {
+        const int64_t M = g.N * g.out[1] * g.out[2];
+        const int64_t kred = g.C * g.taps();
+        HIPQ_REQUIRE(g.C % 16 == 0 && M * kred < (1ll << 31), "im2col takes multiples of 16 channels and matrices below 2 GiB");
+        const int64_t lanes = M * (kred / 16);
+        if (lanes == 0)
+            return HIPQ_OK;
+        im2col_nxc_kernel<<<static_cast<unsigned>((lanes + 255) / 256), 256, 0, s>>>(static_cast<const uint8_t*>(x_nxc), static_cast<uint8_t*>(a), g, static_cast<int32_t>(M),
+                                                                                  static_cast<int32_t>(kred / 16), zp, zp_t);
+        return check_launch("im2col_nxc");
+    }
+
     // Fewer than 16 input channels (a network's first layer): the MFMA kernels take the layer with the
     // channels padded to 16 -- zero weights in the packed filter, a padded copy of the data
     bool conv_pad_eligible(const ConvGeom& g, ConvGeom* padded)

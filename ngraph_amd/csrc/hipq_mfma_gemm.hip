@@ -34,8 +34,11 @@ namespace hipq
                 if (m < M)
                 {
                     const int32_t a = acc_of(i);
-                    const int32_t v = MODE == EPI_INTERP ? epi_interp<KIND>(ec, a) : epi_fused<KIND>(ec, a, bias, scale, false, 0.0f, relu);
                     const int64_t o = static_cast<int64_t>(m) * N + n;
+                    // (a convolution routed here may carry a residual sum input, indexed like the output)
+                    const bool has_sum = MODE == EPI_FUSED && epi.sum_in != nullptr;
+                    const float sv = has_sum ? static_cast<float>(load_q(epi.sum_in, epi.sum_t, o)) : 0.0f;
+                    const int32_t v = MODE == EPI_INTERP ? epi_interp<KIND>(ec, a) : epi_fused<KIND>(ec, a, bias, scale, has_sum, sv, relu);
                     if (KIND == OUT_Q8)
                         static_cast<uint8_t*>(out)[o] = static_cast<uint8_t>(v);
                     else

@@ -2,6 +2,8 @@
 // MFMA kernels and the direct kernels, layout conversion through the device workspace.
 #include <cstdlib>
 
+#include <cstring>
+
 #include "hipq_common.h"
 
 namespace hipq
@@ -49,21 +51,60 @@ namespace hipq
         if (!packed || !conv_mfma_eligible(g) || (epi.mode == EPI_FUSED && g.out_t == HIPQ_I32))
             return launch_conv_direct(g, data, filter, zp, epi, out, s);
 
-        // The kernel reads channels-last data; an NCHW input is transposed through the workspace.
+        // The kernels read channels-last data; an NCHW input is transposed through the workspace.
         // The output is written directly in either layout (sum_in is indexed like the output).
+        // A layer with few output pixels in all (M <= 256: the deep layers of a network at batch 1)
+        // is a skinny GEMM over its receptive-field matrix [M][taps * C] -- the data itself for a 1x1
+        // stride-1 filter, an im2col copy in the workspace otherwise -- and takes the weight-streaming
+        // GEMM kernels, which spread the filter over every CU where tiles of M would fill a few.
         const int64_t in_sp = g.in[1] * g.in[2];
         const bool tr_in = g.data_layout == HIPQ_LAYOUT_NCX && g.C > 1;
+        const int64_t M = g.N * g.out[1] * g.out[2];
+        const int64_t kred = g.C * g.taps();
+        const bool pointwise = g.taps() == 1 && g.st[1] == 1 && g.st[2] == 1 && g.pb[1] == 0 && g.pb[2] == 0 && g.out[1] == g.in[1] && g.out[2] == g.in[2];
+        const bool as_gemm = !(g.out_layout == HIPQ_LAYOUT_NCX && g.K > 1) && M <= 256 && kred % 64 == 0 && kred >= 256 && M * kred < (1ll << 31) &&
+                             g.filter_t == HIPQ_I8 && getenv("HIPQ_NO_SKINNY") == nullptr;
+        const size_t tr_bytes = tr_in ? align_up(static_cast<size_t>(g.in_count()), 256) : 0;
+        const size_t col_bytes = (as_gemm && !pointwise) ? align_up(static_cast<size_t>(M * kred), 256) : 0;
         const void* x = data;
-        if (tr_in)
+        uint8_t* ws = nullptr;
+        if (tr_bytes + col_bytes)
         {
-            void* ws = nullptr;
-            int rc = workspace(align_up(static_cast<size_t>(g.in_count()), 256), &ws);
+            void* p = nullptr;
+            int rc = workspace(tr_bytes + col_bytes, &p);
             if (rc)
                 return rc;
-            rc = launch_transpose(data, ws, g.N, g.C, in_sp, 1, s);
+            ws = static_cast<uint8_t*>(p);
+        }
+        if (tr_in)
+        {
+            int rc = launch_transpose(data, ws, g.N, g.C, in_sp, 1, s);
             if (rc)
                 return rc;
             x = ws;
+        }
+        if (as_gemm)
+        {
+            if (!pointwise)
+            {
+                int rc = launch_im2col_nxc(g, x, ws + tr_bytes, zp.data_zp, zp.data_t, s);
+                if (rc)
+                    return rc;
+                x = ws + tr_bytes;
+            }
+            hipq_dot_desc_t dd;
+            memset(&dd, 0, sizeof(dd));
+            dd.a_t = g.data_t;
+            dd.b_t = g.filter_t;
+            dd.out_t = g.out_t;
+            dd.M = M;
+            dd.K = kred;
+            dd.N = g.K;
+            if (dot_mfma_eligible(dd))
+            {
+                const int32_t* wsum = reinterpret_cast<const int32_t*>(static_cast<const uint8_t*>(packed) + align_up(static_cast<size_t>(g.K * kred), 256));
+                return launch_dot_mfma(dd, x, packed, wsum, zp, epi, out, s);
+            }
         }
         const bool out_ncx = g.out_layout == HIPQ_LAYOUT_NCX && g.K > 1;
         // layers whose filter fits in LDS take the band kernel (HIPQ_NO_BAND=1 forces the generic one)

@@ -193,7 +193,7 @@ def test_conv_reference_vectors(gpu_lib, ref_vectors):
         dl = cases.conv_from_manifest(m, H.NXC, H.NXC)[0]
         for name, got, kern in _conv_both(dl, cases.to_nxc(data), filt, s, z):
             assert np.array_equal(cases.to_ncx(got), arrays[m["name"]]), (m["name"], name, "nxc")
-    assert "conv_direct" in used and any(k.startswith("conv_mfma") for k in used), used
+    assert "conv_direct" in used and any(k.startswith(("conv_mfma", "dot_skinny")) for k in used), used
 
 
 MFMA_SHAPES = [
@@ -225,7 +225,7 @@ def test_conv_mfma_shapes(gpu_lib, i):
         exp = O.quantized_convolution(d, data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
         O.port().orc_set_threads(1)
         got = H.quantized_convolution(d, data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
-        assert H.last_kernel().startswith(("conv_mfma", "conv_band")), H.last_kernel()
+        assert H.last_kernel().startswith(("conv_mfma", "conv_band", "dot_skinny")), H.last_kernel()
         assert np.array_equal(got, exp), (out_t, z)
     # reference layouts in and out (transposed through the workspace)
     d = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t="i8", **kw)
@@ -234,7 +234,7 @@ def test_conv_mfma_shapes(gpu_lib, i):
     exp = O.quantized_convolution(d, data, filt, 0.02, 0, 0.005, 0, 0.9, 0)
     O.port().orc_set_threads(1)
     got = H.quantized_convolution(d, data, filt, 0.02, 0, 0.005, 0, 0.9, 0)
-    assert H.last_kernel().startswith(("conv_mfma", "conv_band")), H.last_kernel()
+    assert H.last_kernel().startswith(("conv_mfma", "conv_band", "dot_skinny")), H.last_kernel()
     assert np.array_equal(got, exp)
 
 
@@ -275,7 +275,7 @@ def test_conv_linearity_at_config1_batch(gpu_lib):
     a = H.quantized_convolution(d, data, f1, 1.0, 0, 1.0, 0, 1.0, 0).astype(np.int64)
     b = H.quantized_convolution(d, data, f2, 1.0, 0, 1.0, 0, 1.0, 0).astype(np.int64)
     c = H.quantized_convolution(d, data, (f1 + f2).astype(np.int8), 1.0, 0, 1.0, 0, 1.0, 0).astype(np.int64)
-    assert H.last_kernel().startswith(("conv_mfma", "conv_band"))
+    assert H.last_kernel().startswith(("conv_mfma", "conv_band", "dot_skinny"))
     assert np.array_equal(a + b, c)
     d1 = H.make_conv_desc(1, 64, 64, (56, 56), (3, 3), **kw)
     O.port().orc_set_threads(8)
@@ -419,6 +419,52 @@ def test_conv_band(gpu_lib, i):
             assert np.array_equal(got, exp), (dl, ol, relu, has_sum, per_channel, H.last_kernel())
     O.port().orc_set_threads(1)
     assert any(k.startswith("conv_band") for k in kernels), kernels
+
+
+SKINNY_CONV_SHAPES = [
+    # N, C, K, in_sp, f_sp, kw : at most 256 output pixels in all and a reduction of whole 64-byte steps
+    (1, 256, 64, (14, 14), (1, 1), dict()),                                                  # the data is the matrix
+    (1, 512, 512, (7, 7), (3, 3), dict(pad_below=(1, 1), pad_above=(1, 1))),                 # im2col, padding taps
+    (2, 64, 96, (12, 12), (3, 3), dict(stride=(2, 2), pad_below=(1, 1), pad_above=(0, 1))),  # stride, ragged K
+    (1, 128, 40, (9, 11), (2, 2), dict(dilation=(2, 1), pad_below=(1, 0), pad_above=(1, 0))),
+    (3, 256, 1000, (1, 1), (1, 1), dict()),                                                  # a classifier as a convolution
+]
+
+
+@pytest.mark.parametrize("i", range(len(SKINNY_CONV_SHAPES)))
+def test_conv_as_skinny_gemm(gpu_lib, i):
+    """layers with few output pixels run as a GEMM over their receptive-field matrix on the
+    weight-streaming kernels: both policies, zero points (padding holds the data zero point; a filter
+    zero point takes the exact path), reference-layout input (transposed, then gathered), residual sum"""
+    N, Cc, K, in_sp, f_sp, kw = SKINNY_CONV_SHAPES[i]
+    say("skinny conv", SKINNY_CONV_SHAPES[i])
+    O.port().orc_set_threads(8)
+    for dl in (H.NXC, H.NCX):
+        for out_t, z in (("i8", (0, 0, -3)), ("u8", (131, 0, 7)), ("i32", (3, 0, 0)), ("i8", (9, -7, 1))):
+            d = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t=out_t, data_layout=dl, out_layout=H.NXC, **kw)
+            dn = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t=out_t, **kw)
+            data = synth.uniform_int(1100 + i, dn.data_shape(), 0, 255, np.uint8)
+            filt = synth.uniform_int(1200 + i, dn.filter_shape(), -128, 127, np.int8)
+            s = (1.0, 1.0, 1.0) if out_t == "i32" else (0.02, 0.005, 0.9)
+            exp = O.quantized_convolution(dn, data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
+            got = H.quantized_convolution(d, cases.to_nxc(data) if dl == H.NXC else data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
+            assert H.last_kernel().startswith("dot_skinny"), H.last_kernel()
+            assert np.array_equal(cases.to_ncx(got), exp), (dl, out_t, z)
+        for relu, has_sum in ((True, True), (False, False)):
+            out_t = "u8" if relu else "i8"
+            d = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t=out_t, data_layout=dl, out_layout=H.NXC, **kw)
+            dn = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t=out_t, **kw)
+            data = synth.uniform_int(1300 + i, dn.data_shape(), 0, 255, np.uint8)
+            filt = synth.uniform_int(1400 + i, dn.filter_shape(), -127, 127, np.int8)
+            bias = synth.uniform_int(1500, (K,), -20000, 20000, np.int32)
+            scales = synth.uniform_f32(1501, (K,), 2e-4, 9e-4)
+            summ = synth.uniform_int(1502, dn.out_shape(), 0, 255, np.uint8) if has_sum else None
+            f = H.make_fused_desc(has_bias=True, has_sum=has_sum, sum_t="u8", with_relu=relu, scale_count=K)
+            exp = O.quantized_convolution_fused(dn, f, data, filt, bias, summ, scales, 0.37 if has_sum else None)
+            got = H.quantized_convolution_fused(d, f, cases.to_nxc(data) if dl == H.NXC else data, filt, bias, cases.to_nxc(summ) if has_sum else None, scales, 0.37 if has_sum else None)
+            assert H.last_kernel().startswith("dot_skinny"), H.last_kernel()
+            assert np.array_equal(cases.to_ncx(got), exp), (dl, relu, has_sum)
+    O.port().orc_set_threads(1)
 
 
 @pytest.mark.parametrize("Cc", [1, 3, 4, 15])

@@ -205,7 +205,7 @@ namespace hipq
 
     // Channels-last data -> the [M][taps * C] matrix of a convolution's receptive fields (M = images x
     // output pixels), 16 bytes a lane; taps in the padding hold the data zero point, which
-    // contributes nothing.  Only for the few-row case (M <= 256), where the matrix is small and the
+    // contributes nothing.  Only for the few-row case (M <= 64), where the matrix is small and the
     // weight-streaming GEMM kernels beat the tiled ones by far.
     __global__ __launch_bounds__(256) void im2col_nxc_kernel(const uint8_t* __restrict__ x, uint8_t* __restrict__ a, ConvGeom g, int32_t M, int32_t chunks_per_row, const void* zp, int32_t zp_t)
     {

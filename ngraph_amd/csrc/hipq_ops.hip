@@ -53,7 +53,7 @@ namespace hipq
 
         // The kernels read channels-last data; an NCHW input is transposed through the workspace.
         // The output is written directly in either layout (sum_in is indexed like the output).
-        // A layer with few output pixels in all (M <= 256: the deep layers of a network at batch 1)
+        // A layer with few output pixels in all (M <= 64: the deepest layers of a network at batch 1)
         // is a skinny GEMM over its receptive-field matrix [M][taps * C] -- the data itself for a 1x1
         // stride-1 filter, an im2col copy in the workspace otherwise -- and takes the weight-streaming
         // GEMM kernels, which spread the filter over every CU where tiles of M would fill a few.
@@ -62,7 +62,7 @@ namespace hipq
         const int64_t M = g.N * g.out[1] * g.out[2];
         const int64_t kred = g.C * g.taps();
         const bool pointwise = g.taps() == 1 && g.st[1] == 1 && g.st[2] == 1 && g.pb[1] == 0 && g.pb[2] == 0 && g.out[1] == g.in[1] && g.out[2] == g.in[2];
-        const bool as_gemm = !(g.out_layout == HIPQ_LAYOUT_NCX && g.K > 1) && M <= 256 && kred % 64 == 0 && kred >= 256 && M * kred < (1ll << 31) &&
+        const bool as_gemm = !(g.out_layout == HIPQ_LAYOUT_NCX && g.K > 1) && M <= 64 && kred % 64 == 0 && kred >= 256 && M * kred < (1ll << 31) &&
                              g.filter_t == HIPQ_I8 && getenv("HIPQ_NO_SKINNY") == nullptr;
         const size_t tr_bytes = tr_in ? align_up(static_cast<size_t>(g.in_count()), 256) : 0;
         const size_t col_bytes = (as_gemm && !pointwise) ? align_up(static_cast<size_t>(M * kred), 256) : 0;

@@ -422,11 +422,11 @@ def test_conv_band(gpu_lib, i):
 
 
 SKINNY_CONV_SHAPES = [
-    # N, C, K, in_sp, f_sp, kw : at most 256 output pixels in all and a reduction of whole 64-byte steps
-    (1, 256, 64, (14, 14), (1, 1), dict()),                                                  # the data is the matrix
+    # N, C, K, in_sp, f_sp, kw : at most 64 output pixels in all and a reduction of whole 64-byte steps
+    (1, 256, 64, (8, 7), (1, 1), dict()),                                                    # the data is the matrix
     (1, 512, 512, (7, 7), (3, 3), dict(pad_below=(1, 1), pad_above=(1, 1))),                 # im2col, padding taps
-    (2, 64, 96, (12, 12), (3, 3), dict(stride=(2, 2), pad_below=(1, 1), pad_above=(0, 1))),  # stride, ragged K
-    (1, 128, 40, (9, 11), (2, 2), dict(dilation=(2, 1), pad_below=(1, 0), pad_above=(1, 0))),
+    (1, 64, 96, (12, 12), (3, 3), dict(stride=(2, 2), pad_below=(1, 1), pad_above=(0, 1))),  # stride, ragged K
+    (1, 128, 40, (7, 8), (2, 2), dict(dilation=(2, 1), pad_below=(1, 0), pad_above=(1, 0))),
     (3, 256, 1000, (1, 1), (1, 1), dict()),                                                  # a classifier as a convolution
 ]
 

@@ -77,8 +77,10 @@ def test_packed_sizes_and_eligibility():
     lib = H.load()
     d = H.make_conv_desc(1, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1))
     assert lib.hipq_conv_packed_filter_bytes(C.byref(d)) == 64 * 64 * 9 + 64 * 4
-    d3 = H.make_conv_desc(1, 3, 64, (224, 224), (7, 7))  # C not a multiple of 16: direct kernel
-    assert lib.hipq_conv_packed_filter_bytes(C.byref(d3)) == 0
+    d3 = H.make_conv_desc(1, 3, 64, (224, 224), (7, 7))  # fewer than 16 channels: packed with the channels padded to 16
+    assert lib.hipq_conv_packed_filter_bytes(C.byref(d3)) == 64 * 16 * 49 + 64 * 4
+    d40 = H.make_conv_desc(1, 40, 64, (8, 8), (3, 3))  # 16 or more channels, not a multiple of 16: direct kernel
+    assert lib.hipq_conv_packed_filter_bytes(C.byref(d40)) == 0
     du = H.make_conv_desc(1, 64, 64, (8, 8), (1, 1), filter_t="u8", out_t="u8")
     assert lib.hipq_conv_packed_filter_bytes(C.byref(du)) == 0
     dd = H.make_dot_desc(32, 4096, 4096, b_layout=H.B_NK)

@@ -876,6 +876,26 @@ namespace hipq
         // requantizes the wavefront's sub-tile into its staging region and writes it out
         auto epilogue = [&]() {
             uint8_t* o8 = static_cast<uint8_t*>(out);
+            if (has_sum)
+            {
+                // the residual input of the sub-tile comes in the way the output leaves: 16 bytes a
+                // lane along the rows, through the staging region (each lane then picks up the dword
+                // that its own output dword will replace)
+                const uint8_t* s8 = static_cast<const uint8_t*>(epi.sum_in);
+#pragma unroll
+                for (int i = 0; i < TM * TN / 16 / 64; ++i)
+                {
+                    const int id = i * 64 + lane;
+                    const int row = id >> 2;
+                    const int piece = id & 3;
+                    const int64_t m = cm0 + wm * TM + row;
+                    const int32_t n = cn0 + wn * TN + piece * 16;
+                    v4i v = {0, 0, 0, 0};
+                    if (m < M && n < N)
+                        v = *reinterpret_cast<const v4i*>(s8 + m * N + n);
+                    *reinterpret_cast<v4i*>(ostage + row * TN + ((piece ^ ((row >> 2) & 3)) << 4)) = v;
+                }
+            }
 #pragma unroll
             for (int ni = 0; ni < WN; ++ni)
 #pragma unroll
@@ -890,12 +910,17 @@ namespace hipq
                     for (int mi = 0; mi < WM; ++mi)
                     {
                         const int row = mi * 32 + (lane & 31);
+                        uint32_t* const cell = reinterpret_cast<uint32_t*>(ostage + row * TN + ((((nl >> 4) ^ ((row >> 2) & 3))) << 4) + (nl & 15));
                         float s4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
                         if (has_sum)
                         {
-                            const int64_t m = cm0 + wm * TM + row;
-                            if (m < M && cn0 + nt < N)
-                                sum4(epi.sum_in, epi.sum_t, m * N + cn0 + nt, true, s4);
+                            const uint32_t sw = *cell;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                            {
+                                const uint32_t b = (sw >> (8 * e)) & 0xFFu;
+                                s4[e] = epi.sum_t == HIPQ_I8 ? static_cast<float>(static_cast<int8_t>(b)) : static_cast<float>(b);
+                            }
                         }
                         int32_t v[4];
 #pragma unroll
@@ -904,7 +929,7 @@ namespace hipq
                             const int32_t a = acc[mi][ni][4 * g + e] + corr4[e];
                             v[e] = MODE == EPI_INTERP ? epi_interp<OUT_Q8>(ec, a) : epi_fused<OUT_Q8>(ec, a, bias4[e], scale4[e], has_sum, s4[e], relu);
                         }
-                        *reinterpret_cast<uint32_t*>(ostage + row * TN + ((((nl >> 4) ^ ((row >> 2) & 3))) << 4) + (nl & 15)) = pack4(v);
+                        *cell = pack4(v);
                     }
                 }
 #pragma unroll

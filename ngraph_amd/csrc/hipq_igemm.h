@@ -874,6 +874,11 @@ namespace hipq
             params_n0 = n0;
         };
         // requantizes the wavefront's sub-tile into its staging region and writes it out
+        const float clamp_lo = fmaxf(ec.lo, ec.relu_floor);
+        const float s256 = __fmul_rn(ec.scale, 256.0f);
+        const int32_t c256 = 128 + 256 * ec.ozp;
+        // the fixed-point form needs |acc * scale| * 256 < 2^31 with room to spare
+        const bool fast_interp = fabsf(ec.scale) * (static_cast<float>(Kred) * (255.0f * 128.0f)) < 4194304.0f;
         auto epilogue = [&]() {
             uint8_t* o8 = static_cast<uint8_t*>(out);
             if (has_sum)
@@ -922,14 +927,32 @@ namespace hipq
                                 s4[e] = epi.sum_t == HIPQ_I8 ? static_cast<float>(static_cast<int8_t>(b)) : static_cast<float>(b);
                             }
                         }
-                        int32_t v[4];
+                        // the output byte ends up in byte BYTE of x[e]: fused policy -- clamp (the ReLU is
+                        // the clamp's lower bound), then 1.5 * 2^23 + v rounds half to even into the low
+                        // mantissa bits; INTERPRETER policy in fixed point -- t = trunc(256 v), and
+                        // round-half-away(v) = (t + 128 - (t < 0)) >> 8 exactly
+                        int32_t x[4];
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
                         {
                             const int32_t a = acc[mi][ni][4 * g + e] + corr4[e];
-                            v[e] = MODE == EPI_INTERP ? epi_interp<OUT_Q8>(ec, a) : epi_fused<OUT_Q8>(ec, a, bias4[e], scale4[e], has_sum, s4[e], relu);
+                            if (MODE == EPI_FUSED)
+                            {
+                                float v = __fmul_rn(__fadd_rn(static_cast<float>(a), bias4[e]), scale4[e]);
+                                if (has_sum)
+                                    v = fmaf(ec.sum_scale, s4[e], v);
+                                x[e] = __float_as_int(__fadd_rn(__builtin_amdgcn_fmed3f(v, clamp_lo, ec.hi), 12582912.0f));
+                            }
+                            else if (fast_interp)
+                            {
+                                const int32_t t = static_cast<int32_t>(__fmul_rn(static_cast<float>(a), s256));
+                                x[e] = t + (t >> 31) + c256;
+                            }
+                            else
+                                x[e] = epi_interp<OUT_Q8>(ec, a) << 8;
                         }
-                        *cell = pack4(v);
+                        const uint32_t sel = MODE == EPI_FUSED ? 0x0c0c0400u : 0x0c0c0501u;
+                        *cell = (__builtin_amdgcn_perm(x[3], x[2], sel) << 16) | __builtin_amdgcn_perm(x[1], x[0], sel);
                     }
                 }
 #pragma unroll

@@ -9,6 +9,8 @@ oracle/_ref has been built (`make -C oracle ref`).  The committed outputs are da
   qlinearconv{2d,3d}_{x,y}.bin    the byte fixtures of test/files/onnx/qlinearconv{2d,3d}/
   pool_vectors.npz + .json        outputs of the compiled reference max_pool / avg_pool (oracle/_ref)
                                   on seeded synthetic inputs (`--pool-only` writes just these)
+  resnet50_logits.npz / .json     the synthetic int8 ResNet-50's logits and per-op byte sums on one seeded
+                                  image, from the C restatement (`--resnet-only` writes just these)
   ref_vectors.npz + .json         outputs of the compiled reference kernels (oracle/_ref) on seeded
                                   synthetic inputs; inputs are regenerated from the seed by
                                   ngraph_amd.synth (or stored, where they are floating point)
@@ -261,7 +263,33 @@ def pool_vectors():
     print("pool_vectors:", len(manifest), "cases")
 
 
+def resnet50_vectors():
+    """The synthetic int8 ResNet-50 of ngraph_amd/resnet50.py on one seeded image, computed by the C
+    restatement in oracle/ (the fused quantized ops it is made of exist only in the reference's CPU
+    backend, which cannot be built here; the restatement of those ops is pinned on the reference's own
+    test values).  Kept: the logits and a checksum of every op's output."""
+    import oracle_lib as O
+    from ngraph_amd import resnet50 as R
+
+    class Oracle:
+        conv = staticmethod(lambda d, f, x, filt, bias, s, sc, ss: O.quantized_convolution_fused(d, f, x, filt, bias, s, sc, ss))
+        pool = staticmethod(lambda d, x: O.pool(d, x))
+        dot_bias = staticmethod(lambda d, f, a, w, bias, sc: O.quantized_dot_bias(d, f, a, w, bias, sc))
+
+    O.port().orc_set_threads(8)
+    t = R.run(Oracle, R.synthetic_images(1))
+    O.port().orc_set_threads(1)
+    sums = {op["name"]: int(t[op["name"]].view(np.uint8).astype(np.uint64).sum()) for op in R.layers()}
+    np.savez_compressed(os.path.join(HERE, "resnet50_logits.npz"), logits=t["logits"])
+    with open(os.path.join(HERE, "resnet50_logits.json"), "w") as f:
+        json.dump(dict(image_seed=42, byte_sums=sums, logits=[float(v) for v in t["logits"].ravel()]), f, indent=0)
+    print("resnet50_logits: 1000 logits,", len(sums), "byte sums")
+
+
 if __name__ == "__main__":
+    if "--resnet-only" in sys.argv:
+        resnet50_vectors()
+        sys.exit(0)
     if "--pool-only" not in sys.argv:
         parse_quantize_dequantize()
         copy_onnx_bins()

@@ -50,6 +50,27 @@ def test_layer_list_is_resnet50():
     assert 4.0e9 < macs < 4.2e9
 
 
+def _golden():
+    import json
+    import os
+
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    with open(os.path.join(here, "resnet50_logits.json")) as f:
+        meta = json.load(f)
+    return meta, np.load(os.path.join(here, "resnet50_logits.npz"))["logits"]
+
+
+def test_oracle_reproduces_committed_logits():
+    """the committed fixture (which the C++ backend test also uses) is what the restatement computes today"""
+    meta, logits = _golden()
+    O.port().orc_set_threads(8)
+    t = R.run(OracleProvider, R.synthetic_images(1, seed=meta["image_seed"]))
+    O.port().orc_set_threads(1)
+    assert np.array_equal(t["logits"], logits)
+    for name, total in meta["byte_sums"].items():
+        assert int(t[name].view(np.uint8).astype(np.uint64).sum()) == total, name
+
+
 @pytest.mark.gpu
 def test_resnet50_every_op_against_oracle(gpu_lib):
     images = R.synthetic_images(1)
@@ -67,6 +88,7 @@ def test_resnet50_every_op_against_oracle(gpu_lib):
     last = exp["s5_b2_out"]
     assert 0.2 < np.count_nonzero(last) / last.size and (last == 255).mean() < 0.2
     assert np.unique(exp["logits"]).size > 900
+    assert np.array_equal(got["logits"], _golden()[1])
 
 
 @pytest.mark.gpu

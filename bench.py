@@ -235,7 +235,7 @@ def cpu_baseline(seconds=12.0):
         el = time.perf_counter() - t0
         if el >= seconds or calls >= 200:
             break
-    return dict(
+    out = dict(
         value=d.ops() * calls / el / 1e12,
         unit="TOP/s",
         cores=1,
@@ -243,6 +243,26 @@ def cpu_baseline(seconds=12.0):
         sample="%d calls of QuantizedConvolution u8[1,64,56,56] x i8[64,64,3,3] -> i8 (config 1, N=1), %.1f s, %s"
         % (calls, el, "runtime::reference::convolution compiled from the nGraph tree" if kind == "reference" else "C restatement of it"),
     )
+    # the synthetic ResNet-50 on the host: one image through the C restatement of its ops (the fused
+    # ops exist only in the reference's CPU backend, which does not build here), all of this box's share of cores
+    try:
+        from ngraph_amd import resnet50 as R
+
+        class Port:
+            conv = staticmethod(lambda d, f, x, filt, bias, s, sc, ss: O.quantized_convolution_fused(d, f, x, filt, bias, s, sc, ss))
+            pool = staticmethod(lambda d, x: O.pool(d, x))
+            dot_bias = staticmethod(lambda d, f, a, w, bias, sc: O.quantized_dot_bias(d, f, a, w, bias, sc))
+
+        threads = 16
+        O.port().orc_set_threads(threads)
+        t0 = time.perf_counter()
+        R.run(Port, R.synthetic_images(1))
+        el = time.perf_counter() - t0
+        O.port().orc_set_threads(1)
+        out["resnet50_int8"] = dict(value=1.0 / el, unit="images/s", cores=threads, kind="port", sample="1 image, %.1f s" % el)
+    except Exception as e:  # the baseline is informative: never fail the bench over it
+        out["resnet50_int8"] = dict(error=str(e))
+    return out
 
 
 def main():
@@ -252,6 +272,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--batch", type=int, default=128)
     ap.add_argument("--quick", action="store_true", help="headline workload only, no CPU baseline")
+    ap.add_argument("--resnet-only", action="store_true", help="only the synthetic int8 ResNet-50 (for profiling); prints its results")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -265,6 +286,10 @@ def main():
     H.check(lib.hipq_stream_create(C.byref(sp)))
     stream = sp.value
     timer = Timer(lib, stream)
+
+    if args.resnet_only:
+        print(json.dumps({"resnet50_int8": bench_resnet50(lib, stream, timer)}))
+        return
 
     # headline: the reference's NCHW tensors in, NCHW out
     head = bench_conv(lib, stream, timer, args.batch, args.steps, args.warmup, H.NCX)

@@ -879,26 +879,36 @@ namespace hipq
         const int32_t c256 = 128 + 256 * ec.ozp;
         // the fixed-point form needs |acc * scale| * 256 < 2^31 with room to spare
         const bool fast_interp = fabsf(ec.scale) * (static_cast<float>(Kred) * (255.0f * 128.0f)) < 4194304.0f;
+        constexpr int SUM_LOADS = TM * TN / 16 / 64;
+        v4i sum_regs[SUM_LOADS];
+        const __amdgpu_buffer_rsrc_t srs = make_rsrc(epi.sum_in, has_sum ? static_cast<uint32_t>(M * N) : 0u);
+        auto sum_fetch = [&]() {
+#pragma unroll
+            for (int i = 0; i < SUM_LOADS; ++i)
+            {
+                const int id = i * 64 + lane;
+                const int row = id >> 2;
+                const int piece = id & 3;
+                const int64_t m = cm0 + wm * TM + row;
+                const int32_t n = cn0 + wn * TN + piece * 16;
+                sum_regs[i] = buffer_load16(srs, (m < M && n < N) ? static_cast<int32_t>(m * N + n) : kOob);
+            }
+        };
         auto epilogue = [&]() {
             uint8_t* o8 = static_cast<uint8_t*>(out);
             if (has_sum)
             {
                 // the residual input of the sub-tile comes in the way the output leaves: 16 bytes a
-                // lane along the rows, through the staging region (each lane then picks up the dword
-                // that its own output dword will replace)
-                const uint8_t* s8 = static_cast<const uint8_t*>(epi.sum_in);
+                // lane along the rows (fetched into registers before the tile's last slice was
+                // multiplied), through the staging region; each lane then picks up the dword that its
+                // own output dword will replace
 #pragma unroll
-                for (int i = 0; i < TM * TN / 16 / 64; ++i)
+                for (int i = 0; i < SUM_LOADS; ++i)
                 {
                     const int id = i * 64 + lane;
                     const int row = id >> 2;
                     const int piece = id & 3;
-                    const int64_t m = cm0 + wm * TM + row;
-                    const int32_t n = cn0 + wn * TN + piece * 16;
-                    v4i v = {0, 0, 0, 0};
-                    if (m < M && n < N)
-                        v = *reinterpret_cast<const v4i*>(s8 + m * N + n);
-                    *reinterpret_cast<v4i*>(ostage + row * TN + ((piece ^ ((row >> 2) & 3)) << 4)) = v;
+                    *reinterpret_cast<v4i*>(ostage + row * TN + ((piece ^ ((row >> 2) & 3)) << 4)) = sum_regs[i];
                 }
             }
 #pragma unroll
@@ -970,6 +980,8 @@ namespace hipq
         // one slice: LDS buffer `buf` feeds the MFMAs, `next` (slice s+1) moves into the other
         // buffer, `free_regs` takes the loads of slice s+2
         auto step = [&](int s, int buf, const Regs& next, Regs& free_regs) {
+            if (has_sum && ckt + 1 == KT) // uniform
+                sum_fetch();
             if (s + 2 < total)
                 gload(free_regs);
             compute(buf);

@@ -37,6 +37,10 @@ namespace hipq
     // Grow-only device workspace, one per device, shared by every call on that device (calls that
     // need it and overlap on different streams would race; the backend serialises per executable).
     int workspace(size_t bytes, void** ptr);
+    // a second block for reductions split over workgroups: zeroed tile counters (kSplitCounterBytes of
+    // them) followed by `partial_bytes` for partial sums
+    constexpr size_t kSplitCounterBytes = 64 * 1024;
+    int split_workspace(size_t partial_bytes, uint32_t** counters, void** partials);
 
     inline size_t dtype_size(int t)
     {
@@ -236,6 +240,9 @@ namespace hipq
                         const Epilogue& epi,
                         void* out,
                         hipStream_t s);
+
+    int launch_rows_mfma(const void* a, bool a_unsigned, const int8_t* w_nk, const int32_t* wsum, int64_t M, int32_t N, int32_t K,
+                         const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s, const char* name);
 
     int launch_transpose(const void* in, void* out, int64_t N, int64_t R, int64_t Cc, int elem_bytes, hipStream_t s);
     int launch_pad_channels(const void* in, void* out, int64_t N, int64_t X, int64_t Cc, bool in_ncx, const void* zp, int zp_t, hipStream_t s);

@@ -27,6 +27,8 @@
 // Workgroup ids are remapped so that each of the 8 XCDs (which receive consecutive ids round-robin
 // and have private L2s) works on a contiguous range of m tiles.
 #pragma once
+#include <type_traits>
+
 #include "hipq_common.h"
 
 namespace hipq
@@ -60,6 +62,26 @@ namespace hipq
     __device__ __forceinline__ v4i buffer_load16(__amdgpu_buffer_rsrc_t r, int32_t off)
     {
         return __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+    }
+
+    // Division of a value below 2^31 by a divisor fixed at launch (1 <= d < 2^31), exact:
+    // with l = ceil(log2 d) and m = 2^(31 + l) / d + 1, n / d = hi32(n * m) >> (l - 1).
+    struct FastDiv
+    {
+        uint32_t m, sh; // m == 0: d == 1
+        __device__ __forceinline__ uint32_t div(uint32_t n) const { return m ? __umulhi(n, m) >> sh : n; }
+    };
+    static inline FastDiv fast_div(int64_t d)
+    {
+        FastDiv r{0u, 0u};
+        if (d <= 1)
+            return r;
+        int l = 0;
+        while ((1ll << l) < d)
+            ++l;
+        r.m = static_cast<uint32_t>((1ull << (31 + l)) / static_cast<uint64_t>(d) + 1);
+        r.sh = static_cast<uint32_t>(l - 1);
+        return r;
     }
 
     struct GemmX
@@ -103,6 +125,7 @@ namespace hipq
         int32_t H, W, C, Q, R, S, sh, sw, dh, dw, pbh, pbw;
         int64_t PQ;
         uint32_t bytes; // N * H * W * C
+        FastDiv by_pq, by_q, by_c, by_s; // by_pq.sh == 0xffffffff: more than 2^31 output pixels, plain division
 
         struct Row
         {
@@ -117,18 +140,28 @@ namespace hipq
         {
             const bool valid = m < M;
             const int64_t mm = valid ? m : 0;
-            const int64_t n = mm / PQ;
-            const int32_t rem = static_cast<int32_t>(mm - n * PQ);
-            const int32_t p = rem / Q;
+            int32_t n, rem;
+            if (by_pq.sh == 0xffffffffu) // uniform
+            {
+                const int64_t n64 = mm / PQ;
+                n = static_cast<int32_t>(n64);
+                rem = static_cast<int32_t>(mm - n64 * PQ);
+            }
+            else
+            {
+                n = static_cast<int32_t>(by_pq.div(static_cast<uint32_t>(mm)));
+                rem = static_cast<int32_t>(mm) - n * static_cast<int32_t>(PQ);
+            }
+            const int32_t p = static_cast<int32_t>(by_q.div(static_cast<uint32_t>(rem)));
             const int32_t q = rem - p * Q;
-            rw.base = valid ? static_cast<int32_t>(n) * H * W * C : kOob;
+            rw.base = valid ? n * H * W * C : kOob;
             rw.yx = ((p * sh - pbh) << 16) | ((q * sw - pbw) & 0xffff);
         }
         __device__ __forceinline__ void init_cursor(Cursor& c, int kbyte) const
         {
-            const int tap = kbyte / C;
+            const int tap = static_cast<int>(by_c.div(static_cast<uint32_t>(kbyte)));
             c.c = kbyte - tap * C;
-            c.r = tap / S;
+            c.r = static_cast<int>(by_s.div(static_cast<uint32_t>(tap)));
             c.s = tap - c.r * S;
         }
         __device__ __forceinline__ void advance(Cursor& c, int bytes_) const
@@ -671,6 +704,20 @@ namespace hipq
     }
 
 
+    // Optional clocks (development builds only): the first lane of every wavefront of workgroup 0
+    // records the shader clock at points of its first 12 slices.
+#ifdef HIPQ_PIPE_CLOCKS
+    static __device__ long long g_pipe_clock[12][4][8];
+#define HIPQ_PIPE_MARK(step, point)                                                                \
+    do                                                                                             \
+    {                                                                                              \
+        if (blockIdx.x == 0 && (threadIdx.x & 63) == 0 && (step) < 12)                              \
+            g_pipe_clock[step][threadIdx.x >> 6][point] = clock64();                                \
+    } while (0)
+#else
+#define HIPQ_PIPE_MARK(step, point) ((void)0)
+#endif
+
     // ---- persistent, software-pipelined variant ---------------------------------------------------
     // For 8-bit channels-last / row-major outputs whose rows are whole 16-byte pieces.  A workgroup
     // walks its tiles (tile = vb + j * grid) and treats all their 64-byte reduction slices as one
@@ -689,6 +736,10 @@ namespace hipq
                                                                 int32_t x_unsigned,
                                                                 int32_t m_tiles,
                                                                 int32_t n_tiles,
+                                                                int32_t split_shift,
+                                                                FastDiv by_m_tiles,
+                                                                int32_t* __restrict__ partials,
+                                                                uint32_t* __restrict__ counters,
                                                                 ZeroPoints zp,
                                                                 Epilogue epi,
                                                                 OutMap om,
@@ -714,15 +765,25 @@ namespace hipq
         const int wm = wave / WAVES_N;
         const int N = om.N;
         const int grid = static_cast<int>(gridDim.x);
-        const int total_tiles = m_tiles * n_tiles;
+        // With `splits` > 1 the reduction of every tile is cut into that many equal runs of slices,
+        // each a work item of its own (neighbouring ids: they finish together); the items of a tile
+        // leave their raw sums in `partials` and the last one to arrive adds them up and finishes.
+        const int splits = 1 << split_shift;
+        const int total_tiles = (m_tiles * n_tiles) << split_shift;
         const int vb = (grid & 7) == 0 ? (static_cast<int>(blockIdx.x) & 7) * (grid >> 3) + (static_cast<int>(blockIdx.x) >> 3) : static_cast<int>(blockIdx.x);
         if (vb >= total_tiles)
             return;
         const int my_tiles = (total_tiles - vb + grid - 1) / grid;
         // tiles of one column block are consecutive, so a workgroup rarely changes its column block
-        auto tile_origin = [&](int j, int64_t& m0, int32_t& n0) {
+        auto tile_index = [&](int j, int& tile, int& split) {
             const int t = vb + j * grid;
-            const int nt = t / m_tiles;
+            tile = t >> split_shift;
+            split = t & (splits - 1);
+        };
+        auto tile_origin = [&](int j, int64_t& m0, int32_t& n0) {
+            int t, ks;
+            tile_index(j, t, ks);
+            const int nt = static_cast<int>(by_m_tiles.div(static_cast<uint32_t>(t)));
             m0 = static_cast<int64_t>(t - nt * m_tiles) * BM;
             n0 = nt * BN;
         };
@@ -736,7 +797,10 @@ namespace hipq
                 int64_t m0;
                 int32_t n0;
                 tile_origin(j, m0, n0);
-                slow_tile(xl, w, M, Kred, x_unsigned, xzp, wzp, epi, om, out, m0, n0, BM, BN);
+                int t, ks;
+                tile_index(j, t, ks);
+                if (ks == 0)
+                    slow_tile(xl, w, M, Kred, x_unsigned, xzp, wzp, epi, om, out, m0, n0, BM, BN);
             }
             return;
         }
@@ -752,7 +816,7 @@ namespace hipq
         const int fill = (xzp & 0xFF) * 0x01010101;
         const __amdgpu_buffer_rsrc_t xrs = make_rsrc(xl.x, xl.bytes);
         const __amdgpu_buffer_rsrc_t wrs = make_rsrc(w, static_cast<uint32_t>(N) * static_cast<uint32_t>(Kred));
-        const int KT = (Kred + BK - 1) / BK;
+        const int KT = ((Kred + BK - 1) / BK) >> split_shift; // slices per work item (the launcher makes the split even)
         const int total = my_tiles * KT;
         typename XL::Row xr[XLOADS];
         typename XL::Cursor cur;
@@ -763,17 +827,20 @@ namespace hipq
             int64_t m0;
             int32_t n0;
             tile_origin(j, m0, n0);
+            int t, ks;
+            tile_index(j, t, ks);
+            const int kbyte0 = ks * KT * BK + lchunk * 16;
 #pragma unroll
             for (int i = 0; i < XLOADS; ++i)
                 xl.init_row(xr[i], m0 + lrow + 64 * i, M);
-            xl.init_cursor(cur, lchunk * 16);
+            xl.init_cursor(cur, kbyte0);
 #pragma unroll
             for (int i = 0; i < WLOADS; ++i)
             {
                 const int32_t r = lrow + 64 * i;
                 woff[i] = (n0 + r < N && r < BN) ? (n0 + r) * Kred : kOob;
             }
-            kb = lchunk * 16;
+            kb = kbyte0;
         };
         struct Regs
         {
@@ -827,16 +894,23 @@ namespace hipq
 
         // ---- consumer ------------------------------------------------------------------------
         v16i acc[WM][WN];
-        auto clear = [&]() {
+        // The accumulators start from the zero-point correction of their channels (a register row of
+        // an MFMA result is one output channel), so nothing is cleared and the epilogue adds nothing:
+        // the first slice of a tile multiplies onto `corrv`, read from the per-channel constants.
+        v16i corrv[WN];
+        auto corr_load = [&](bool zero) {
 #pragma unroll
-            for (int mi = 0; mi < WM; ++mi)
+            for (int ni = 0; ni < WN; ++ni)
 #pragma unroll
-                for (int ni = 0; ni < WN; ++ni)
+                for (int g = 0; g < 4; ++g)
+                {
+                    const v4i c4 = zero ? v4i{0, 0, 0, 0} : *reinterpret_cast<const v4i*>(reinterpret_cast<const int32_t*>(params) + wn * TN + ni * 32 + 8 * g + 4 * (lane >> 5));
 #pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        acc[mi][ni][r] = 0;
+                    for (int e = 0; e < 4; ++e)
+                        corrv[ni][4 * g + e] = c4[e];
+                }
         };
-        auto compute = [&](int buf) {
+        auto compute = [&](int buf, auto first) {
             const uint8_t* xs = lds + buf * STAGE;
             const uint8_t* ws = xs + BM * BK;
 #pragma unroll
@@ -854,7 +928,7 @@ namespace hipq
                 for (int mi = 0; mi < WM; ++mi)
 #pragma unroll
                     for (int ni = 0; ni < WN; ++ni)
-                        acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ni], xf[mi], acc[mi][ni], 0, 0, 0);
+                        acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ni], xf[mi], (decltype(first)::value && ks == 0) ? corrv[ni] : acc[mi][ni], 0, 0, 0);
             }
         };
         int cj = 0, ckt = 0;
@@ -875,6 +949,7 @@ namespace hipq
         };
         // requantizes the wavefront's sub-tile into its staging region and writes it out
         const float clamp_lo = fmaxf(ec.lo, ec.relu_floor);
+        const float magic = 12582912.0f; // 1.5 * 2^23: adding it rounds half to even into the low mantissa bits
         const float s256 = __fmul_rn(ec.scale, 256.0f);
         const int32_t c256 = 128 + 256 * ec.ozp;
         // the fixed-point form needs |acc * scale| * 256 < 2^31 with room to spare
@@ -894,7 +969,8 @@ namespace hipq
                 sum_regs[i] = buffer_load16(srs, (m < M && n < N) ? static_cast<int32_t>(m * N + n) : kOob);
             }
         };
-        auto epilogue = [&]() {
+        auto epilogue = [&](auto with_sum) {
+            constexpr bool has_sum = decltype(with_sum)::value; // (shadows the run-time flag: one copy of the code each)
             uint8_t* o8 = static_cast<uint8_t*>(out);
             if (has_sum)
             {
@@ -918,7 +994,6 @@ namespace hipq
                 {
                     const int nl = ni * 32 + 8 * g + 4 * (lane >> 5); // channel within the wavefront's 64
                     const int nt = wn * TN + nl;                     // within the column block
-                    const v4i corr4 = *reinterpret_cast<const v4i*>(reinterpret_cast<const int32_t*>(params) + nt);
                     const v4f bias4 = *reinterpret_cast<const v4f*>(params + BN + nt);
                     const v4f scale4 = *reinterpret_cast<const v4f*>(params + 2 * BN + nt);
 #pragma unroll
@@ -942,16 +1017,26 @@ namespace hipq
                         // mantissa bits; INTERPRETER policy in fixed point -- t = trunc(256 v), and
                         // round-half-away(v) = (t + 128 - (t < 0)) >> 8 exactly
                         int32_t x[4];
+                        uint32_t packed = 0;
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
                         {
-                            const int32_t a = acc[mi][ni][4 * g + e] + corr4[e];
+                            const int32_t a = acc[mi][ni][4 * g + e];
                             if (MODE == EPI_FUSED)
                             {
                                 float v = __fmul_rn(__fadd_rn(static_cast<float>(a), bias4[e]), scale4[e]);
                                 if (has_sum)
                                     v = fmaf(ec.sum_scale, s4[e], v);
-                                x[e] = __float_as_int(__fadd_rn(__builtin_amdgcn_fmed3f(v, clamp_lo, ec.hi), 12582912.0f));
+                                v = __builtin_amdgcn_fmed3f(v, clamp_lo, ec.hi);
+                                // the rounding add drops its low byte straight into byte e of the word
+                                if (e == 0)
+                                    packed = __float_as_uint(__fadd_rn(v, magic)); // the bytes above are replaced below
+                                else if (e == 1)
+                                    asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(packed) : "v"(v), "v"(magic));
+                                else if (e == 2)
+                                    asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(packed) : "v"(v), "v"(magic));
+                                else
+                                    asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(packed) : "v"(v), "v"(magic));
                             }
                             else if (fast_interp)
                             {
@@ -961,8 +1046,10 @@ namespace hipq
                             else
                                 x[e] = epi_interp<OUT_Q8>(ec, a) << 8;
                         }
-                        const uint32_t sel = MODE == EPI_FUSED ? 0x0c0c0400u : 0x0c0c0501u;
-                        *cell = (__builtin_amdgcn_perm(x[3], x[2], sel) << 16) | __builtin_amdgcn_perm(x[1], x[0], sel);
+                        if (MODE == EPI_FUSED)
+                            *cell = packed;
+                        else
+                            *cell = (__builtin_amdgcn_perm(x[3], x[2], 0x0c0c0501u) << 16) | __builtin_amdgcn_perm(x[1], x[0], 0x0c0c0501u);
                     }
                 }
 #pragma unroll
@@ -977,26 +1064,104 @@ namespace hipq
                     *reinterpret_cast<v4i*>(o8 + m * N + n) = *reinterpret_cast<const v4i*>(ostage + row * TN + ((piece ^ ((row >> 2) & 3)) << 4));
             }
         };
+        // split reductions: leaves this item's raw sums in `partials`; the last item of the tile to
+        // arrive (counted in `counters`, which it resets) adds all of them into its accumulators and
+        // returns true: it runs the epilogue.  Every wavefront of the workgroup takes the same path.
+        // The sums travel between compute dies, each with an L2 of its own: they are stored and
+        // loaded at device scope (sc1: written through to, and fetched from, the memory side), so no
+        // whole-cache write-back or invalidate is needed; the barrier in front of the counter
+        // update waits for the stores.
+        uint32_t* const arrival = reinterpret_cast<uint32_t*>(params + 3 * BN);
+        constexpr int kDeviceScope = 16; // the sc1 bit of a buffer instruction
+        auto gather_splits = [&]() {
+            int tile, ks;
+            tile_index(cj, tile, ks);
+            const __amdgpu_buffer_rsrc_t prs = make_rsrc(partials + static_cast<size_t>(tile) * splits * (BM * BN), static_cast<uint32_t>(splits) * BM * BN * 4u);
+            // register order: a wavefront's store covers 1 KiB in one piece
+            const int32_t lane_off = (wave * (WM * WN * 4) * 64 + lane) * 16;
+#pragma unroll
+            for (int mi = 0; mi < WM; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < WN; ++ni)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                        __builtin_amdgcn_raw_buffer_store_b128(v4i{acc[mi][ni][4 * g], acc[mi][ni][4 * g + 1], acc[mi][ni][4 * g + 2], acc[mi][ni][4 * g + 3]},
+                                                               prs,
+                                                               ks * (BM * BN * 4) + lane_off + ((mi * WN + ni) * 4 + g) * 1024,
+                                                               0,
+                                                               kDeviceScope);
+            __syncthreads(); // every wavefront's stores have been acknowledged
+            if (tid == 0)
+            {
+                const uint32_t seen = atomicAdd(counters + tile, 1u);
+                if (seen == static_cast<uint32_t>(splits - 1))
+                    atomicExch(counters + tile, 0u);
+                *arrival = seen;
+            }
+            __syncthreads();
+            const bool last = *arrival == static_cast<uint32_t>(splits - 1);
+            __syncthreads(); // `arrival` may be rewritten by the next tile
+            if (!last)
+                return false;
+            for (int k = 0; k < splits; ++k)
+            {
+                if (k == ks)
+                    continue;
+#pragma unroll
+                for (int mi = 0; mi < WM; ++mi)
+#pragma unroll
+                    for (int ni = 0; ni < WN; ++ni)
+#pragma unroll
+                        for (int g = 0; g < 4; ++g)
+                        {
+                            const v4i p4 = __builtin_amdgcn_raw_buffer_load_b128(prs, k * (BM * BN * 4) + lane_off + ((mi * WN + ni) * 4 + g) * 1024, 0, kDeviceScope);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                acc[mi][ni][4 * g + e] += p4[e];
+                        }
+            }
+            return true;
+        };
         // one slice: LDS buffer `buf` feeds the MFMAs, `next` (slice s+1) moves into the other
         // buffer, `free_regs` takes the loads of slice s+2
         auto step = [&](int s, int buf, const Regs& next, Regs& free_regs) {
+            HIPQ_PIPE_MARK(s, 0);
             if (has_sum && ckt + 1 == KT) // uniform
                 sum_fetch();
             if (s + 2 < total)
                 gload(free_regs);
-            compute(buf);
+            HIPQ_PIPE_MARK(s, 1);
+            if (ckt == 0) // uniform
+            {
+                int t, ks = 0;
+                if (splits > 1)
+                    tile_index(cj, t, ks);
+                corr_load(ks != 0); // the correction enters a split reduction once
+                compute(buf, std::true_type{});
+            }
+            else
+                compute(buf, std::false_type{});
+            HIPQ_PIPE_MARK(s, 2);
             const bool tile_done = ++ckt == KT;
             if (tile_done)
             {
-                epilogue();
-                clear();
+                if (splits == 1 || gather_splits()) // uniform
+                {
+                    if (has_sum)
+                        epilogue(std::true_type{});
+                    else
+                        epilogue(std::false_type{});
+                }
                 ckt = 0;
                 if (++cj < my_tiles)
                     tile_origin(cj, cm0, cn0);
             }
+            HIPQ_PIPE_MARK(s, 3);
             if (s + 1 < total)
                 lstore(next, buf ^ 1);
+            HIPQ_PIPE_MARK(s, 4);
             __syncthreads();
+            HIPQ_PIPE_MARK(s, 5);
             if (tile_done && cj < my_tiles && cn0 != params_n0) // uniform
             {
                 load_params(cn0);
@@ -1010,7 +1175,6 @@ namespace hipq
         if (total > 1)
             gload(r1);
         load_params(cn0);
-        clear();
         lstore(r0, 0);
         __syncthreads();
         for (int s = 0; s < total; s += 2)
@@ -1074,7 +1238,7 @@ namespace hipq
                            const char* name)
     {
         constexpr int BM = WAVES_M * 64, BN = WAVES_N * 64;
-        constexpr size_t lds_bytes = 2 * static_cast<size_t>(BM + BN) * BK + 4 * 64 * 64 + 3 * BN * sizeof(float);
+        constexpr size_t lds_bytes = 2 * static_cast<size_t>(BM + BN) * BK + 4 * 64 * 64 + 3 * BN * sizeof(float) + 16;
         auto kernel = igemm_pipe_kernel<XL, 2, 2, WAVES_M, WAVES_N, MODE>;
         static bool configured[16] = {};
         static int cus[16] = {};
@@ -1093,8 +1257,38 @@ namespace hipq
         HIPQ_REQUIRE(fits_i32(m_tiles * n_tiles), "too many tiles");
         const int64_t resident = static_cast<int64_t>(dev >= 0 && dev < 16 && cus[dev] > 0 ? cus[dev] : 256) * (160 * 1024 / lds_bytes);
         const int64_t tiles = m_tiles * n_tiles;
-        const unsigned grid = static_cast<unsigned>(tiles < resident ? tiles : resident);
-        kernel<<<grid, 256, lds_bytes, s>>>(xl, w, wsum, M, Kred, x_unsigned, static_cast<int32_t>(m_tiles), static_cast<int32_t>(n_tiles), zp, epi, om, out);
+        // Few tiles with long reductions leave most of the chip idle: cut every reduction into
+        // `splits` runs of whole slices (at least four each) as long as the work items still find a
+        // compute unit each.
+        int splits = 1;
+        const int64_t slices = (Kred + BK - 1) / BK;
+        const char* const split_env = getenv("HIPQ_SPLIT_K");
+        if (split_env)
+        {
+            const int want = atoi(split_env);
+            splits = want > 0 && (want & (want - 1)) == 0 && slices % want == 0 ? want : 1;
+        }
+        else
+            while (splits < 16 && tiles * splits * 2 <= (dev >= 0 && dev < 16 && cus[dev] > 0 ? cus[dev] : 256) && slices % (splits * 2) == 0 && slices / (splits * 2) >= 4)
+                splits *= 2;
+        int32_t* partials = nullptr;
+        uint32_t* counters = nullptr;
+        if (splits > 1 && tiles * sizeof(uint32_t) <= kSplitCounterBytes)
+        {
+            void* p = nullptr;
+            int rc = split_workspace(static_cast<size_t>(tiles) * splits * BM * BN * sizeof(int32_t), &counters, &p);
+            if (rc != HIPQ_OK)
+                return rc;
+            partials = static_cast<int32_t*>(p);
+        }
+        else
+            splits = 1;
+        const int64_t items = tiles * splits;
+        int split_shift = 0;
+        while ((1 << split_shift) < splits)
+            ++split_shift;
+        const unsigned grid = static_cast<unsigned>(items < resident ? items : resident);
+        kernel<<<grid, 256, lds_bytes, s>>>(xl, w, wsum, M, Kred, x_unsigned, static_cast<int32_t>(m_tiles), static_cast<int32_t>(n_tiles), split_shift, fast_div(m_tiles), partials, counters, zp, epi, om, out);
         return check_launch(name);
     }
 

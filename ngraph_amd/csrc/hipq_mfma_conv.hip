@@ -56,6 +56,12 @@ namespace hipq
         xl.PQ = g.out[1] * g.out[2];
         xl.bytes = static_cast<uint32_t>(g.in_count());
         const int64_t M = g.N * xl.PQ;
+        xl.by_pq = fast_div(xl.PQ);
+        if (M >= (1ll << 31))
+            xl.by_pq.sh = 0xffffffffu;
+        xl.by_q = fast_div(xl.Q);
+        xl.by_c = fast_div(xl.C);
+        xl.by_s = fast_div(xl.S);
         const int32_t N = static_cast<int32_t>(g.K);
         const int32_t Kred = static_cast<int32_t>(g.C * g.taps());
         const int8_t* w = static_cast<const int8_t*>(packed);
@@ -63,8 +69,19 @@ namespace hipq
             reinterpret_cast<const int32_t*>(static_cast<const uint8_t*>(packed) + align_up(static_cast<size_t>(g.K) * Kred, 256));
         OutMap om{out_ncx ? 1 : 0, N, xl.PQ};
         const int xu = g.data_t == HIPQ_U8 ? 1 : 0;
+        // a 1 x 1 filter over every pixel: the channels-last data is the [pixels][C] matrix itself
+        if (!out_ncx && g.taps() == 1 && g.st[1] == 1 && g.st[2] == 1 && g.pb[1] == 0 && g.pb[2] == 0 && g.out[1] == g.in[1] && g.out[2] == g.in[2] &&
+            g.C % 16 == 0)
+            return launch_rows_mfma(data_nxc, xu != 0, w, wsum, M, N, Kred, zp, epi, out, s, "conv_mfma_i8_32x32x32");
         if (out_ncx)
             return launch_epilogue<ConvX, true>(xl, w, wsum, M, N, Kred, xu, zp, epi, om, out, s, "conv_mfma_i8_32x32x32");
         return launch_epilogue<ConvX, false>(xl, w, wsum, M, N, Kred, xu, zp, epi, om, out, s, "conv_mfma_i8_32x32x32");
     }
 }
+
+#ifdef HIPQ_PIPE_CLOCKS
+extern "C" HIPQ_API int hipq_debug_pipe_clocks(long long* out384)
+{
+    return hipMemcpyFromSymbol(out384, HIP_SYMBOL(hipq::g_pipe_clock), sizeof(long long) * 384) == hipSuccess ? 0 : 1;
+}
+#endif

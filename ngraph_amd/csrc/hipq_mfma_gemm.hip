@@ -328,6 +328,20 @@ namespace hipq
         return check_launch("dot_skinny_wide_i8_16x16x64");
     }
 
+    // rows of `a` ([M][K] bytes) against packed weights, channels-last 8-bit or wider output: the
+    // tile kernels with the row-matrix loader (also the path of 1 x 1 convolutions, whose
+    // channels-last data is such a matrix)
+    int launch_rows_mfma(const void* a, bool a_unsigned, const int8_t* w_nk, const int32_t* wsum, int64_t M, int32_t N, int32_t K,
+                         const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s, const char* name)
+    {
+        GemmX xl;
+        xl.x = static_cast<const uint8_t*>(a);
+        xl.K = K;
+        xl.bytes = static_cast<uint32_t>(M * K);
+        OutMap om{0, N, 1};
+        return launch_epilogue<GemmX, false>(xl, w_nk, wsum, M, N, K, a_unsigned ? 1 : 0, zp, epi, om, out, s, name);
+    }
+
     bool dot_mfma_eligible(const hipq_dot_desc_t& d)
     {
         if (d.b_t != HIPQ_I8 || (d.a_t != HIPQ_U8 && d.a_t != HIPQ_I8))
@@ -364,12 +378,7 @@ namespace hipq
                 return launch_skinny_wide<8>(d, a, w_nk, wsum, zp, epi, out, s);
             return launch_skinny_wide<16>(d, a, w_nk, wsum, zp, epi, out, s);
         }
-        GemmX xl;
-        xl.x = static_cast<const uint8_t*>(a);
-        xl.K = static_cast<int32_t>(d.K);
-        xl.bytes = static_cast<uint32_t>(d.M * d.K);
-        OutMap om{0, static_cast<int32_t>(d.N), 1};
-        return launch_epilogue<GemmX, false>(xl, static_cast<const int8_t*>(w_nk), wsum, d.M, static_cast<int32_t>(d.N),
-                                         static_cast<int32_t>(d.K), d.a_t == HIPQ_U8 ? 1 : 0, zp, epi, om, out, s, "dot_mfma_i8_32x32x32");
+        return launch_rows_mfma(a, d.a_t == HIPQ_U8, static_cast<const int8_t*>(w_nk), wsum, d.M, static_cast<int32_t>(d.N), static_cast<int32_t>(d.K), zp, epi,
+                                out, s, "dot_mfma_i8_32x32x32");
     }
 }

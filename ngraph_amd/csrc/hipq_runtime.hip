@@ -60,6 +60,40 @@ namespace hipq
         return HIPQ_OK;
     }
 
+    // Second grow-only block: partial sums of reductions split over workgroups, with a counter per
+    // output tile at its head.  The counters are zeroed when the block is (re)allocated and every
+    // kernel that uses them leaves them at zero.
+    static void* g_split_ptr[kMaxDevices] = {};
+    static size_t g_split_bytes[kMaxDevices] = {};
+    int split_workspace(size_t partial_bytes, uint32_t** counters, void** partials)
+    {
+        int dev = 0;
+        HIPQ_HIP(hipGetDevice(&dev));
+        if (dev < 0 || dev >= kMaxDevices)
+            return fail(HIPQ_ERR_LIMIT, "device ordinal %d beyond %d", dev, kMaxDevices);
+        std::lock_guard<std::mutex> lock(g_ws_mutex);
+        const size_t need = kSplitCounterBytes + partial_bytes;
+        if (g_split_bytes[dev] < need)
+        {
+            if (g_split_ptr[dev])
+            {
+                HIPQ_HIP(hipDeviceSynchronize());
+                HIPQ_HIP(hipFree(g_split_ptr[dev]));
+                g_split_ptr[dev] = nullptr;
+                g_split_bytes[dev] = 0;
+            }
+            size_t want = align_up(need + need / 4, 1 << 20);
+            HIPQ_HIP(hipMalloc(&g_split_ptr[dev], want));
+            HIPQ_HIP(hipMemset(g_split_ptr[dev], 0, kSplitCounterBytes));
+            HIPQ_HIP(hipDeviceSynchronize());
+            g_split_bytes[dev] = want;
+            ++g_ws_epoch[dev];
+        }
+        *counters = static_cast<uint32_t*>(g_split_ptr[dev]);
+        *partials = static_cast<uint8_t*>(g_split_ptr[dev]) + kSplitCounterBytes;
+        return HIPQ_OK;
+    }
+
     __global__ void fill_bytes_kernel(uint8_t* dst, uint32_t pattern, size_t bytes)
     {
         size_t i = (static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 16;

@@ -467,6 +467,50 @@ def test_conv_as_skinny_gemm(gpu_lib, i):
     O.port().orc_set_threads(1)
 
 
+SPLIT_CONV_SHAPES = [
+    # N, C, K, in_sp, f_sp, kw : few output tiles, long reductions that divide into runs of slices
+    (1, 256, 256, (14, 14), (3, 3), dict(pad_below=(1, 1), pad_above=(1, 1))),   # 36 slices, 2 x 2 tiles
+    (1, 1024, 64, (14, 14), (1, 1), dict()),                                     # 16 slices, one narrow tile
+    (2, 512, 144, (9, 9), (1, 1), dict()),                                       # ragged tiles on both sides
+    (1, 128, 128, (10, 12), (4, 4), dict(stride=(1, 1), pad_below=(2, 1), pad_above=(1, 2))),
+]
+
+
+@pytest.mark.parametrize("i", range(len(SPLIT_CONV_SHAPES)))
+def test_conv_split_reduction(gpu_lib, i):
+    """few tiles with long reductions: the pipelined kernel cuts each reduction over several
+    workgroups, which meet through partial sums and a counter that the last one resets; called
+    several times in a row (the counters must be back at zero), both policies, zero points, residual"""
+    N, Cc, K, in_sp, f_sp, kw = SPLIT_CONV_SHAPES[i]
+    say("split conv", SPLIT_CONV_SHAPES[i])
+    O.port().orc_set_threads(8)
+    d = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t="u8", data_layout=H.NXC, out_layout=H.NXC, **kw)
+    dn = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t="u8", **kw)
+    for rep, z in enumerate(((0, 0, 0), (131, 0, 7), (9, -7, 1))):
+        data = synth.uniform_int(2100 + i + rep, dn.data_shape(), 0, 255, np.uint8)
+        filt = synth.uniform_int(2200 + i, dn.filter_shape(), -128, 127, np.int8)
+        s = (0.02, 0.005, 0.9)
+        exp = O.quantized_convolution(dn, data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
+        got = H.quantized_convolution(d, cases.to_nxc(data), filt, s[0], z[0], s[1], z[1], s[2], z[2])
+        assert H.last_kernel().startswith("conv_mfma"), H.last_kernel()
+        assert np.array_equal(cases.to_ncx(got), exp), z
+    for rep, (relu, has_sum) in enumerate(((True, True), (False, False), (True, True))):
+        out_t = "u8" if relu else "i8"
+        d = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t=out_t, data_layout=H.NXC, out_layout=H.NXC, **kw)
+        dn = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t=out_t, **kw)
+        data = synth.uniform_int(2300 + i + rep, dn.data_shape(), 0, 255, np.uint8)
+        filt = synth.uniform_int(2400 + i, dn.filter_shape(), -127, 127, np.int8)
+        bias = synth.uniform_int(2500, (K,), -20000, 20000, np.int32)
+        scales = synth.uniform_f32(2501, (K,), 2e-4, 9e-4)
+        summ = synth.uniform_int(2502, dn.out_shape(), 0, 255, np.uint8) if has_sum else None
+        f = H.make_fused_desc(has_bias=True, has_sum=has_sum, sum_t="u8", with_relu=relu, scale_count=K)
+        exp = O.quantized_convolution_fused(dn, f, data, filt, bias, summ, scales, 0.37 if has_sum else None)
+        got = H.quantized_convolution_fused(d, f, cases.to_nxc(data), filt, bias, cases.to_nxc(summ) if has_sum else None, scales, 0.37 if has_sum else None)
+        assert H.last_kernel().startswith("conv_mfma"), H.last_kernel()
+        assert np.array_equal(cases.to_ncx(got), exp), (relu, has_sum)
+    O.port().orc_set_threads(1)
+
+
 @pytest.mark.parametrize("Cc", [1, 3, 4, 15])
 def test_conv_few_input_channels(gpu_lib, Cc):
     """a network's first layer (3 input channels, 7x7 stride 2): the data is padded to 16 channels on

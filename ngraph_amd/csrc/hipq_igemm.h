@@ -727,7 +727,7 @@ namespace hipq
     // tiles' arithmetic and epilogues, and long ones have two slices of latency cover.  Each
     // wavefront requantizes its own 64 x 64 sub-tile into a private swizzled LDS region and writes it
     // out 16 bytes a lane; per-channel constants of the current column tile sit in LDS.
-    template <class XL, int WM, int WN, int WAVES_M, int WAVES_N, int MODE>
+    template <class XL, int WM, int WN, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM>
     __global__ __launch_bounds__(256, 2) void igemm_pipe_kernel(XL xl,
                                                                 const int8_t* __restrict__ w,
                                                                 const int32_t* __restrict__ wsum,
@@ -806,8 +806,8 @@ namespace hipq
         }
         const int32_t mult = (x_unsigned ? 128 : 0) - xzp;
         const EpiConst ec = epi_const(epi);
-        const bool has_sum = MODE == EPI_FUSED && epi.sum_in != nullptr;
-        const bool relu = epi.relu != 0;
+        constexpr bool has_sum = HAS_SUM; // residual input (fused policy only)
+        static_assert(!HAS_SUM || MODE == EPI_FUSED, "only the fused policy adds a residual");
 
         // ---- loader --------------------------------------------------------------------------
         const int lrow = tid >> 2;
@@ -817,7 +817,11 @@ namespace hipq
         const __amdgpu_buffer_rsrc_t xrs = make_rsrc(xl.x, xl.bytes);
         const __amdgpu_buffer_rsrc_t wrs = make_rsrc(w, static_cast<uint32_t>(N) * static_cast<uint32_t>(Kred));
         const int KT = ((Kred + BK - 1) / BK) >> split_shift; // slices per work item (the launcher makes the split even)
-        const int total = my_tiles * KT;
+        // Every slice issues the loads of the slice after next and stores the next one's into LDS,
+        // without conditions (a condition the compiler cannot see through makes it wait for loads in
+        // flight before their registers are loaded again): past the end the loader reads nothing
+        // (every offset out of range), and an odd sequence gets one idle slice whose tile stores nothing.
+        const int total = (my_tiles * KT + 1) & ~1;
         typename XL::Row xr[XLOADS];
         typename XL::Cursor cur;
         int32_t woff[WLOADS];
@@ -865,6 +869,15 @@ namespace hipq
                 lkt = 0;
                 if (++lj < my_tiles)
                     loader_tile(lj);
+                else
+                {
+#pragma unroll
+                    for (int i = 0; i < XLOADS; ++i)
+                        xl.init_row(xr[i], M, M);
+#pragma unroll
+                    for (int i = 0; i < WLOADS; ++i)
+                        woff[i] = kOob;
+                }
             }
             else
             {
@@ -969,8 +982,7 @@ namespace hipq
                 sum_regs[i] = buffer_load16(srs, (m < M && n < N) ? static_cast<int32_t>(m * N + n) : kOob);
             }
         };
-        auto epilogue = [&](auto with_sum) {
-            constexpr bool has_sum = decltype(with_sum)::value; // (shadows the run-time flag: one copy of the code each)
+        auto epilogue = [&]() {
             uint8_t* o8 = static_cast<uint8_t*>(out);
             if (has_sum)
             {
@@ -1124,13 +1136,7 @@ namespace hipq
         };
         // one slice: LDS buffer `buf` feeds the MFMAs, `next` (slice s+1) moves into the other
         // buffer, `free_regs` takes the loads of slice s+2
-        auto step = [&](int s, int buf, const Regs& next, Regs& free_regs) {
-            HIPQ_PIPE_MARK(s, 0);
-            if (has_sum && ckt + 1 == KT) // uniform
-                sum_fetch();
-            if (s + 2 < total)
-                gload(free_regs);
-            HIPQ_PIPE_MARK(s, 1);
+        auto multiply = [&](int buf) {
             if (ckt == 0) // uniform
             {
                 int t, ks = 0;
@@ -1141,24 +1147,36 @@ namespace hipq
             }
             else
                 compute(buf, std::false_type{});
-            HIPQ_PIPE_MARK(s, 2);
-            const bool tile_done = ++ckt == KT;
-            if (tile_done)
+        };
+        auto step = [&](int s, int buf, const Regs& next, Regs& free_regs) {
+            HIPQ_PIPE_MARK(s, 0);
+            const bool tile_done = ckt + 1 == KT;
+            if (tile_done) // uniform; the residual is fetched and used inside one branch
             {
-                if (splits == 1 || gather_splits()) // uniform
-                {
-                    if (has_sum)
-                        epilogue(std::true_type{});
-                    else
-                        epilogue(std::false_type{});
-                }
+                if (has_sum)
+                    sum_fetch();
+                gload(free_regs);
+                HIPQ_PIPE_MARK(s, 1);
+                multiply(buf);
+                HIPQ_PIPE_MARK(s, 2);
+                if (splits == 1 || (cm0 < M && gather_splits())) // uniform
+                    epilogue();
                 ckt = 0;
                 if (++cj < my_tiles)
                     tile_origin(cj, cm0, cn0);
+                else
+                    cm0 = M; // the idle slice's tile: nothing fetched, nothing stored
+            }
+            else
+            {
+                gload(free_regs);
+                HIPQ_PIPE_MARK(s, 1);
+                multiply(buf);
+                HIPQ_PIPE_MARK(s, 2);
+                ++ckt;
             }
             HIPQ_PIPE_MARK(s, 3);
-            if (s + 1 < total)
-                lstore(next, buf ^ 1);
+            lstore(next, buf ^ 1);
             HIPQ_PIPE_MARK(s, 4);
             __syncthreads();
             HIPQ_PIPE_MARK(s, 5);
@@ -1172,16 +1190,14 @@ namespace hipq
         Regs r0, r1;
         loader_tile(0);
         gload(r0);
-        if (total > 1)
-            gload(r1);
+        gload(r1);
         load_params(cn0);
         lstore(r0, 0);
         __syncthreads();
         for (int s = 0; s < total; s += 2)
         {
             step(s, 0, r1, r0);
-            if (s + 1 < total)
-                step(s + 1, 1, r0, r1);
+            step(s + 1, 1, r0, r1);
         }
     }
 
@@ -1222,7 +1238,7 @@ namespace hipq
         return check_launch(name);
     }
 
-    template <class XL, int WAVES_M, int WAVES_N, int MODE>
+    template <class XL, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM>
     static int launch_pipe(const XL& xl,
                            const int8_t* w,
                            const int32_t* wsum,
@@ -1239,7 +1255,7 @@ namespace hipq
     {
         constexpr int BM = WAVES_M * 64, BN = WAVES_N * 64;
         constexpr size_t lds_bytes = 2 * static_cast<size_t>(BM + BN) * BK + 4 * 64 * 64 + 3 * BN * sizeof(float) + 16;
-        auto kernel = igemm_pipe_kernel<XL, 2, 2, WAVES_M, WAVES_N, MODE>;
+        auto kernel = igemm_pipe_kernel<XL, 2, 2, WAVES_M, WAVES_N, MODE, HAS_SUM>;
         static bool configured[16] = {};
         static int cus[16] = {};
         int dev = 0;
@@ -1311,9 +1327,15 @@ namespace hipq
         // 8-bit channels-last outputs in whole 16-byte pieces: the persistent pipelined kernel
         if (!X_ON_A && KIND == OUT_Q8 && (N & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 && getenv("HIPQ_NO_PIPE") == nullptr)
         {
+            if (MODE == EPI_FUSED && epi.sum_in != nullptr)
+            {
+                if (N <= 64)
+                    return launch_pipe<XL, 4, 1, EPI_FUSED, true>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+                return launch_pipe<XL, 2, 2, EPI_FUSED, true>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+            }
             if (N <= 64)
-                return launch_pipe<XL, 4, 1, MODE>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
-            return launch_pipe<XL, 2, 2, MODE>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+                return launch_pipe<XL, 4, 1, MODE, false>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+            return launch_pipe<XL, 2, 2, MODE, false>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
         }
         // short reductions are bound by latency, not by LDS traffic: small wavefront tiles (64 x 64)
         // take half the registers, so twice as many workgroups are resident to hide it

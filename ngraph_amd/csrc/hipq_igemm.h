@@ -84,11 +84,36 @@ namespace hipq
         return r;
     }
 
+    // ---- loads straight into LDS -----------------------------------------------------------------
+    __device__ __forceinline__ v4i rsrc_words(const void* p, uint32_t bytes)
+    {
+        const uint64_t a = reinterpret_cast<uint64_t>(p);
+        return v4i{static_cast<int>(a), static_cast<int>((a >> 32) & 0xffffu), static_cast<int>(bytes), 0x00020000};
+    }
+    __device__ __forceinline__ uint32_t lds_address(const void* p)
+    {
+        return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const uint8_t*)p));
+    }
+    // every lane's 16 bytes at `off` of the buffer go to LDS address lds_base + 16 * lane (zeros
+    // when `off` is out of range); lds_base is uniform.  Counted by vmcnt like any load.
+    __device__ __forceinline__ void lds_dma16(v4i rsrc, int32_t off, uint32_t lds_base)
+    {
+        asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base), "v"(off), "s"(rsrc) : "memory");
+    }
+    template <int N>
+    __device__ __forceinline__ void wait_vmcnt()
+    {
+        static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+    }
+
     struct GemmX
     {
         const uint8_t* x;
         int32_t K;
         uint32_t bytes; // M * K
+        static constexpr bool kUniform = false;
+        static constexpr bool kPads = false; // (only read by the kernels that load straight into LDS)
 
         struct Row
         {
@@ -121,6 +146,8 @@ namespace hipq
 
     struct ConvX
     {
+        static constexpr bool kUniform = false;
+        static constexpr bool kPads = false; // (only read by the kernels that load straight into LDS)
         const uint8_t* x; // [N][H][W][C]
         int32_t H, W, C, Q, R, S, sh, sw, dh, dw, pbh, pbw;
         int64_t PQ;
@@ -206,6 +233,106 @@ namespace hipq
                     }
                 }
             return acc;
+        }
+    };
+
+    // ---- loaders of the kernels that load straight into LDS -------------------------------------
+    // Their reduction cursor is the same for every lane of the workgroup (scalar registers); a lane
+    // adds the offset of its own 16-byte chunk.
+    struct RowsU
+    {
+        const uint8_t* x;
+        int32_t K;
+        uint32_t bytes; // M * K
+        static constexpr bool kUniform = true;
+        static constexpr bool kPads = false; // no reads of padding: an out-of-range chunk is never used
+        struct Row
+        {
+            int32_t off;
+        };
+        struct Cursor
+        {
+            int32_t kbyte;
+        };
+        __device__ __forceinline__ void init_row(Row& r, int64_t m, int64_t M) const { r.off = m < M ? static_cast<int32_t>(m) * K : kOob; }
+        __device__ __forceinline__ void init_cursor(Cursor& c, int kbyte) const { c.kbyte = kbyte; }
+        __device__ __forceinline__ void advance(Cursor& c, int bytes_) const { c.kbyte += bytes_; }
+        __device__ __forceinline__ int32_t offset(const Row& r, const Cursor& c, int lane_bytes) const
+        {
+            return (r.off != kOob && c.kbyte + lane_bytes < K) ? r.off + c.kbyte + lane_bytes : kOob;
+        }
+        __device__ __forceinline__ int32_t direct(int64_t m, const int8_t* wrow, int32_t xzp, int32_t wzp, bool x_unsigned) const
+        {
+            GemmX g{x, K, bytes};
+            return g.direct(m, wrow, xzp, wzp, x_unsigned);
+        }
+    };
+
+    // channels-last convolution whose channel count is a multiple of 64: a 64-byte slice lies inside one tap
+    struct ConvU
+    {
+        ConvX cx;
+        const uint8_t* x; // = cx.x
+        uint32_t bytes;   // = cx.bytes
+        static constexpr bool kUniform = true;
+        static constexpr bool kPads = true;
+        struct Row
+        {
+            int32_t pix; // byte offset of the window's first tap (may lie before the image), kOob when beyond M
+            int32_t yx;  // (top input row << 16) | (left input column & 0xffff) of the window
+        };
+        struct Cursor
+        {
+            int32_t r, s, c;  // tap and channel offset of the slice
+            int32_t ry, sx;   // r * dh, s * dw
+            int32_t tap_off;  // ((r * dh) * W + s * dw) * C + c
+        };
+        __device__ __forceinline__ void init_row(Row& rw, int64_t m, int64_t M) const
+        {
+            ConvX::Row r;
+            cx.init_row(r, m, M);
+            rw.yx = r.yx;
+            rw.pix = r.base == kOob ? kOob : r.base + ((r.yx >> 16) * cx.W + static_cast<int16_t>(r.yx & 0xffff)) * cx.C;
+        }
+        __device__ __forceinline__ void set(Cursor& c) const
+        {
+            c.ry = c.r * cx.dh;
+            c.sx = c.s * cx.dw;
+            c.tap_off = (c.ry * cx.W + c.sx) * cx.C + c.c;
+        }
+        __device__ __forceinline__ void init_cursor(Cursor& c, int kbyte) const
+        {
+            const int tap = static_cast<int>(cx.by_c.div(static_cast<uint32_t>(kbyte)));
+            c.c = kbyte - tap * cx.C;
+            c.r = static_cast<int>(cx.by_s.div(static_cast<uint32_t>(tap)));
+            c.s = tap - c.r * cx.S;
+            set(c);
+        }
+        __device__ __forceinline__ void advance(Cursor& c, int bytes_) const
+        {
+            c.c += bytes_;
+            if (c.c >= cx.C) // at most one tap further: bytes_ <= 64 <= C
+            {
+                c.c -= cx.C;
+                if (++c.s == cx.S)
+                {
+                    c.s = 0;
+                    ++c.r;
+                }
+            }
+            set(c);
+        }
+        __device__ __forceinline__ int32_t offset(const Row& rw, const Cursor& c, int lane_bytes) const
+        {
+            const int32_t y = (rw.yx >> 16) + c.ry;
+            const int32_t xx = static_cast<int16_t>(rw.yx & 0xffff) + c.sx;
+            const bool ok = (rw.pix != kOob) & (c.r < cx.R) & (static_cast<uint32_t>(y) < static_cast<uint32_t>(cx.H)) &
+                            (static_cast<uint32_t>(xx) < static_cast<uint32_t>(cx.W));
+            return ok ? rw.pix + c.tap_off + lane_bytes : kOob;
+        }
+        __device__ __forceinline__ int32_t direct(int64_t m, const int8_t* wrow, int32_t xzp, int32_t wzp, bool x_unsigned) const
+        {
+            return cx.direct(m, wrow, xzp, wzp, x_unsigned);
         }
     };
 
@@ -727,7 +854,15 @@ namespace hipq
     // tiles' arithmetic and epilogues, and long ones have two slices of latency cover.  Each
     // wavefront requantizes its own 64 x 64 sub-tile into a private swizzled LDS region and writes it
     // out 16 bytes a lane; per-channel constants of the current column tile sit in LDS.
-    template <class XL, int WM, int WN, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM>
+    //
+    // DMA variant (loaders with a uniform cursor): the slices go from global memory straight into
+    // LDS (buffer loads with the lds modifier, 16 bytes a lane, a wavefront's 64 lanes filling one
+    // contiguous KiB, so the swizzle is applied to what a lane reads instead of where it writes),
+    // three buffers deep: no staging registers, no LDS stores, and the sign flip of unsigned data
+    // moves to the MFMA fragments.  These loads are written in assembly, so the waits for them are
+    // explicit: a wait for "at most n operations in flight" only ever errs on the long side when
+    // the compiler's own loads and stores are in the queue as well.
+    template <class XL, int WM, int WN, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM, bool DMA>
     __global__ __launch_bounds__(256, 2) void igemm_pipe_kernel(XL xl,
                                                                 const int8_t* __restrict__ w,
                                                                 const int32_t* __restrict__ wsum,
@@ -754,9 +889,10 @@ namespace hipq
         constexpr int STAGE = (BM + BN) * BK;
         constexpr int OUT_STAGE = TM * TN; // per wavefront
         static_assert(TN == 64, "the output staging swizzle is written for 64-byte rows");
-        extern __shared__ __attribute__((aligned(16))) uint8_t lds[]; // [2][x | w] operands, 4 output regions, per-channel constants
-        uint8_t* const ostage = lds + 2 * STAGE + (threadIdx.x >> 6) * OUT_STAGE;
-        float* const params = reinterpret_cast<float*>(lds + 2 * STAGE + 4 * OUT_STAGE); // [3][BN]: correction (as int), bias, scale
+        constexpr int NSTAGE = DMA ? 3 : 2;
+        extern __shared__ __attribute__((aligned(16))) uint8_t lds[]; // [NSTAGE][x | w] operands, 4 output regions, per-channel constants
+        uint8_t* const ostage = lds + NSTAGE * STAGE + (threadIdx.x >> 6) * OUT_STAGE;
+        float* const params = reinterpret_cast<float*>(lds + NSTAGE * STAGE + 4 * OUT_STAGE); // [3][BN]: correction (as int), bias, scale
 
         const int tid = threadIdx.x;
         const int lane = tid & 63;
@@ -811,7 +947,8 @@ namespace hipq
 
         // ---- loader --------------------------------------------------------------------------
         const int lrow = tid >> 2;
-        const int lchunk = tid & 3;
+        // (DMA: the lane's LDS slot is fixed, chunk position tid & 3 of row lrow: it reads the chunk that belongs there)
+        const int lchunk = DMA ? ((tid & 3) ^ ((lrow >> 2) & 3)) : (tid & 3);
         const int xor_mask = x_unsigned ? static_cast<int>(0x80808080u) : 0;
         const int fill = (xzp & 0xFF) * 0x01010101;
         const __amdgpu_buffer_rsrc_t xrs = make_rsrc(xl.x, xl.bytes);
@@ -821,7 +958,7 @@ namespace hipq
         // without conditions (a condition the compiler cannot see through makes it wait for loads in
         // flight before their registers are loaded again): past the end the loader reads nothing
         // (every offset out of range), and an odd sequence gets one idle slice whose tile stores nothing.
-        const int total = (my_tiles * KT + 1) & ~1;
+        const int total = DMA ? my_tiles * KT : ((my_tiles * KT + 1) & ~1);
         typename XL::Row xr[XLOADS];
         typename XL::Cursor cur;
         int32_t woff[WLOADS];
@@ -833,7 +970,7 @@ namespace hipq
             tile_origin(j, m0, n0);
             int t, ks;
             tile_index(j, t, ks);
-            const int kbyte0 = ks * KT * BK + lchunk * 16;
+            const int kbyte0 = ks * KT * BK + (DMA ? 0 : lchunk * 16);
 #pragma unroll
             for (int i = 0; i < XLOADS; ++i)
                 xl.init_row(xr[i], m0 + lrow + 64 * i, M);
@@ -854,16 +991,19 @@ namespace hipq
         };
         auto gload = [&](Regs& r) {
             r.oob = 0;
-#pragma unroll
-            for (int i = 0; i < XLOADS; ++i)
+            if constexpr (!DMA)
             {
-                const int32_t off = xl.offset(xr[i], cur);
-                r.oob |= (off == kOob ? 1u : 0u) << i;
-                r.x[i] = buffer_load16(xrs, off);
-            }
 #pragma unroll
-            for (int i = 0; i < WLOADS; ++i)
-                r.w[i] = buffer_load16(wrs, (woff[i] != kOob && kb < Kred) ? woff[i] + kb : kOob);
+                for (int i = 0; i < XLOADS; ++i)
+                {
+                    const int32_t off = xl.offset(xr[i], cur);
+                    r.oob |= (off == kOob ? 1u : 0u) << i;
+                    r.x[i] = buffer_load16(xrs, off);
+                }
+#pragma unroll
+                for (int i = 0; i < WLOADS; ++i)
+                    r.w[i] = buffer_load16(wrs, (woff[i] != kOob && kb < Kred) ? woff[i] + kb : kOob);
+            }
             if (++lkt == KT)
             {
                 lkt = 0;
@@ -905,6 +1045,54 @@ namespace hipq
                     *reinterpret_cast<v4i*>(ws + lds_offset(lrow + 64 * i, lchunk)) = r.w[i];
         };
 
+        // DMA: the next slice of the loader's sequence goes into operand buffer `buf`; returns which
+        // of the lane's data chunks were out of range (they arrive as zeros)
+        const v4i xrs_words = rsrc_words(xl.x, xl.bytes);
+        const v4i wrs_words = rsrc_words(w, static_cast<uint32_t>(N) * static_cast<uint32_t>(Kred));
+        const uint32_t lds_wave = lds_address(lds) + static_cast<uint32_t>(wave) * 1024u;
+        auto dma_load = [&](int buf) -> uint32_t {
+            uint32_t oob = 0;
+            if constexpr (DMA)
+            {
+                const uint32_t base = __builtin_amdgcn_readfirstlane(lds_wave + static_cast<uint32_t>(buf) * STAGE);
+#pragma unroll
+                for (int i = 0; i < XLOADS; ++i)
+                {
+                    const int32_t off = xl.offset(xr[i], cur, lchunk * 16);
+                    oob |= (off == kOob ? 1u : 0u) << i;
+                    lds_dma16(xrs_words, off, base + i * 4096);
+                }
+#pragma unroll
+                for (int i = 0; i < WLOADS; ++i)
+                    lds_dma16(wrs_words, (woff[i] != kOob && kb + lchunk * 16 < Kred) ? woff[i] + kb + lchunk * 16 : kOob, base + BM * BK + i * 4096);
+                if (++lkt == KT)
+                {
+                    lkt = 0;
+                    if (++lj < my_tiles)
+                        loader_tile(lj);
+                }
+                else
+                {
+                    xl.advance(cur, BK);
+                    kb += BK;
+                }
+            }
+            return oob;
+        };
+        // DMA with a non-zero data zero point: chunks in the padding must hold that byte, not zero
+        auto fill_fix = [&](int buf, uint32_t oob) {
+            if constexpr (DMA && XL::kPads)
+            {
+                if (fill != 0 && oob != 0)
+                {
+#pragma unroll
+                    for (int i = 0; i < XLOADS; ++i)
+                        if ((oob >> i) & 1u)
+                            *reinterpret_cast<v4i*>(lds + buf * STAGE + lds_offset(lrow + 64 * i, lchunk)) = v4i{fill, fill, fill, fill};
+                }
+            }
+        };
+
         // ---- consumer ------------------------------------------------------------------------
         v16i acc[WM][WN];
         // The accumulators start from the zero-point correction of their channels (a register row of
@@ -936,7 +1124,11 @@ namespace hipq
                     wf[i] = *reinterpret_cast<const v4i*>(ws + lds_offset((wn * WN + i) * 32 + (lane & 31), chunk));
 #pragma unroll
                 for (int i = 0; i < WM; ++i)
+                {
                     xf[i] = *reinterpret_cast<const v4i*>(xs + lds_offset((wm * WM + i) * 32 + (lane & 31), chunk));
+                    if constexpr (DMA) // the data sits in LDS as it came: unsigned bytes become signed here
+                        xf[i] = v4i{xf[i][0] ^ xor_mask, xf[i][1] ^ xor_mask, xf[i][2] ^ xor_mask, xf[i][3] ^ xor_mask};
+                }
 #pragma unroll
                 for (int mi = 0; mi < WM; ++mi)
 #pragma unroll
@@ -1187,17 +1379,80 @@ namespace hipq
             }
         };
 
-        Regs r0, r1;
-        loader_tile(0);
-        gload(r0);
-        gload(r1);
-        load_params(cn0);
-        lstore(r0, 0);
-        __syncthreads();
-        for (int s = 0; s < total; s += 2)
+        if constexpr (DMA)
         {
-            step(s, 0, r1, r0);
-            step(s + 1, 1, r0, r1);
+            constexpr int L = XLOADS + WLOADS; // operand loads of one slice per lane
+            loader_tile(0);
+            uint32_t oob_next = dma_load(0);
+            uint32_t oob_new = total > 1 ? dma_load(1) : 0u;
+            load_params(cn0);
+            if (total > 1)
+                wait_vmcnt<L>();
+            else
+                wait_vmcnt<0>();
+            fill_fix(0, oob_next);
+            oob_next = oob_new;
+            __syncthreads();
+            int cb = 0, lb = 2; // buffer of the slice being multiplied, buffer the loads go to
+            for (int s = 0; s < total; ++s)
+            {
+                HIPQ_PIPE_MARK(s, 0);
+                if (s + 2 < total) // uniform
+                    oob_new = dma_load(lb);
+                HIPQ_PIPE_MARK(s, 1);
+                const bool tile_done = ckt + 1 == KT;
+                if (tile_done) // uniform
+                {
+                    if (has_sum)
+                        sum_fetch();
+                    multiply(cb);
+                    HIPQ_PIPE_MARK(s, 2);
+                    if (splits == 1 || gather_splits()) // uniform
+                        epilogue();
+                    ckt = 0;
+                    if (++cj < my_tiles)
+                        tile_origin(cj, cm0, cn0);
+                }
+                else
+                {
+                    multiply(cb);
+                    HIPQ_PIPE_MARK(s, 2);
+                    ++ckt;
+                }
+                HIPQ_PIPE_MARK(s, 3);
+                cb = cb == 2 ? 0 : cb + 1;
+                lb = lb == 2 ? 0 : lb + 1;
+                // the next slice has landed once at most the loads of the one after it are in flight
+                if (s + 2 < total)
+                    wait_vmcnt<L>();
+                else
+                    wait_vmcnt<0>();
+                fill_fix(cb, oob_next);
+                oob_next = oob_new;
+                HIPQ_PIPE_MARK(s, 4);
+                __syncthreads();
+                HIPQ_PIPE_MARK(s, 5);
+                if (tile_done && cj < my_tiles && cn0 != params_n0) // uniform
+                {
+                    load_params(cn0);
+                    __syncthreads();
+                }
+            }
+        }
+        else
+        {
+            Regs r0, r1;
+            loader_tile(0);
+            gload(r0);
+            gload(r1);
+            load_params(cn0);
+            lstore(r0, 0);
+            __syncthreads();
+            for (int s = 0; s < total; s += 2)
+            {
+                step(s, 0, r1, r0);
+                step(s + 1, 1, r0, r1);
+            }
         }
     }
 
@@ -1254,8 +1509,9 @@ namespace hipq
                            const char* name)
     {
         constexpr int BM = WAVES_M * 64, BN = WAVES_N * 64;
-        constexpr size_t lds_bytes = 2 * static_cast<size_t>(BM + BN) * BK + 4 * 64 * 64 + 3 * BN * sizeof(float) + 16;
-        auto kernel = igemm_pipe_kernel<XL, 2, 2, WAVES_M, WAVES_N, MODE, HAS_SUM>;
+        constexpr bool DMA = XL::kUniform;
+        constexpr size_t lds_bytes = (DMA ? 3 : 2) * static_cast<size_t>(BM + BN) * BK + 4 * 64 * 64 + 3 * BN * sizeof(float) + 16;
+        auto kernel = igemm_pipe_kernel<XL, 2, 2, WAVES_M, WAVES_N, MODE, HAS_SUM, DMA>;
         static bool configured[16] = {};
         static int cus[16] = {};
         int dev = 0;
@@ -1306,6 +1562,43 @@ namespace hipq
         const unsigned grid = static_cast<unsigned>(items < resident ? items : resident);
         kernel<<<grid, 256, lds_bytes, s>>>(xl, w, wsum, M, Kred, x_unsigned, static_cast<int32_t>(m_tiles), static_cast<int32_t>(n_tiles), split_shift, fast_div(m_tiles), partials, counters, zp, epi, om, out);
         return check_launch(name);
+    }
+
+    // The kernels that load straight into LDS, for 8-bit channels-last outputs in whole 16-byte
+    // pieces; returns HIPQ_ERR_UNSUPPORTED (nothing launched, no error text) when the call is not of that kind.
+    template <class XL>
+    static int launch_uniform(const XL& xl,
+                              const int8_t* w,
+                              const int32_t* wsum,
+                              int64_t M,
+                              int32_t N,
+                              int32_t Kred,
+                              int x_unsigned,
+                              const ZeroPoints& zp,
+                              const Epilogue& epi,
+                              const OutMap& om,
+                              void* out,
+                              hipStream_t s,
+                              const char* name)
+    {
+        const bool q8 = epi.out_t == HIPQ_U8 || epi.out_t == HIPQ_I8;
+        if (!q8 || om.ncx || (N & 15) != 0 || (reinterpret_cast<uintptr_t>(out) & 15) != 0 || getenv("HIPQ_NO_DMA") != nullptr || getenv("HIPQ_NO_PIPE") != nullptr)
+            return HIPQ_ERR_UNSUPPORTED;
+        if (epi.mode == EPI_INTERP)
+        {
+            if (N <= 64)
+                return launch_pipe<XL, 4, 1, EPI_INTERP, false>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+            return launch_pipe<XL, 2, 2, EPI_INTERP, false>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+        }
+        if (epi.sum_in != nullptr)
+        {
+            if (N <= 64)
+                return launch_pipe<XL, 4, 1, EPI_FUSED, true>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+            return launch_pipe<XL, 2, 2, EPI_FUSED, true>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+        }
+        if (N <= 64)
+            return launch_pipe<XL, 4, 1, EPI_FUSED, false>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+        return launch_pipe<XL, 2, 2, EPI_FUSED, false>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
     }
 
     // tile choice: narrow outputs (N <= 64) take 512 x 64 so each wavefront still owns 128 x 64

@@ -334,11 +334,20 @@ namespace hipq
     int launch_rows_mfma(const void* a, bool a_unsigned, const int8_t* w_nk, const int32_t* wsum, int64_t M, int32_t N, int32_t K,
                          const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s, const char* name)
     {
+        OutMap om{0, N, 1};
+        {
+            RowsU xu;
+            xu.x = static_cast<const uint8_t*>(a);
+            xu.K = K;
+            xu.bytes = static_cast<uint32_t>(M * K);
+            const int rc = launch_uniform(xu, w_nk, wsum, M, N, K, a_unsigned ? 1 : 0, zp, epi, om, out, s, name);
+            if (rc != HIPQ_ERR_UNSUPPORTED)
+                return rc;
+        }
         GemmX xl;
         xl.x = static_cast<const uint8_t*>(a);
         xl.K = K;
         xl.bytes = static_cast<uint32_t>(M * K);
-        OutMap om{0, N, 1};
         return launch_epilogue<GemmX, false>(xl, w_nk, wsum, M, N, K, a_unsigned ? 1 : 0, zp, epi, om, out, s, name);
     }
 
@@ -374,9 +383,15 @@ namespace hipq
                 return launch_skinny<2, 16>(d, a, w_nk, wsum, zp, epi, out, s);
             if (d.M <= 64)
                 return launch_skinny<4, 8>(d, a, w_nk, wsum, zp, epi, out, s);
-            if (d.M <= 128)
-                return launch_skinny_wide<8>(d, a, w_nk, wsum, zp, epi, out, s);
-            return launch_skinny_wide<16>(d, a, w_nk, wsum, zp, epi, out, s);
+            // above 64 rows an 8-bit output is faster on the tile kernels, whose reductions are
+            // split over workgroups when the tiles are few (config 2, 256 rows: 22 us against 44)
+            const bool q8 = epi.out_t == HIPQ_U8 || epi.out_t == HIPQ_I8;
+            if (!(q8 && d.N % 16 == 0) || getenv("HIPQ_NO_PIPE") != nullptr)
+            {
+                if (d.M <= 128)
+                    return launch_skinny_wide<8>(d, a, w_nk, wsum, zp, epi, out, s);
+                return launch_skinny_wide<16>(d, a, w_nk, wsum, zp, epi, out, s);
+            }
         }
         return launch_rows_mfma(a, d.a_t == HIPQ_U8, static_cast<const int8_t*>(w_nk), wsum, d.M, static_cast<int32_t>(d.N), static_cast<int32_t>(d.K), zp, epi,
                                 out, s, "dot_mfma_i8_32x32x32");

@@ -477,6 +477,14 @@ SPLIT_CONV_SHAPES = [
 
 
 @pytest.mark.parametrize("i", range(len(SPLIT_CONV_SHAPES)))
+def test_conv_loads_into_lds(gpu_lib, i, monkeypatch):
+    """the same shapes through the kernels whose loads go straight into LDS (opt-in for filters
+    with more than one tap): padding with a non-zero data zero point is patched in after the load"""
+    monkeypatch.setenv("HIPQ_CONV_DMA", "1")
+    test_conv_split_reduction(gpu_lib, i)
+
+
+@pytest.mark.parametrize("i", range(len(SPLIT_CONV_SHAPES)))
 def test_conv_split_reduction(gpu_lib, i):
     """few tiles with long reductions: the pipelined kernel cuts each reduction over several
     workgroups, which meet through partial sums and a counter that the last one resets; called
@@ -678,7 +686,9 @@ def test_dot_skinny(gpu_lib, M):
                 d = H.make_dot_desc(M, K, N, a_t=a_t, out_t=out_t, b_layout=H.B_NK)
                 exp = O.quantized_dot(d, a, w, s[0], z[0], s[1], z[1], s[2], z[2])
                 got = H.quantized_dot(d, a, w, s[0], z[0], s[1], z[1], s[2], z[2])
-                assert H.last_kernel().startswith("dot_skinny"), H.last_kernel()
+                # (more than 64 rows with an 8-bit output in whole 16-byte rows go to the tile kernels)
+                tiles = M > 64 and out_t != "i32" and N % 16 == 0
+                assert H.last_kernel().startswith("dot_mfma" if tiles else "dot_skinny"), H.last_kernel()
                 assert np.array_equal(got, exp), (K, N, a_t, out_t, z)
             bias = synth.uniform_int(803, (N,), -(2**15), 2**15, np.int32)
             scales = synth.uniform_f32(804, (N,), 0.001, 0.01) * np.float32(0.05)
@@ -687,7 +697,8 @@ def test_dot_skinny(gpu_lib, M):
                 f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
                 exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
                 got = H.quantized_dot_bias(d, f, a, w, bias, scales)
-                assert H.last_kernel().startswith("dot_skinny"), H.last_kernel()
+                tiles = M > 64 and out_t != "f32" and N % 16 == 0
+                assert H.last_kernel().startswith("dot_mfma" if tiles else "dot_skinny"), H.last_kernel()
                 assert np.array_equal(got, exp), (K, N, a_t, out_t, relu)
     O.port().orc_set_threads(1)
 

@@ -248,5 +248,14 @@ namespace hipq
     int launch_pad_channels(const void* in, void* out, int64_t N, int64_t X, int64_t Cc, bool in_ncx, const void* zp, int zp_t, hipStream_t s);
     bool conv_pad_eligible(const ConvGeom& g, ConvGeom* padded);
     int launch_im2col_nxc(const ConvGeom& g, const void* x_nxc, void* a, const void* zp, int zp_t, hipStream_t s);
+    // first layers (at most four channels): staged copy with materialised padding + row-packed filter
+    struct RowPack
+    {
+        int64_t Hp, Wp; // staged image extent
+        int64_t kp;     // packed reduction bytes per output channel: filter rows x 32, rounded up to 64
+    };
+    bool conv_rowpack_eligible(const ConvGeom& g, RowPack* rp);
+    int launch_stage_rows(const ConvGeom& g, const RowPack& rp, const void* in, void* staged, const void* zp, int zp_t, hipStream_t s);
+    int launch_conv_rowpack(const ConvGeom& g, const RowPack& rp, const void* staged, const void* packed, const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s);
     int launch_row_sums_i8(const void* w, int64_t rows, int64_t cols, int32_t* sums, hipStream_t s);
 }

@@ -1,0 +1,109 @@
+// Convolutions over at most four input channels (a network's first layer) on the tile kernels that
+// load straight into LDS: eligibility, the staged copy of the data, launch.
+#include <cstdlib>
+
+#include "hipq_igemm.h"
+
+namespace hipq
+{
+    bool conv_rowpack_eligible(const ConvGeom& g, RowPack* rp)
+    {
+        if (g.in[0] != 1 || g.f[0] != 1 || g.out[0] != 1) // 1-D / 2-D only
+            return false;
+        for (int i = 0; i < 3; ++i)
+            if (g.dd[i] != 1 || g.dl[i] != 1)
+                return false;
+        if (g.filter_t != HIPQ_I8 || (g.data_t != HIPQ_U8 && g.data_t != HIPQ_I8))
+            return false;
+        if (g.out_t != HIPQ_U8 && g.out_t != HIPQ_I8)
+            return false;
+        if (g.C < 1 || g.C > 4 || g.f[2] > 8 || g.K % 16 != 0)
+            return false;
+        if (g.out_layout != HIPQ_LAYOUT_NXC && g.K > 1)
+            return false;
+        if (g.pb[1] < 0 || g.pb[2] < 0 || g.out[1] < 1 || g.out[2] < 1)
+            return false;
+        RowPack r;
+        r.Hp = (g.out[1] - 1) * g.st[1] + g.f[1];
+        r.Wp = (g.out[2] - 1) * g.st[2] + 8;
+        r.kp = static_cast<int64_t>(align_up(static_cast<size_t>(g.f[1] * 32), 64));
+        if (!fits_i32(g.N * r.Hp * r.Wp * 4 + 64) || !fits_i32(g.in_count()) || !fits_i32(g.out_count()) || !fits_i32(g.K * r.kp))
+            return false;
+        if (getenv("HIPQ_NO_ROWPACK") != nullptr || getenv("HIPQ_NO_PIPE") != nullptr || getenv("HIPQ_NO_DMA") != nullptr)
+            return false;
+        if (rp)
+            *rp = r;
+        return true;
+    }
+
+    // [N][C][H][W] or [N][H][W][C] bytes -> [N][Hp][Wp][4]: staged pixel (y, x) is input pixel
+    // (y - pad_h, x - pad_w) where that exists; everything else, and the channels beyond C, hold the
+    // data zero point.  One staged pixel (one dword) a lane.
+    __global__ __launch_bounds__(256) void stage_rows_kernel(const uint8_t* __restrict__ in, uint32_t* __restrict__ out, int64_t pixels, int32_t Hp, int32_t Wp, int32_t H, int32_t W,
+                                                             int32_t Cc, int32_t pbh, int32_t pbw, int32_t in_ncx, const void* zp, int32_t zp_t)
+    {
+        const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+        if (i >= pixels)
+            return;
+        const int32_t xp = static_cast<int32_t>(i % Wp);
+        const int64_t t = i / Wp;
+        const int32_t yp = static_cast<int32_t>(t % Hp);
+        const int64_t n = t / Hp;
+        const int32_t y = yp - pbh, x = xp - pbw;
+        uint32_t v = (static_cast<uint32_t>(load_zp(zp, zp_t)) & 0xffu) * 0x01010101u;
+        if (static_cast<uint32_t>(y) < static_cast<uint32_t>(H) && static_cast<uint32_t>(x) < static_cast<uint32_t>(W))
+        {
+            const int64_t pix = static_cast<int64_t>(y) * W + x;
+            const int64_t X = static_cast<int64_t>(H) * W;
+            for (int c = 0; c < Cc; ++c)
+            {
+                const uint32_t b = in_ncx ? in[(n * Cc + c) * X + pix] : in[(n * X + pix) * Cc + c];
+                v = (v & ~(0xffu << (8 * c))) | (b << (8 * c));
+            }
+        }
+        out[i] = v;
+    }
+
+    int launch_stage_rows(const ConvGeom& g, const RowPack& rp, const void* in, void* staged, const void* zp, int zp_t, hipStream_t s)
+    {
+        const int64_t pixels = g.N * rp.Hp * rp.Wp;
+        if (pixels == 0)
+            return HIPQ_OK;
+        HIPQ_REQUIRE((pixels + 255) / 256 < (1ll << 31), "tensor too large for one launch");
+        stage_rows_kernel<<<static_cast<unsigned>((pixels + 255) / 256), 256, 0, s>>>(static_cast<const uint8_t*>(in), static_cast<uint32_t*>(staged), pixels, static_cast<int32_t>(rp.Hp),
+                                                                                     static_cast<int32_t>(rp.Wp), static_cast<int32_t>(g.in[1]), static_cast<int32_t>(g.in[2]),
+                                                                                     static_cast<int32_t>(g.C), static_cast<int32_t>(g.pb[1]), static_cast<int32_t>(g.pb[2]),
+                                                                                     g.data_layout == HIPQ_LAYOUT_NCX ? 1 : 0, zp, zp_t);
+        return check_launch("stage_rows");
+    }
+
+    int launch_conv_rowpack(const ConvGeom& g, const RowPack& rp, const void* staged, const void* packed, const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s)
+    {
+        HIPQ_REQUIRE((reinterpret_cast<uintptr_t>(staged) & 15) == 0 && (reinterpret_cast<uintptr_t>(packed) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0,
+                     "MFMA convolution needs 16-byte aligned tensors");
+        ConvR xl;
+        xl.x = static_cast<const uint8_t*>(staged);
+        xl.bytes = static_cast<uint32_t>(g.N * rp.Hp * rp.Wp * 4);
+        xl.R = static_cast<int32_t>(g.f[1]);
+        xl.S = static_cast<int32_t>(g.f[2]);
+        xl.C = static_cast<int32_t>(g.C);
+        xl.row_pitch = static_cast<int32_t>(rp.Wp * 4);
+        xl.img_pitch = static_cast<int32_t>(rp.Hp * rp.Wp * 4);
+        xl.sh_pitch = static_cast<int32_t>(g.st[1] * rp.Wp * 4);
+        xl.sw4 = static_cast<int32_t>(g.st[2] * 4);
+        xl.Q = static_cast<int32_t>(g.out[2]);
+        xl.PQ = static_cast<int32_t>(g.out[1] * g.out[2]);
+        xl.by_pq = fast_div(xl.PQ);
+        xl.by_q = fast_div(xl.Q);
+        const int64_t M = g.N * g.out[1] * g.out[2];
+        const int32_t N = static_cast<int32_t>(g.K);
+        const int32_t Kred = static_cast<int32_t>(rp.kp);
+        const int8_t* w = static_cast<const int8_t*>(packed);
+        const int32_t* wsum = reinterpret_cast<const int32_t*>(static_cast<const uint8_t*>(packed) + align_up(static_cast<size_t>(g.K) * Kred, 256));
+        OutMap om{0, N, xl.PQ};
+        const int rc = launch_uniform(xl, w, wsum, M, N, Kred, g.data_t == HIPQ_U8 ? 1 : 0, zp, epi, om, out, s, "conv_mfma_i8_32x32x32");
+        if (rc == HIPQ_ERR_UNSUPPORTED)
+            return fail(HIPQ_ERR_INVALID, "row-packed convolution: output is not an aligned 8-bit channels-last tensor");
+        return rc;
+    }
+}

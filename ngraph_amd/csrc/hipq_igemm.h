@@ -336,6 +336,66 @@ namespace hipq
         }
     };
 
+    // Convolution over at most four channels (a network's first layer), on a staged copy of the
+    // data: [image][Hp][Wp][4] with the padding materialised (data zero point) so that every window
+    // lies inside it.  A filter row is one 32-byte run of the copy -- 8 taps x 4 channels, the taps
+    // and channels beyond the filter's meeting zero weights -- so the reduction is R runs of 32
+    // bytes instead of R x S taps padded to 16 channels each (a 7 x 7 filter: 224 bytes, not 784).
+    struct ConvR
+    {
+        const uint8_t* x;
+        uint32_t bytes;
+        int32_t R, S, C;                 // filter rows, taps per row (<= 8), channels (<= 4)
+        int32_t row_pitch, img_pitch;    // Wp * 4, Hp * Wp * 4
+        int32_t sh_pitch, sw4;           // stride_h * Wp * 4, stride_w * 4
+        int32_t Q, PQ;
+        FastDiv by_pq, by_q;
+        static constexpr bool kUniform = true;
+        static constexpr bool kPads = false;
+        struct Row
+        {
+            int32_t off;
+        };
+        struct Cursor
+        {
+            int32_t kbyte;
+        };
+        __device__ __forceinline__ void init_row(Row& r, int64_t m, int64_t M) const
+        {
+            const bool valid = m < M;
+            const uint32_t mm = valid ? static_cast<uint32_t>(m) : 0u;
+            const int32_t n = static_cast<int32_t>(by_pq.div(mm));
+            const int32_t rem = static_cast<int32_t>(mm) - n * PQ;
+            const int32_t p = static_cast<int32_t>(by_q.div(static_cast<uint32_t>(rem)));
+            const int32_t q = rem - p * Q;
+            r.off = valid ? n * img_pitch + p * sh_pitch + q * sw4 : kOob;
+        }
+        __device__ __forceinline__ void init_cursor(Cursor& c, int kbyte) const { c.kbyte = kbyte; }
+        __device__ __forceinline__ void advance(Cursor& c, int bytes_) const { c.kbyte += bytes_; }
+        __device__ __forceinline__ int32_t offset(const Row& r, const Cursor& c, int lane_bytes) const
+        {
+            const int32_t q = (c.kbyte + lane_bytes) >> 4; // 16-byte piece of the packed reduction: filter row q / 2, half q % 2
+            const int32_t fr = q >> 1;
+            return (r.off != kOob && fr < R) ? r.off + fr * row_pitch + (q & 1) * 16 : kOob;
+        }
+        // exact accumulator over the filter's own taps and channels; wrow is the packed row [R][8][4]
+        __device__ __forceinline__ int32_t direct(int64_t m, const int8_t* wrow, int32_t xzp, int32_t wzp, bool x_unsigned) const
+        {
+            Row rw;
+            init_row(rw, m, m + 1);
+            int32_t acc = 0;
+            for (int32_t fr = 0; fr < R; ++fr)
+                for (int32_t fs = 0; fs < S; ++fs)
+                    for (int32_t c = 0; c < C; ++c)
+                    {
+                        const uint8_t b = x[rw.off + fr * row_pitch + fs * 4 + c];
+                        const int32_t a = x_unsigned ? static_cast<int32_t>(b) : static_cast<int32_t>(static_cast<int8_t>(b));
+                        acc += (a - xzp) * (static_cast<int32_t>(wrow[fr * 32 + fs * 4 + c]) - wzp);
+                    }
+            return acc;
+        }
+    };
+
     // Exact but slow tile for a non-zero weight zero point (w - wzp does not fit a signed byte).
     struct OutMap
     {
@@ -1307,22 +1367,29 @@ namespace hipq
             __syncthreads(); // `arrival` may be rewritten by the next tile
             if (!last)
                 return false;
+            // the other items' sums, half a sub-tile's registers at a time: all loads of a batch are
+            // issued before the first is added
             for (int k = 0; k < splits; ++k)
             {
                 if (k == ks)
                     continue;
 #pragma unroll
                 for (int mi = 0; mi < WM; ++mi)
+                {
+                    v4i p4[WN][4];
 #pragma unroll
                     for (int ni = 0; ni < WN; ++ni)
 #pragma unroll
                         for (int g = 0; g < 4; ++g)
-                        {
-                            const v4i p4 = __builtin_amdgcn_raw_buffer_load_b128(prs, k * (BM * BN * 4) + lane_off + ((mi * WN + ni) * 4 + g) * 1024, 0, kDeviceScope);
+                            p4[ni][g] = __builtin_amdgcn_raw_buffer_load_b128(prs, k * (BM * BN * 4) + lane_off + ((mi * WN + ni) * 4 + g) * 1024, 0, kDeviceScope);
+#pragma unroll
+                    for (int ni = 0; ni < WN; ++ni)
+#pragma unroll
+                        for (int g = 0; g < 4; ++g)
 #pragma unroll
                             for (int e = 0; e < 4; ++e)
-                                acc[mi][ni][4 * g + e] += p4[e];
-                        }
+                                acc[mi][ni][4 * g + e] += p4[ni][g][e];
+                }
             }
             return true;
         };

@@ -169,6 +169,22 @@ namespace hipq
         }
     }
 
+    // filter [K][C][R][S] -> row-packed [K][kp]: byte r * 32 + s * 4 + c holds tap (r, s) of channel c,
+    // everything else (taps s >= S, channels c >= C, the tail up to kp) is zero
+    __global__ __launch_bounds__(256) void pack_filter_rows_kernel(const int8_t* __restrict__ f, int8_t* __restrict__ p, int64_t K, int32_t Cc, int32_t R, int32_t S, int32_t kp)
+    {
+        const int64_t total = K * kp;
+        int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+        const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+        for (; i < total; i += step)
+        {
+            const int64_t k = i / kp;
+            const int32_t b = static_cast<int32_t>(i - k * kp);
+            const int32_t r = b >> 5, s = (b >> 2) & 7, c = b & 3;
+            p[i] = (r < R && s < S && c < Cc) ? f[((k * Cc + c) * R + r) * S + s] : static_cast<int8_t>(0);
+        }
+    }
+
     // [N][C][X] or [N][X][C] bytes -> [N][X][16] with the channels C .. 15 holding the data zero point
     // (they meet zero weights; as the zero point they also vanish on the exact path for a non-zero
     // filter zero point); one pixel a lane, one 16-byte store
@@ -284,6 +300,9 @@ size_t hipq_conv_packed_filter_bytes(const hipq_conv_desc_t* desc)
     ConvGeom g;
     if (make_geom(desc, &g) != HIPQ_OK)
         return 0;
+    RowPack rp;
+    if (conv_rowpack_eligible(g, &rp))
+        return align_up(static_cast<size_t>(g.K * rp.kp), 256) + static_cast<size_t>(g.K) * sizeof(int32_t);
     if (!conv_mfma_eligible(g) && !conv_pad_eligible(g, &g))
         return 0;
     size_t w = align_up(static_cast<size_t>(g.K * g.C * g.taps()), 256);
@@ -297,6 +316,23 @@ int hipq_conv_pack_filter(const hipq_conv_desc_t* desc, const void* filter, void
     if (rc)
         return rc;
     const int64_t src_c = g.C;
+    RowPack rp;
+    if (conv_rowpack_eligible(g, &rp))
+    {
+        HIPQ_REQUIRE(filter && packed, "null pointer");
+        hipStream_t s = as_stream(stream);
+        const int64_t total = g.K * rp.kp;
+        int64_t blocks = (total + 255) / 256;
+        if (blocks > 65536)
+            blocks = 65536;
+        pack_filter_rows_kernel<<<static_cast<unsigned>(blocks), 256, 0, s>>>(static_cast<const int8_t*>(filter), static_cast<int8_t*>(packed), g.K, static_cast<int32_t>(g.C),
+                                                                              static_cast<int32_t>(g.f[1]), static_cast<int32_t>(g.f[2]), static_cast<int32_t>(rp.kp));
+        rc = check_launch("pack_filter_rows");
+        if (rc)
+            return rc;
+        int32_t* sums = reinterpret_cast<int32_t*>(static_cast<uint8_t*>(packed) + align_up(static_cast<size_t>(total), 256));
+        return launch_row_sums_i8(packed, g.K, rp.kp, sums, s);
+    }
     if (!conv_mfma_eligible(g) && !conv_pad_eligible(g, &g))
         return fail(HIPQ_ERR_UNSUPPORTED, "shape is not eligible for the MFMA path (hipq_conv_packed_filter_bytes is 0)");
     HIPQ_REQUIRE(filter && packed, "null pointer");

@@ -34,6 +34,20 @@ namespace hipq
                         hipStream_t s)
     {
         // the MFMA kernels have no fused-policy instantiation with int32 output (no nGraph op asks for one)
+        RowPack rp;
+        if (packed && conv_rowpack_eligible(g, &rp))
+        {
+            // a first layer's three or four channels: a copy with the padding materialised, whose
+            // filter rows are single 32-byte runs, then the tile kernel that loads straight into LDS
+            void* ws = nullptr;
+            int rc = workspace(align_up(static_cast<size_t>(g.N * rp.Hp * rp.Wp * 4), 256), &ws);
+            if (rc)
+                return rc;
+            rc = launch_stage_rows(g, rp, data, ws, zp.data_zp, zp.data_t, s);
+            if (rc)
+                return rc;
+            return launch_conv_rowpack(g, rp, ws, packed, zp, epi, out, s);
+        }
         ConvGeom padded;
         if (packed && !conv_mfma_eligible(g) && conv_pad_eligible(g, &padded) && !(epi.mode == EPI_FUSED && g.out_t == HIPQ_I32))
         {

@@ -79,6 +79,9 @@ def test_packed_sizes_and_eligibility():
     assert lib.hipq_conv_packed_filter_bytes(C.byref(d)) == 64 * 64 * 9 + 64 * 4
     d3 = H.make_conv_desc(1, 3, 64, (224, 224), (7, 7))  # fewer than 16 channels: packed with the channels padded to 16
     assert lib.hipq_conv_packed_filter_bytes(C.byref(d3)) == 64 * 16 * 49 + 64 * 4
+    # ... unless the output is 8-bit channels-last: then every filter row is packed as 8 taps x 4 channels (7 rows -> 224 -> 256 bytes)
+    d3r = H.make_conv_desc(1, 3, 64, (224, 224), (7, 7), out_t="u8", out_layout=H.NXC)
+    assert lib.hipq_conv_packed_filter_bytes(C.byref(d3r)) == 64 * 256 + 64 * 4
     d40 = H.make_conv_desc(1, 40, 64, (8, 8), (3, 3))  # 16 or more channels, not a multiple of 16: direct kernel
     assert lib.hipq_conv_packed_filter_bytes(C.byref(d40)) == 0
     du = H.make_conv_desc(1, 64, 64, (8, 8), (1, 1), filter_t="u8", out_t="u8")

@@ -1201,15 +1201,36 @@ namespace hipq
         int32_t cn0, params_n0 = -1;
         tile_origin(0, cm0, cn0);
         // per-channel constants of column block n0 -> LDS; callers put a barrier behind it
+        // With a short reduction (|accumulator| <= 2^24) and biases of that size, float(acc) +
+        // float(bias) is float(acc + bias): no rounding happens before the sum's own.  The bias of such
+        // a column block joins the correction in the accumulators' start value and the epilogue
+        // skips its add (decided per column block; every lane of the workgroup calls this).
+        // (only in the kernels that load straight into LDS: they take the short reductions, and the
+        // register-staged ones have no registers to spare for a second epilogue)
+        constexpr bool kFold = DMA && MODE == EPI_FUSED;
+        const bool fold_possible = kFold && static_cast<int64_t>(Kred) * (255 * 128) <= (1 << 24);
+        bool bias_folded = false;
         auto load_params = [&](int32_t n0) {
+            int32_t corr = 0, b = 0;
+            float sc = ec.scale;
             if (tid < BN)
             {
                 const int32_t n = n0 + tid;
                 const bool ok = n < N;
-                reinterpret_cast<int32_t*>(params)[tid] = ok ? mult * wsum[n] : 0;
-                params[BN + tid] = (MODE == EPI_FUSED && epi.bias && ok) ? static_cast<float>(epi.bias[n]) : 0.0f;
-                params[2 * BN + tid] = (MODE == EPI_FUSED && epi.per_channel && ok) ? epi.scale[n] : ec.scale;
+                corr = ok ? mult * wsum[n] : 0;
+                b = (MODE == EPI_FUSED && epi.bias && ok) ? epi.bias[n] : 0;
+                sc = (MODE == EPI_FUSED && epi.per_channel && ok) ? epi.scale[n] : ec.scale;
             }
+            bool fold = false;
+            if (fold_possible) // uniform
+                fold = __syncthreads_and(b >= -(1 << 24) && b <= (1 << 24)) != 0;
+            if (tid < BN)
+            {
+                reinterpret_cast<int32_t*>(params)[tid] = fold ? corr + b : corr;
+                params[BN + tid] = fold ? 0.0f : static_cast<float>(b);
+                params[2 * BN + tid] = sc;
+            }
+            bias_folded = fold;
             params_n0 = n0;
         };
         // requantizes the wavefront's sub-tile into its staging region and writes it out
@@ -1234,7 +1255,8 @@ namespace hipq
                 sum_regs[i] = buffer_load16(srs, (m < M && n < N) ? static_cast<int32_t>(m * N + n) : kOob);
             }
         };
-        auto epilogue = [&]() {
+        auto epilogue = [&](auto folded) {
+            constexpr bool FOLD = decltype(folded)::value; // the bias is already in the accumulators
             uint8_t* o8 = static_cast<uint8_t*>(out);
             if (has_sum)
             {
@@ -1258,7 +1280,9 @@ namespace hipq
                 {
                     const int nl = ni * 32 + 8 * g + 4 * (lane >> 5); // channel within the wavefront's 64
                     const int nt = wn * TN + nl;                     // within the column block
-                    const v4f bias4 = *reinterpret_cast<const v4f*>(params + BN + nt);
+                    v4f bias4 = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+                    if (!FOLD)
+                        bias4 = *reinterpret_cast<const v4f*>(params + BN + nt);
                     const v4f scale4 = *reinterpret_cast<const v4f*>(params + 2 * BN + nt);
 #pragma unroll
                     for (int mi = 0; mi < WM; ++mi)
@@ -1288,7 +1312,7 @@ namespace hipq
                             const int32_t a = acc[mi][ni][4 * g + e];
                             if (MODE == EPI_FUSED)
                             {
-                                float v = __fmul_rn(__fadd_rn(static_cast<float>(a), bias4[e]), scale4[e]);
+                                float v = __fmul_rn(FOLD ? static_cast<float>(a) : __fadd_rn(static_cast<float>(a), bias4[e]), scale4[e]);
                                 if (has_sum)
                                     v = fmaf(ec.sum_scale, s4[e], v);
                                 v = __builtin_amdgcn_fmed3f(v, clamp_lo, ec.hi);
@@ -1367,29 +1391,30 @@ namespace hipq
             __syncthreads(); // `arrival` may be rewritten by the next tile
             if (!last)
                 return false;
-            // the other items' sums, half a sub-tile's registers at a time: all loads of a batch are
-            // issued before the first is added
+            // the other items' sums, a batch of loads at a time (all issued before the first is added;
+            // the register-staged kernels can spare registers for two)
+            constexpr int GB = DMA ? 4 : 2;
             for (int k = 0; k < splits; ++k)
             {
                 if (k == ks)
                     continue;
 #pragma unroll
                 for (int mi = 0; mi < WM; ++mi)
-                {
-                    v4i p4[WN][4];
 #pragma unroll
                     for (int ni = 0; ni < WN; ++ni)
 #pragma unroll
-                        for (int g = 0; g < 4; ++g)
-                            p4[ni][g] = __builtin_amdgcn_raw_buffer_load_b128(prs, k * (BM * BN * 4) + lane_off + ((mi * WN + ni) * 4 + g) * 1024, 0, kDeviceScope);
+                        for (int g0 = 0; g0 < 4; g0 += GB)
+                        {
+                            v4i p4[GB];
 #pragma unroll
-                    for (int ni = 0; ni < WN; ++ni)
+                            for (int g = 0; g < GB; ++g)
+                                p4[g] = __builtin_amdgcn_raw_buffer_load_b128(prs, k * (BM * BN * 4) + lane_off + ((mi * WN + ni) * 4 + g0 + g) * 1024, 0, kDeviceScope);
 #pragma unroll
-                        for (int g = 0; g < 4; ++g)
+                            for (int g = 0; g < GB; ++g)
 #pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                acc[mi][ni][4 * g + e] += p4[ni][g][e];
-                }
+                                for (int e = 0; e < 4; ++e)
+                                    acc[mi][ni][4 * (g0 + g) + e] += p4[g][e];
+                        }
             }
             return true;
         };
@@ -1419,7 +1444,12 @@ namespace hipq
                 multiply(buf);
                 HIPQ_PIPE_MARK(s, 2);
                 if (splits == 1 || (cm0 < M && gather_splits())) // uniform
-                    epilogue();
+                {
+                    if (kFold && bias_folded) // uniform
+                        epilogue(std::true_type{});
+                    else
+                        epilogue(std::false_type{});
+                }
                 ckt = 0;
                 if (++cj < my_tiles)
                     tile_origin(cj, cm0, cn0);
@@ -1475,7 +1505,12 @@ namespace hipq
                     multiply(cb);
                     HIPQ_PIPE_MARK(s, 2);
                     if (splits == 1 || gather_splits()) // uniform
-                        epilogue();
+                    {
+                    if (kFold && bias_folded) // uniform
+                        epilogue(std::true_type{});
+                    else
+                        epilogue(std::false_type{});
+                }
                     ckt = 0;
                     if (++cj < my_tiles)
                         tile_origin(cj, cm0, cn0);
@@ -1597,8 +1632,7 @@ namespace hipq
         const int64_t resident = static_cast<int64_t>(dev >= 0 && dev < 16 && cus[dev] > 0 ? cus[dev] : 256) * (160 * 1024 / lds_bytes);
         const int64_t tiles = m_tiles * n_tiles;
         // Few tiles with long reductions leave most of the chip idle: cut every reduction into
-        // `splits` runs of whole slices (at least four each) as long as the work items still find a
-        // compute unit each.
+        // `splits` runs of whole slices.
         int splits = 1;
         const int64_t slices = (Kred + BK - 1) / BK;
         const char* const split_env = getenv("HIPQ_SPLIT_K");
@@ -1608,8 +1642,14 @@ namespace hipq
             splits = want > 0 && (want & (want - 1)) == 0 && slices % want == 0 ? want : 1;
         }
         else
-            while (splits < 16 && tiles * splits * 2 <= (dev >= 0 && dev < 16 && cus[dev] > 0 ? cus[dev] : 256) && slices % (splits * 2) == 0 && slices / (splits * 2) >= 4)
+        {
+            // doubled while the items still find a compute unit each and keep four slices, or find
+            // a resident slot each and keep eight (the partial sums cost about two slices' time)
+            const int64_t units = dev >= 0 && dev < 16 && cus[dev] > 0 ? cus[dev] : 256;
+            while (splits < 16 && slices % (splits * 2) == 0 &&
+                   ((tiles * splits * 2 <= units && slices / (splits * 2) >= 4) || (tiles * splits * 2 <= resident && slices / (splits * 2) >= 8)))
                 splits *= 2;
+        }
         int32_t* partials = nullptr;
         uint32_t* counters = nullptr;
         if (splits > 1 && tiles * sizeof(uint32_t) <= kSplitCounterBytes)

@@ -476,6 +476,34 @@ SPLIT_CONV_SHAPES = [
 ]
 
 
+def test_conv_bias_in_accumulator(gpu_lib):
+    """short reductions add small biases to the accumulators as integers (exact: no float rounding
+    happens below 2^24); a column block holding a bias beyond 2^24 keeps the float add -- both kinds
+    in one call, with and without a residual, against the oracle"""
+    say("bias folding")
+    O.port().orc_set_threads(8)
+    N, Cc, K, sp = 2, 64, 256, (12, 11)
+    dn = H.make_conv_desc(N, Cc, K, sp, (1, 1), out_t="u8")
+    d = H.make_conv_desc(N, Cc, K, sp, (1, 1), out_t="u8", data_layout=H.NXC, out_layout=H.NXC)
+    data = synth.uniform_int(3100, dn.data_shape(), 0, 255, np.uint8)
+    filt = synth.uniform_int(3101, dn.filter_shape(), -127, 127, np.int8)
+    bias = synth.uniform_int(3102, (K,), -(2**24), 2**24, np.int32)
+    bias[5] = 2**24          # still exact
+    bias[7] = -(2**24)
+    bias[200] = 2**25 + 3    # second column block: rounds as a float, so that block must not fold
+    bias[201] = -(2**26) - 5
+    scales = synth.uniform_f32(3103, (K,), 2e-6, 6e-6)
+    for has_sum in (False, True):
+        summ = synth.uniform_int(3104, dn.out_shape(), 0, 255, np.uint8) if has_sum else None
+        f = H.make_fused_desc(has_bias=True, has_sum=has_sum, sum_t="u8", with_relu=True, scale_count=K)
+        exp = O.quantized_convolution_fused(dn, f, data, filt, bias, summ, scales, 0.21 if has_sum else None)
+        got = H.quantized_convolution_fused(d, f, cases.to_nxc(data), filt, bias, cases.to_nxc(summ) if has_sum else None, scales, 0.21 if has_sum else None)
+        assert H.last_kernel().startswith("conv_mfma"), H.last_kernel()
+        assert np.array_equal(cases.to_ncx(got), exp), has_sum
+        assert len(np.unique(exp)) > 50  # the outputs are spread, not saturated
+    O.port().orc_set_threads(1)
+
+
 @pytest.mark.parametrize("i", range(len(SPLIT_CONV_SHAPES)))
 def test_conv_loads_into_lds(gpu_lib, i, monkeypatch):
     """the same shapes through the kernels whose loads go straight into LDS (opt-in for filters

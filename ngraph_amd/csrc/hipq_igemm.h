@@ -1243,16 +1243,38 @@ namespace hipq
         constexpr int SUM_LOADS = TM * TN / 16 / 64;
         v4i sum_regs[SUM_LOADS];
         const __amdgpu_buffer_rsrc_t srs = make_rsrc(epi.sum_in, has_sum ? static_cast<uint32_t>(M * N) : 0u);
+        const v4i srs_words = rsrc_words(epi.sum_in, has_sum ? static_cast<uint32_t>(M * N) : 0u);
+        const uint32_t ostage_lds = lds_address(lds) + NSTAGE * STAGE + static_cast<uint32_t>(wave) * OUT_STAGE;
+        bool loads_behind_sum = false; // DMA: operand loads were issued after the residual's
         auto sum_fetch = [&]() {
-#pragma unroll
-            for (int i = 0; i < SUM_LOADS; ++i)
+            if constexpr (DMA)
             {
-                const int id = i * 64 + lane;
-                const int row = id >> 2;
-                const int piece = id & 3;
-                const int64_t m = cm0 + wm * TM + row;
-                const int32_t n = cn0 + wn * TN + piece * 16;
-                sum_regs[i] = buffer_load16(srs, (m < M && n < N) ? static_cast<int32_t>(m * N + n) : kOob);
+                // straight into the wavefront's staging region, in the layout the epilogue reads: the
+                // lane's slot is piece id % 4 of row id / 4, so it fetches the piece that belongs there
+                const uint32_t base = __builtin_amdgcn_readfirstlane(ostage_lds);
+#pragma unroll
+                for (int i = 0; i < SUM_LOADS; ++i)
+                {
+                    const int id = i * 64 + lane;
+                    const int row = id >> 2;
+                    const int piece = (id & 3) ^ ((row >> 2) & 3);
+                    const int64_t m = cm0 + wm * TM + row;
+                    const int32_t n = cn0 + wn * TN + piece * 16;
+                    lds_dma16(srs_words, (m < M && n < N) ? static_cast<int32_t>(m * N + n) : kOob, base + i * 1024);
+                }
+            }
+            else
+            {
+#pragma unroll
+                for (int i = 0; i < SUM_LOADS; ++i)
+                {
+                    const int id = i * 64 + lane;
+                    const int row = id >> 2;
+                    const int piece = id & 3;
+                    const int64_t m = cm0 + wm * TM + row;
+                    const int32_t n = cn0 + wn * TN + piece * 16;
+                    sum_regs[i] = buffer_load16(srs, (m < M && n < N) ? static_cast<int32_t>(m * N + n) : kOob);
+                }
             }
         };
         auto epilogue = [&](auto folded) {
@@ -1261,16 +1283,26 @@ namespace hipq
             if (has_sum)
             {
                 // the residual input of the sub-tile comes in the way the output leaves: 16 bytes a
-                // lane along the rows (fetched into registers before the tile's last slice was
-                // multiplied), through the staging region; each lane then picks up the dword that its
-                // own output dword will replace
-#pragma unroll
-                for (int i = 0; i < SUM_LOADS; ++i)
+                // lane along the rows, fetched before the tile's last slice was multiplied -- into
+                // registers and from there into the staging region, or (DMA) straight into it; each
+                // lane then picks up the dword that its own output dword will replace
+                if constexpr (DMA)
                 {
-                    const int id = i * 64 + lane;
-                    const int row = id >> 2;
-                    const int piece = id & 3;
-                    *reinterpret_cast<v4i*>(ostage + row * TN + ((piece ^ ((row >> 2) & 3)) << 4)) = sum_regs[i];
+                    if (loads_behind_sum) // uniform
+                        wait_vmcnt<XLOADS + WLOADS>();
+                    else
+                        wait_vmcnt<0>();
+                }
+                else
+                {
+#pragma unroll
+                    for (int i = 0; i < SUM_LOADS; ++i)
+                    {
+                        const int id = i * 64 + lane;
+                        const int row = id >> 2;
+                        const int piece = id & 3;
+                        *reinterpret_cast<v4i*>(ostage + row * TN + ((piece ^ ((row >> 2) & 3)) << 4)) = sum_regs[i];
+                    }
                 }
             }
 #pragma unroll
@@ -1494,14 +1526,15 @@ namespace hipq
             for (int s = 0; s < total; ++s)
             {
                 HIPQ_PIPE_MARK(s, 0);
+                const bool tile_done = ckt + 1 == KT;
+                if (has_sum && tile_done) // uniform; ahead of the operand loads, so that waiting for it leaves them in flight
+                    sum_fetch();
+                loads_behind_sum = s + 2 < total;
                 if (s + 2 < total) // uniform
                     oob_new = dma_load(lb);
                 HIPQ_PIPE_MARK(s, 1);
-                const bool tile_done = ckt + 1 == KT;
                 if (tile_done) // uniform
                 {
-                    if (has_sum)
-                        sum_fetch();
                     multiply(cb);
                     HIPQ_PIPE_MARK(s, 2);
                     if (splits == 1 || gather_splits()) // uniform

@@ -197,6 +197,36 @@ def bench_glue(lib, stream, timer, steps, warmup, batch=128):
     return out
 
 
+def bench_fp32_glue(lib, stream, timer, steps, warmup):
+    """fp32 glue of a BERT-base encoder layer between its quantized projections (batch 32, sequence 128):
+    attention softmax f32[32*12*128, 128], Gelu f32[4096, 3072], LayerNorm f32[4096, 768] with affine and stats"""
+    f, vp, i64 = C.c_float, C.c_void_p, C.c_int64
+    lib.hipq_softmax_f32.argtypes = [vp, vp, i64, i64, i64, vp]
+    lib.hipq_gelu_f32.argtypes = [vp, vp, i64, vp]
+    lib.hipq_layer_norm_f32.argtypes = [vp] * 6 + [i64, i64, C.c_double, vp]
+    n_max = 4096 * 3072
+    src = dev(synth.normal_f32(31, (n_max,)))
+    dst = H.DeviceBuffer(n_max * 4)
+    scale, bias = dev(synth.uniform_f32(32, (768,), 0.5, 1.5)), dev(synth.uniform_f32(33, (768,), -0.5, 0.5))
+    mean, var = H.DeviceBuffer(4096 * 4), H.DeviceBuffer(4096 * 4)
+    ops = {
+        "softmax_f32[49152,128]": (lambda: lib.hipq_softmax_f32(src.ptr, dst.ptr, 32 * 12 * 128, 128, 1, stream), 32 * 12 * 128 * 128),
+        "gelu_f32[4096,3072]": (lambda: lib.hipq_gelu_f32(src.ptr, dst.ptr, n_max, stream), n_max),
+        "layer_norm_f32[4096,768]": (lambda: lib.hipq_layer_norm_f32(src.ptr, scale.ptr, bias.ptr, dst.ptr, mean.ptr, var.ptr, 4096, 768, 1e-5, stream), 4096 * 768),
+    }
+    out = []
+    for name, (fn, n) in ops.items():
+        def step():
+            rc = fn()
+            if rc:
+                H.check(rc)
+
+        _, ev = timer.run(step, steps, warmup)
+        gbs = 8 * n / (ev * 1e-3) / 1e9  # one f32 read, one f32 written per element
+        out.append(dict(op=name, elements=n, ms_event=ev, gbs=gbs, frac_hbm=gbs / PEAK_HBM_GBS, kernel=H.last_kernel()))
+    return out
+
+
 def bench_resnet50(lib, stream, timer, batches=(1, 32, 128)):
     """synthetic int8 ResNet-50 (ngraph_amd/resnet50.py), every tensor resident in HBM, channels-last,
     one forward pass = 53 convolutions, 2 pools, 1 GEMM; replayed as one HIP graph"""
@@ -323,6 +353,7 @@ def main():
         results["quantize_dequantize_config3"] = bench_qdq(lib, stream, timer, small, 5)
         results["pool_resnet50_u8"] = bench_pool(lib, stream, timer, small, 5, args.batch)
         results["glue_resnet50_u8"] = bench_glue(lib, stream, timer, small, 5, args.batch)
+        results["fp32_glue_bert_base"] = bench_fp32_glue(lib, stream, timer, small, 5)
         results["resnet50_int8"] = bench_resnet50(lib, stream, timer)
         cpu = cpu_baseline()
 

@@ -429,6 +429,40 @@ HIPQ_API int hipq_concat(int32_t elem_bytes,
                          void* out,
                          void* stream);
 
+/* ---- fp32 glue of a transformer encoder (between the quantized projections) ----------------------
+ * Floating point: results agree with the reference's to 1e-5 relative (the reference sums
+ * sequentially with Kahan compensation, src/ngraph/runtime/reference/sum.hpp:56-88, and calls the
+ * host's expf / erff; the kernels reduce in parallel and call the device's). */
+
+/* op::v0::Softmax over a contiguous run of axes, the tensor seen as [outer][axis][inner]:
+ * out = exp(x - max) / sum(exp(x - max)) along `axis`
+ * (src/ngraph/runtime/reference/softmax.hpp:31-57). */
+HIPQ_API int hipq_softmax_f32(const float* in, float* out, int64_t outer, int64_t axis, int64_t inner, void* stream);
+
+/* op::v0::Erf (src/ngraph/runtime/reference/erf.hpp:29-35). */
+HIPQ_API int hipq_erf_f32(const float* in, float* out, int64_t count, void* stream);
+
+/* op::v0::Gelu as FusedOpDecomposition lowers it (src/ngraph/op/gelu.cpp:46-60):
+ * (0.5 * x) * (1 + erf(x / sqrt(2))), every step in f32. */
+HIPQ_API int hipq_gelu_f32(const float* in, float* out, int64_t count, void* stream);
+
+/* op::v0::LayerNorm forward as it decomposes (src/ngraph/op/layer_norm.cpp:68-150,
+ * src/ngraph/builder/reduce_ops.cpp:68-124): the tensor is [rows][cols] with cols the product of the
+ * normalised trailing axes; mean = sum(x) / cols, var = sum((x - mean)^2) / cols,
+ * out = (x - mean) / sqrt(var + epsilon) * scale + bias.  scale and bias ([cols]) may both be null
+ * (use_affine = false); mean and var ([rows]) may be null (keep_stats = false). */
+HIPQ_API int hipq_layer_norm_f32(const float* in,
+                                 const float* scale,
+                                 const float* bias,
+                                 float* out,
+                                 float* mean,
+                                 float* var,
+                                 int64_t rows,
+                                 int64_t cols,
+                                 double epsilon,
+                                 void* stream);
+
+
 /* Which kernel the last hipq_quantized_* call on this thread used: "mfma", "direct", ... (host
  * string, never NULL).  For tests and profiles. */
 HIPQ_API const char* hipq_last_kernel(void);

@@ -1,0 +1,351 @@
+// fp32 glue of a transformer encoder between the quantized projections: Softmax, Erf, Gelu,
+// LayerNorm.  All of them stream their tensors once through HBM; a row (the normalised axis) is
+// owned by one wavefront and kept in registers when it has at most 2048 elements.
+#include <cmath>
+
+#include "hipq_common.h"
+
+namespace hipq
+{
+    namespace
+    {
+        typedef float f4 __attribute__((ext_vector_type(4)));
+
+        // reductions over aligned groups of W lanes of a wavefront
+        template <int W = 64>
+        __device__ __forceinline__ float wave_max(float v)
+        {
+#pragma unroll
+            for (int o = W / 2; o > 0; o >>= 1)
+                v = fmaxf(v, __shfl_xor(v, o));
+            return v;
+        }
+        template <int W = 64>
+        __device__ __forceinline__ float wave_sum(float v)
+        {
+#pragma unroll
+            for (int o = W / 2; o > 0; o >>= 1)
+                v += __shfl_xor(v, o);
+            return v;
+        }
+
+        constexpr int kRowVecs = 8; // float4 pieces of a row a lane keeps: rows up to 64 * 4 * 8 = 2048 elements
+
+        // out = exp(x - max(x)) / sum(exp(x - max(x))) along contiguous rows
+        // (src/ngraph/runtime/reference/softmax.hpp:31-57); one wavefront a row.
+        template <bool CACHED>
+        __global__ __launch_bounds__(256) void softmax_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int64_t rows, int32_t cols)
+        {
+            const int lane = threadIdx.x & 63;
+            const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+            if (row >= rows)
+                return;
+            const float* x = in + row * cols;
+            float* y = out + row * cols;
+            if (CACHED) // cols % 4 == 0, 16-byte aligned rows, cols <= 2048
+            {
+                const int vecs = cols >> 2;
+                f4 v[kRowVecs];
+                float m = -INFINITY;
+#pragma unroll
+                for (int i = 0; i < kRowVecs; ++i)
+                {
+                    const int j = i * 64 + lane;
+                    if (j < vecs)
+                    {
+                        v[i] = reinterpret_cast<const f4*>(x)[j];
+                        m = fmaxf(fmaxf(fmaxf(m, v[i][0]), fmaxf(v[i][1], v[i][2])), v[i][3]);
+                    }
+                }
+                m = wave_max(m);
+                float s = 0.0f;
+#pragma unroll
+                for (int i = 0; i < kRowVecs; ++i)
+                    if (i * 64 + lane < vecs)
+                    {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                        {
+                            v[i][e] = expf(v[i][e] - m);
+                            s += v[i][e];
+                        }
+                    }
+                s = wave_sum(s);
+#pragma unroll
+                for (int i = 0; i < kRowVecs; ++i)
+                {
+                    const int j = i * 64 + lane;
+                    if (j < vecs)
+                        reinterpret_cast<f4*>(y)[j] = f4{v[i][0] / s, v[i][1] / s, v[i][2] / s, v[i][3] / s};
+                }
+            }
+            else
+            {
+                float m = -INFINITY;
+                for (int j = lane; j < cols; j += 64)
+                    m = fmaxf(m, x[j]);
+                m = wave_max(m);
+                float s = 0.0f;
+                for (int j = lane; j < cols; j += 64)
+                    s += expf(x[j] - m);
+                s = wave_sum(s);
+                for (int j = lane; j < cols; j += 64)
+                    y[j] = expf(x[j] - m) / s;
+            }
+        }
+
+        // short rows (at most W float4 pieces, W = 32, 16 or 8 lanes): 64 / W rows a wavefront, one
+        // piece a lane, so that every lane has work (an attention row of 128 is 32 pieces)
+        template <int W>
+        __global__ __launch_bounds__(256) void softmax_short_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int64_t rows, int32_t cols)
+        {
+            constexpr int RPW = 64 / W;
+            const int lane = threadIdx.x & 63;
+            const int sub = lane & (W - 1);
+            const int64_t row = (static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6)) * RPW + lane / W;
+            const int vecs = cols >> 2;
+            const bool live = row < rows && sub < vecs;
+            f4 v = f4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+            if (live)
+                v = reinterpret_cast<const f4*>(in + row * cols)[sub];
+            const float m = wave_max<W>(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
+            float s = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+            {
+                v[e] = live ? expf(v[e] - m) : 0.0f;
+                s += v[e];
+            }
+            s = wave_sum<W>(s);
+            if (live)
+                reinterpret_cast<f4*>(out + row * cols)[sub] = f4{v[0] / s, v[1] / s, v[2] / s, v[3] / s};
+        }
+
+        // the same over a strided axis: the tensor is [outer][axis][inner], one lane a column (o, i)
+        __global__ __launch_bounds__(256) void softmax_strided_kernel(const float* __restrict__ in, float* __restrict__ out, int64_t outer, int32_t axis, int64_t inner)
+        {
+            const int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+            if (t >= outer * inner)
+                return;
+            const int64_t o = t / inner, i = t - o * inner;
+            const float* x = in + o * axis * inner + i;
+            float* y = out + o * axis * inner + i;
+            float m = -INFINITY;
+            for (int a = 0; a < axis; ++a)
+                m = fmaxf(m, x[a * inner]);
+            float s = 0.0f;
+            for (int a = 0; a < axis; ++a)
+                s += expf(x[a * inner] - m);
+            for (int a = 0; a < axis; ++a)
+                y[a * inner] = expf(x[a * inner] - m) / s;
+        }
+
+        // Gelu as the reference decomposes it (src/ngraph/op/gelu.cpp:46-60):
+        // (0.5 * x) * (1 + erf(x / float(sqrt(2.0)))), every step rounded to f32
+        __device__ __forceinline__ float gelu1(float x)
+        {
+            const float sqrt_two = 1.41421354f; // float(std::sqrt(2.0))
+            return __fmul_rn(__fmul_rn(0.5f, x), __fadd_rn(1.0f, erff(__fdiv_rn(x, sqrt_two))));
+        }
+
+        template <bool GELU>
+        __global__ __launch_bounds__(256) void erf_kernel(const float* __restrict__ in, float* __restrict__ out, int64_t count, int32_t vec_ok)
+        {
+            const int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+            if (vec_ok)
+            {
+                if (t * 4 >= count)
+                    return;
+                const f4 v = reinterpret_cast<const f4*>(in)[t];
+                f4 r;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    r[e] = GELU ? gelu1(v[e]) : erff(v[e]);
+                reinterpret_cast<f4*>(out)[t] = r;
+            }
+            else if (t < count)
+                out[t] = GELU ? gelu1(in[t]) : erff(in[t]);
+        }
+
+        // LayerNorm over the trailing `cols` elements of every row, as the reference decomposes it
+        // (src/ngraph/op/layer_norm.cpp:96-139 with builder::mean / builder::variance,
+        // src/ngraph/builder/reduce_ops.cpp:68-124): mean = sum(x) / n, var = sum((x - mean)^2) / n,
+        // out = (x - mean) / sqrt(var + eps) * scale + bias.  One wavefront a row.
+        template <bool CACHED>
+        __global__ __launch_bounds__(256) void layer_norm_kernel(const float* __restrict__ in, const float* __restrict__ scale, const float* __restrict__ bias, float* __restrict__ out,
+                                                                 float* __restrict__ mean_out, float* __restrict__ var_out, int64_t rows, int32_t cols, float eps)
+        {
+            const int lane = threadIdx.x & 63;
+            const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+            if (row >= rows)
+                return;
+            const float* x = in + row * cols;
+            float* y = out + row * cols;
+            const float n = static_cast<float>(cols);
+            if (CACHED)
+            {
+                const int vecs = cols >> 2;
+                f4 v[kRowVecs];
+                float s = 0.0f;
+#pragma unroll
+                for (int i = 0; i < kRowVecs; ++i)
+                    if (i * 64 + lane < vecs)
+                    {
+                        v[i] = reinterpret_cast<const f4*>(x)[i * 64 + lane];
+                        s += (v[i][0] + v[i][1]) + (v[i][2] + v[i][3]);
+                    }
+                const float mean = __fdiv_rn(wave_sum(s), n);
+                float q = 0.0f;
+#pragma unroll
+                for (int i = 0; i < kRowVecs; ++i)
+                    if (i * 64 + lane < vecs)
+                    {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                        {
+                            v[i][e] = v[i][e] - mean;
+                            q = fmaf(v[i][e], v[i][e], q);
+                        }
+                    }
+                const float var = __fdiv_rn(wave_sum(q), n);
+                const float sd = sqrtf(var + eps);
+#pragma unroll
+                for (int i = 0; i < kRowVecs; ++i)
+                {
+                    const int j = i * 64 + lane;
+                    if (j < vecs)
+                    {
+                        f4 r;
+                        const f4 sc = scale ? reinterpret_cast<const f4*>(scale)[j] : f4{1.0f, 1.0f, 1.0f, 1.0f};
+                        const f4 bi = scale ? reinterpret_cast<const f4*>(bias)[j] : f4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                        {
+                            const float nv = __fdiv_rn(v[i][e], sd);
+                            r[e] = scale ? __fadd_rn(__fmul_rn(nv, sc[e]), bi[e]) : nv;
+                        }
+                        reinterpret_cast<f4*>(y)[j] = r;
+                    }
+                }
+                if (lane == 0)
+                {
+                    if (mean_out)
+                        mean_out[row] = mean;
+                    if (var_out)
+                        var_out[row] = var;
+                }
+            }
+            else
+            {
+                float s = 0.0f;
+                for (int j = lane; j < cols; j += 64)
+                    s += x[j];
+                const float mean = __fdiv_rn(wave_sum(s), n);
+                float q = 0.0f;
+                for (int j = lane; j < cols; j += 64)
+                {
+                    const float d = x[j] - mean;
+                    q = fmaf(d, d, q);
+                }
+                const float var = __fdiv_rn(wave_sum(q), n);
+                const float sd = sqrtf(var + eps);
+                for (int j = lane; j < cols; j += 64)
+                {
+                    const float nv = __fdiv_rn(x[j] - mean, sd);
+                    y[j] = scale ? __fadd_rn(__fmul_rn(nv, scale[j]), bias[j]) : nv;
+                }
+                if (lane == 0)
+                {
+                    if (mean_out)
+                        mean_out[row] = mean;
+                    if (var_out)
+                        var_out[row] = var;
+                }
+            }
+        }
+
+        bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+    }
+}
+
+using namespace hipq;
+
+int hipq_softmax_f32(const float* in, float* out, int64_t outer, int64_t axis, int64_t inner, void* stream)
+{
+    HIPQ_REQUIRE(outer >= 0 && axis >= 0 && inner >= 0, "negative extent");
+    if (outer == 0 || axis == 0 || inner == 0)
+        return HIPQ_OK;
+    HIPQ_REQUIRE(in && out, "null pointer");
+    HIPQ_REQUIRE(axis < (1ll << 31) && outer * inner < (1ll << 40), "tensor too large for one launch");
+    hipStream_t s = as_stream(stream);
+    if (inner == 1)
+    {
+        const bool cached = axis % 4 == 0 && axis <= 64 * 4 * kRowVecs && aligned16(in) && aligned16(out);
+        if (cached && axis <= 128)
+        {
+            const int w = axis > 64 ? 32 : (axis > 32 ? 16 : 8);
+            const int64_t rows_per_block = 4 * (64 / w);
+            const unsigned blocks = static_cast<unsigned>((outer + rows_per_block - 1) / rows_per_block);
+            if (w == 32)
+                softmax_short_rows_kernel<32><<<blocks, 256, 0, s>>>(in, out, outer, static_cast<int32_t>(axis));
+            else if (w == 16)
+                softmax_short_rows_kernel<16><<<blocks, 256, 0, s>>>(in, out, outer, static_cast<int32_t>(axis));
+            else
+                softmax_short_rows_kernel<8><<<blocks, 256, 0, s>>>(in, out, outer, static_cast<int32_t>(axis));
+            return check_launch("softmax_rows");
+        }
+        const unsigned grid = static_cast<unsigned>((outer + 3) / 4);
+        if (cached)
+            softmax_rows_kernel<true><<<grid, 256, 0, s>>>(in, out, outer, static_cast<int32_t>(axis));
+        else
+            softmax_rows_kernel<false><<<grid, 256, 0, s>>>(in, out, outer, static_cast<int32_t>(axis));
+        return check_launch("softmax_rows");
+    }
+    softmax_strided_kernel<<<static_cast<unsigned>((outer * inner + 255) / 256), 256, 0, s>>>(in, out, outer, static_cast<int32_t>(axis), inner);
+    return check_launch("softmax_strided");
+}
+
+static int launch_erf(const float* in, float* out, int64_t count, void* stream, bool gelu)
+{
+    HIPQ_REQUIRE(count >= 0, "negative count");
+    if (count == 0)
+        return HIPQ_OK;
+    HIPQ_REQUIRE(in && out, "null pointer");
+    const bool vec = count % 4 == 0 && aligned16(in) && aligned16(out);
+    const int64_t lanes = vec ? count / 4 : count;
+    HIPQ_REQUIRE((lanes + 255) / 256 < (1ll << 31), "tensor too large for one launch");
+    const unsigned grid = static_cast<unsigned>((lanes + 255) / 256);
+    if (gelu)
+        erf_kernel<true><<<grid, 256, 0, as_stream(stream)>>>(in, out, count, vec ? 1 : 0);
+    else
+        erf_kernel<false><<<grid, 256, 0, as_stream(stream)>>>(in, out, count, vec ? 1 : 0);
+    return check_launch(gelu ? "gelu_vec" : "erf_vec");
+}
+
+int hipq_erf_f32(const float* in, float* out, int64_t count, void* stream)
+{
+    return launch_erf(in, out, count, stream, false);
+}
+
+int hipq_gelu_f32(const float* in, float* out, int64_t count, void* stream)
+{
+    return launch_erf(in, out, count, stream, true);
+}
+
+int hipq_layer_norm_f32(const float* in, const float* scale, const float* bias, float* out, float* mean, float* var, int64_t rows, int64_t cols, double epsilon, void* stream)
+{
+    HIPQ_REQUIRE(rows >= 0 && cols >= 0, "negative extent");
+    if (rows == 0 || cols == 0)
+        return HIPQ_OK;
+    HIPQ_REQUIRE(in && out, "null pointer");
+    HIPQ_REQUIRE((scale == nullptr) == (bias == nullptr), "scale and bias come together");
+    HIPQ_REQUIRE(cols < (1ll << 31) && (rows + 3) / 4 < (1ll << 31), "tensor too large for one launch");
+    const bool cached = cols % 4 == 0 && cols <= 64 * 4 * kRowVecs && aligned16(in) && aligned16(out) && (!scale || (aligned16(scale) && aligned16(bias)));
+    const unsigned grid = static_cast<unsigned>((rows + 3) / 4);
+    hipStream_t s = as_stream(stream);
+    if (cached)
+        layer_norm_kernel<true><<<grid, 256, 0, s>>>(in, scale, bias, out, mean, var, rows, static_cast<int32_t>(cols), static_cast<float>(epsilon));
+    else
+        layer_norm_kernel<false><<<grid, 256, 0, s>>>(in, scale, bias, out, mean, var, rows, static_cast<int32_t>(cols), static_cast<float>(epsilon));
+    return check_launch("layer_norm_rows");
+}

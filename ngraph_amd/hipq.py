@@ -295,6 +295,10 @@ EXPORTS = [
     "hipq_pool",
     "hipq_concat",
     "hipq_last_kernel",
+    "hipq_softmax_f32",
+    "hipq_erf_f32",
+    "hipq_gelu_f32",
+    "hipq_layer_norm_f32",
 ]
 
 _lib = None
@@ -619,3 +623,66 @@ def quantized_dot_bias(desc, fused, a, w, bias, scale, prepare=True):
     )
     check(lib.hipq_stream_sync(None))
     return out.to_numpy(NP_OF[desc.out_t], (int(desc.M), int(desc.N)))
+
+
+# ---- fp32 glue of a transformer encoder -----------------------------------------------------------
+
+def _axes_run(shape, axes):
+    """(outer, axis, inner) of a contiguous run of axes (all axes when `axes` is empty, as op::v0::Softmax reads it)"""
+    rank = len(shape)
+    axes = sorted(set(range(rank)) if len(axes) == 0 else set(axes))
+    if axes != list(range(axes[0], axes[-1] + 1)):
+        raise ValueError("the library takes a contiguous run of axes")
+    outer = int(np.prod(shape[: axes[0]], dtype=np.int64))
+    axis = int(np.prod(shape[axes[0] : axes[-1] + 1], dtype=np.int64))
+    inner = int(np.prod(shape[axes[-1] + 1 :], dtype=np.int64))
+    return outer, axis, inner
+
+
+def softmax(x, axes=()):
+    lib = load()
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    outer, axis, inner = _axes_run(x.shape, axes)
+    src, dst = _dev(x), DeviceBuffer(max(x.nbytes, 4))
+    lib.hipq_softmax_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_void_p]
+    check(lib.hipq_softmax_f32(src.ptr, dst.ptr, outer, axis, inner, None))
+    check(lib.hipq_stream_sync(None))
+    return dst.to_numpy(np.float32, x.shape)
+
+
+def _unary_f32(name, x):
+    lib = load()
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    src, dst = _dev(x), DeviceBuffer(max(x.nbytes, 4))
+    fn = getattr(lib, name)
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
+    check(fn(src.ptr, dst.ptr, x.size, None))
+    check(lib.hipq_stream_sync(None))
+    return dst.to_numpy(np.float32, x.shape)
+
+
+def erf(x):
+    return _unary_f32("hipq_erf_f32", x)
+
+
+def gelu(x):
+    return _unary_f32("hipq_gelu_f32", x)
+
+
+def layer_norm(x, scale=None, bias=None, begin_norm_axis=1, epsilon=1e-5, keep_stats=True):
+    """op::v0::LayerNorm forward: returns (norm, mean, var), mean and var None without keep_stats"""
+    lib = load()
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    n_axis = begin_norm_axis if begin_norm_axis >= 0 else x.ndim + begin_norm_axis
+    rows = int(np.prod(x.shape[:n_axis], dtype=np.int64))
+    cols = int(np.prod(x.shape[n_axis:], dtype=np.int64))
+    src, dst = _dev(x), DeviceBuffer(max(x.nbytes, 4))
+    sc = _dev(np.ascontiguousarray(scale, dtype=np.float32)) if scale is not None else None
+    bi = _dev(np.ascontiguousarray(bias, dtype=np.float32)) if bias is not None else None
+    mean = DeviceBuffer(max(rows, 1) * 4) if keep_stats else None
+    var = DeviceBuffer(max(rows, 1) * 4) if keep_stats else None
+    lib.hipq_layer_norm_f32.argtypes = [C.c_void_p] * 6 + [C.c_int64, C.c_int64, C.c_double, C.c_void_p]
+    check(lib.hipq_layer_norm_f32(src.ptr, sc.ptr if sc else None, bi.ptr if bi else None, dst.ptr, mean.ptr if mean else None, var.ptr if var else None, rows, cols, float(epsilon), None))
+    check(lib.hipq_stream_sync(None))
+    stats_shape = x.shape[:n_axis]
+    return (dst.to_numpy(np.float32, x.shape), mean.to_numpy(np.float32, stats_shape) if keep_stats else None, var.to_numpy(np.float32, stats_shape) if keep_stats else None)

@@ -30,6 +30,13 @@
  *                                   scales, |acc+bias| > 2^24, fused-multiply-add of the sum term)
  *                                   PARITY IS UNPINNED and defined by the closed form below.
  *   orc_get_*scale                  the same builder tests (they feed min/max, not scales).
+ *   orc_softmax_f32, orc_erf_f32    the compiled reference templates (oracle/_ref: softmax.hpp, sum.hpp,
+ *                                   erf.hpp) bit for bit on seeded tensors, and the closed-form
+ *                                   expectations of test/backend/softmax.in.cpp:66-293.
+ *   orc_gelu_f32                    the formula the reference's own test evaluates
+ *                                   (test/backend/gelu.in.cpp:73-75) and its f64 points (:89-95).
+ *   orc_layer_norm_f32              the literal vectors of test/backend/layer_norm.in.cpp:48-91; its
+ *                                   sums against the compiled reference sum (oracle/_ref).
  */
 #include "../include/hipq.h"
 
@@ -830,4 +837,120 @@ ORC_API int orc_concat(int elem_bytes, int n_inputs, const void* const* inputs, 
 ORC_API size_t orc_dtype_size(int t)
 {
     return dtype_size(t);
+}
+
+
+/* ---- fp32 glue of a transformer encoder ---------------------------------------------------------- */
+
+/* src/ngraph/runtime/reference/sum.hpp:56-88: sequential, Kahan-compensated while both operands are finite */
+static void kahan_add(float* z, float* c, float x)
+{
+    if (isfinite(x) && isfinite(*z))
+    {
+        volatile float y = x - *c;
+        volatile float t = *z + y;
+        *c = (t - *z) - y;
+        *z = t;
+    }
+    else
+        *z = *z + x;
+}
+
+/* src/ngraph/runtime/reference/softmax.hpp:31-57 on a tensor seen as [outer][axis][inner]:
+ * max over the axis (reference/max.hpp: starts from -inf, keeps the larger), exp(x - max) with the
+ * host's expf, the compensated sum above in row-major input order, then the division. */
+ORC_API int orc_softmax_f32(const float* in, float* out, int64_t outer, int64_t axis, int64_t inner)
+{
+    if (outer < 0 || axis < 0 || inner < 0)
+        return HIPQ_ERR_INVALID;
+#pragma omp parallel for num_threads(g_threads) if (g_threads > 1)
+    for (int64_t o = 0; o < outer; ++o)
+        for (int64_t i = 0; i < inner; ++i)
+        {
+            const float* x = in + o * axis * inner + i;
+            float* y = out + o * axis * inner + i;
+            float m = -INFINITY;
+            for (int64_t a = 0; a < axis; ++a)
+                if (x[a * inner] > m)
+                    m = x[a * inner];
+            float z = 0.0f, c = 0.0f;
+            for (int64_t a = 0; a < axis; ++a)
+            {
+                y[a * inner] = expf(x[a * inner] - m);
+                kahan_add(&z, &c, y[a * inner]);
+            }
+            for (int64_t a = 0; a < axis; ++a)
+                y[a * inner] = y[a * inner] / z;
+        }
+    return HIPQ_OK;
+}
+
+/* src/ngraph/runtime/reference/erf.hpp:29-35 */
+ORC_API int orc_erf_f32(const float* in, float* out, int64_t count)
+{
+    for (int64_t i = 0; i < count; ++i)
+        out[i] = erff(in[i]);
+    return HIPQ_OK;
+}
+
+/* src/ngraph/op/gelu.cpp:46-60: half * data * (one + Erf(data / sqrt_two)) with f32 constants
+ * (sqrt_two = float(std::sqrt(2.0))), every node rounding to f32 */
+ORC_API int orc_gelu_f32(const float* in, float* out, int64_t count)
+{
+    const float sqrt_two = (float)sqrt(2.0);
+    for (int64_t i = 0; i < count; ++i)
+    {
+        volatile float t = in[i] / sqrt_two;
+        volatile float e = 1.0f + erff(t);
+        volatile float h = 0.5f * in[i];
+        out[i] = h * e;
+    }
+    return HIPQ_OK;
+}
+
+/* src/ngraph/op/layer_norm.cpp:96-139 with builder::mean and builder::variance
+ * (src/ngraph/builder/reduce_ops.cpp:68-124): mean = Sum(x) / n; var = Sum((x - mean)^2) / n, both
+ * sums compensated as above; norm = (x - mean) / sqrt(var + eps); affine: norm * scale + bias */
+ORC_API int orc_layer_norm_f32(const float* in, const float* scale, const float* bias, float* out, float* mean, float* var, int64_t rows, int64_t cols, double epsilon)
+{
+    if (rows < 0 || cols < 0 || ((scale == NULL) != (bias == NULL)))
+        return HIPQ_ERR_INVALID;
+    const float n = (float)cols, eps = (float)epsilon;
+#pragma omp parallel for num_threads(g_threads) if (g_threads > 1)
+    for (int64_t r = 0; r < rows; ++r)
+    {
+        const float* x = in + r * cols;
+        float z = 0.0f, c = 0.0f;
+        for (int64_t j = 0; j < cols; ++j)
+            kahan_add(&z, &c, x[j]);
+        const float mu = z / n;
+        z = 0.0f;
+        c = 0.0f;
+        for (int64_t j = 0; j < cols; ++j)
+        {
+            volatile float d = x[j] - mu;
+            volatile float dd = d * d;
+            kahan_add(&z, &c, dd);
+        }
+        const float v = z / n;
+        volatile float ve = v + eps;
+        const float sd = sqrtf(ve);
+        for (int64_t j = 0; j < cols; ++j)
+        {
+            volatile float d = x[j] - mu;
+            volatile float nv = d / sd;
+            if (scale)
+            {
+                volatile float p = nv * scale[j];
+                out[r * cols + j] = p + bias[j];
+            }
+            else
+                out[r * cols + j] = nv;
+        }
+        if (mean)
+            mean[r] = mu;
+        if (var)
+            var[r] = v;
+    }
+    return HIPQ_OK;
 }

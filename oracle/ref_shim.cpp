@@ -15,7 +15,10 @@
 #include "ngraph/runtime/reference/dequantize.hpp"
 #include "ngraph/runtime/reference/dot.hpp"
 #include "ngraph/runtime/reference/max_pool.hpp"
+#include "ngraph/runtime/reference/erf.hpp"
 #include "ngraph/runtime/reference/quantize.hpp"
+#include "ngraph/runtime/reference/softmax.hpp"
+#include "ngraph/runtime/reference/sum.hpp"
 #include "ngraph/shape.hpp"
 #include "ngraph/strides.hpp"
 
@@ -335,6 +338,50 @@ __attribute__((visibility("default"))) int ref_pool(int op,
     {
         return -2;
     }
+    return 0;
+}
+
+// runtime::reference::softmax<float> over the axes whose bit is set in axes_mask
+__attribute__((visibility("default"))) int ref_softmax_f32(const float* in, float* out, const int64_t* shape, int rank, uint32_t axes_mask)
+{
+    Shape sh = make_shape(shape, rank);
+    AxisSet axes;
+    for (int i = 0; i < rank; ++i)
+        if (axes_mask & (1u << i))
+            axes.insert(static_cast<size_t>(i));
+    try
+    {
+        runtime::reference::softmax<float>(in, out, sh, axes);
+    }
+    catch (const std::exception&)
+    {
+        return -2;
+    }
+    return 0;
+}
+
+// runtime::reference::sum<float> (the Kahan-compensated sequential sum LayerNorm's mean and variance use)
+__attribute__((visibility("default"))) int ref_sum_f32(const float* in, float* out, const int64_t* shape, int rank, uint32_t axes_mask)
+{
+    Shape sh = make_shape(shape, rank);
+    AxisSet axes;
+    for (int i = 0; i < rank; ++i)
+        if (axes_mask & (1u << i))
+            axes.insert(static_cast<size_t>(i));
+    try
+    {
+        runtime::reference::sum<float>(in, out, sh, axes);
+    }
+    catch (const std::exception&)
+    {
+        return -2;
+    }
+    return 0;
+}
+
+__attribute__((visibility("default"))) int ref_erf_f32(const float* in, float* out, int64_t count)
+{
+    runtime::reference::erf<float>(in, out, static_cast<size_t>(count));
     return 0;
 }
 }

@@ -49,6 +49,10 @@ def port():
         lib.orc_get_dot_scale.argtypes = [f] * 6 + [C.c_int] * 3
         lib.orc_get_conv_requant_scale.restype = f
         lib.orc_get_conv_requant_scale.argtypes = [f, f, C.c_int, f, f, C.c_int, f, f, C.c_int]
+        lib.orc_softmax_f32.argtypes = [vp, vp, C.c_int64, C.c_int64, C.c_int64]
+        lib.orc_erf_f32.argtypes = [vp, vp, C.c_int64]
+        lib.orc_gelu_f32.argtypes = [vp, vp, C.c_int64]
+        lib.orc_layer_norm_f32.argtypes = [vp] * 6 + [C.c_int64, C.c_int64, C.c_double]
         _port = lib
     return _port
 
@@ -67,6 +71,10 @@ def ref():
         lib.ref_quantize.argtypes = [C.c_int, i64p, C.c_uint32, C.c_int, C.c_int, C.c_int] + [vp] * 4
         lib.ref_dequantize.argtypes = [C.c_int, i64p, C.c_uint32, C.c_int, C.c_int] + [vp] * 4
         lib.ref_pool.argtypes = [C.c_int] * 3 + [i64p] * 6 + [C.c_int, vp, vp]
+        if hasattr(lib, "ref_softmax_f32"):
+            lib.ref_softmax_f32.argtypes = [vp, vp, i64p, C.c_int, C.c_uint32]
+            lib.ref_sum_f32.argtypes = [vp, vp, i64p, C.c_int, C.c_uint32]
+            lib.ref_erf_f32.argtypes = [vp, vp, C.c_int64]
         _ref = lib
     return _ref
 
@@ -284,4 +292,71 @@ def concat(arrays, axis):
     ptrs = (C.c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
     ext = (C.c_int64 * len(arrays))(*extents)
     _ok(port().orc_concat(arrays[0].dtype.itemsize, len(arrays), ptrs, ext, outer, inner, _ptr(out)))
+    return out
+
+
+# ---- fp32 glue ------------------------------------------------------------------------------------
+
+def softmax(x, axes=()):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    outer, axis, inner = H._axes_run(x.shape, axes)
+    out = np.empty_like(x)
+    _ok(port().orc_softmax_f32(_ptr(x), _ptr(out), outer, axis, inner))
+    return out
+
+
+def erf(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    _ok(port().orc_erf_f32(_ptr(x), _ptr(out), x.size))
+    return out
+
+
+def gelu(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    _ok(port().orc_gelu_f32(_ptr(x), _ptr(out), x.size))
+    return out
+
+
+def layer_norm(x, scale=None, bias=None, begin_norm_axis=1, epsilon=1e-5):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    n_axis = begin_norm_axis if begin_norm_axis >= 0 else x.ndim + begin_norm_axis
+    rows = int(np.prod(x.shape[:n_axis], dtype=np.int64))
+    cols = int(np.prod(x.shape[n_axis:], dtype=np.int64))
+    sc = np.ascontiguousarray(scale, dtype=np.float32) if scale is not None else None
+    bi = np.ascontiguousarray(bias, dtype=np.float32) if bias is not None else None
+    out = np.empty_like(x)
+    mean = np.empty(x.shape[:n_axis], dtype=np.float32)
+    var = np.empty(x.shape[:n_axis], dtype=np.float32)
+    _ok(port().orc_layer_norm_f32(_ptr(x), _ptr(sc), _ptr(bi), _ptr(out), _ptr(mean), _ptr(var), rows, cols, float(epsilon)))
+    return out, mean, var
+
+
+def _mask(axes):
+    m = 0
+    for a in axes:
+        m |= 1 << a
+    return m
+
+
+def ref_softmax(x, axes):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    axes = range(x.ndim) if len(axes) == 0 else axes
+    assert ref().ref_softmax_f32(_ptr(x), _ptr(out), _i64(x.shape), x.ndim, _mask(axes)) == 0
+    return out
+
+
+def ref_sum(x, axes):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty([d for i, d in enumerate(x.shape) if i not in axes], dtype=np.float32)
+    assert ref().ref_sum_f32(_ptr(x), _ptr(out), _i64(x.shape), x.ndim, _mask(axes)) == 0
+    return out
+
+
+def ref_erf(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    assert ref().ref_erf_f32(_ptr(x), _ptr(out), x.size) == 0
     return out

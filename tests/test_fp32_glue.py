@@ -1,0 +1,140 @@
+"""fp32 glue of a transformer encoder on the device against the oracle: Softmax, Erf, Gelu, LayerNorm.
+
+Floating point, so the bar is a tolerance: 1e-5 relative (the reference sums sequentially with Kahan
+compensation and calls the host's expf / erff; the kernels reduce in parallel and call the
+device's), with an absolute floor where a result is a difference of nearly equal numbers (stated
+at each check).  The shapes cross every kernel variant: rows kept in registers, rows re-read,
+ragged rows, strided axes, and the BERT-base sizes (batch 32, 12 heads, sequence 128, hidden 768,
+FFN 3072).
+"""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from ngraph_amd import hipq as H
+from ngraph_amd import synth
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+RTOL = 1e-5
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+
+
+SOFTMAX_CASES = [
+    ((32 * 12 * 128, 128), (1,)),   # BERT-base attention rows: kept in registers
+    ((3, 5, 2048), (2,)),           # the longest row that stays in registers
+    ((7, 2052), (1,)),              # longer: re-read
+    ((9, 131), (1,)),               # not a multiple of four
+    ((77, 64), (1,)),               # short rows: four to a wavefront
+    ((50, 20), (1,)),               # eight to a wavefront, five of eight lanes used
+    ((13, 4), (1,)),
+    ((4, 6, 10), (1,)),             # strided axis
+    ((5, 3, 4, 6), (1, 2)),         # a run of two axes with an inner extent
+    ((2, 3), ()),                   # all axes (op::v0::Softmax with an empty AxisSet)
+    ((6, 1, 5), (1,)),              # one element along the axis
+    ((0, 8), (1,)),                 # empty
+]
+
+
+@pytest.mark.parametrize("shape,axes", SOFTMAX_CASES)
+def test_softmax(gpu_lib, shape, axes):
+    say("softmax", shape, axes)
+    O.port().orc_set_threads(8)
+    x = synth.normal_f32(21, shape) * f32(5.0)
+    exp = O.softmax(x, axes)
+    got = H.softmax(x, axes)
+    O.port().orc_set_threads(1)
+    assert got.shape == exp.shape
+    if x.size == 0:
+        return
+    assert np.allclose(got, exp, rtol=RTOL, atol=1e-30), float(np.max(np.abs(got - exp) / np.maximum(exp, 1e-30)))
+    # rows sum to one
+    outer, axis, inner = H._axes_run(x.shape, axes)
+    assert np.allclose(got.reshape(outer, axis, inner).astype(np.float64).sum(axis=1), 1.0, atol=1e-5)
+    assert H.last_kernel() == ("softmax_rows" if inner == 1 else "softmax_strided")
+
+
+def test_softmax_extremes(gpu_lib):
+    """test/backend/softmax.in.cpp:241-293: lowest() and max() in a column neither underflow to NaN nor overflow"""
+    say("softmax extremes")
+    for v in (np.finfo(f32).min, np.finfo(f32).max):
+        x = np.array([[v, 1, 2], [3, 4, 5]], dtype=f32)
+        got, exp = H.softmax(x, (0,)), O.softmax(x, (0,))
+        assert np.all(np.isfinite(got)) and np.allclose(got, exp, rtol=RTOL, atol=1e-30)
+        got, exp = H.softmax(x, (1,)), O.softmax(x, (1,))
+        assert np.all(np.isfinite(got)) and np.allclose(got, exp, rtol=RTOL, atol=1e-30)
+
+
+@pytest.mark.parametrize("n", [1, 3, 4096, 4099, 4096 * 3072])
+def test_erf_and_gelu(gpu_lib, n):
+    say("erf / gelu", n)
+    x = synth.uniform_f32(22, (n,), -6.0, 6.0)
+    # erf: |erf| <= 1 and the functions agree to a couple of ulps of 1
+    assert np.max(np.abs(H.erf(x) - O.erf(x))) <= 2.4e-7
+    assert H.last_kernel() == "erf_vec"
+    # gelu: the f32 rounding of (1 + erf) is an absolute ~1e-7 scaled by 0.5 |x|; relative elsewhere
+    got, exp = H.gelu(x), O.gelu(x)
+    assert np.all(np.abs(got - exp) <= RTOL * np.abs(exp) + 3e-7 * np.maximum(np.abs(x), 1.0))
+    assert H.last_kernel() == "gelu_vec"
+    # special values
+    sp = np.array([0.0, -0.0, np.inf, -np.inf, 50.0, -50.0], dtype=f32)
+    assert np.array_equal(H.erf(sp), np.array([0.0, -0.0, 1.0, -1.0, 1.0, -1.0], dtype=f32))
+    g = H.gelu(sp[[0, 4, 5]])
+    assert g[0] == 0.0 and g[1] == 50.0 and g[2] == 0.0
+
+
+LN_CASES = [
+    ((32 * 128, 768), 1, True),     # BERT-base hidden states
+    ((4, 2048), 1, True),           # the longest row that stays in registers
+    ((5, 2056), 1, True),           # longer: re-read
+    ((6, 130), 1, False),           # ragged row, no affine
+    ((2, 3, 4, 5), 2, True),        # several trailing axes
+    ((3, 7, 64), -1, True),         # negative begin_norm_axis
+    ((0, 16), 1, True),             # empty
+]
+
+
+@pytest.mark.parametrize("shape,axis,affine", LN_CASES)
+def test_layer_norm(gpu_lib, shape, axis, affine):
+    say("layer_norm", shape, axis, affine)
+    O.port().orc_set_threads(8)
+    x = synth.normal_f32(23, shape) * f32(2.0) + f32(0.75)
+    n_axis = axis if axis >= 0 else len(shape) + axis
+    cols = int(np.prod(shape[n_axis:]))
+    scale = synth.uniform_f32(24, (cols,), 0.5, 1.5) if affine else None
+    bias = synth.uniform_f32(25, (cols,), -0.5, 0.5) if affine else None
+    en, em, ev = O.layer_norm(x, scale, bias, begin_norm_axis=axis, epsilon=1e-5)
+    gn, gm, gv = H.layer_norm(x, scale, bias, begin_norm_axis=axis, epsilon=1e-5)
+    O.port().orc_set_threads(1)
+    assert gn.shape == en.shape and gm.shape == em.shape
+    if x.size == 0:
+        return
+    # the mean is a difference-prone quantity only against |x| ~ 2: absolute floor 1e-6
+    assert np.allclose(gm, em, rtol=RTOL, atol=1e-6) and np.allclose(gv, ev, rtol=RTOL, atol=1e-7)
+    # (x - mean) cancels near the mean: absolute floor 1e-5 on values of order one
+    assert np.allclose(gn, en, rtol=RTOL, atol=1e-5), float(np.max(np.abs(gn - en)))
+    g2, m2, v2 = H.layer_norm(x, scale, bias, begin_norm_axis=axis, epsilon=1e-5, keep_stats=False)
+    assert m2 is None and v2 is None and np.array_equal(g2, gn)
+    assert H.last_kernel() == "layer_norm_rows"
+
+
+def test_layer_norm_reference_vectors(gpu_lib):
+    """test/backend/layer_norm.in.cpp:48-91"""
+    say("layer_norm reference vectors")
+    x = np.array([[-4, -3, -2, -1], [0, 1, 2, 3]], dtype=f32)
+    norm, mean, var = H.layer_norm(x, np.array([-1, 1, 2, 3], dtype=f32), np.array([-4, -3, -2, -1], dtype=f32), begin_norm_axis=1, epsilon=1e-5)
+    exp = np.array([-2.658364534378051758, -3.447211742401123047, -1.105576276779174805, 3.024906158447265625] * 2, dtype=f32).reshape(2, 4)
+    assert np.allclose(norm, exp, rtol=RTOL) and np.array_equal(mean, [-2.5, 1.5]) and np.array_equal(var, [1.25, 1.25])
+
+
+def test_argument_errors(gpu_lib):
+    lib = gpu_lib
+    lib.hipq_softmax_f32.argtypes = [H.C.c_void_p, H.C.c_void_p, H.C.c_int64, H.C.c_int64, H.C.c_int64, H.C.c_void_p]
+    assert lib.hipq_softmax_f32(None, None, 2, 3, 1, None) == H.ERR_INVALID
+    assert lib.hipq_softmax_f32(None, None, -1, 3, 1, None) == H.ERR_INVALID
+    lib.hipq_layer_norm_f32.argtypes = [H.C.c_void_p] * 6 + [H.C.c_int64, H.C.c_int64, H.C.c_double, H.C.c_void_p]
+    buf = H.DeviceBuffer(64)
+    assert lib.hipq_layer_norm_f32(buf.ptr, buf.ptr, None, buf.ptr, None, None, 1, 4, 1e-5, None) == H.ERR_INVALID  # scale without bias

@@ -224,6 +224,19 @@ def bench_fp32_glue(lib, stream, timer, steps, warmup):
         _, ev = timer.run(step, steps, warmup)
         gbs = 8 * n / (ev * 1e-3) / 1e9  # one f32 read, one f32 written per element
         out.append(dict(op=name, elements=n, ms_event=ev, gbs=gbs, frac_hbm=gbs / PEAK_HBM_GBS, kernel=H.last_kernel()))
+    # attention's two batched products per (image, head): scores = Q K^T [128,64]x[128,64]^T, context = P V [128,128]x[128,64]
+    lib.hipq_batch_matmul_f32.argtypes = [vp] * 3 + [i64] * 4 + [C.c_int32] * 2 + [vp]
+    heads = 32 * 12
+    for name, (m, k, n, tb) in {"scores_f32[384x128x64x128]": (128, 64, 128, 1), "context_f32[384x128x128x64]": (128, 128, 64, 0)}.items():
+        def step():
+            rc = lib.hipq_batch_matmul_f32(src.ptr, src.ptr + 4 * heads * m * k, dst.ptr, heads, m, k, n, 0, tb, stream)
+            if rc:
+                H.check(rc)
+
+        _, ev = timer.run(step, steps, warmup)
+        nbytes = 4 * heads * (m * k + k * n + m * n)
+        out.append(dict(op=name, elements=heads * m * n, ms_event=ev, gbs=nbytes / (ev * 1e-3) / 1e9, frac_hbm=nbytes / (ev * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                        tflops=2.0 * heads * m * k * n / (ev * 1e-3) / 1e12, kernel=H.last_kernel()))
     return out
 
 

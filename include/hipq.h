@@ -462,6 +462,24 @@ HIPQ_API int hipq_layer_norm_f32(const float* in,
                                  double epsilon,
                                  void* stream);
 
+/* op::v0::BatchMatMul (src/ngraph/runtime/reference/batch_mat_mul.hpp:31-57: runtime::reference::dot,
+ * dot.hpp:34-167 with one reduction axis, on every pair of the batch), op::v0::Dot of two f32
+ * matrices (batch = 1), and op::v0::BatchMatMulTranspose (src/ngraph/op/batch_mat_mul_transpose.hpp),
+ * which reads either operand transposed: out[b] = op(a[b]) * op(b[b]), a[b] stored [M][K] (or [K][M]
+ * with transpose_a), b[b] stored [K][N] (or [N][K] with transpose_b), out[b] [M][N].  The reference
+ * accumulates in double, k ascending, and rounds once to f32 (dot.hpp:37: ACCUMULATION =
+ * widen<float>::type, convolution.hpp:34-44); so does the kernel: the results are bit-exact. */
+HIPQ_API int hipq_batch_matmul_f32(const float* a,
+                                   const float* b,
+                                   float* out,
+                                   int64_t batch,
+                                   int64_t M,
+                                   int64_t K,
+                                   int64_t N,
+                                   int32_t transpose_a,
+                                   int32_t transpose_b,
+                                   void* stream);
+
 
 /* Which kernel the last hipq_quantized_* call on this thread used: "mfma", "direct", ... (host
  * string, never NULL).  For tests and profiles. */

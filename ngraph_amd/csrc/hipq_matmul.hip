@@ -1,0 +1,160 @@
+// f32 batched matrix product (attention scores and contexts of a transformer encoder; op::v0::Dot on
+// two matrices is the batch of one).  64 x 64 output tiles, 16-deep steps through LDS, 4 x 4 outputs a
+// lane in registers.  The reference accumulates f32 products in double, k ascending
+// (src/ngraph/runtime/reference/dot.hpp:34-37 with widen<float> = double,
+// convolution.hpp:34-44), and rounds the sum to f32 once; so does this kernel: a product of two
+// floats is exact in double, hence the fused multiply-add rounds exactly as the reference's separate
+// multiply and add, and the results are the reference's bit for bit.
+#include "hipq_common.h"
+
+namespace hipq
+{
+    namespace
+    {
+        typedef float f4 __attribute__((ext_vector_type(4)));
+        constexpr int TM = 64, TN = 64, TK = 16;
+
+        // out[b] = op(A[b]) * op(B[b]): A is [M][K] (or [K][M] with ta), B is [K][N] (or [N][K] with tb)
+        __global__ __launch_bounds__(256) void batch_matmul_f32_kernel(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ out, int32_t M, int32_t K, int32_t N, int32_t ta,
+                                                                       int32_t tb, int32_t m_tiles, int32_t n_tiles, int32_t vec_a, int32_t vec_b)
+        {
+            __shared__ __attribute__((aligned(16))) float as[TK][TM + 4]; // [k][m]
+            __shared__ __attribute__((aligned(16))) float bs[TK][TN + 4]; // [k][n]
+            const int tid = threadIdx.x;
+            int t = blockIdx.x;
+            const int nt = t % n_tiles;
+            t /= n_tiles;
+            const int mt = t % m_tiles;
+            const int64_t batch = t / m_tiles;
+            const float* A = a + batch * static_cast<int64_t>(M) * K;
+            const float* B = b + batch * static_cast<int64_t>(K) * N;
+            float* O = out + batch * static_cast<int64_t>(M) * N;
+            const int m0 = mt * TM, n0 = nt * TN;
+            const int tm = (tid >> 4) * 4, tn = (tid & 15) * 4; // this lane's 4 x 4 outputs within the tile
+            double acc[4][4] = {};
+            for (int k0 = 0; k0 < K; k0 += TK)
+            {
+                // 64 x 16 elements of each operand, four a lane, contiguous along the operand's rows in memory
+                if (!ta)
+                {
+                    const int r = tid >> 2, kq = (tid & 3) * 4; // A[m0 + r][k0 + kq ..]
+                    f4 v = f4{0.0f, 0.0f, 0.0f, 0.0f};
+                    if (vec_a && m0 + r < M && k0 + kq + 3 < K)
+                        v = *reinterpret_cast<const f4*>(A + static_cast<int64_t>(m0 + r) * K + k0 + kq);
+                    else
+                    {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            v[i] = (m0 + r < M && k0 + kq + i < K) ? A[static_cast<int64_t>(m0 + r) * K + k0 + kq + i] : 0.0f;
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        as[kq + i][r] = v[i];
+                }
+                else
+                {
+                    const int kk = tid >> 4, mq = (tid & 15) * 4; // A[k0 + kk][m0 + mq ..]
+                    f4 v = f4{0.0f, 0.0f, 0.0f, 0.0f};
+                    if (vec_a && k0 + kk < K && m0 + mq + 3 < M)
+                        v = *reinterpret_cast<const f4*>(A + static_cast<int64_t>(k0 + kk) * M + m0 + mq);
+                    else
+                    {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            v[i] = (k0 + kk < K && m0 + mq + i < M) ? A[static_cast<int64_t>(k0 + kk) * M + m0 + mq + i] : 0.0f;
+                    }
+                    *reinterpret_cast<f4*>(&as[kk][mq]) = v;
+                }
+                if (!tb)
+                {
+                    const int kk = tid >> 4, nq = (tid & 15) * 4; // B[k0 + kk][n0 + nq ..]
+                    f4 v = f4{0.0f, 0.0f, 0.0f, 0.0f};
+                    if (vec_b && k0 + kk < K && n0 + nq + 3 < N)
+                        v = *reinterpret_cast<const f4*>(B + static_cast<int64_t>(k0 + kk) * N + n0 + nq);
+                    else
+                    {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            v[i] = (k0 + kk < K && n0 + nq + i < N) ? B[static_cast<int64_t>(k0 + kk) * N + n0 + nq + i] : 0.0f;
+                    }
+                    *reinterpret_cast<f4*>(&bs[kk][nq]) = v;
+                }
+                else
+                {
+                    const int r = tid >> 2, kq = (tid & 3) * 4; // B[n0 + r][k0 + kq ..]
+                    f4 v = f4{0.0f, 0.0f, 0.0f, 0.0f};
+                    if (vec_b && n0 + r < N && k0 + kq + 3 < K)
+                        v = *reinterpret_cast<const f4*>(B + static_cast<int64_t>(n0 + r) * K + k0 + kq);
+                    else
+                    {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            v[i] = (n0 + r < N && k0 + kq + i < K) ? B[static_cast<int64_t>(n0 + r) * K + k0 + kq + i] : 0.0f;
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        bs[kq + i][r] = v[i];
+                }
+                __syncthreads();
+#pragma unroll
+                for (int k = 0; k < TK; ++k)
+                {
+                    // (past K both operands hold zeros: + 0 * 0 leaves a sum as it is -- a sum that started from +0 is never -0)
+                    const f4 av = *reinterpret_cast<const f4*>(&as[k][tm]);
+                    const f4 bv = *reinterpret_cast<const f4*>(&bs[k][tn]);
+                    double ad[4], bd[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                    {
+                        ad[i] = static_cast<double>(av[i]);
+                        bd[i] = static_cast<double>(bv[i]);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            acc[i][j] = fma(ad[i], bd[j], acc[i][j]);
+                }
+                __syncthreads();
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                const int m = m0 + tm + i;
+                if (m >= M)
+                    continue;
+                float* row = O + static_cast<int64_t>(m) * N + n0 + tn;
+                if (n0 + tn + 3 < N && (N & 3) == 0)
+                    *reinterpret_cast<f4*>(row) = f4{static_cast<float>(acc[i][0]), static_cast<float>(acc[i][1]), static_cast<float>(acc[i][2]), static_cast<float>(acc[i][3])};
+                else
+                {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (n0 + tn + j < N)
+                            row[j] = static_cast<float>(acc[i][j]);
+                }
+            }
+        }
+    }
+}
+
+using namespace hipq;
+
+int hipq_batch_matmul_f32(const float* a, const float* b, float* out, int64_t batch, int64_t M, int64_t K, int64_t N, int32_t transpose_a, int32_t transpose_b, void* stream)
+{
+    HIPQ_REQUIRE(batch >= 0 && M >= 0 && K >= 0 && N >= 0, "negative extent");
+    if (batch == 0 || M == 0 || N == 0)
+        return HIPQ_OK;
+    HIPQ_REQUIRE(out && (K == 0 || (a && b)), "null pointer");
+    HIPQ_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15) == 0, "the output must be 16-byte aligned");
+    HIPQ_REQUIRE(M < (1ll << 31) && K < (1ll << 31) && N < (1ll << 31), "extent too large");
+    const int64_t m_tiles = (M + TM - 1) / TM, n_tiles = (N + TN - 1) / TN;
+    // 16-byte loads along the operands' rows when every row starts aligned
+    const int vec_a = (reinterpret_cast<uintptr_t>(a) & 15) == 0 && (transpose_a ? M : K) % 4 == 0;
+    const int vec_b = (reinterpret_cast<uintptr_t>(b) & 15) == 0 && (transpose_b ? K : N) % 4 == 0;
+    HIPQ_REQUIRE(batch * m_tiles * n_tiles < (1ll << 31), "too many tiles for one launch");
+    batch_matmul_f32_kernel<<<static_cast<unsigned>(batch * m_tiles * n_tiles), 256, 0, as_stream(stream)>>>(a, b, out, static_cast<int32_t>(M), static_cast<int32_t>(K), static_cast<int32_t>(N),
+                                                                                                              transpose_a ? 1 : 0, transpose_b ? 1 : 0, static_cast<int32_t>(m_tiles),
+                                                                                                              static_cast<int32_t>(n_tiles), vec_a, vec_b);
+    return check_launch("batch_matmul_f32");
+}

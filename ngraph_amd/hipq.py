@@ -299,6 +299,7 @@ EXPORTS = [
     "hipq_erf_f32",
     "hipq_gelu_f32",
     "hipq_layer_norm_f32",
+    "hipq_batch_matmul_f32",
 ]
 
 _lib = None
@@ -686,3 +687,23 @@ def layer_norm(x, scale=None, bias=None, begin_norm_axis=1, epsilon=1e-5, keep_s
     check(lib.hipq_stream_sync(None))
     stats_shape = x.shape[:n_axis]
     return (dst.to_numpy(np.float32, x.shape), mean.to_numpy(np.float32, stats_shape) if keep_stats else None, var.to_numpy(np.float32, stats_shape) if keep_stats else None)
+
+
+def batch_matmul(a, b, transpose_a=False, transpose_b=False):
+    """out[i] = op(a[i]) @ op(b[i]) for f32 [batch, ., .] operands (two matrices: a batch of one)"""
+    lib = load()
+    a, b = np.ascontiguousarray(a, dtype=np.float32), np.ascontiguousarray(b, dtype=np.float32)
+    squeeze = a.ndim == 2
+    if squeeze:
+        a, b = a[None], b[None]
+    batch = a.shape[0]
+    M, K = (a.shape[2], a.shape[1]) if transpose_a else (a.shape[1], a.shape[2])
+    N = b.shape[1] if transpose_b else b.shape[2]
+    assert (b.shape[2] if transpose_b else b.shape[1]) == K and b.shape[0] == batch
+    da, db = _dev(a) if a.size else None, _dev(b) if b.size else None
+    out = DeviceBuffer(max(batch * M * N * 4, 4))
+    lib.hipq_batch_matmul_f32.argtypes = [C.c_void_p] * 3 + [C.c_int64] * 4 + [C.c_int32] * 2 + [C.c_void_p]
+    check(lib.hipq_batch_matmul_f32(da.ptr if da else None, db.ptr if db else None, out.ptr, batch, M, K, N, int(transpose_a), int(transpose_b), None))
+    check(lib.hipq_stream_sync(None))
+    r = out.to_numpy(np.float32, (batch, M, N))
+    return r[0] if squeeze else r

@@ -35,6 +35,9 @@
  *                                   expectations of test/backend/softmax.in.cpp:66-293.
  *   orc_gelu_f32                    the formula the reference's own test evaluates
  *                                   (test/backend/gelu.in.cpp:73-75) and its f64 points (:89-95).
+ *   orc_batch_matmul_f32            the compiled reference (oracle/_ref: batch_mat_mul.hpp over dot.hpp) bit
+ *                                   for bit on seeded tensors (transposes through numpy), the vectors
+ *                                   of test/backend/batch_mat_mul.in.cpp, float64 products.
  *   orc_layer_norm_f32              the literal vectors of test/backend/layer_norm.in.cpp:48-91; its
  *                                   sums against the compiled reference sum (oracle/_ref).
  */
@@ -952,5 +955,32 @@ ORC_API int orc_layer_norm_f32(const float* in, const float* scale, const float*
         if (var)
             var[r] = v;
     }
+    return HIPQ_OK;
+}
+
+
+/* src/ngraph/runtime/reference/batch_mat_mul.hpp:31-57 calling dot.hpp:34-167 for every pair of the
+ * batch (non-quantized branch, :146-151: sum = sum + ACCUMULATION(a) * ACCUMULATION(b), k ascending,
+ * with ACCUMULATION = widen<float>::type = double, dot.hpp:37 and convolution.hpp:34-44; the sum is
+ * cast to f32 once, dot.hpp:163); the transposes are those of op::v0::BatchMatMulTranspose, which only change how the
+ * operands are indexed */
+ORC_API int orc_batch_matmul_f32(const float* a, const float* b, float* out, int64_t batch, int64_t M, int64_t K, int64_t N, int transpose_a, int transpose_b)
+{
+    if (batch < 0 || M < 0 || K < 0 || N < 0)
+        return HIPQ_ERR_INVALID;
+#pragma omp parallel for collapse(2) num_threads(g_threads) if (g_threads > 1)
+    for (int64_t bi = 0; bi < batch; ++bi)
+        for (int64_t m = 0; m < M; ++m)
+        {
+            const float* A = a + bi * M * K;
+            const float* B = b + bi * K * N;
+            for (int64_t n = 0; n < N; ++n)
+            {
+                double sum = 0.0;
+                for (int64_t k = 0; k < K; ++k)
+                    sum = sum + (double)(transpose_a ? A[k * M + m] : A[m * K + k]) * (double)(transpose_b ? B[n * K + k] : B[k * N + n]);
+                out[(bi * M + m) * N + n] = (float)sum;
+            }
+        }
     return HIPQ_OK;
 }

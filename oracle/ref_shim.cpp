@@ -11,6 +11,7 @@
 #include "ngraph/axis_set.hpp"
 #include "ngraph/coordinate_diff.hpp"
 #include "ngraph/runtime/reference/avg_pool.hpp"
+#include "ngraph/runtime/reference/batch_mat_mul.hpp"
 #include "ngraph/runtime/reference/convolution.hpp"
 #include "ngraph/runtime/reference/dequantize.hpp"
 #include "ngraph/runtime/reference/dot.hpp"
@@ -382,6 +383,25 @@ __attribute__((visibility("default"))) int ref_sum_f32(const float* in, float* o
 __attribute__((visibility("default"))) int ref_erf_f32(const float* in, float* out, int64_t count)
 {
     runtime::reference::erf<float>(in, out, static_cast<size_t>(count));
+    return 0;
+}
+
+// runtime::reference::batch_mat_mul<float>: a [batch, M, K], b [batch, K, N]
+__attribute__((visibility("default"))) int ref_batch_mat_mul_f32(const float* a, const float* b, float* out, int64_t batch, int64_t M, int64_t K, int64_t N)
+{
+    try
+    {
+        runtime::reference::batch_mat_mul<float>(a,
+                                                 b,
+                                                 out,
+                                                 Shape{static_cast<size_t>(batch), static_cast<size_t>(M), static_cast<size_t>(K)},
+                                                 Shape{static_cast<size_t>(batch), static_cast<size_t>(K), static_cast<size_t>(N)},
+                                                 Shape{static_cast<size_t>(batch), static_cast<size_t>(M), static_cast<size_t>(N)});
+    }
+    catch (const std::exception&)
+    {
+        return -2;
+    }
     return 0;
 }
 }

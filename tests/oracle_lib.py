@@ -53,6 +53,7 @@ def port():
         lib.orc_erf_f32.argtypes = [vp, vp, C.c_int64]
         lib.orc_gelu_f32.argtypes = [vp, vp, C.c_int64]
         lib.orc_layer_norm_f32.argtypes = [vp] * 6 + [C.c_int64, C.c_int64, C.c_double]
+        lib.orc_batch_matmul_f32.argtypes = [vp] * 3 + [C.c_int64] * 4 + [C.c_int] * 2
         _port = lib
     return _port
 
@@ -75,6 +76,8 @@ def ref():
             lib.ref_softmax_f32.argtypes = [vp, vp, i64p, C.c_int, C.c_uint32]
             lib.ref_sum_f32.argtypes = [vp, vp, i64p, C.c_int, C.c_uint32]
             lib.ref_erf_f32.argtypes = [vp, vp, C.c_int64]
+        if hasattr(lib, "ref_batch_mat_mul_f32"):
+            lib.ref_batch_mat_mul_f32.argtypes = [vp] * 3 + [C.c_int64] * 4
         _ref = lib
     return _ref
 
@@ -359,4 +362,23 @@ def ref_erf(x):
     x = np.ascontiguousarray(x, dtype=np.float32)
     out = np.empty_like(x)
     assert ref().ref_erf_f32(_ptr(x), _ptr(out), x.size) == 0
+    return out
+
+
+def batch_matmul(a, b, transpose_a=False, transpose_b=False):
+    a, b = np.ascontiguousarray(a, dtype=np.float32), np.ascontiguousarray(b, dtype=np.float32)
+    batch = a.shape[0]
+    M, K = (a.shape[2], a.shape[1]) if transpose_a else (a.shape[1], a.shape[2])
+    N = b.shape[1] if transpose_b else b.shape[2]
+    out = np.empty((batch, M, N), dtype=np.float32)
+    _ok(port().orc_batch_matmul_f32(_ptr(a), _ptr(b), _ptr(out), batch, M, K, N, int(transpose_a), int(transpose_b)))
+    return out
+
+
+def ref_batch_matmul(a, b):
+    a, b = np.ascontiguousarray(a, dtype=np.float32), np.ascontiguousarray(b, dtype=np.float32)
+    batch, M, K = a.shape
+    N = b.shape[2]
+    out = np.empty((batch, M, N), dtype=np.float32)
+    assert ref().ref_batch_mat_mul_f32(_ptr(a), _ptr(b), _ptr(out), batch, M, K, N) == 0
     return out

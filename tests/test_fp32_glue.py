@@ -138,3 +138,51 @@ def test_argument_errors(gpu_lib):
     lib.hipq_layer_norm_f32.argtypes = [H.C.c_void_p] * 6 + [H.C.c_int64, H.C.c_int64, H.C.c_double, H.C.c_void_p]
     buf = H.DeviceBuffer(64)
     assert lib.hipq_layer_norm_f32(buf.ptr, buf.ptr, None, buf.ptr, None, None, 1, 4, 1e-5, None) == H.ERR_INVALID  # scale without bias
+
+
+MATMUL_CASES = [
+    # batch, M, K, N
+    (32 * 12, 128, 64, 128),   # BERT-base attention scores (Q K^T takes transpose_b)
+    (32 * 12, 128, 128, 64),   # attention context
+    (3, 70, 37, 129),          # ragged on every side
+    (2, 64, 16, 64),           # exactly one tile, one step
+    (1, 200, 300, 100),        # op::v0::Dot of two matrices
+    (5, 1, 9, 1),
+    (2, 8, 0, 8),              # empty reduction: zeros
+    (0, 4, 4, 4),
+]
+
+
+@pytest.mark.parametrize("batch,M,K,N", MATMUL_CASES)
+def test_batch_matmul(gpu_lib, batch, M, K, N):
+    """bit-exact: like the reference (dot.hpp:37, widen<float> = double) the kernel accumulates the exact
+    products in double, k ascending, and rounds to f32 once"""
+    say("batch_matmul", batch, M, K, N)
+    O.port().orc_set_threads(8)
+    a, b = synth.normal_f32(51, (batch, M, K)), synth.normal_f32(52, (batch, K, N))
+    small = batch * M * N * max(K, 1) <= 40_000_000
+    for ta in (False, True):
+        for tb in (False, True):
+            if not small and (ta, tb) not in ((False, False), (False, True)):
+                continue
+            aa = np.ascontiguousarray(a.transpose(0, 2, 1)) if ta else a
+            bb = np.ascontiguousarray(b.transpose(0, 2, 1)) if tb else b
+            got = H.batch_matmul(aa, bb, ta, tb)
+            assert got.shape == (batch, M, N)
+            if got.size == 0:
+                continue
+            exp = O.batch_matmul(aa, bb, ta, tb)
+            assert np.array_equal(got, exp), (ta, tb, float(np.max(np.abs(got - exp))))
+            assert H.last_kernel() == "batch_matmul_f32"
+    O.port().orc_set_threads(1)
+
+
+def test_batch_matmul_reference_vectors(gpu_lib):
+    """test/backend/batch_mat_mul.in.cpp:51-102 (small integers: exact)"""
+    a = np.array([1, 1, 1, 2, 2, 2, 3, 3, 3, 4, 4, 4], dtype=f32)
+    b = np.array([1, 1, 1, 1, 2, 2, 2, 2, 3, 3, 3, 3] * 2, dtype=f32).reshape(2, 3, 4)
+    assert np.array_equal(H.batch_matmul(a.reshape(2, 2, 3), b).ravel(), [6, 6, 6, 6, 12, 12, 12, 12, 18, 18, 18, 18, 24, 24, 24, 24])
+    assert np.array_equal(H.batch_matmul(a.reshape(2, 3, 2), b, transpose_a=True).ravel(), [9, 9, 9, 9, 11, 11, 11, 11, 21, 21, 21, 21, 23, 23, 23, 23])
+    # two matrices
+    x, y = synth.normal_f32(53, (10, 20)), synth.normal_f32(54, (20, 6))
+    assert np.allclose(H.batch_matmul(x, y), x.astype(np.float64) @ y.astype(np.float64), rtol=1e-5, atol=1e-5)

@@ -140,3 +140,28 @@ def test_layer_norm_sums_equal_compiled_reference():
     assert np.array_equal(mean, s / f32(700))
     d = (x - mean[:, None]).astype(f32)
     assert np.array_equal(var, O.ref_sum((d * d).astype(f32), (1,)) / f32(700))
+
+
+def test_batch_matmul_reference_tests():
+    """test/backend/batch_mat_mul.in.cpp:51-102: BatchMatMulTranspose without and with a transposed first operand"""
+    a = np.array([1, 1, 1, 2, 2, 2, 3, 3, 3, 4, 4, 4], dtype=f32)
+    b = np.array([1, 1, 1, 1, 2, 2, 2, 2, 3, 3, 3, 3] * 2, dtype=f32).reshape(2, 3, 4)
+    got = O.batch_matmul(a.reshape(2, 2, 3), b)
+    assert np.array_equal(got.ravel(), [6, 6, 6, 6, 12, 12, 12, 12, 18, 18, 18, 18, 24, 24, 24, 24])
+    got = O.batch_matmul(a.reshape(2, 3, 2), b, transpose_a=True)
+    assert np.array_equal(got.ravel(), [9, 9, 9, 9, 11, 11, 11, 11, 21, 21, 21, 21, 23, 23, 23, 23])
+
+
+@pytest.mark.skipif(not (O.have_ref() and hasattr(O.ref(), "ref_batch_mat_mul_f32")), reason="oracle/_ref not built with batch_mat_mul")
+@pytest.mark.parametrize("batch,M,K,N", [(3, 5, 7, 4), (2, 16, 33, 9), (1, 1, 50, 1), (4, 8, 1, 8)])
+def test_batch_matmul_equals_compiled_reference(batch, M, K, N):
+    """runtime::reference::batch_mat_mul<float> (dot.hpp's sequential f32 sum) bit for bit; the transposed
+    forms must give the same bits on operands transposed in numpy"""
+    a, b = synth.normal_f32(41, (batch, M, K)), synth.normal_f32(42, (batch, K, N))
+    exp = O.ref_batch_matmul(a, b)
+    assert np.array_equal(O.batch_matmul(a, b), exp)
+    at, bt = np.ascontiguousarray(a.transpose(0, 2, 1)), np.ascontiguousarray(b.transpose(0, 2, 1))
+    assert np.array_equal(O.batch_matmul(at, b, transpose_a=True), exp)
+    assert np.array_equal(O.batch_matmul(a, bt, transpose_b=True), exp)
+    assert np.array_equal(O.batch_matmul(at, bt, transpose_a=True, transpose_b=True), exp)
+    assert np.allclose(exp, np.einsum("bmk,bkn->bmn", a.astype(np.float64), b.astype(np.float64)), rtol=1e-5, atol=1e-5)

@@ -240,6 +240,26 @@ def bench_fp32_glue(lib, stream, timer, steps, warmup):
     return out
 
 
+def bench_bert(lib, stream, timer, batches=(1, 32)):
+    """synthetic int8 BERT-base-shaped encoder (ngraph_amd/bert.py): 12 layers of QuantizedDotBias projections
+    with f32 attention, Softmax, Gelu and LayerNorm between them, sequence 128, every tensor resident in HBM"""
+    from ngraph_amd import bert as B
+
+    out = []
+    for n in batches:
+        plan = B.DevicePlan(lib, stream, n)
+        plan.set_input(B.embeddings(B.BASE, n))
+        steps = 10 if n <= 8 else 5
+        _, eager = timer.run(plan.launch, steps, 2)
+        plan.capture()
+        _, graph = timer.run(plan.replay, steps, 2)
+        H.check(lib.hipq_graph_destroy(plan.graph))
+        best = min(eager, graph)
+        out.append(dict(batch=n, ms_eager=eager, ms_graph=graph, sequences_per_s=n / (best * 1e-3), int8_tops=2 * B.BASE.macs_per_sequence() * n / (best * 1e-3) / 1e12, launches=len(plan.calls)))
+        del plan
+    return out
+
+
 def bench_resnet50(lib, stream, timer, batches=(1, 32, 128)):
     """synthetic int8 ResNet-50 (ngraph_amd/resnet50.py), every tensor resident in HBM, channels-last,
     one forward pass = 53 convolutions, 2 pools, 1 GEMM; replayed as one HIP graph"""
@@ -367,6 +387,7 @@ def main():
         results["pool_resnet50_u8"] = bench_pool(lib, stream, timer, small, 5, args.batch)
         results["glue_resnet50_u8"] = bench_glue(lib, stream, timer, small, 5, args.batch)
         results["fp32_glue_bert_base"] = bench_fp32_glue(lib, stream, timer, small, 5)
+        results["bert_base_int8"] = bench_bert(lib, stream, timer)
         results["resnet50_int8"] = bench_resnet50(lib, stream, timer)
         cpu = cpu_baseline()
 

@@ -154,6 +154,30 @@ namespace hipq
         }
     }
 
+    // the same with 32-bit index arithmetic (tensors below 2^31 elements) on 16-byte pieces: for orders
+    // that keep the innermost axis, whose rows are whole pieces (splitting and merging attention heads)
+    struct PermuteInfo32
+    {
+        int32_t rank;
+        uint32_t out_shape[HIPQ_MAX_RANK];
+        uint32_t in_stride[HIPQ_MAX_RANK];
+    };
+
+    __global__ __launch_bounds__(256) void permute_rows16_kernel(const uint4* __restrict__ in, uint4* __restrict__ out, uint32_t n, PermuteInfo32 pi)
+    {
+        const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+        if (i >= n)
+            return;
+        uint32_t r = i, j = 0;
+        for (int a = pi.rank - 1; a >= 0; --a)
+        {
+            const uint32_t q = r / pi.out_shape[a];
+            j += (r - q * pi.out_shape[a]) * pi.in_stride[a];
+            r = q;
+        }
+        out[i] = in[j];
+    }
+
     // 16 bytes per lane for the element types networks move in bulk: the same scalar expression per
     // element, on registers
     template <typename T, int OP>
@@ -449,6 +473,27 @@ int hipq_permute(int32_t elem_bytes, const void* in, void* out, int32_t rank, co
             if (R < 65535 * 64 && Cc < (1ll << 31) && B < 65536)
                 return launch_transpose(in, out, B, R, Cc, elem_bytes, s);
         }
+    }
+    // the innermost axis stays innermost and its rows are whole 16-byte pieces: move pieces
+    if (rank >= 2 && order[rank - 1] == rank - 1 && (in_shape[rank - 1] * elem_bytes) % 16 == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 &&
+        n * elem_bytes / 16 < (1ll << 31))
+    {
+        const int64_t per = 16 / elem_bytes; // elements per piece
+        PermuteInfo32 p32;
+        p32.rank = rank;
+        for (int i = 0; i < HIPQ_MAX_RANK; ++i)
+        {
+            p32.out_shape[i] = 1;
+            p32.in_stride[i] = 0;
+        }
+        for (int i = 0; i < rank; ++i)
+        {
+            p32.out_shape[i] = static_cast<uint32_t>(i == rank - 1 ? pi.out_shape[i] / per : pi.out_shape[i]);
+            p32.in_stride[i] = static_cast<uint32_t>(i == rank - 1 ? 1 : pi.in_stride[i] / per);
+        }
+        const uint32_t pieces = static_cast<uint32_t>(n / per);
+        permute_rows16_kernel<<<(pieces + 255) / 256, 256, 0, s>>>(static_cast<const uint4*>(in), static_cast<uint4*>(out), pieces, p32);
+        return check_launch("permute_rows16");
     }
     switch (elem_bytes)
     {

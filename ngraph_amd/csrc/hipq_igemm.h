@@ -1771,8 +1771,11 @@ namespace hipq
             return launch_pipe<XL, 2, 2, MODE, false>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
         }
         // short reductions are bound by latency, not by LDS traffic: small wavefront tiles (64 x 64)
-        // take half the registers, so twice as many workgroups are resident to hide it
-        if (Kred <= 512 && N > 64 && getenv("HIPQ_NO_SMALL_TILE") == nullptr)
+        // take half the registers, so twice as many workgroups are resident to hide it; and when the
+        // large tiles are too few to give every compute unit two (a 4096 x 768 output is 96 of them),
+        // the small ones fill the chip better than the large ones use it
+        const int64_t large_tiles = ((M + 255) / 256) * ((N + 127) / 128);
+        if ((Kred <= 512 || large_tiles < 512) && N > 64 && getenv("HIPQ_NO_SMALL_TILE") == nullptr)
             return launch_tile<XL, 2, 2, 2, 2, X_ON_A, MODE, KIND>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
         if (N <= 64)
             return launch_tile<XL, 4, 2, 4, 1, X_ON_A, MODE, KIND>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);

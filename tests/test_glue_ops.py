@@ -95,6 +95,9 @@ PERMUTES = [
     ((2, 3, 4, 5), (0, 1, 2, 3)),   # identity
     ((2, 3, 4, 5), (3, 1, 0, 2)),   # a general permutation
     ((2, 3, 4, 5), (0, 2, 1, 3)),   # middle axes swapped: not a two-block order
+    ((2, 5, 3, 4, 16), (2, 0, 3, 1, 4)),  # attention heads split: innermost axis kept, rows of whole 16-byte pieces
+    ((3, 4, 6, 64), (0, 2, 1, 3)),        # heads merged
+    ((3, 4, 6, 12), (0, 2, 1, 3)),        # the same with rows that are whole pieces for f32 only
 ]
 
 

@@ -552,7 +552,8 @@ namespace
             op::v0::Abs::type_info, op::v0::Relu::type_info, op::v0::Convert::type_info, op::v0::Broadcast::type_info,
             op::v0::Reshape::type_info, op::v1::Add::type_info, op::v1::Subtract::type_info, op::v1::Multiply::type_info,
             op::v1::Divide::type_info, op::v1::Maximum::type_info, op::v1::Minimum::type_info, op::v0::MaxPool::type_info,
-            op::v0::AvgPool::type_info, op::v0::Concat::type_info};
+            op::v0::AvgPool::type_info, op::v0::Concat::type_info, op::v0::Softmax::type_info, op::v0::Erf::type_info,
+            op::v0::Gelu::type_info, op::v0::LayerNorm::type_info, op::v0::BatchMatMul::type_info, op::v0::BatchMatMulTranspose::type_info};
         for (const auto& ti : ops)
             if (n.get_type_info() == ti)
                 return true;
@@ -695,6 +696,77 @@ namespace
         else if (is_type<op::v0::MaxPool>(n) || is_type<op::v0::AvgPool>(n))
         {
             lower_pool(n, st);
+        }
+        else if (auto sm = as_type_ptr<op::v0::Softmax>(n))
+        {
+            // src/ngraph/runtime/reference/softmax.hpp:31-57; the library takes a contiguous run of axes
+            if (et != element::f32)
+                throw unsupported_op("HIP backend: Softmax on " + et.get_type_name());
+            const Shape& s = n->get_input_shape(0);
+            const AxisSet& axes = sm->get_axes();
+            const size_t first = *axes.begin(), last = *axes.rbegin();
+            if (last - first + 1 != axes.size())
+                throw unsupported_op("HIP backend: Softmax over axes that are not a contiguous run");
+            int64_t outer = 1, axis = 1, inner = 1;
+            for (size_t i = 0; i < s.size(); ++i)
+                (i < first ? outer : (i <= last ? axis : inner)) *= static_cast<int64_t>(s[i]);
+            st.launch = [outer, axis, inner](const vector<void*>& in, void* out, void* stream) {
+                check(hipq_softmax_f32(static_cast<const float*>(in[0]), static_cast<float*>(out), outer, axis, inner, stream), "Softmax");
+            };
+        }
+        else if (is_type<op::v0::Erf>(n) || is_type<op::v0::Gelu>(n))
+        {
+            // src/ngraph/runtime/reference/erf.hpp:29-35; src/ngraph/op/gelu.cpp:46-60
+            if (et != element::f32)
+                throw unsupported_op("HIP backend: " + n->description() + " on " + et.get_type_name());
+            const int64_t count = static_cast<int64_t>(shape_size(n->get_output_shape(0)));
+            const bool gelu = is_type<op::v0::Gelu>(n);
+            st.launch = [count, gelu](const vector<void*>& in, void* out, void* stream) {
+                if (gelu)
+                    check(hipq_gelu_f32(static_cast<const float*>(in[0]), static_cast<float*>(out), count, stream), "Gelu");
+                else
+                    check(hipq_erf_f32(static_cast<const float*>(in[0]), static_cast<float*>(out), count, stream), "Erf");
+            };
+        }
+        else if (auto ln = as_type_ptr<op::v0::LayerNorm>(n))
+        {
+            // src/ngraph/op/layer_norm.cpp:68-150 (the statistics outputs need multi-output steps: not yet)
+            if (et != element::f32)
+                throw unsupported_op("HIP backend: LayerNorm on " + et.get_type_name());
+            const Shape& s = n->get_input_shape(0);
+            const int64_t rank = static_cast<int64_t>(s.size());
+            const int64_t n_axis = ln->get_begin_norm_axis() >= 0 ? ln->get_begin_norm_axis() : rank + ln->get_begin_norm_axis();
+            int64_t rows = 1, cols = 1;
+            for (int64_t i = 0; i < rank; ++i)
+                (i < n_axis ? rows : cols) *= static_cast<int64_t>(s[i]);
+            const bool affine = ln->get_use_affine();
+            if (affine && static_cast<int64_t>(shape_size(n->get_input_shape(1))) != cols)
+                throw unsupported_op("HIP backend: LayerNorm scale that does not cover the normalised axes");
+            const double eps = ln->get_epsilon();
+            st.launch = [rows, cols, affine, eps](const vector<void*>& in, void* out, void* stream) {
+                check(hipq_layer_norm_f32(static_cast<const float*>(in[0]), affine ? static_cast<const float*>(in[1]) : nullptr, affine ? static_cast<const float*>(in[2]) : nullptr,
+                                          static_cast<float*>(out), nullptr, nullptr, rows, cols, eps, stream),
+                      "LayerNorm");
+            };
+        }
+        else if (is_type<op::v0::BatchMatMul>(n) || is_type<op::v0::BatchMatMulTranspose>(n))
+        {
+            // src/ngraph/runtime/reference/batch_mat_mul.hpp:31-57
+            if (et != element::f32)
+                throw unsupported_op("HIP backend: " + n->description() + " on " + et.get_type_name());
+            bool t0 = false, t1 = false;
+            if (auto bt = as_type_ptr<op::v0::BatchMatMulTranspose>(n))
+            {
+                t0 = bt->get_transpose_arg0();
+                t1 = bt->get_transpose_arg1();
+            }
+            const Shape& a = n->get_input_shape(0);
+            const Shape& o = n->get_output_shape(0);
+            const int64_t batch = static_cast<int64_t>(o[0]), M = static_cast<int64_t>(o[1]), N = static_cast<int64_t>(o[2]), K = static_cast<int64_t>(t0 ? a[1] : a[2]);
+            st.launch = [batch, M, K, N, t0, t1](const vector<void*>& in, void* out, void* stream) {
+                check(hipq_batch_matmul_f32(static_cast<const float*>(in[0]), static_cast<const float*>(in[1]), static_cast<float*>(out), batch, M, K, N, t0 ? 1 : 0, t1 ? 1 : 0, stream),
+                      "BatchMatMul");
+            };
         }
         else if (auto cc = as_type_ptr<op::v0::Concat>(n))
         {

@@ -467,6 +467,89 @@ namespace ngraph
                 int64_t m_axis;
                 int64_t m_concat_axis = -1;
             };
+
+            // ---- fp32 glue of a transformer encoder --------------------------------------------------
+            // src/ngraph/op/softmax.hpp:28-60 (static axes)
+            class NGRAPH_API Softmax : public Op
+            {
+            public:
+                NGRAPH_OP_DECL("Softmax", 0)
+                Softmax(const Output<Node>& arg, const AxisSet& axes);
+                void validate_and_infer_types() override;
+                const AxisSet& get_axes() const { return m_axes; }
+                std::shared_ptr<Node> clone_with_new_inputs(const OutputVector& new_args) const override;
+
+            private:
+                AxisSet m_axes;
+            };
+
+            // src/ngraph/op/erf.hpp
+            class NGRAPH_API Erf : public Op
+            {
+            public:
+                NGRAPH_OP_DECL("Erf", 0)
+                explicit Erf(const Output<Node>& arg);
+                void validate_and_infer_types() override;
+                std::shared_ptr<Node> clone_with_new_inputs(const OutputVector& new_args) const override;
+            };
+
+            // src/ngraph/op/gelu.hpp:30-50: 0.5 * x * (1 + erf(x / sqrt(2)))
+            class NGRAPH_API Gelu : public Op
+            {
+            public:
+                NGRAPH_OP_DECL("Gelu", 0)
+                explicit Gelu(const Output<Node>& arg);
+                void validate_and_infer_types() override;
+                std::shared_ptr<Node> clone_with_new_inputs(const OutputVector& new_args) const override;
+            };
+
+            // src/ngraph/op/layer_norm.hpp:31-80 (forward): outputs norm, and mean and variance
+            // over the normalised axes when keep_stats
+            class NGRAPH_API LayerNorm : public Op
+            {
+            public:
+                NGRAPH_OP_DECL("LayerNorm", 0)
+                LayerNorm(const Output<Node>& data, const Output<Node>& scale, const Output<Node>& bias, bool keep_stats = true, int64_t begin_norm_axis = 1, double epsilon = 1e-5);
+                LayerNorm(const Output<Node>& data, bool keep_stats = true, int64_t begin_norm_axis = 1, double epsilon = 1e-5);
+                void validate_and_infer_types() override;
+                std::shared_ptr<Node> clone_with_new_inputs(const OutputVector& new_args) const override;
+                bool get_keep_stats() const { return m_keep_stats; }
+                bool get_use_affine() const { return m_use_affine; }
+                double get_epsilon() const { return m_epsilon; }
+                int64_t get_begin_norm_axis() const { return m_begin_norm_axis; }
+
+            private:
+                bool m_keep_stats{true};
+                bool m_use_affine{true};
+                int64_t m_begin_norm_axis{1};
+                double m_epsilon{1e-5};
+            };
+
+            // src/ngraph/op/experimental/batch_mat_mul.hpp: [b, m, k] x [b, k, n] -> [b, m, n]
+            class NGRAPH_API BatchMatMul : public Op
+            {
+            public:
+                NGRAPH_OP_DECL("BatchMatMul", 0)
+                BatchMatMul(const Output<Node>& arg0, const Output<Node>& arg1);
+                void validate_and_infer_types() override;
+                std::shared_ptr<Node> clone_with_new_inputs(const OutputVector& new_args) const override;
+            };
+
+            // src/ngraph/op/batch_mat_mul_transpose.hpp: the same with either operand read transposed
+            class NGRAPH_API BatchMatMulTranspose : public Op
+            {
+            public:
+                NGRAPH_OP_DECL("BatchMatMulTranspose", 0)
+                BatchMatMulTranspose(const Output<Node>& arg0, const Output<Node>& arg1, bool transpose_arg0 = false, bool transpose_arg1 = false);
+                void validate_and_infer_types() override;
+                std::shared_ptr<Node> clone_with_new_inputs(const OutputVector& new_args) const override;
+                bool get_transpose_arg0() const { return m_transpose_arg0; }
+                bool get_transpose_arg1() const { return m_transpose_arg1; }
+
+            private:
+                bool m_transpose_arg0;
+                bool m_transpose_arg1;
+            };
         }
 
         namespace v1
@@ -509,11 +592,16 @@ namespace ngraph
         // the opset-0 names the tests use without a version
         using v0::Abs;
         using v0::AvgPool;
+        using v0::BatchMatMul;
+        using v0::BatchMatMulTranspose;
         using v0::Broadcast;
         using v0::Concat;
         using v0::Constant;
         using v0::Convert;
         using v0::Dequantize;
+        using v0::Erf;
+        using v0::Gelu;
+        using v0::LayerNorm;
         using v0::MaxPool;
         using v0::Parameter;
         using v0::Quantize;
@@ -527,6 +615,7 @@ namespace ngraph
         using v0::Relu;
         using v0::Reshape;
         using v0::Result;
+        using v0::Softmax;
     }
 
     NGRAPH_API std::shared_ptr<Node> operator+(const Output<Node>& a, const Output<Node>& b);

@@ -780,6 +780,134 @@ namespace ngraph
                 return make_shared<AvgPool>(a.at(0), m_window_shape, m_strides, m_padding_below, m_padding_above, m_include_padding);
             }
 
+            // ---- fp32 glue of a transformer encoder --------------------------------------------------
+            constexpr NodeTypeInfo Softmax::type_info;
+            Softmax::Softmax(const Output<Node>& arg, const AxisSet& axes) : Op({arg}), m_axes(axes) { constructor_validate_and_infer_types(); }
+            void Softmax::validate_and_infer_types()
+            {
+                // src/ngraph/op/softmax.cpp:56-70; an empty set means every axis (:45-52)
+                const Shape& s = get_input_shape(0);
+                if (m_axes.empty())
+                    for (size_t i = 0; i < s.size(); ++i)
+                        m_axes.insert(i);
+                for (auto axis : m_axes)
+                    NODE_VALIDATION_CHECK(this, axis < s.size(), "Reduction axis (", axis, ") is out of bounds (argument shape: ", s, ").");
+                set_output_type(0, get_input_element_type(0), s);
+            }
+            shared_ptr<Node> Softmax::clone_with_new_inputs(const OutputVector& a) const
+            {
+                check_new_args_count(this, a);
+                return make_shared<Softmax>(a.at(0), m_axes);
+            }
+
+            constexpr NodeTypeInfo Erf::type_info;
+            Erf::Erf(const Output<Node>& arg) : Op({arg}) { constructor_validate_and_infer_types(); }
+            void Erf::validate_and_infer_types() { set_output_type(0, get_input_element_type(0), get_input_shape(0)); }
+            shared_ptr<Node> Erf::clone_with_new_inputs(const OutputVector& a) const
+            {
+                check_new_args_count(this, a);
+                return make_shared<Erf>(a.at(0));
+            }
+
+            constexpr NodeTypeInfo Gelu::type_info;
+            Gelu::Gelu(const Output<Node>& arg) : Op({arg}) { constructor_validate_and_infer_types(); }
+            void Gelu::validate_and_infer_types()
+            {
+                // src/ngraph/op/gelu.cpp:71-90
+                NODE_VALIDATION_CHECK(this, get_input_element_type(0).is_real(), "Argument element type must be f16, bf16, f32, f64 or dynamic (got ", get_input_element_type(0), ").");
+                set_output_type(0, get_input_element_type(0), get_input_shape(0));
+            }
+            shared_ptr<Node> Gelu::clone_with_new_inputs(const OutputVector& a) const
+            {
+                check_new_args_count(this, a);
+                return make_shared<Gelu>(a.at(0));
+            }
+
+            constexpr NodeTypeInfo LayerNorm::type_info;
+            LayerNorm::LayerNorm(const Output<Node>& data, const Output<Node>& scale, const Output<Node>& bias, bool keep_stats, int64_t begin_norm_axis, double epsilon)
+                : Op({data, scale, bias}), m_keep_stats(keep_stats), m_use_affine(true), m_begin_norm_axis(begin_norm_axis), m_epsilon(epsilon)
+            {
+                constructor_validate_and_infer_types();
+            }
+            LayerNorm::LayerNorm(const Output<Node>& data, bool keep_stats, int64_t begin_norm_axis, double epsilon)
+                : Op({data}), m_keep_stats(keep_stats), m_use_affine(false), m_begin_norm_axis(begin_norm_axis), m_epsilon(epsilon)
+            {
+                constructor_validate_and_infer_types();
+            }
+            void LayerNorm::validate_and_infer_types()
+            {
+                // src/ngraph/op/layer_norm.cpp:173-235, static shapes
+                const element::Type& et = get_input_element_type(0);
+                NODE_VALIDATION_CHECK(this, et.is_real(), "Argument element type must be f16, bf16, f32, f64 or dynamic (got ", et, ").");
+                const Shape& ds = get_input_shape(0);
+                const int64_t d_rank = static_cast<int64_t>(ds.size());
+                const int64_t n_axis = m_begin_norm_axis >= 0 ? m_begin_norm_axis : d_rank + m_begin_norm_axis;
+                NODE_VALIDATION_CHECK(this, n_axis >= 0 && n_axis < d_rank, "begin_norm_axis is out of range");
+                if (m_use_affine)
+                {
+                    const int64_t s_rank = static_cast<int64_t>(get_input_shape(1).size()), b_rank = static_cast<int64_t>(get_input_shape(2).size());
+                    NODE_VALIDATION_CHECK(this, s_rank == b_rank && (s_rank == d_rank - n_axis || s_rank == 1), "Scale and/or bias rank is incorrect");
+                }
+                if (m_keep_stats)
+                {
+                    set_output_size(3);
+                    const Shape stats(ds.begin(), ds.begin() + n_axis);
+                    set_output_type(1, et, stats);
+                    set_output_type(2, et, stats);
+                }
+                set_output_type(0, et, ds);
+            }
+            shared_ptr<Node> LayerNorm::clone_with_new_inputs(const OutputVector& a) const
+            {
+                // src/ngraph/op/layer_norm.cpp:148-170
+                if (a.size() != 1 && a.size() != 3)
+                    throw ngraph_error("Incorrect number of new arguments");
+                if (!m_use_affine)
+                    return make_shared<LayerNorm>(a.at(0), m_keep_stats, m_begin_norm_axis, m_epsilon);
+                return make_shared<LayerNorm>(a.at(0), a.at(1), a.at(2), m_keep_stats, m_begin_norm_axis, m_epsilon);
+            }
+
+            namespace
+            {
+                // src/ngraph/op/experimental/batch_mat_mul.cpp:39-77 and batch_mat_mul_transpose.cpp:113-160
+                Shape batch_mat_mul_shape(const Node* n, const char* name, bool t0, bool t1)
+                {
+                    NODE_VALIDATION_CHECK(n, n->get_input_element_type(0) == n->get_input_element_type(1), "Inputs arg0 and arg1 must have compatible element type.");
+                    const Shape& a = n->get_input_shape(0);
+                    const Shape& b = n->get_input_shape(1);
+                    NODE_VALIDATION_CHECK(n, a.size() == 3, "Input arg0 shape must have rank 3, got ", a.size(), ".");
+                    NODE_VALIDATION_CHECK(n, b.size() == 3, "Input arg1 shape must have rank 3, got ", b.size(), ".");
+                    NODE_VALIDATION_CHECK(n, a[0] == b[0], "Batch size dimensions are not equal while creating ", name, ".");
+                    const size_t m = t0 ? a[2] : a[1], k0 = t0 ? a[1] : a[2], k1 = t1 ? b[2] : b[1], nn = t1 ? b[1] : b[2];
+                    NODE_VALIDATION_CHECK(n, k0 == k1, "Product dimensions are not equal while creating ", name, ".");
+                    return Shape{a[0], m, nn};
+                }
+            }
+
+            constexpr NodeTypeInfo BatchMatMul::type_info;
+            BatchMatMul::BatchMatMul(const Output<Node>& arg0, const Output<Node>& arg1) : Op({arg0, arg1}) { constructor_validate_and_infer_types(); }
+            void BatchMatMul::validate_and_infer_types() { set_output_type(0, get_input_element_type(0), batch_mat_mul_shape(this, "BatchMatMul", false, false)); }
+            shared_ptr<Node> BatchMatMul::clone_with_new_inputs(const OutputVector& a) const
+            {
+                check_new_args_count(this, a);
+                return make_shared<BatchMatMul>(a.at(0), a.at(1));
+            }
+
+            constexpr NodeTypeInfo BatchMatMulTranspose::type_info;
+            BatchMatMulTranspose::BatchMatMulTranspose(const Output<Node>& arg0, const Output<Node>& arg1, bool t0, bool t1) : Op({arg0, arg1}), m_transpose_arg0(t0), m_transpose_arg1(t1)
+            {
+                constructor_validate_and_infer_types();
+            }
+            void BatchMatMulTranspose::validate_and_infer_types()
+            {
+                set_output_type(0, get_input_element_type(0), batch_mat_mul_shape(this, "BatchMatMulTranspose", m_transpose_arg0, m_transpose_arg1));
+            }
+            shared_ptr<Node> BatchMatMulTranspose::clone_with_new_inputs(const OutputVector& a) const
+            {
+                check_new_args_count(this, a);
+                return make_shared<BatchMatMulTranspose>(a.at(0), a.at(1), m_transpose_arg0, m_transpose_arg1);
+            }
+
             constexpr NodeTypeInfo Concat::type_info;
             Concat::Concat(const OutputVector& args, int64_t axis) : Op(args), m_axis(axis) { constructor_validate_and_infer_types(); }
             void Concat::validate_and_infer_types()

@@ -1,0 +1,192 @@
+// Softmax / Erf / Gelu / LayerNorm / BatchMatMul / BatchMatMulTranspose through backend "HIP", with
+// the values of the reference's test/backend/softmax.in.cpp:66-221, erf.in.cpp:47-66,
+// gelu.in.cpp:49-108, layer_norm.in.cpp:48-91 and batch_mat_mul.in.cpp:51-102; type propagation
+// after src/ngraph/op/{softmax,gelu,layer_norm}.cpp and op/experimental/batch_mat_mul.cpp.
+#include <cmath>
+
+#include "test_util.hpp"
+
+using namespace std;
+using namespace ngraph;
+
+namespace
+{
+    bool close(const vector<float>& a, const vector<float>& b, float rtol = 1e-5f, float atol = 1e-7f)
+    {
+        if (a.size() != b.size())
+            return false;
+        for (size_t i = 0; i < a.size(); ++i)
+            if (!(fabs(a[i] - b[i]) <= atol + rtol * fabs(b[i])))
+                return false;
+        return true;
+    }
+
+    vector<float> run(const shared_ptr<Function>& f, const vector<pair<Shape, vector<float>>>& args, const Shape& out_shape)
+    {
+        auto backend = runtime::Backend::create("HIP");
+        vector<shared_ptr<runtime::Tensor>> in;
+        for (const auto& a : args)
+        {
+            in.push_back(backend->create_tensor(element::f32, a.first));
+            copy_data(in.back(), a.second);
+        }
+        auto result = backend->create_tensor(element::f32, out_shape);
+        auto handle = backend->compile(f);
+        handle->call_with_validate({result}, in);
+        return read_vector<float>(result);
+    }
+}
+
+GPU_TEST(HIP, softmax_all_and_empty_axis_set)
+{
+    Shape shape{2, 3};
+    const vector<float> x{-3, -2, -1, 0, 1, 2};
+    const float d = expf(-3) + expf(-2) + expf(-1) + expf(0) + expf(1) + expf(2);
+    const vector<float> expected{expf(-3) / d, expf(-2) / d, expf(-1) / d, expf(0) / d, expf(1) / d, expf(2) / d};
+    for (const AxisSet& axes : {AxisSet{0, 1}, AxisSet{}})
+    {
+        auto A = make_shared<op::v0::Parameter>(element::f32, shape);
+        auto f = make_shared<Function>(OutputVector{make_shared<op::v0::Softmax>(A, axes)}, ParameterVector{A});
+        EXPECT_TRUE(close(run(f, {{shape, x}}, shape), expected));
+    }
+}
+
+GPU_TEST(HIP, softmax_axis_3d)
+{
+    Shape shape{2, 2, 3};
+    const vector<float> x{-10, -20, -30, -40, -50, -60, -1, -2, -3, -4, -5, -6};
+    auto A = make_shared<op::v0::Parameter>(element::f32, shape);
+    auto f = make_shared<Function>(OutputVector{make_shared<op::v0::Softmax>(A, AxisSet{0})}, ParameterVector{A});
+    vector<float> expected(12);
+    for (int i = 0; i < 6; ++i)
+    {
+        const float d = expf(x[i]) + expf(x[i + 6]);
+        expected[i] = expf(x[i]) / d;
+        expected[i + 6] = expf(x[i + 6]) / d;
+    }
+    EXPECT_TRUE(close(run(f, {{shape, x}}, shape), expected, 1e-5f, 1e-8f));
+}
+
+GPU_TEST(HIP, softmax_axis_rows_and_columns)
+{
+    Shape shape{2, 3};
+    const vector<float> x{-10, -20, -30, -40, -50, -60};
+    {
+        auto A = make_shared<op::v0::Parameter>(element::f32, shape);
+        auto f = make_shared<Function>(OutputVector{make_shared<op::v0::Softmax>(A, AxisSet{1})}, ParameterVector{A});
+        const float d0 = expf(-10) + expf(-20) + expf(-30), d1 = expf(-40) + expf(-50) + expf(-60);
+        EXPECT_TRUE(close(run(f, {{shape, x}}, shape), {expf(-10) / d0, expf(-20) / d0, expf(-30) / d0, expf(-40) / d1, expf(-50) / d1, expf(-60) / d1}));
+    }
+    {
+        auto A = make_shared<op::v0::Parameter>(element::f32, shape);
+        auto f = make_shared<Function>(OutputVector{make_shared<op::v0::Softmax>(A, AxisSet{0})}, ParameterVector{A});
+        const float d0 = expf(-10) + expf(-40), d1 = expf(-20) + expf(-50), d2 = expf(-30) + expf(-60);
+        EXPECT_TRUE(close(run(f, {{shape, x}}, shape), {expf(-10) / d0, expf(-20) / d1, expf(-30) / d2, expf(-40) / d0, expf(-50) / d1, expf(-60) / d2}));
+    }
+}
+
+GPU_TEST(HIP, erf_and_gelu)
+{
+    Shape shape{4096};
+    vector<float> x(4096), e(4096), g(4096);
+    for (size_t i = 0; i < x.size(); ++i)
+    {
+        x[i] = -100.0f + 200.0f * static_cast<float>((i * 2654435761u) % 100003) / 100003.0f;
+        if (i % 2)
+            x[i] *= 0.03f; // half of the points where erf is not saturated
+        e[i] = erff(x[i]);
+        g[i] = 0.5f * x[i] * (1.0f + erff(x[i] / sqrtf(2.0f)));
+    }
+    auto A = make_shared<op::v0::Parameter>(element::f32, shape);
+    auto fe = make_shared<Function>(OutputVector{make_shared<op::v0::Erf>(A)}, ParameterVector{A});
+    EXPECT_TRUE(close(run(fe, {{shape, x}}, shape), e, 1e-6f, 3e-7f));
+    auto B = make_shared<op::v0::Parameter>(element::f32, shape);
+    auto fg = make_shared<Function>(OutputVector{make_shared<op::v0::Gelu>(B)}, ParameterVector{B});
+    // the reference's own tolerance for this op (test/backend/gelu.in.cpp:78) and a tighter one
+    auto got = run(fg, {{shape, x}}, shape);
+    EXPECT_TRUE(close(got, g, .007f, .007f));
+    EXPECT_TRUE(close(got, g, 1e-5f, 3e-5f));
+}
+
+GPU_TEST(HIP, layer_norm_affine)
+{
+    // layer_norm_affine_stats of the reference without the statistics outputs
+    auto data = make_shared<op::v0::Parameter>(element::f32, Shape{2, 4});
+    auto scale = make_shared<op::v0::Parameter>(element::f32, Shape{4});
+    auto bias = make_shared<op::v0::Parameter>(element::f32, Shape{4});
+    auto ln = make_shared<op::v0::LayerNorm>(data, scale, bias, false);
+    auto f = make_shared<Function>(OutputVector{ln}, ParameterVector{data, scale, bias});
+    auto got = run(f, {{Shape{2, 4}, {-4, -3, -2, -1, 0, 1, 2, 3}}, {Shape{4}, {-1, 1, 2, 3}}, {Shape{4}, {-4, -3, -2, -1}}}, Shape{2, 4});
+    const vector<float> expected{-2.658364534378051758f, -3.447211742401123047f, -1.105576276779174805f, 3.024906158447265625f,
+                                 -2.658364534378051758f, -3.447211742401123047f, -1.105576276779174805f, 3.024906158447265625f};
+    EXPECT_TRUE(close(got, expected, 1e-5f, 1e-6f));
+    // without affine, normalising the last axis of a 3-D tensor
+    auto d3 = make_shared<op::v0::Parameter>(element::f32, Shape{1, 2, 4});
+    auto f3 = make_shared<Function>(OutputVector{make_shared<op::v0::LayerNorm>(d3, false, -1)}, ParameterVector{d3});
+    auto n3 = run(f3, {{Shape{1, 2, 4}, {-4, -3, -2, -1, 0, 1, 2, 3}}}, Shape{1, 2, 4});
+    const float sd = sqrtf(1.25f + 1e-5f);
+    EXPECT_TRUE(close(n3, {-1.5f / sd, -0.5f / sd, 0.5f / sd, 1.5f / sd, -1.5f / sd, -0.5f / sd, 0.5f / sd, 1.5f / sd}, 1e-5f, 1e-6f));
+}
+
+GPU_TEST(HIP, layer_norm_with_statistics_is_reported_unsupported)
+{
+    auto data = make_shared<op::v0::Parameter>(element::f32, Shape{2, 4});
+    auto ln = make_shared<op::v0::LayerNorm>(data, true);
+    EXPECT_EQ(ln->get_output_size(), size_t(3));
+    auto f = make_shared<Function>(OutputVector{ln->output(0), ln->output(1), ln->output(2)}, ParameterVector{data});
+    auto backend = runtime::Backend::create("HIP");
+    EXPECT_THROW(backend->compile(f), unsupported_op);
+}
+
+GPU_TEST(HIP, batch_mat_mul_and_transpose)
+{
+    const vector<float> a{1, 1, 1, 2, 2, 2, 3, 3, 3, 4, 4, 4};
+    const vector<float> b{1, 1, 1, 1, 2, 2, 2, 2, 3, 3, 3, 3, 1, 1, 1, 1, 2, 2, 2, 2, 3, 3, 3, 3};
+    {
+        auto A = make_shared<op::v0::Parameter>(element::f32, Shape{2, 2, 3});
+        auto B = make_shared<op::v0::Parameter>(element::f32, Shape{2, 3, 4});
+        auto f = make_shared<Function>(OutputVector{make_shared<op::v0::BatchMatMulTranspose>(A, B, false, false)}, ParameterVector{A, B});
+        EXPECT_VEC_EQ((vector<float>{6, 6, 6, 6, 12, 12, 12, 12, 18, 18, 18, 18, 24, 24, 24, 24}), run(f, {{Shape{2, 2, 3}, a}, {Shape{2, 3, 4}, b}}, Shape{2, 2, 4}));
+        auto A2 = make_shared<op::v0::Parameter>(element::f32, Shape{2, 2, 3});
+        auto B2 = make_shared<op::v0::Parameter>(element::f32, Shape{2, 3, 4});
+        auto f2 = make_shared<Function>(OutputVector{make_shared<op::v0::BatchMatMul>(A2, B2)}, ParameterVector{A2, B2});
+        EXPECT_VEC_EQ((vector<float>{6, 6, 6, 6, 12, 12, 12, 12, 18, 18, 18, 18, 24, 24, 24, 24}), run(f2, {{Shape{2, 2, 3}, a}, {Shape{2, 3, 4}, b}}, Shape{2, 2, 4}));
+    }
+    {
+        auto A = make_shared<op::v0::Parameter>(element::f32, Shape{2, 3, 2});
+        auto B = make_shared<op::v0::Parameter>(element::f32, Shape{2, 3, 4});
+        auto f = make_shared<Function>(OutputVector{make_shared<op::v0::BatchMatMulTranspose>(A, B, true, false)}, ParameterVector{A, B});
+        EXPECT_VEC_EQ((vector<float>{9, 9, 9, 9, 11, 11, 11, 11, 21, 21, 21, 21, 23, 23, 23, 23}), run(f, {{Shape{2, 3, 2}, a}, {Shape{2, 3, 4}, b}}, Shape{2, 2, 4}));
+    }
+}
+
+CPU_TEST(type_prop, fp32_glue_shapes_and_failures)
+{
+    auto x = make_shared<op::v0::Parameter>(element::f32, Shape{2, 3, 4});
+    EXPECT_EQ(make_shared<op::v0::Softmax>(x, AxisSet{2})->get_output_shape(0), (Shape{2, 3, 4}));
+    EXPECT_EQ(make_shared<op::v0::Softmax>(x, AxisSet{})->get_axes().size(), size_t(3));
+    EXPECT_THROW(make_shared<op::v0::Softmax>(x, AxisSet{3}), NodeValidationFailure);
+    auto q = make_shared<op::v0::Parameter>(element::i8, Shape{4});
+    EXPECT_THROW(make_shared<op::v0::Gelu>(q), NodeValidationFailure);
+    EXPECT_THROW(make_shared<op::v0::LayerNorm>(q, false), NodeValidationFailure);
+    auto ln = make_shared<op::v0::LayerNorm>(x, true, 1);
+    EXPECT_EQ(ln->get_output_size(), size_t(3));
+    EXPECT_EQ(ln->get_output_shape(1), (Shape{2}));
+    EXPECT_EQ(make_shared<op::v0::LayerNorm>(x, true, -1)->get_output_shape(2), (Shape{2, 3}));
+    EXPECT_THROW(make_shared<op::v0::LayerNorm>(x, true, 3), NodeValidationFailure);
+    auto s2 = make_shared<op::v0::Parameter>(element::f32, Shape{3, 4});
+    auto s1 = make_shared<op::v0::Parameter>(element::f32, Shape{4});
+    EXPECT_NO_THROW(make_shared<op::v0::LayerNorm>(x, s2, s2, false, 1));
+    EXPECT_NO_THROW(make_shared<op::v0::LayerNorm>(x, s1, s1, false, 2));
+    auto s3 = make_shared<op::v0::Parameter>(element::f32, Shape{2, 3, 4});
+    EXPECT_THROW(make_shared<op::v0::LayerNorm>(x, s3, s3, false, 1), NodeValidationFailure);
+    auto a = make_shared<op::v0::Parameter>(element::f32, Shape{5, 2, 3});
+    auto b = make_shared<op::v0::Parameter>(element::f32, Shape{5, 3, 7});
+    EXPECT_EQ(make_shared<op::v0::BatchMatMul>(a, b)->get_output_shape(0), (Shape{5, 2, 7}));
+    EXPECT_EQ(make_shared<op::v0::BatchMatMulTranspose>(b, b, true, false)->get_output_shape(0), (Shape{5, 7, 7}));
+    EXPECT_THROW(make_shared<op::v0::BatchMatMul>(a, a), NodeValidationFailure);
+    auto c = make_shared<op::v0::Parameter>(element::f32, Shape{4, 3, 7});
+    EXPECT_THROW(make_shared<op::v0::BatchMatMul>(a, c), NodeValidationFailure);
+    auto m = make_shared<op::v0::Parameter>(element::f32, Shape{3, 7});
+    EXPECT_THROW(make_shared<op::v0::BatchMatMul>(a, m), NodeValidationFailure);
+}

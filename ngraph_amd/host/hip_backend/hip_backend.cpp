@@ -143,7 +143,8 @@ namespace
         }
 
     private:
-        int value_of(const Output<Node>& o) const { return m_value_of.at(o.get_node()); }
+        // the outputs of a node have consecutive value ids
+        int value_of(const Output<Node>& o) const { return m_value_of.at(o.get_node()) + static_cast<int>(o.get_index()); }
         void* constant_ptr(const Output<Node>& o) const;
         void lower(const shared_ptr<Node>& n);
         void lower_conv(const shared_ptr<Node>& n, Step& st);
@@ -161,7 +162,7 @@ namespace
         int m_device;
         bool m_perf;
         shared_ptr<Function> m_function;
-        unordered_map<const Node*, int> m_value_of; // node (output 0) -> value id
+        unordered_map<const Node*, int> m_value_of; // node -> value id of its output 0
         unordered_map<const Node*, bool> m_nxc;     // nodes whose output tensor is kept channels-last
         vector<void*> m_value_ptr;                  // persistent device pointer, or null when bound per call
         vector<size_t> m_value_bytes;
@@ -564,7 +565,9 @@ namespace
     {
         if (!backend_supports(*n))
             throw unsupported_op(string("Unsupported op '") + n->description() + "'");
-        if (n->get_output_size() != 1)
+        // one output a step, except LayerNorm with its statistics: further outputs get the following
+        // value ids and reach the launch as pointers after the inputs
+        if (n->get_output_size() != 1 && !is_type<op::v0::LayerNorm>(n))
             throw unsupported_op(string("HIP backend: op '") + n->description() + "' with " + to_string(n->get_output_size()) + " outputs");
         const auto et = n->get_output_element_type(0);
         const size_t bytes = shape_size(n->get_output_shape(0)) * et.size();
@@ -597,10 +600,16 @@ namespace
         st.output = id;
         for (size_t i = 0; i < n->get_input_size(); ++i)
         {
-            if (n->input_value(i).get_index() != 0)
-                throw unsupported_op("HIP backend: multi-output producers are not supported");
             st.inputs.push_back(value_of(n->input_value(i)));
             m_value_uses[st.inputs.back()] += 1;
+        }
+        for (size_t o = 1; o < n->get_output_size(); ++o)
+        {
+            const size_t obytes = shape_size(n->get_output_shape(o)) * n->get_output_element_type(o).size();
+            m_value_ptr.push_back(alloc(obytes)->ptr);
+            m_value_bytes.push_back(obytes);
+            m_value_uses.push_back(0);
+            st.inputs.push_back(id + static_cast<int>(o)); // written, not read: no use counted
         }
         const int64_t count = static_cast<int64_t>(shape_size(n->get_output_shape(0)));
         const int dt = dtype_of(et);
@@ -730,7 +739,7 @@ namespace
         }
         else if (auto ln = as_type_ptr<op::v0::LayerNorm>(n))
         {
-            // src/ngraph/op/layer_norm.cpp:68-150 (the statistics outputs need multi-output steps: not yet)
+            // src/ngraph/op/layer_norm.cpp:68-150; with keep_stats the mean and variance tensors follow the inputs
             if (et != element::f32)
                 throw unsupported_op("HIP backend: LayerNorm on " + et.get_type_name());
             const Shape& s = n->get_input_shape(0);
@@ -743,9 +752,12 @@ namespace
             if (affine && static_cast<int64_t>(shape_size(n->get_input_shape(1))) != cols)
                 throw unsupported_op("HIP backend: LayerNorm scale that does not cover the normalised axes");
             const double eps = ln->get_epsilon();
-            st.launch = [rows, cols, affine, eps](const vector<void*>& in, void* out, void* stream) {
+            const bool stats = ln->get_keep_stats();
+            const size_t first_stat = affine ? 3 : 1;
+            st.launch = [rows, cols, affine, eps, stats, first_stat](const vector<void*>& in, void* out, void* stream) {
                 check(hipq_layer_norm_f32(static_cast<const float*>(in[0]), affine ? static_cast<const float*>(in[1]) : nullptr, affine ? static_cast<const float*>(in[2]) : nullptr,
-                                          static_cast<float*>(out), nullptr, nullptr, rows, cols, eps, stream),
+                                          static_cast<float*>(out), stats ? static_cast<float*>(in[first_stat]) : nullptr, stats ? static_cast<float*>(in[first_stat + 1]) : nullptr, rows,
+                                          cols, eps, stream),
                       "LayerNorm");
             };
         }

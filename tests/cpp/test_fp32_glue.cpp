@@ -128,14 +128,41 @@ GPU_TEST(HIP, layer_norm_affine)
     EXPECT_TRUE(close(n3, {-1.5f / sd, -0.5f / sd, 0.5f / sd, 1.5f / sd, -1.5f / sd, -0.5f / sd, 0.5f / sd, 1.5f / sd}, 1e-5f, 1e-6f));
 }
 
-GPU_TEST(HIP, layer_norm_with_statistics_is_reported_unsupported)
+GPU_TEST(HIP, layer_norm_affine_stats)
 {
-    auto data = make_shared<op::v0::Parameter>(element::f32, Shape{2, 4});
-    auto ln = make_shared<op::v0::LayerNorm>(data, true);
+    // test/backend/layer_norm.in.cpp:48-91: three outputs
+    auto p_data = make_shared<op::v0::Parameter>(element::f32, Shape{2, 4});
+    auto p_scale = make_shared<op::v0::Parameter>(element::f32, Shape{4});
+    auto p_bias = make_shared<op::v0::Parameter>(element::f32, Shape{4});
+    auto ln = make_shared<op::v0::LayerNorm>(p_data, p_scale, p_bias);
     EXPECT_EQ(ln->get_output_size(), size_t(3));
-    auto f = make_shared<Function>(OutputVector{ln->output(0), ln->output(1), ln->output(2)}, ParameterVector{data});
+    auto f = make_shared<Function>(OutputVector{ln->output(0), ln->output(1), ln->output(2)}, ParameterVector{p_data, p_scale, p_bias});
     auto backend = runtime::Backend::create("HIP");
-    EXPECT_THROW(backend->compile(f), unsupported_op);
+    auto data = backend->create_tensor(element::f32, Shape{2, 4});
+    auto scale = backend->create_tensor(element::f32, Shape{4});
+    auto bias = backend->create_tensor(element::f32, Shape{4});
+    copy_data(data, vector<float>{-4, -3, -2, -1, 0, 1, 2, 3});
+    copy_data(scale, vector<float>{-1, 1, 2, 3});
+    copy_data(bias, vector<float>{-4, -3, -2, -1});
+    auto norm = backend->create_tensor(element::f32, Shape{2, 4});
+    auto mean = backend->create_tensor(element::f32, Shape{2});
+    auto var = backend->create_tensor(element::f32, Shape{2});
+    auto handle = backend->compile(f);
+    const vector<float> exp_norm{-2.658364534378051758f, -3.447211742401123047f, -1.105576276779174805f, 3.024906158447265625f,
+                                 -2.658364534378051758f, -3.447211742401123047f, -1.105576276779174805f, 3.024906158447265625f};
+    for (int rep = 0; rep < 3; ++rep) // eager, captured, replayed
+    {
+        handle->call_with_validate({norm, mean, var}, {data, scale, bias});
+        EXPECT_TRUE(close(read_vector<float>(norm), exp_norm, 1e-5f, 1e-6f));
+        EXPECT_VEC_EQ((vector<float>{-2.5f, 1.5f}), read_vector<float>(mean));
+        EXPECT_VEC_EQ((vector<float>{1.25f, 1.25f}), read_vector<float>(var));
+    }
+    // a statistic consumed inside the graph: variance + mean
+    auto d2 = make_shared<op::v0::Parameter>(element::f32, Shape{2, 4});
+    auto ln2 = make_shared<op::v0::LayerNorm>(d2, true, 1);
+    auto sum = make_shared<op::v1::Add>(ln2->output(1), ln2->output(2));
+    auto f2 = make_shared<Function>(OutputVector{sum}, ParameterVector{d2});
+    EXPECT_VEC_EQ((vector<float>{-1.25f, 2.75f}), run(f2, {{Shape{2, 4}, {-4, -3, -2, -1, 0, 1, 2, 3}}}, Shape{2}));
 }
 
 GPU_TEST(HIP, batch_mat_mul_and_transpose)

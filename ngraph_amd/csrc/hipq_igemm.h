@@ -1523,51 +1523,68 @@ namespace hipq
             oob_next = oob_new;
             __syncthreads();
             int cb = 0, lb = 2; // buffer of the slice being multiplied, buffer the loads go to
-            for (int s = 0; s < total; ++s)
-            {
-                HIPQ_PIPE_MARK(s, 0);
-                const bool tile_done = ckt + 1 == KT;
-                if (has_sum && tile_done) // uniform; ahead of the operand loads, so that waiting for it leaves them in flight
-                    sum_fetch();
+            int s = 0;          // position in the workgroup's sequence of slices
+            // One loop nest per tile, the tile's middle slices in a loop of their own that holds
+            // nothing but loads, waits and MFMAs: the accumulators then have one definition per
+            // tile (the first slice's product onto the correction) and the compiler neither copies
+            // them around a merged loop nor puts waits of its own into the steady state.
+            auto issue = [&]() {
                 loads_behind_sum = s + 2 < total;
                 if (s + 2 < total) // uniform
                     oob_new = dma_load(lb);
-                HIPQ_PIPE_MARK(s, 1);
-                if (tile_done) // uniform
-                {
-                    multiply(cb);
-                    HIPQ_PIPE_MARK(s, 2);
-                    if (splits == 1 || gather_splits()) // uniform
-                    {
-                    if (kFold && bias_folded) // uniform
-                        epilogue(std::true_type{});
-                    else
-                        epilogue(std::false_type{});
-                }
-                    ckt = 0;
-                    if (++cj < my_tiles)
-                        tile_origin(cj, cm0, cn0);
-                }
-                else
-                {
-                    multiply(cb);
-                    HIPQ_PIPE_MARK(s, 2);
-                    ++ckt;
-                }
-                HIPQ_PIPE_MARK(s, 3);
+            };
+            // the slice after this one has landed once at most the loads of the one after it are in flight
+            auto slice_end = [&]() {
                 cb = cb == 2 ? 0 : cb + 1;
                 lb = lb == 2 ? 0 : lb + 1;
-                // the next slice has landed once at most the loads of the one after it are in flight
                 if (s + 2 < total)
                     wait_vmcnt<L>();
                 else
                     wait_vmcnt<0>();
                 fill_fix(cb, oob_next);
                 oob_next = oob_new;
-                HIPQ_PIPE_MARK(s, 4);
+                ++s;
                 __syncthreads();
-                HIPQ_PIPE_MARK(s, 5);
-                if (tile_done && cj < my_tiles && cn0 != params_n0) // uniform
+            };
+            for (cj = 0; cj < my_tiles; ++cj)
+            {
+                int t, ks = 0;
+                if (splits > 1)
+                    tile_index(cj, t, ks);
+                HIPQ_PIPE_MARK(s, 0);
+                if (has_sum && KT == 1) // ahead of the operand loads, so that waiting for it leaves them in flight
+                    sum_fetch();
+                issue();
+                HIPQ_PIPE_MARK(s, 1);
+                corr_load(ks != 0); // the correction enters a split reduction once
+                compute(cb, std::true_type{});
+                HIPQ_PIPE_MARK(s, 2);
+                if (KT > 1) // uniform
+                {
+                    slice_end();
+                    for (int kt = 1; kt + 1 < KT; ++kt)
+                    {
+                        issue();
+                        compute(cb, std::false_type{});
+                        slice_end();
+                    }
+                    if (has_sum)
+                        sum_fetch();
+                    issue();
+                    compute(cb, std::false_type{});
+                }
+                if (splits == 1 || gather_splits()) // uniform
+                {
+                    if (kFold && bias_folded) // uniform
+                        epilogue(std::true_type{});
+                    else
+                        epilogue(std::false_type{});
+                }
+                HIPQ_PIPE_MARK(s, 3);
+                if (cj + 1 < my_tiles)
+                    tile_origin(cj + 1, cm0, cn0);
+                slice_end();
+                if (cj + 1 < my_tiles && cn0 != params_n0) // uniform
                 {
                     load_params(cn0);
                     __syncthreads();

@@ -933,6 +933,8 @@ namespace hipq
                                                                 int32_t n_tiles,
                                                                 int32_t split_shift,
                                                                 FastDiv by_m_tiles,
+                                                                FastDiv by_group,
+                                                                int32_t group_shift,
                                                                 int32_t* __restrict__ partials,
                                                                 uint32_t* __restrict__ counters,
                                                                 ZeroPoints zp,
@@ -951,8 +953,13 @@ namespace hipq
         static_assert(TN == 64, "the output staging swizzle is written for 64-byte rows");
         constexpr int NSTAGE = DMA ? 3 : 2;
         extern __shared__ __attribute__((aligned(16))) uint8_t lds[]; // [NSTAGE][x | w] operands, 4 output regions, per-channel constants
-        uint8_t* const ostage = lds + NSTAGE * STAGE + (threadIdx.x >> 6) * OUT_STAGE;
-        float* const params = reinterpret_cast<float*>(lds + NSTAGE * STAGE + 4 * OUT_STAGE); // [3][BN]: correction (as int), bias, scale
+        // Without a residual input the output regions need no room of their own: a tile's outputs are
+        // staged in the operand buffer that its last slice has just been multiplied out of (one more
+        // barrier per tile), which lets a third workgroup fit on a compute unit.
+        constexpr bool ALIAS_OUT = DMA && !HAS_SUM;
+        static_assert(!ALIAS_OUT || 4 * OUT_STAGE <= STAGE, "the output regions must fit an operand buffer");
+        uint8_t* ostage = lds + NSTAGE * STAGE + (threadIdx.x >> 6) * OUT_STAGE;
+        float* const params = reinterpret_cast<float*>(lds + NSTAGE * STAGE + (ALIAS_OUT ? 0 : 4 * OUT_STAGE)); // [3][BN]: correction (as int), bias, scale
 
         const int tid = threadIdx.x;
         const int lane = tid & 63;
@@ -970,7 +977,13 @@ namespace hipq
         if (vb >= total_tiles)
             return;
         const int my_tiles = (total_tiles - vb + grid - 1) / grid;
-        // tiles of one column block are consecutive, so a workgroup rarely changes its column block
+        // Tile order: column blocks go in groups of 2^group_shift; inside a group the tiles run
+        // along the group's column blocks first, then down the rows.  The workgroups of one compute
+        // die work on consecutive tiles (see `vb`), so with groups of eight they cover a square of
+        // 8 x 8 tiles and fetch 16 operand tiles into their L2 where the plain order (group_shift
+        // 0: down the rows of one column block) fetches 65.  The launcher only groups when the grid
+        // is a multiple of the group, so a workgroup keeps its column block from tile to tile;
+        // a last, narrower group runs in the plain order.
         auto tile_index = [&](int j, int& tile, int& split) {
             const int t = vb + j * grid;
             tile = t >> split_shift;
@@ -979,8 +992,21 @@ namespace hipq
         auto tile_origin = [&](int j, int64_t& m0, int32_t& n0) {
             int t, ks;
             tile_index(j, t, ks);
-            const int nt = static_cast<int>(by_m_tiles.div(static_cast<uint32_t>(t)));
-            m0 = static_cast<int64_t>(t - nt * m_tiles) * BM;
+            const int g = static_cast<int>(by_group.div(static_cast<uint32_t>(t)));
+            const int r = t - g * (m_tiles << group_shift);
+            int mt, nt;
+            if (((g + 1) << group_shift) <= n_tiles) // uniform
+            {
+                mt = r >> group_shift;
+                nt = (g << group_shift) + (r & ((1 << group_shift) - 1));
+            }
+            else
+            {
+                const int c = static_cast<int>(by_m_tiles.div(static_cast<uint32_t>(r)));
+                mt = r - c * m_tiles;
+                nt = (g << group_shift) + c;
+            }
+            m0 = static_cast<int64_t>(mt) * BM;
             n0 = nt * BN;
         };
 
@@ -1573,6 +1599,11 @@ namespace hipq
                     issue();
                     compute(cb, std::false_type{});
                 }
+                if constexpr (ALIAS_OUT)
+                {
+                    __syncthreads(); // every wavefront has read its last fragments
+                    ostage = lds + cb * STAGE + wave * OUT_STAGE;
+                }
                 if (splits == 1 || gather_splits()) // uniform
                 {
                     if (kFold && bias_folded) // uniform
@@ -1662,7 +1693,8 @@ namespace hipq
     {
         constexpr int BM = WAVES_M * 64, BN = WAVES_N * 64;
         constexpr bool DMA = XL::kUniform;
-        constexpr size_t lds_bytes = (DMA ? 3 : 2) * static_cast<size_t>(BM + BN) * BK + 4 * 64 * 64 + 3 * BN * sizeof(float) + 16;
+        // (the kernels that load into LDS and take no residual stage their outputs in an operand buffer)
+        constexpr size_t lds_bytes = (DMA ? 3 : 2) * static_cast<size_t>(BM + BN) * BK + (DMA && !HAS_SUM ? 0 : 4 * 64 * 64) + 3 * BN * sizeof(float) + 16;
         auto kernel = igemm_pipe_kernel<XL, 2, 2, WAVES_M, WAVES_N, MODE, HAS_SUM, DMA>;
         static bool configured[16] = {};
         static int cus[16] = {};
@@ -1717,7 +1749,13 @@ namespace hipq
         while ((1 << split_shift) < splits)
             ++split_shift;
         const unsigned grid = static_cast<unsigned>(items < resident ? items : resident);
-        kernel<<<grid, 256, lds_bytes, s>>>(xl, w, wsum, M, Kred, x_unsigned, static_cast<int32_t>(m_tiles), static_cast<int32_t>(n_tiles), split_shift, fast_div(m_tiles), partials, counters, zp, epi, om, out);
+        // column blocks in groups of up to eight (a power of two that divides the grid: a workgroup
+        // then stays in its column block), for operand reuse inside each compute die's L2
+        int group_shift = 0;
+        if (getenv("HIPQ_NO_TILE_GROUPS") == nullptr)
+            while (group_shift < 3 && (2ll << group_shift) <= n_tiles && ((grid >> split_shift) % (2u << group_shift)) == 0 && (grid & ((1u << split_shift) - 1)) == 0)
+                ++group_shift;
+        kernel<<<grid, 256, lds_bytes, s>>>(xl, w, wsum, M, Kred, x_unsigned, static_cast<int32_t>(m_tiles), static_cast<int32_t>(n_tiles), split_shift, fast_div(m_tiles), fast_div(m_tiles << group_shift), group_shift, partials, counters, zp, epi, om, out);
         return check_launch(name);
     }
 

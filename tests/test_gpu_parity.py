@@ -505,10 +505,11 @@ def test_conv_bias_in_accumulator(gpu_lib):
 
 
 @pytest.mark.parametrize("i", range(len(SPLIT_CONV_SHAPES)))
-def test_conv_loads_into_lds(gpu_lib, i, monkeypatch):
-    """the same shapes through the kernels whose loads go straight into LDS (opt-in for filters
-    with more than one tap): padding with a non-zero data zero point is patched in after the load"""
-    monkeypatch.setenv("HIPQ_CONV_DMA", "1")
+def test_conv_register_staged(gpu_lib, i, monkeypatch):
+    """the same shapes through the register-staged kernels (windows over multiples of 64 channels
+    take the kernels whose loads go straight into LDS unless this switch is set; there, padding
+    with a non-zero data zero point is patched in after the load)"""
+    monkeypatch.setenv("HIPQ_NO_CONV_DMA", "1")
     test_conv_split_reduction(gpu_lib, i)
 
 

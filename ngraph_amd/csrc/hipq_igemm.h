@@ -245,6 +245,7 @@ namespace hipq
         int32_t K;
         uint32_t bytes; // M * K
         static constexpr bool kUniform = true;
+        static constexpr bool kFloatOut = true; // GEMM outputs may be floats
         static constexpr bool kPads = false; // no reads of padding: an out-of-range chunk is never used
         struct Row
         {
@@ -275,6 +276,7 @@ namespace hipq
         const uint8_t* x; // = cx.x
         uint32_t bytes;   // = cx.bytes
         static constexpr bool kUniform = true;
+        static constexpr bool kFloatOut = false;
         static constexpr bool kPads = true;
         struct Row
         {
@@ -351,6 +353,7 @@ namespace hipq
         int32_t Q, PQ;
         FastDiv by_pq, by_q;
         static constexpr bool kUniform = true;
+        static constexpr bool kFloatOut = false;
         static constexpr bool kPads = false;
         struct Row
         {
@@ -922,7 +925,9 @@ namespace hipq
     // moves to the MFMA fragments.  These loads are written in assembly, so the waits for them are
     // explicit: a wait for "at most n operations in flight" only ever errs on the long side when
     // the compiler's own loads and stores are in the queue as well.
-    template <class XL, int WM, int WN, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM, bool DMA>
+    // KIND OUT_F32 (fused policy without a residual, loaders with a uniform cursor): the scaled sums
+    // leave as floats, 16 bytes a lane straight from the accumulators.
+    template <class XL, int WM, int WN, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM, bool DMA, int KIND = OUT_Q8>
     __global__ __launch_bounds__(256, 2) void igemm_pipe_kernel(XL xl,
                                                                 const int8_t* __restrict__ w,
                                                                 const int32_t* __restrict__ wsum,
@@ -1030,6 +1035,7 @@ namespace hipq
         const EpiConst ec = epi_const(epi);
         constexpr bool has_sum = HAS_SUM; // residual input (fused policy only)
         static_assert(!HAS_SUM || MODE == EPI_FUSED, "only the fused policy adds a residual");
+        static_assert(KIND == OUT_Q8 || (KIND == OUT_F32 && DMA && MODE == EPI_FUSED && !HAS_SUM), "float outputs: fused policy, no residual, loads straight into LDS");
 
         // ---- loader --------------------------------------------------------------------------
         const int lrow = tid >> 2;
@@ -1305,6 +1311,39 @@ namespace hipq
         };
         auto epilogue = [&](auto folded) {
             constexpr bool FOLD = decltype(folded)::value; // the bias is already in the accumulators
+            if constexpr (KIND == OUT_F32)
+            {
+                float* const of = static_cast<float*>(out);
+                const bool relu = epi.relu != 0;
+#pragma unroll
+                for (int ni = 0; ni < WN; ++ni)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                    {
+                        const int nt = wn * TN + ni * 32 + 8 * g + 4 * (lane >> 5); // within the column block
+                        v4f bias4 = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+                        if (!FOLD)
+                            bias4 = *reinterpret_cast<const v4f*>(params + BN + nt);
+                        const v4f scale4 = *reinterpret_cast<const v4f*>(params + 2 * BN + nt);
+                        const int32_t n = cn0 + nt;
+#pragma unroll
+                        for (int mi = 0; mi < WM; ++mi)
+                        {
+                            const int64_t m = cm0 + wm * TM + mi * 32 + (lane & 31);
+                            v4f v;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                            {
+                                const float a = static_cast<float>(acc[mi][ni][4 * g + e]);
+                                const float x = __fmul_rn(FOLD ? a : __fadd_rn(a, bias4[e]), scale4[e]);
+                                v[e] = relu ? ((x > 0.0f) ? x : __fmul_rn(x, -0.0f)) : x;
+                            }
+                            if (m < M && n < N)
+                                *reinterpret_cast<v4f*>(of + m * N + n) = v;
+                        }
+                    }
+                return;
+            }
             uint8_t* o8 = static_cast<uint8_t*>(out);
             if (has_sum)
             {
@@ -1676,7 +1715,7 @@ namespace hipq
         return check_launch(name);
     }
 
-    template <class XL, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM>
+    template <class XL, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM, int KIND = OUT_Q8>
     static int launch_pipe(const XL& xl,
                            const int8_t* w,
                            const int32_t* wsum,
@@ -1695,7 +1734,7 @@ namespace hipq
         constexpr bool DMA = XL::kUniform;
         // (the kernels that load into LDS and take no residual stage their outputs in an operand buffer)
         constexpr size_t lds_bytes = (DMA ? 3 : 2) * static_cast<size_t>(BM + BN) * BK + (DMA && !HAS_SUM ? 0 : 4 * 64 * 64) + 3 * BN * sizeof(float) + 16;
-        auto kernel = igemm_pipe_kernel<XL, 2, 2, WAVES_M, WAVES_N, MODE, HAS_SUM, DMA>;
+        auto kernel = igemm_pipe_kernel<XL, 2, 2, WAVES_M, WAVES_N, MODE, HAS_SUM, DMA, KIND>;
         static bool configured[16] = {};
         static int cus[16] = {};
         int dev = 0;
@@ -1777,8 +1816,18 @@ namespace hipq
                               const char* name)
     {
         const bool q8 = epi.out_t == HIPQ_U8 || epi.out_t == HIPQ_I8;
-        if (!q8 || om.ncx || (N & 15) != 0 || (reinterpret_cast<uintptr_t>(out) & 15) != 0 || getenv("HIPQ_NO_DMA") != nullptr || getenv("HIPQ_NO_PIPE") != nullptr)
+        const bool f32 = epi.out_t == HIPQ_F32 && epi.mode == EPI_FUSED && epi.sum_in == nullptr;
+        if ((!q8 && !f32) || om.ncx || (N & 15) != 0 || (reinterpret_cast<uintptr_t>(out) & 15) != 0 || getenv("HIPQ_NO_DMA") != nullptr || getenv("HIPQ_NO_PIPE") != nullptr)
             return HIPQ_ERR_UNSUPPORTED;
+        if (f32 && !XL::kFloatOut)
+            return HIPQ_ERR_UNSUPPORTED;
+        if constexpr (XL::kFloatOut)
+            if (f32)
+            {
+                if (N <= 64)
+                    return launch_pipe<XL, 4, 1, EPI_FUSED, false, OUT_F32>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+                return launch_pipe<XL, 2, 2, EPI_FUSED, false, OUT_F32>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+            }
         if (epi.mode == EPI_INTERP)
         {
             if (N <= 64)

@@ -383,10 +383,12 @@ namespace hipq
                 return launch_skinny<2, 16>(d, a, w_nk, wsum, zp, epi, out, s);
             if (d.M <= 64)
                 return launch_skinny<4, 8>(d, a, w_nk, wsum, zp, epi, out, s);
-            // above 64 rows an 8-bit output is faster on the tile kernels, whose reductions are
-            // split over workgroups when the tiles are few (config 2, 256 rows: 22 us against 44)
+            // above 64 rows an 8-bit or (fused policy) float output is faster on the tile kernels,
+            // whose reductions are split over workgroups when the tiles are few (config 2, 256 rows:
+            // 22 us against 44)
             const bool q8 = epi.out_t == HIPQ_U8 || epi.out_t == HIPQ_I8;
-            if (!(q8 && d.N % 16 == 0) || getenv("HIPQ_NO_PIPE") != nullptr)
+            const bool f32 = epi.out_t == HIPQ_F32 && epi.mode == EPI_FUSED && epi.sum_in == nullptr;
+            if (!((q8 || f32) && d.N % 16 == 0) || getenv("HIPQ_NO_PIPE") != nullptr || (f32 && getenv("HIPQ_NO_DMA") != nullptr))
             {
                 if (d.M <= 128)
                     return launch_skinny_wide<8>(d, a, w_nk, wsum, zp, epi, out, s);

@@ -683,6 +683,32 @@ def test_dot_bias_config2_shape(gpu_lib, M):
     O.port().orc_set_threads(1)
 
 
+@pytest.mark.parametrize("shape", [(200, 192, 144), (130, 4096, 64), (333, 768, 272), (4096, 64, 128)])
+def test_dot_bias_f32_tiles(gpu_lib, shape):
+    """float outputs of QuantizedDotBias through the tile kernels: ragged row and column tiles, a
+    long reduction that is split over workgroups, a single-slice reduction; small biases (added to
+    the accumulators as integers) and one beyond 2^24 (kept as a float add); with and without relu"""
+    M, K, N = shape
+    say("dot bias f32 tiles", shape)
+    O.port().orc_set_threads(8)
+    for a_t, lo, hi in (("u8", 0, 255), ("i8", -128, 127)):
+        a = synth.uniform_int(1201, (M, K), lo, hi, np.uint8 if a_t == "u8" else np.int8)
+        w = synth.uniform_int(1202, (N, K), -127, 127, np.int8)
+        for big_bias in (False, True):
+            bias = synth.uniform_int(1203, (N,), -(2**15), 2**15, np.int32)
+            if big_bias:
+                bias[N // 2] = 2**26 + 12345
+            scales = synth.uniform_f32(1204, (N,), 0.001, 0.01) * np.float32(0.03)
+            for relu in (False, True):
+                d = H.make_dot_desc(M, K, N, a_t=a_t, out_t="f32", b_layout=H.B_NK)
+                f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
+                exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
+                got = H.quantized_dot_bias(d, f, a, w, bias, scales)
+                assert H.last_kernel().startswith("dot_mfma"), H.last_kernel()
+                assert np.array_equal(got.view(np.uint32), exp.view(np.uint32)), (a_t, big_bias, relu)
+    O.port().orc_set_threads(1)
+
+
 def test_dot_config2_full_size_properties(gpu_lib):
     """config 2 at its real size [256,4096] x [4096,4096]: rows of the M=256 result equal the
     M=1 / M=32 results (launch geometry independence), and int32 accumulators of a row subset
@@ -729,7 +755,7 @@ def test_dot_skinny(gpu_lib, M):
                 f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
                 exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
                 got = H.quantized_dot_bias(d, f, a, w, bias, scales)
-                tiles = M > 64 and out_t != "f32" and N % 16 == 0
+                tiles = M > 64 and N % 16 == 0
                 assert H.last_kernel().startswith("dot_mfma" if tiles else "dot_skinny"), H.last_kernel()
                 assert np.array_equal(got, exp), (K, N, a_t, out_t, relu)
     O.port().orc_set_threads(1)

@@ -514,6 +514,13 @@ def test_conv_register_staged(gpu_lib, i, monkeypatch):
 
 
 @pytest.mark.parametrize("i", range(len(SPLIT_CONV_SHAPES)))
+def test_conv_split_forced(gpu_lib, i, monkeypatch):
+    """the same shapes with every reduction cut in two whatever the launch heuristic would choose"""
+    monkeypatch.setenv("HIPQ_SPLIT_K", "2")
+    test_conv_split_reduction(gpu_lib, i)
+
+
+@pytest.mark.parametrize("i", range(len(SPLIT_CONV_SHAPES)))
 def test_conv_split_reduction(gpu_lib, i):
     """few tiles with long reductions: the pipelined kernel cuts each reduction over several
     workgroups, which meet through partial sums and a counter that the last one resets; called

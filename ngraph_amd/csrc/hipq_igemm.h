@@ -113,6 +113,7 @@ namespace hipq
         int32_t K;
         uint32_t bytes; // M * K
         static constexpr bool kUniform = false;
+        static constexpr bool kFloatOut = false;
         static constexpr bool kPads = false; // (only read by the kernels that load straight into LDS)
 
         struct Row
@@ -147,6 +148,7 @@ namespace hipq
     struct ConvX
     {
         static constexpr bool kUniform = false;
+        static constexpr bool kFloatOut = false;
         static constexpr bool kPads = false; // (only read by the kernels that load straight into LDS)
         const uint8_t* x; // [N][H][W][C]
         int32_t H, W, C, Q, R, S, sh, sw, dh, dw, pbh, pbw;
@@ -245,7 +247,7 @@ namespace hipq
         int32_t K;
         uint32_t bytes; // M * K
         static constexpr bool kUniform = true;
-        static constexpr bool kFloatOut = true; // GEMM outputs may be floats
+        static constexpr bool kFloatOut = true; // GEMM outputs may be floats; also: the loader is light enough on registers for three workgroups per compute unit
         static constexpr bool kPads = false; // no reads of padding: an out-of-range chunk is never used
         struct Row
         {
@@ -928,7 +930,7 @@ namespace hipq
     // KIND OUT_F32 (fused policy without a residual, loaders with a uniform cursor): the scaled sums
     // leave as floats, 16 bytes a lane straight from the accumulators.
     template <class XL, int WM, int WN, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM, bool DMA, int KIND = OUT_Q8>
-    __global__ __launch_bounds__(256, 2) void igemm_pipe_kernel(XL xl,
+    __global__ __launch_bounds__(256, (DMA && !HAS_SUM && XL::kFloatOut) ? 3 : 2) void igemm_pipe_kernel(XL xl,
                                                                 const int8_t* __restrict__ w,
                                                                 const int32_t* __restrict__ wsum,
                                                                 int64_t M,
@@ -1309,8 +1311,9 @@ namespace hipq
                 }
             }
         };
-        auto epilogue = [&](auto folded) {
+        auto epilogue = [&](auto folded, auto to_u8) {
             constexpr bool FOLD = decltype(folded)::value; // the bias is already in the accumulators
+            constexpr bool PK_U8 = decltype(to_u8)::value; // fused policy, u8 output: one instruction saturates, rounds and packs
             if constexpr (KIND == OUT_F32)
             {
                 float* const of = static_cast<float*>(out);
@@ -1412,6 +1415,13 @@ namespace hipq
                                 float v = __fmul_rn(FOLD ? static_cast<float>(a) : __fadd_rn(static_cast<float>(a), bias4[e]), scale4[e]);
                                 if (has_sum)
                                     v = fmaf(ec.sum_scale, s4[e], v);
+                                if constexpr (PK_U8)
+                                {
+                                    // float -> u8 with saturation to [0, 255] (the ReLU included) and
+                                    // round half to even, written into byte e of the word; a NaN gives 0
+                                    packed = __builtin_amdgcn_cvt_pk_u8_f32(v, e, packed);
+                                    continue;
+                                }
                                 v = __builtin_amdgcn_fmed3f(v, clamp_lo, ec.hi);
                                 // the rounding add drops its low byte straight into byte e of the word
                                 if (e == 0)
@@ -1447,6 +1457,25 @@ namespace hipq
                 const int32_t n = cn0 + wn * TN + piece * 16;
                 if (m < M && n < N)
                     *reinterpret_cast<v4i*>(o8 + m * N + n) = *reinterpret_cast<const v4i*>(ostage + row * TN + ((piece ^ ((row >> 2) & 3)) << 4));
+            }
+        };
+        // (the variants exist in the kernels that load straight into LDS; see kFold)
+        constexpr bool kPackU8 = DMA && MODE == EPI_FUSED && KIND == OUT_Q8;
+        const bool pack_u8 = kPackU8 && epi.out_t == HIPQ_U8;
+        auto run_epilogue = [&]() {
+            if (kFold && bias_folded) // uniform
+            {
+                if (kPackU8 && pack_u8) // uniform
+                    epilogue(std::true_type{}, std::true_type{});
+                else
+                    epilogue(std::true_type{}, std::false_type{});
+            }
+            else
+            {
+                if (kPackU8 && pack_u8) // uniform
+                    epilogue(std::false_type{}, std::true_type{});
+                else
+                    epilogue(std::false_type{}, std::false_type{});
             }
         };
         // split reductions: leaves this item's raw sums in `partials`; the last item of the tile to
@@ -1542,10 +1571,7 @@ namespace hipq
                 HIPQ_PIPE_MARK(s, 2);
                 if (splits == 1 || (cm0 < M && gather_splits())) // uniform
                 {
-                    if (kFold && bias_folded) // uniform
-                        epilogue(std::true_type{});
-                    else
-                        epilogue(std::false_type{});
+                    run_epilogue();
                 }
                 ckt = 0;
                 if (++cj < my_tiles)
@@ -1645,10 +1671,7 @@ namespace hipq
                 }
                 if (splits == 1 || gather_splits()) // uniform
                 {
-                    if (kFold && bias_folded) // uniform
-                        epilogue(std::true_type{});
-                    else
-                        epilogue(std::false_type{});
+                    run_epilogue();
                 }
                 HIPQ_PIPE_MARK(s, 3);
                 if (cj + 1 < my_tiles)
@@ -1737,6 +1760,7 @@ namespace hipq
         auto kernel = igemm_pipe_kernel<XL, 2, 2, WAVES_M, WAVES_N, MODE, HAS_SUM, DMA, KIND>;
         static bool configured[16] = {};
         static int cus[16] = {};
+        static int per_cu[16] = {}; // workgroups of this kernel that fit a compute unit (LDS and registers)
         int dev = 0;
         HIPQ_HIP(hipGetDevice(&dev));
         if (dev >= 0 && dev < 16 && !configured[dev])
@@ -1745,12 +1769,16 @@ namespace hipq
             hipDeviceProp_t prop;
             HIPQ_HIP(hipGetDeviceProperties(&prop, dev));
             cus[dev] = prop.multiProcessorCount;
+            int fit = 0;
+            HIPQ_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&fit, reinterpret_cast<const void*>(kernel), 256, lds_bytes));
+            const int by_lds = static_cast<int>(160 * 1024 / lds_bytes);
+            per_cu[dev] = fit >= 1 && fit < by_lds ? fit : by_lds;
             configured[dev] = true;
         }
         const int64_t m_tiles = (M + BM - 1) / BM;
         const int64_t n_tiles = (N + BN - 1) / BN;
         HIPQ_REQUIRE(fits_i32(m_tiles * n_tiles), "too many tiles");
-        const int64_t resident = static_cast<int64_t>(dev >= 0 && dev < 16 && cus[dev] > 0 ? cus[dev] : 256) * (160 * 1024 / lds_bytes);
+        const int64_t resident = static_cast<int64_t>(dev >= 0 && dev < 16 && cus[dev] > 0 ? cus[dev] : 256) * (dev >= 0 && dev < 16 && per_cu[dev] > 0 ? per_cu[dev] : static_cast<int>(160 * 1024 / lds_bytes));
         const int64_t tiles = m_tiles * n_tiles;
         // Few tiles with long reductions leave most of the chip idle: cut every reduction into
         // `splits` runs of whole slices.

@@ -336,6 +336,8 @@ def main():
     ap.add_argument("--batch", type=int, default=128)
     ap.add_argument("--quick", action="store_true", help="headline workload only, no CPU baseline")
     ap.add_argument("--resnet-only", action="store_true", help="only the synthetic int8 ResNet-50 (for profiling); prints its results")
+    ap.add_argument("--bert-only", action="store_true", help="only the synthetic int8 BERT-base encoder (for profiling); prints its results")
+    ap.add_argument("--skip-models", action="store_true", help="leave out the BERT and ResNet-50 sections (kernel traces of the single operators; the models have runs of their own)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -352,6 +354,9 @@ def main():
 
     if args.resnet_only:
         print(json.dumps({"resnet50_int8": bench_resnet50(lib, stream, timer)}))
+        return
+    if args.bert_only:
+        print(json.dumps({"bert_base_int8": bench_bert(lib, stream, timer)}))
         return
 
     # headline: the reference's NCHW tensors in, NCHW out
@@ -387,8 +392,9 @@ def main():
         results["pool_resnet50_u8"] = bench_pool(lib, stream, timer, small, 5, args.batch)
         results["glue_resnet50_u8"] = bench_glue(lib, stream, timer, small, 5, args.batch)
         results["fp32_glue_bert_base"] = bench_fp32_glue(lib, stream, timer, small, 5)
-        results["bert_base_int8"] = bench_bert(lib, stream, timer)
-        results["resnet50_int8"] = bench_resnet50(lib, stream, timer)
+        if not args.skip_models:
+            results["bert_base_int8"] = bench_bert(lib, stream, timer)
+            results["resnet50_int8"] = bench_resnet50(lib, stream, timer)
         cpu = cpu_baseline()
 
     derived_peak = info.compute_units * info.clock_mhz * 1e6 * 8192 / 1e12

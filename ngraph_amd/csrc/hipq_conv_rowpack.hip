@@ -38,42 +38,44 @@ namespace hipq
 
     // [N][C][H][W] or [N][H][W][C] bytes -> [N][Hp][Wp][4]: staged pixel (y, x) is input pixel
     // (y - pad_h, x - pad_w) where that exists; everything else, and the channels beyond C, hold the
-    // data zero point.  One staged pixel (one dword) a lane.
-    __global__ __launch_bounds__(256) void stage_rows_kernel(const uint8_t* __restrict__ in, uint32_t* __restrict__ out, int64_t pixels, int32_t Hp, int32_t Wp, int32_t H, int32_t W,
+    // data zero point.  One staged pixel (one dword) a lane, one staged row (image, y) a block
+    // column: the only division is the block's own, of its row number by Hp.
+    __global__ __launch_bounds__(256) void stage_rows_kernel(const uint8_t* __restrict__ in, uint32_t* __restrict__ out, int32_t Hp, int32_t Wp, int32_t H, int32_t W,
                                                              int32_t Cc, int32_t pbh, int32_t pbw, int32_t in_ncx, const void* zp, int32_t zp_t)
     {
-        const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-        if (i >= pixels)
+        const int32_t xp = static_cast<int32_t>(blockIdx.y) * 256 + static_cast<int32_t>(threadIdx.x);
+        if (xp >= Wp)
             return;
-        const int32_t xp = static_cast<int32_t>(i % Wp);
-        const int64_t t = i / Wp;
-        const int32_t yp = static_cast<int32_t>(t % Hp);
-        const int64_t n = t / Hp;
+        const uint32_t row = blockIdx.x; // image * Hp + yp
+        const uint32_t n = row / static_cast<uint32_t>(Hp);
+        const int32_t yp = static_cast<int32_t>(row - n * static_cast<uint32_t>(Hp));
         const int32_t y = yp - pbh, x = xp - pbw;
         uint32_t v = (static_cast<uint32_t>(load_zp(zp, zp_t)) & 0xffu) * 0x01010101u;
         if (static_cast<uint32_t>(y) < static_cast<uint32_t>(H) && static_cast<uint32_t>(x) < static_cast<uint32_t>(W))
         {
-            const int64_t pix = static_cast<int64_t>(y) * W + x;
             const int64_t X = static_cast<int64_t>(H) * W;
+            const int64_t pix = static_cast<int64_t>(y) * W + x;
+            const uint8_t* p = in_ncx ? in + static_cast<int64_t>(n) * Cc * X + pix : in + (static_cast<int64_t>(n) * X + pix) * Cc;
+            const int64_t step = in_ncx ? X : 1;
             for (int c = 0; c < Cc; ++c)
             {
-                const uint32_t b = in_ncx ? in[(n * Cc + c) * X + pix] : in[(n * X + pix) * Cc + c];
+                const uint32_t b = p[c * step];
                 v = (v & ~(0xffu << (8 * c))) | (b << (8 * c));
             }
         }
-        out[i] = v;
+        out[static_cast<int64_t>(row) * Wp + xp] = v;
     }
 
     int launch_stage_rows(const ConvGeom& g, const RowPack& rp, const void* in, void* staged, const void* zp, int zp_t, hipStream_t s)
     {
-        const int64_t pixels = g.N * rp.Hp * rp.Wp;
-        if (pixels == 0)
+        const int64_t rows = g.N * rp.Hp;
+        if (rows == 0 || rp.Wp == 0)
             return HIPQ_OK;
-        HIPQ_REQUIRE((pixels + 255) / 256 < (1ll << 31), "tensor too large for one launch");
-        stage_rows_kernel<<<static_cast<unsigned>((pixels + 255) / 256), 256, 0, s>>>(static_cast<const uint8_t*>(in), static_cast<uint32_t*>(staged), pixels, static_cast<int32_t>(rp.Hp),
-                                                                                     static_cast<int32_t>(rp.Wp), static_cast<int32_t>(g.in[1]), static_cast<int32_t>(g.in[2]),
-                                                                                     static_cast<int32_t>(g.C), static_cast<int32_t>(g.pb[1]), static_cast<int32_t>(g.pb[2]),
-                                                                                     g.data_layout == HIPQ_LAYOUT_NCX ? 1 : 0, zp, zp_t);
+        HIPQ_REQUIRE(rows < (1ll << 31) && (rp.Wp + 255) / 256 <= 65535, "tensor too large for one launch");
+        dim3 grid(static_cast<unsigned>(rows), static_cast<unsigned>((rp.Wp + 255) / 256));
+        stage_rows_kernel<<<grid, 256, 0, s>>>(static_cast<const uint8_t*>(in), static_cast<uint32_t*>(staged), static_cast<int32_t>(rp.Hp), static_cast<int32_t>(rp.Wp),
+                                               static_cast<int32_t>(g.in[1]), static_cast<int32_t>(g.in[2]), static_cast<int32_t>(g.C), static_cast<int32_t>(g.pb[1]),
+                                               static_cast<int32_t>(g.pb[2]), g.data_layout == HIPQ_LAYOUT_NCX ? 1 : 0, zp, zp_t);
         return check_launch("stage_rows");
     }
 

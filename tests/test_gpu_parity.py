@@ -716,6 +716,29 @@ def test_dot_bias_f32_tiles(gpu_lib, shape):
     O.port().orc_set_threads(1)
 
 
+@pytest.mark.parametrize("shape", [(512, 256, 384), (1024, 128, 640), (12288, 64, 1024), (16384, 64, 1152), (5000, 192, 400)])
+def test_dot_tile_order(gpu_lib, shape):
+    """the persistent tile kernels number their tiles in groups of column blocks (squares per
+    compute die): full groups of 2, 4 and 8, a narrower last group, more tiles than resident
+    workgroups, ragged edges -- every output element must still be written exactly once"""
+    M, K, N = shape
+    say("dot tile order", shape)
+    O.port().orc_set_threads(8)
+    a = synth.uniform_int(1301, (M, K), 0, 255, np.uint8)
+    w = synth.uniform_int(1302, (N, K), -127, 127, np.int8)
+    bias = synth.uniform_int(1303, (N,), -(2**15), 2**15, np.int32)
+    scales = synth.uniform_f32(1304, (N,), 0.001, 0.01) * np.float32(0.05)
+    for out_t, relu in (("i8", False), ("u8", True), ("f32", False)):
+        d = H.make_dot_desc(M, K, N, a_t="u8", out_t=out_t, b_layout=H.B_NK)
+        f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
+        exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
+        got = H.quantized_dot_bias(d, f, a, w, bias, scales)
+        assert H.last_kernel().startswith("dot_mfma"), H.last_kernel()
+        assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), (out_t, relu)
+        assert len(np.unique(exp)) > 20
+    O.port().orc_set_threads(1)
+
+
 def test_dot_config2_full_size_properties(gpu_lib):
     """config 2 at its real size [256,4096] x [4096,4096]: rows of the M=256 result equal the
     M=1 / M=32 results (launch geometry independence), and int32 accumulators of a row subset

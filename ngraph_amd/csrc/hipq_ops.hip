@@ -123,7 +123,12 @@ namespace hipq
         const bool out_ncx = g.out_layout == HIPQ_LAYOUT_NCX && g.K > 1;
         // layers whose filter fits in LDS take the band kernel (HIPQ_NO_BAND=1 forces the generic one)
         const bool no_band = getenv("HIPQ_NO_BAND") != nullptr;
-        if (!no_band && conv_band_eligible(g, out_ncx))
+        // (a 1 x 1 filter over every pixel, 8-bit channels-last output in whole 16-byte rows: the data
+        // is a row matrix and the tile kernels that load it straight into LDS are faster -- 64 -> 64
+        // channels at 56 x 56, batch 128: 15.8 us against 23 us)
+        const bool row_matrix = !out_ncx && g.taps() == 1 && g.st[1] == 1 && g.st[2] == 1 && g.pb[1] == 0 && g.pb[2] == 0 && g.out[1] == g.in[1] && g.out[2] == g.in[2] &&
+                                (g.out_t == HIPQ_U8 || g.out_t == HIPQ_I8) && g.K % 16 == 0 && getenv("HIPQ_NO_DMA") == nullptr && getenv("HIPQ_NO_PIPE") == nullptr;
+        if (!no_band && !row_matrix && conv_band_eligible(g, out_ncx))
             return launch_conv_band(g, x, packed, zp, epi, out, out_ncx, s);
         return launch_conv_mfma(g, x, packed, zp, epi, out, out_ncx, s);
     }

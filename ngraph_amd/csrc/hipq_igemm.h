@@ -929,8 +929,11 @@ namespace hipq
     // the compiler's own loads and stores are in the queue as well.
     // KIND OUT_F32 (fused policy without a residual, loaders with a uniform cursor): the scaled sums
     // leave as floats, 16 bytes a lane straight from the accumulators.
-    template <class XL, int WM, int WN, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM, bool DMA, int KIND = OUT_Q8>
-    __global__ __launch_bounds__(256, (DMA && !HAS_SUM && XL::kFloatOut) ? 3 : 2) void igemm_pipe_kernel(XL xl,
+    // BKT = 128 (row-matrix loader, no residual, reductions in whole 128-byte pieces): slices twice
+    // as deep, two operand buffers.  A row piece is then a whole 128-byte line, which the path from
+    // L2 into LDS moves half again as fast as two 64-byte halves, and a slice has half the barriers.
+    template <class XL, int WM, int WN, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM, bool DMA, int KIND = OUT_Q8, int BKT = BK>
+    __global__ __launch_bounds__(256, (DMA && !HAS_SUM && XL::kFloatOut && BKT == BK) ? 3 : 2) void igemm_pipe_kernel(XL xl,
                                                                 const int8_t* __restrict__ w,
                                                                 const int32_t* __restrict__ wsum,
                                                                 int64_t M,
@@ -953,12 +956,15 @@ namespace hipq
         constexpr int BM = WAVES_M * WM * 32;
         constexpr int BN = WAVES_N * WN * 32;
         constexpr int TM = WM * 32, TN = WN * 32; // a wavefront's sub-tile
-        constexpr int XLOADS = BM * 4 / 256;
-        constexpr int WLOADS = (BN * 4 + 255) / 256;
-        constexpr int STAGE = (BM + BN) * BK;
+        static_assert(BKT == BK || (BKT == 2 * BK && DMA && !HAS_SUM && !XL::kPads), "deep slices: loads straight into LDS, no residual, no padding");
+        constexpr int LPR = BKT / 16;  // lanes that load one row's piece of a slice
+        constexpr int RPI = 256 / LPR; // rows one load instruction of the workgroup covers
+        constexpr int XLOADS = BM / RPI;
+        constexpr int WLOADS = (BN + RPI - 1) / RPI;
+        constexpr int STAGE = (BM + BN) * BKT;
         constexpr int OUT_STAGE = TM * TN; // per wavefront
         static_assert(TN == 64, "the output staging swizzle is written for 64-byte rows");
-        constexpr int NSTAGE = DMA ? 3 : 2;
+        constexpr int NSTAGE = DMA && BKT == BK ? 3 : 2;
         extern __shared__ __attribute__((aligned(16))) uint8_t lds[]; // [NSTAGE][x | w] operands, 4 output regions, per-channel constants
         // Without a residual input the output regions need no room of their own: a tile's outputs are
         // staged in the operand buffer that its last slice has just been multiplied out of (one more
@@ -1040,14 +1046,14 @@ namespace hipq
         static_assert(KIND == OUT_Q8 || (KIND == OUT_F32 && DMA && MODE == EPI_FUSED && !HAS_SUM), "float outputs: fused policy, no residual, loads straight into LDS");
 
         // ---- loader --------------------------------------------------------------------------
-        const int lrow = tid >> 2;
-        // (DMA: the lane's LDS slot is fixed, chunk position tid & 3 of row lrow: it reads the chunk that belongs there)
-        const int lchunk = DMA ? ((tid & 3) ^ ((lrow >> 2) & 3)) : (tid & 3);
+        const int lrow = tid / LPR;
+        // (DMA: the lane's LDS slot is fixed, chunk position tid % LPR of row lrow: it reads the chunk that belongs there)
+        const int lchunk = !DMA ? (tid & 3) : BKT == BK ? ((tid & 3) ^ ((lrow >> 2) & 3)) : ((tid & 7) ^ ((lrow >> 1) & 7));
         const int xor_mask = x_unsigned ? static_cast<int>(0x80808080u) : 0;
         const int fill = (xzp & 0xFF) * 0x01010101;
         const __amdgpu_buffer_rsrc_t xrs = make_rsrc(xl.x, xl.bytes);
         const __amdgpu_buffer_rsrc_t wrs = make_rsrc(w, static_cast<uint32_t>(N) * static_cast<uint32_t>(Kred));
-        const int KT = ((Kred + BK - 1) / BK) >> split_shift; // slices per work item (the launcher makes the split even)
+        const int KT = ((Kred + BKT - 1) / BKT) >> split_shift; // slices per work item (the launcher makes the split even)
         // Every slice issues the loads of the slice after next and stores the next one's into LDS,
         // without conditions (a condition the compiler cannot see through makes it wait for loads in
         // flight before their registers are loaded again): past the end the loader reads nothing
@@ -1064,15 +1070,15 @@ namespace hipq
             tile_origin(j, m0, n0);
             int t, ks;
             tile_index(j, t, ks);
-            const int kbyte0 = ks * KT * BK + (DMA ? 0 : lchunk * 16);
+            const int kbyte0 = ks * KT * BKT + (DMA ? 0 : lchunk * 16);
 #pragma unroll
             for (int i = 0; i < XLOADS; ++i)
-                xl.init_row(xr[i], m0 + lrow + 64 * i, M);
+                xl.init_row(xr[i], m0 + lrow + RPI * i, M);
             xl.init_cursor(cur, kbyte0);
 #pragma unroll
             for (int i = 0; i < WLOADS; ++i)
             {
-                const int32_t r = lrow + 64 * i;
+                const int32_t r = lrow + RPI * i;
                 woff[i] = (n0 + r < N && r < BN) ? (n0 + r) * Kred : kOob;
             }
             kb = kbyte0;
@@ -1158,7 +1164,7 @@ namespace hipq
                 }
 #pragma unroll
                 for (int i = 0; i < WLOADS; ++i)
-                    lds_dma16(wrs_words, (woff[i] != kOob && kb + lchunk * 16 < Kred) ? woff[i] + kb + lchunk * 16 : kOob, base + BM * BK + i * 4096);
+                    lds_dma16(wrs_words, (woff[i] != kOob && kb + lchunk * 16 < Kred) ? woff[i] + kb + lchunk * 16 : kOob, base + BM * BKT + i * 4096);
                 if (++lkt == KT)
                 {
                     lkt = 0;
@@ -1167,8 +1173,8 @@ namespace hipq
                 }
                 else
                 {
-                    xl.advance(cur, BK);
-                    kb += BK;
+                    xl.advance(cur, BKT);
+                    kb += BKT;
                 }
             }
             return oob;
@@ -1205,21 +1211,23 @@ namespace hipq
                         corrv[ni][4 * g + e] = c4[e];
                 }
         };
+        // byte offset of 16-byte chunk `chunk` of operand row `row` inside its LDS block
+        auto frag_offset = [](int row, int chunk) { return BKT == BK ? lds_offset(row, chunk) : row * BKT + ((chunk ^ ((row >> 1) & 7)) << 4); };
         auto compute = [&](int buf, auto first) {
             const uint8_t* xs = lds + buf * STAGE;
-            const uint8_t* ws = xs + BM * BK;
+            const uint8_t* ws = xs + BM * BKT;
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
+            for (int ks = 0; ks < BKT / 32; ++ks)
             {
                 v4i wf[WN], xf[WM];
                 const int chunk = ks * 2 + (lane >> 5);
 #pragma unroll
                 for (int i = 0; i < WN; ++i)
-                    wf[i] = *reinterpret_cast<const v4i*>(ws + lds_offset((wn * WN + i) * 32 + (lane & 31), chunk));
+                    wf[i] = *reinterpret_cast<const v4i*>(ws + frag_offset((wn * WN + i) * 32 + (lane & 31), chunk));
 #pragma unroll
                 for (int i = 0; i < WM; ++i)
                 {
-                    xf[i] = *reinterpret_cast<const v4i*>(xs + lds_offset((wm * WM + i) * 32 + (lane & 31), chunk));
+                    xf[i] = *reinterpret_cast<const v4i*>(xs + frag_offset((wm * WM + i) * 32 + (lane & 31), chunk));
                     if constexpr (DMA) // the data sits in LDS as it came: unsigned bytes become signed here
                         xf[i] = v4i{xf[i][0] ^ xor_mask, xf[i][1] ^ xor_mask, xf[i][2] ^ xor_mask, xf[i][3] ^ xor_mask};
                 }
@@ -1602,33 +1610,34 @@ namespace hipq
         if constexpr (DMA)
         {
             constexpr int L = XLOADS + WLOADS; // operand loads of one slice per lane
+            constexpr int PF = NSTAGE - 1;     // slices in flight ahead of the one being multiplied
             loader_tile(0);
             uint32_t oob_next = dma_load(0);
-            uint32_t oob_new = total > 1 ? dma_load(1) : 0u;
+            uint32_t oob_new = (PF > 1 && total > 1) ? dma_load(1) : 0u;
             load_params(cn0);
-            if (total > 1)
+            if (PF > 1 && total > 1)
                 wait_vmcnt<L>();
             else
                 wait_vmcnt<0>();
             fill_fix(0, oob_next);
             oob_next = oob_new;
             __syncthreads();
-            int cb = 0, lb = 2; // buffer of the slice being multiplied, buffer the loads go to
+            int cb = 0, lb = PF; // buffer of the slice being multiplied, buffer the loads go to
             int s = 0;          // position in the workgroup's sequence of slices
             // One loop nest per tile, the tile's middle slices in a loop of their own that holds
             // nothing but loads, waits and MFMAs: the accumulators then have one definition per
             // tile (the first slice's product onto the correction) and the compiler neither copies
             // them around a merged loop nor puts waits of its own into the steady state.
             auto issue = [&]() {
-                loads_behind_sum = s + 2 < total;
-                if (s + 2 < total) // uniform
+                loads_behind_sum = s + PF < total;
+                if (s + PF < total) // uniform
                     oob_new = dma_load(lb);
             };
             // the slice after this one has landed once at most the loads of the one after it are in flight
             auto slice_end = [&]() {
-                cb = cb == 2 ? 0 : cb + 1;
-                lb = lb == 2 ? 0 : lb + 1;
-                if (s + 2 < total)
+                cb = cb == NSTAGE - 1 ? 0 : cb + 1;
+                lb = lb == NSTAGE - 1 ? 0 : lb + 1;
+                if (PF > 1 && s + 2 < total)
                     wait_vmcnt<L>();
                 else
                     wait_vmcnt<0>();
@@ -1738,7 +1747,22 @@ namespace hipq
         return check_launch(name);
     }
 
-    template <class XL, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM, int KIND = OUT_Q8>
+    // compute units of the current device (cached per device)
+    static inline int device_compute_units()
+    {
+        static int cus[16] = {};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16)
+            return 256;
+        if (cus[dev] == 0)
+        {
+            hipDeviceProp_t prop;
+            cus[dev] = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        }
+        return cus[dev];
+    }
+
+    template <class XL, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM, int KIND = OUT_Q8, int BKT = BK>
     static int launch_pipe(const XL& xl,
                            const int8_t* w,
                            const int32_t* wsum,
@@ -1756,8 +1780,8 @@ namespace hipq
         constexpr int BM = WAVES_M * 64, BN = WAVES_N * 64;
         constexpr bool DMA = XL::kUniform;
         // (the kernels that load into LDS and take no residual stage their outputs in an operand buffer)
-        constexpr size_t lds_bytes = (DMA ? 3 : 2) * static_cast<size_t>(BM + BN) * BK + (DMA && !HAS_SUM ? 0 : 4 * 64 * 64) + 3 * BN * sizeof(float) + 16;
-        auto kernel = igemm_pipe_kernel<XL, 2, 2, WAVES_M, WAVES_N, MODE, HAS_SUM, DMA, KIND>;
+        constexpr size_t lds_bytes = (DMA && BKT == BK ? 3 : 2) * static_cast<size_t>(BM + BN) * BKT + (DMA && !HAS_SUM ? 0 : 4 * 64 * 64) + 3 * BN * sizeof(float) + 16;
+        auto kernel = igemm_pipe_kernel<XL, 2, 2, WAVES_M, WAVES_N, MODE, HAS_SUM, DMA, KIND, BKT>;
         static bool configured[16] = {};
         static int cus[16] = {};
         static int per_cu[16] = {}; // workgroups of this kernel that fit a compute unit (LDS and registers)
@@ -1783,7 +1807,8 @@ namespace hipq
         // Few tiles with long reductions leave most of the chip idle: cut every reduction into
         // `splits` runs of whole slices.
         int splits = 1;
-        const int64_t slices = (Kred + BK - 1) / BK;
+        const int64_t slices = (Kred + BKT - 1) / BKT;
+        constexpr int64_t kDeep = BKT / BK; // the thresholds below are in 64-byte slices
         const char* const split_env = getenv("HIPQ_SPLIT_K");
         if (split_env)
         {
@@ -1798,7 +1823,7 @@ namespace hipq
             // measured on ResNet-50's layers at batches 1, 32 and 128 and on GEMMs of 128 to 512 rows
             const int64_t units = dev >= 0 && dev < 16 && cus[dev] > 0 ? cus[dev] : 256;
             while (splits < 16 && slices % (splits * 2) == 0 &&
-                   ((tiles * splits * 2 * 4 <= units * 3 && slices / (splits * 2) >= 8) || (tiles * splits * 2 <= resident && slices / (splits * 2) >= 16)))
+                   ((tiles * splits * 2 * 4 <= units * 3 && slices * kDeep / (splits * 2) >= 8) || (tiles * splits * 2 <= resident && slices * kDeep / (splits * 2) >= 16)))
                 splits *= 2;
         }
         int32_t* partials = nullptr;
@@ -1851,12 +1876,39 @@ namespace hipq
             return HIPQ_ERR_UNSUPPORTED;
         if (f32 && !XL::kFloatOut)
             return HIPQ_ERR_UNSUPPORTED;
+        // row matrices with reductions in whole 128-byte pieces, no residual, wide outputs: deep slices
+        bool deep = false;
+        if constexpr (XL::kFloatOut)
+        {
+            deep = Kred % (2 * BK) == 0 && Kred >= 4 * BK && N > 64 && epi.sum_in == nullptr && getenv("HIPQ_NO_DEEP_SLICES") == nullptr;
+            // two of those workgroups fit a compute unit where three of the regular ones do: a
+            // tile count that the regular kernel takes in one round and the deep one in two stays
+            // regular (4096 x 2304 outputs, 576 tiles on 256 units: 18.9 us against 22.9)
+            const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+            const int64_t units = device_compute_units();
+            if (tiles > 2 * units && tiles <= 3 * units)
+                deep = false;
+            // few tiles with long reductions are split over workgroups, which then hold few slices
+            // each: three buffers of regular slices do better there (config 2 at 256 rows: 19.5 us
+            // against 20.9)
+            if (tiles * 8 <= units * 3 && Kred >= 16 * BK)
+                deep = false;
+        }
         if constexpr (XL::kFloatOut)
             if (f32)
             {
                 if (N <= 64)
                     return launch_pipe<XL, 4, 1, EPI_FUSED, false, OUT_F32>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+                if (deep)
+                    return launch_pipe<XL, 2, 2, EPI_FUSED, false, OUT_F32, 2 * BK>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
                 return launch_pipe<XL, 2, 2, EPI_FUSED, false, OUT_F32>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+            }
+        if constexpr (XL::kFloatOut)
+            if (deep)
+            {
+                if (epi.mode == EPI_INTERP)
+                    return launch_pipe<XL, 2, 2, EPI_INTERP, false, OUT_Q8, 2 * BK>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+                return launch_pipe<XL, 2, 2, EPI_FUSED, false, OUT_Q8, 2 * BK>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
             }
         if (epi.mode == EPI_INTERP)
         {

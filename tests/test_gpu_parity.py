@@ -716,7 +716,7 @@ def test_dot_bias_f32_tiles(gpu_lib, shape):
     O.port().orc_set_threads(1)
 
 
-@pytest.mark.parametrize("shape", [(512, 256, 384), (1024, 128, 640), (12288, 64, 1024), (16384, 64, 1152), (5000, 192, 400)])
+@pytest.mark.parametrize("shape", [(512, 256, 384), (1024, 128, 640), (12288, 64, 1024), (16384, 64, 1152), (5000, 192, 400), (2048, 512, 1152)])
 def test_dot_tile_order(gpu_lib, shape):
     """the persistent tile kernels number their tiles in groups of column blocks (squares per
     compute die): full groups of 2, 4 and 8, a narrower last group, more tiles than resident
@@ -736,6 +736,32 @@ def test_dot_tile_order(gpu_lib, shape):
         assert H.last_kernel().startswith("dot_mfma"), H.last_kernel()
         assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), (out_t, relu)
         assert len(np.unique(exp)) > 20
+    O.port().orc_set_threads(1)
+
+
+@pytest.mark.parametrize("split", ["2", "4"])
+def test_dot_deep_slices_split(gpu_lib, split, monkeypatch):
+    """reductions in whole 128-byte pieces run with slices twice as deep and two operand buffers;
+    here with the reduction also cut over workgroups, and against the regular slices"""
+    say("dot deep slices, split", split)
+    M, K, N = 300, 1024, 272
+    O.port().orc_set_threads(8)
+    a = synth.uniform_int(1401, (M, K), -128, 127, np.int8)
+    w = synth.uniform_int(1402, (N, K), -127, 127, np.int8)
+    bias = synth.uniform_int(1403, (N,), -(2**15), 2**15, np.int32)
+    scales = synth.uniform_f32(1404, (N,), 0.001, 0.01) * np.float32(0.05)
+    for out_t in ("i8", "f32"):
+        d = H.make_dot_desc(M, K, N, a_t="i8", out_t=out_t, b_layout=H.B_NK)
+        f = H.make_fused_desc(has_bias=True, with_relu=False, scale_count=N)
+        exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
+        monkeypatch.setenv("HIPQ_SPLIT_K", split)
+        got = H.quantized_dot_bias(d, f, a, w, bias, scales)
+        monkeypatch.setenv("HIPQ_NO_DEEP_SLICES", "1")
+        regular = H.quantized_dot_bias(d, f, a, w, bias, scales)
+        monkeypatch.delenv("HIPQ_NO_DEEP_SLICES")
+        monkeypatch.delenv("HIPQ_SPLIT_K")
+        assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), out_t
+        assert np.array_equal(regular.view(np.uint8), exp.view(np.uint8)), out_t
     O.port().orc_set_threads(1)
 
 

@@ -248,6 +248,8 @@ namespace hipq
         uint32_t bytes; // M * K
         static constexpr bool kUniform = true;
         static constexpr bool kFloatOut = true; // GEMM outputs may be floats; also: the loader is light enough on registers for three workgroups per compute unit
+        static constexpr bool kDeep = true;     // 128-byte-deep slices are possible
+        bool deep_ok() const { return true; }
         static constexpr bool kPads = false; // no reads of padding: an out-of-range chunk is never used
         struct Row
         {
@@ -279,6 +281,8 @@ namespace hipq
         uint32_t bytes;   // = cx.bytes
         static constexpr bool kUniform = true;
         static constexpr bool kFloatOut = false;
+        static constexpr bool kDeep = true;
+        bool deep_ok() const { return cx.C % 128 == 0; } // a 128-byte slice then lies inside one tap
         static constexpr bool kPads = true;
         struct Row
         {
@@ -315,7 +319,7 @@ namespace hipq
         __device__ __forceinline__ void advance(Cursor& c, int bytes_) const
         {
             c.c += bytes_;
-            if (c.c >= cx.C) // at most one tap further: bytes_ <= 64 <= C
+            if (c.c >= cx.C) // at most one tap further: bytes_ <= C
             {
                 c.c -= cx.C;
                 if (++c.s == cx.S)
@@ -356,6 +360,7 @@ namespace hipq
         FastDiv by_pq, by_q;
         static constexpr bool kUniform = true;
         static constexpr bool kFloatOut = false;
+        static constexpr bool kDeep = false;
         static constexpr bool kPads = false;
         struct Row
         {
@@ -929,7 +934,7 @@ namespace hipq
     // the compiler's own loads and stores are in the queue as well.
     // KIND OUT_F32 (fused policy without a residual, loaders with a uniform cursor): the scaled sums
     // leave as floats, 16 bytes a lane straight from the accumulators.
-    // BKT = 128 (row-matrix loader, no residual, reductions in whole 128-byte pieces): slices twice
+    // BKT = 128 (loads straight into LDS, no residual, reductions -- per tap -- in whole 128-byte pieces): slices twice
     // as deep, two operand buffers.  A row piece is then a whole 128-byte line, which the path from
     // L2 into LDS moves half again as fast as two 64-byte halves, and a slice has half the barriers.
     template <class XL, int WM, int WN, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM, bool DMA, int KIND = OUT_Q8, int BKT = BK>
@@ -956,7 +961,7 @@ namespace hipq
         constexpr int BM = WAVES_M * WM * 32;
         constexpr int BN = WAVES_N * WN * 32;
         constexpr int TM = WM * 32, TN = WN * 32; // a wavefront's sub-tile
-        static_assert(BKT == BK || (BKT == 2 * BK && DMA && !HAS_SUM && !XL::kPads), "deep slices: loads straight into LDS, no residual, no padding");
+        static_assert(BKT == BK || (BKT == 2 * BK && DMA && !HAS_SUM), "deep slices: loads straight into LDS, no residual");
         constexpr int LPR = BKT / 16;  // lanes that load one row's piece of a slice
         constexpr int RPI = 256 / LPR; // rows one load instruction of the workgroup covers
         constexpr int XLOADS = BM / RPI;
@@ -1179,6 +1184,8 @@ namespace hipq
             }
             return oob;
         };
+        // byte offset of 16-byte chunk `chunk` of operand row `row` inside its LDS block
+        auto frag_offset = [](int row, int chunk) { return BKT == BK ? lds_offset(row, chunk) : row * BKT + ((chunk ^ ((row >> 1) & 7)) << 4); };
         // DMA with a non-zero data zero point: chunks in the padding must hold that byte, not zero
         auto fill_fix = [&](int buf, uint32_t oob) {
             if constexpr (DMA && XL::kPads)
@@ -1188,7 +1195,7 @@ namespace hipq
 #pragma unroll
                     for (int i = 0; i < XLOADS; ++i)
                         if ((oob >> i) & 1u)
-                            *reinterpret_cast<v4i*>(lds + buf * STAGE + lds_offset(lrow + 64 * i, lchunk)) = v4i{fill, fill, fill, fill};
+                            *reinterpret_cast<v4i*>(lds + buf * STAGE + frag_offset(lrow + RPI * i, lchunk)) = v4i{fill, fill, fill, fill};
                 }
             }
         };
@@ -1211,8 +1218,6 @@ namespace hipq
                         corrv[ni][4 * g + e] = c4[e];
                 }
         };
-        // byte offset of 16-byte chunk `chunk` of operand row `row` inside its LDS block
-        auto frag_offset = [](int row, int chunk) { return BKT == BK ? lds_offset(row, chunk) : row * BKT + ((chunk ^ ((row >> 1) & 7)) << 4); };
         auto compute = [&](int buf, auto first) {
             const uint8_t* xs = lds + buf * STAGE;
             const uint8_t* ws = xs + BM * BKT;
@@ -1641,7 +1646,7 @@ namespace hipq
                     wait_vmcnt<L>();
                 else
                     wait_vmcnt<0>();
-                fill_fix(cb, oob_next);
+                fill_fix(cb, PF > 1 ? oob_next : oob_new); // the flags of the slice that has just landed
                 oob_next = oob_new;
                 ++s;
                 __syncthreads();
@@ -1878,9 +1883,9 @@ namespace hipq
             return HIPQ_ERR_UNSUPPORTED;
         // row matrices with reductions in whole 128-byte pieces, no residual, wide outputs: deep slices
         bool deep = false;
-        if constexpr (XL::kFloatOut)
+        if constexpr (XL::kDeep)
         {
-            deep = Kred % (2 * BK) == 0 && Kred >= 4 * BK && N > 64 && epi.sum_in == nullptr && getenv("HIPQ_NO_DEEP_SLICES") == nullptr;
+            deep = xl.deep_ok() && Kred % (2 * BK) == 0 && Kred >= 4 * BK && N > 64 && epi.sum_in == nullptr && getenv("HIPQ_NO_DEEP_SLICES") == nullptr;
             // two of those workgroups fit a compute unit where three of the regular ones do: a
             // tile count that the regular kernel takes in one round and the deep one in two stays
             // regular (4096 x 2304 outputs, 576 tiles on 256 units: 18.9 us against 22.9)
@@ -1903,7 +1908,7 @@ namespace hipq
                     return launch_pipe<XL, 2, 2, EPI_FUSED, false, OUT_F32, 2 * BK>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
                 return launch_pipe<XL, 2, 2, EPI_FUSED, false, OUT_F32>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
             }
-        if constexpr (XL::kFloatOut)
+        if constexpr (XL::kDeep)
             if (deep)
             {
                 if (epi.mode == EPI_INTERP)

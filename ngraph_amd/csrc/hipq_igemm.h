@@ -969,7 +969,7 @@ namespace hipq
         constexpr int STAGE = (BM + BN) * BKT;
         constexpr int OUT_STAGE = TM * TN; // per wavefront
         static_assert(TN == 64, "the output staging swizzle is written for 64-byte rows");
-        constexpr int NSTAGE = DMA && BKT == BK && !HAS_SUM ? 3 : 2; // (with a residual the output regions need room of their own: two buffers, so that three workgroups fit a compute unit)
+        constexpr int NSTAGE = DMA && BKT == BK && !HAS_SUM && WAVES_N > 1 ? 3 : 2; // (with a residual the output regions need room of their own: two buffers, so that three workgroups fit a compute unit)
         extern __shared__ __attribute__((aligned(16))) uint8_t lds[]; // [NSTAGE][x | w] operands, 4 output regions, per-channel constants
         // Without a residual input the output regions need no room of their own: a tile's outputs are
         // staged in the operand buffer that its last slice has just been multiplied out of (one more
@@ -1785,7 +1785,7 @@ namespace hipq
         constexpr int BM = WAVES_M * 64, BN = WAVES_N * 64;
         constexpr bool DMA = XL::kUniform;
         // (the kernels that load into LDS and take no residual stage their outputs in an operand buffer)
-        constexpr size_t lds_bytes = (DMA && BKT == BK && !HAS_SUM ? 3 : 2) * static_cast<size_t>(BM + BN) * BKT + (DMA && !HAS_SUM ? 0 : 4 * 64 * 64) + 3 * BN * sizeof(float) + 16;
+        constexpr size_t lds_bytes = (DMA && BKT == BK && !HAS_SUM && WAVES_N > 1 ? 3 : 2) * static_cast<size_t>(BM + BN) * BKT + (DMA && !HAS_SUM ? 0 : 4 * 64 * 64) + 3 * BN * sizeof(float) + 16;
         auto kernel = igemm_pipe_kernel<XL, 2, 2, WAVES_M, WAVES_N, MODE, HAS_SUM, DMA, KIND, BKT>;
         static bool configured[16] = {};
         static int cus[16] = {};

@@ -924,14 +924,18 @@ namespace hipq
     // tiles' arithmetic and epilogues, and long ones have two slices of latency cover.  Each
     // wavefront requantizes its own 64 x 64 sub-tile into a private swizzled LDS region and writes it
     // out 16 bytes a lane; per-channel constants of the current column tile sit in LDS.
+    // (That is the register-staged variant; the one below prefetches one or two slices and is
+    // written as a loop nest per tile.)
     //
     // DMA variant (loaders with a uniform cursor): the slices go from global memory straight into
     // LDS (buffer loads with the lds modifier, 16 bytes a lane, a wavefront's 64 lanes filling one
     // contiguous KiB, so the swizzle is applied to what a lane reads instead of where it writes),
-    // three buffers deep: no staging registers, no LDS stores, and the sign flip of unsigned data
-    // moves to the MFMA fragments.  These loads are written in assembly, so the waits for them are
-    // explicit: a wait for "at most n operations in flight" only ever errs on the long side when
-    // the compiler's own loads and stores are in the queue as well.
+    // three buffers deep (two where LDS is better spent on a third workgroup per compute unit: the
+    // kernels with a residual input, the narrow tiles, the deep slices): no staging registers, no
+    // LDS stores, and the sign flip of unsigned data moves to the MFMA fragments.  These loads are
+    // written in assembly, so the waits for them are explicit: a wait for "at most n operations in
+    // flight" only ever errs on the long side when the compiler's own loads and stores are in the
+    // queue as well.
     // KIND OUT_F32 (fused policy without a residual, loaders with a uniform cursor): the scaled sums
     // leave as floats, 16 bytes a lane straight from the accumulators.
     // BKT = 128 (loads straight into LDS, no residual, reductions -- per tap -- in whole 128-byte pieces): slices twice

@@ -263,7 +263,7 @@ int hipq_capture_end(void* stream, void** graph_exec)
     HIPQ_HIP(hipStreamEndCapture(as_stream(stream), &graph));
     hipGraphExec_t exec = nullptr;
     hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-    hipGraphDestroy(graph);
+    (void)hipGraphDestroy(graph); // the executable graph keeps what it needs
     if (e != hipSuccess)
         return fail(HIPQ_ERR_HIP, "hipGraphInstantiate: %s", hipGetErrorString(e));
     *graph_exec = exec;

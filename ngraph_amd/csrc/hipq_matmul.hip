@@ -32,13 +32,13 @@ namespace hipq
             const int m0 = mt * TM, n0 = nt * TN;
             const int tm = (tid >> 4) * 4, tn = (tid & 15) * 4; // this lane's 4 x 4 outputs within the tile
             double acc[4][4] = {};
-            for (int k0 = 0; k0 < K; k0 += TK)
-            {
-                // 64 x 16 elements of each operand, four a lane, contiguous along the operand's rows in memory
+            // 64 x 16 elements of each operand, four a lane, contiguous along the operand's rows in
+            // memory; the next step's elements are fetched into registers while this step multiplies
+            auto fetch_a = [&](int k0) -> f4 {
+                f4 v = f4{0.0f, 0.0f, 0.0f, 0.0f};
                 if (!ta)
                 {
                     const int r = tid >> 2, kq = (tid & 3) * 4; // A[m0 + r][k0 + kq ..]
-                    f4 v = f4{0.0f, 0.0f, 0.0f, 0.0f};
                     if (vec_a && m0 + r < M && k0 + kq + 3 < K)
                         v = *reinterpret_cast<const f4*>(A + static_cast<int64_t>(m0 + r) * K + k0 + kq);
                     else
@@ -47,14 +47,10 @@ namespace hipq
                         for (int i = 0; i < 4; ++i)
                             v[i] = (m0 + r < M && k0 + kq + i < K) ? A[static_cast<int64_t>(m0 + r) * K + k0 + kq + i] : 0.0f;
                     }
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        as[kq + i][r] = v[i];
                 }
                 else
                 {
                     const int kk = tid >> 4, mq = (tid & 15) * 4; // A[k0 + kk][m0 + mq ..]
-                    f4 v = f4{0.0f, 0.0f, 0.0f, 0.0f};
                     if (vec_a && k0 + kk < K && m0 + mq + 3 < M)
                         v = *reinterpret_cast<const f4*>(A + static_cast<int64_t>(k0 + kk) * M + m0 + mq);
                     else
@@ -63,12 +59,28 @@ namespace hipq
                         for (int i = 0; i < 4; ++i)
                             v[i] = (k0 + kk < K && m0 + mq + i < M) ? A[static_cast<int64_t>(k0 + kk) * M + m0 + mq + i] : 0.0f;
                     }
+                }
+                return v;
+            };
+            auto put_a = [&](f4 v) {
+                if (!ta)
+                {
+                    const int r = tid >> 2, kq = (tid & 3) * 4;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        as[kq + i][r] = v[i];
+                }
+                else
+                {
+                    const int kk = tid >> 4, mq = (tid & 15) * 4;
                     *reinterpret_cast<f4*>(&as[kk][mq]) = v;
                 }
+            };
+            auto fetch_b = [&](int k0) -> f4 {
+                f4 v = f4{0.0f, 0.0f, 0.0f, 0.0f};
                 if (!tb)
                 {
                     const int kk = tid >> 4, nq = (tid & 15) * 4; // B[k0 + kk][n0 + nq ..]
-                    f4 v = f4{0.0f, 0.0f, 0.0f, 0.0f};
                     if (vec_b && k0 + kk < K && n0 + nq + 3 < N)
                         v = *reinterpret_cast<const f4*>(B + static_cast<int64_t>(k0 + kk) * N + n0 + nq);
                     else
@@ -77,12 +89,10 @@ namespace hipq
                         for (int i = 0; i < 4; ++i)
                             v[i] = (k0 + kk < K && n0 + nq + i < N) ? B[static_cast<int64_t>(k0 + kk) * N + n0 + nq + i] : 0.0f;
                     }
-                    *reinterpret_cast<f4*>(&bs[kk][nq]) = v;
                 }
                 else
                 {
                     const int r = tid >> 2, kq = (tid & 3) * 4; // B[n0 + r][k0 + kq ..]
-                    f4 v = f4{0.0f, 0.0f, 0.0f, 0.0f};
                     if (vec_b && n0 + r < N && k0 + kq + 3 < K)
                         v = *reinterpret_cast<const f4*>(B + static_cast<int64_t>(n0 + r) * K + k0 + kq);
                     else
@@ -91,11 +101,34 @@ namespace hipq
                         for (int i = 0; i < 4; ++i)
                             v[i] = (n0 + r < N && k0 + kq + i < K) ? B[static_cast<int64_t>(n0 + r) * K + k0 + kq + i] : 0.0f;
                     }
+                }
+                return v;
+            };
+            auto put_b = [&](f4 v) {
+                if (!tb)
+                {
+                    const int kk = tid >> 4, nq = (tid & 15) * 4;
+                    *reinterpret_cast<f4*>(&bs[kk][nq]) = v;
+                }
+                else
+                {
+                    const int r = tid >> 2, kq = (tid & 3) * 4;
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
                         bs[kq + i][r] = v[i];
                 }
+            };
+            f4 va = fetch_a(0), vb = fetch_b(0);
+            for (int k0 = 0; k0 < K; k0 += TK)
+            {
+                put_a(va);
+                put_b(vb);
                 __syncthreads();
+                if (k0 + TK < K) // uniform
+                {
+                    va = fetch_a(k0 + TK);
+                    vb = fetch_b(k0 + TK);
+                }
 #pragma unroll
                 for (int k = 0; k < TK; ++k)
                 {

@@ -513,6 +513,42 @@ def test_conv_register_staged(gpu_lib, i, monkeypatch):
     test_conv_split_reduction(gpu_lib, i)
 
 
+@pytest.mark.parametrize("stride", [1, 2])
+def test_conv_deep_slices_padding(gpu_lib, stride, monkeypatch):
+    """windows over 128 channels with enough tiles to take the 128-byte-deep slices (two operand
+    buffers): padded borders with a non-zero data zero point are patched in after the loads land,
+    one slice ahead instead of two; both policies, against the oracle and the regular slices"""
+    say("conv deep slices with padding, stride", stride)
+    N, Cc, K = (4, 128, 128) if stride == 1 else (16, 128, 256)
+    in_sp, f_sp = (56, 56), (3, 3)
+    kw = dict(stride=(stride, stride), pad_below=(1, 1), pad_above=(1, 1))
+    O.port().orc_set_threads(8)
+    d = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t="u8", data_layout=H.NXC, out_layout=H.NXC, **kw)
+    dn = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t="u8", **kw)
+    data = synth.uniform_int(3100 + stride, dn.data_shape(), 0, 255, np.uint8)
+    filt = synth.uniform_int(3200, dn.filter_shape(), -128, 127, np.int8)
+    for z in ((131, 0, 7), (0, 0, 0)):
+        s = (0.02, 0.005, 2.5)
+        exp = O.quantized_convolution(dn, data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
+        got = H.quantized_convolution(d, cases.to_nxc(data), filt, s[0], z[0], s[1], z[1], s[2], z[2])
+        assert H.last_kernel().startswith("conv_mfma"), H.last_kernel()
+        assert np.array_equal(cases.to_ncx(got), exp), z
+        assert len(np.unique(exp)) > 50
+        monkeypatch.setenv("HIPQ_NO_DEEP_SLICES", "1")
+        regular = H.quantized_convolution(d, cases.to_nxc(data), filt, s[0], z[0], s[1], z[1], s[2], z[2])
+        monkeypatch.delenv("HIPQ_NO_DEEP_SLICES")
+        assert np.array_equal(regular, got), z
+    df = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t="i8", data_layout=H.NXC, out_layout=H.NXC, **kw)
+    dfn = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t="i8", **kw)
+    f = H.make_fused_desc(has_bias=True, with_relu=False, scale_count=K)
+    bias = synth.uniform_int(3300, (K,), -20000, 20000, np.int32)
+    scales = synth.uniform_f32(3301, (K,), 2e-4, 9e-4)
+    exp = O.quantized_convolution_fused(dfn, f, data, filt, bias, None, scales, None)
+    got = H.quantized_convolution_fused(df, f, cases.to_nxc(data), filt, bias, None, scales, None)
+    assert np.array_equal(cases.to_ncx(got), exp)
+    O.port().orc_set_threads(1)
+
+
 @pytest.mark.parametrize("i", range(len(SPLIT_CONV_SHAPES)))
 def test_conv_split_forced(gpu_lib, i, monkeypatch):
     """the same shapes with every reduction cut in two whatever the launch heuristic would choose"""

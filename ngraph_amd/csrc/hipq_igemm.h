@@ -1803,7 +1803,11 @@ namespace hipq
             HIPQ_HIP(hipGetDeviceProperties(&prop, dev));
             cus[dev] = prop.multiProcessorCount;
             int fit = 0;
-            HIPQ_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&fit, reinterpret_cast<const void*>(kernel), 256, lds_bytes));
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&fit, reinterpret_cast<const void*>(kernel), 256, lds_bytes) != hipSuccess)
+            {
+                (void)hipGetLastError(); // no answer: size the grid by LDS alone
+                fit = 0;
+            }
             const int by_lds = static_cast<int>(160 * 1024 / lds_bytes);
             per_cu[dev] = fit >= 1 && fit < by_lds ? fit : by_lds;
             configured[dev] = true;

@@ -38,32 +38,48 @@ namespace hipq
 
     // [N][C][H][W] or [N][H][W][C] bytes -> [N][Hp][Wp][4]: staged pixel (y, x) is input pixel
     // (y - pad_h, x - pad_w) where that exists; everything else, and the channels beyond C, hold the
-    // data zero point.  One staged pixel (one dword) a lane, one staged row (image, y) a block
-    // column: the only division is the block's own, of its row number by Hp.
-    __global__ __launch_bounds__(256) void stage_rows_kernel(const uint8_t* __restrict__ in, uint32_t* __restrict__ out, int32_t Hp, int32_t Wp, int32_t H, int32_t W,
+    // data zero point.  One staged pixel (one dword) a lane and kStageRows staged rows (image, y) a
+    // block column, their loads all issued before the first store: a block that moves one row
+    // lives for one memory round trip, and a compute unit holds too few of those to cover it.
+    constexpr int kStageRows = 8;
+    __global__ __launch_bounds__(256) void stage_rows_kernel(const uint8_t* __restrict__ in, uint32_t* __restrict__ out, uint32_t rows, int32_t Hp, int32_t Wp, int32_t H, int32_t W,
                                                              int32_t Cc, int32_t pbh, int32_t pbw, int32_t in_ncx, const void* zp, int32_t zp_t)
     {
         const int32_t xp = static_cast<int32_t>(blockIdx.y) * 256 + static_cast<int32_t>(threadIdx.x);
         if (xp >= Wp)
             return;
-        const uint32_t row = blockIdx.x; // image * Hp + yp
-        const uint32_t n = row / static_cast<uint32_t>(Hp);
-        const int32_t yp = static_cast<int32_t>(row - n * static_cast<uint32_t>(Hp));
-        const int32_t y = yp - pbh, x = xp - pbw;
-        uint32_t v = (static_cast<uint32_t>(load_zp(zp, zp_t)) & 0xffu) * 0x01010101u;
-        if (static_cast<uint32_t>(y) < static_cast<uint32_t>(H) && static_cast<uint32_t>(x) < static_cast<uint32_t>(W))
+        const uint32_t fill = (static_cast<uint32_t>(load_zp(zp, zp_t)) & 0xffu) * 0x01010101u;
+        const int32_t x = xp - pbw;
+        const int64_t X = static_cast<int64_t>(H) * W;
+        const int64_t step = in_ncx ? X : 1;
+        uint32_t v[kStageRows];
+#pragma unroll
+        for (int i = 0; i < kStageRows; ++i)
         {
-            const int64_t X = static_cast<int64_t>(H) * W;
-            const int64_t pix = static_cast<int64_t>(y) * W + x;
-            const uint8_t* p = in_ncx ? in + static_cast<int64_t>(n) * Cc * X + pix : in + (static_cast<int64_t>(n) * X + pix) * Cc;
-            const int64_t step = in_ncx ? X : 1;
-            for (int c = 0; c < Cc; ++c)
+            const uint32_t row = blockIdx.x * kStageRows + i; // image * Hp + yp
+            v[i] = fill;
+            if (row >= rows)
+                continue;
+            const uint32_t n = row / static_cast<uint32_t>(Hp);
+            const int32_t y = static_cast<int32_t>(row - n * static_cast<uint32_t>(Hp)) - pbh;
+            if (static_cast<uint32_t>(y) < static_cast<uint32_t>(H) && static_cast<uint32_t>(x) < static_cast<uint32_t>(W))
             {
-                const uint32_t b = p[c * step];
-                v = (v & ~(0xffu << (8 * c))) | (b << (8 * c));
+                const int64_t pix = static_cast<int64_t>(y) * W + x;
+                const uint8_t* p = in_ncx ? in + static_cast<int64_t>(n) * Cc * X + pix : in + (static_cast<int64_t>(n) * X + pix) * Cc;
+                for (int c = 0; c < Cc; ++c)
+                {
+                    const uint32_t b = p[c * step];
+                    v[i] = (v[i] & ~(0xffu << (8 * c))) | (b << (8 * c));
+                }
             }
         }
-        out[static_cast<int64_t>(row) * Wp + xp] = v;
+#pragma unroll
+        for (int i = 0; i < kStageRows; ++i)
+        {
+            const uint32_t row = blockIdx.x * kStageRows + i;
+            if (row < rows)
+                out[static_cast<int64_t>(row) * Wp + xp] = v[i];
+        }
     }
 
     int launch_stage_rows(const ConvGeom& g, const RowPack& rp, const void* in, void* staged, const void* zp, int zp_t, hipStream_t s)
@@ -72,10 +88,10 @@ namespace hipq
         if (rows == 0 || rp.Wp == 0)
             return HIPQ_OK;
         HIPQ_REQUIRE(rows < (1ll << 31) && (rp.Wp + 255) / 256 <= 65535, "tensor too large for one launch");
-        dim3 grid(static_cast<unsigned>(rows), static_cast<unsigned>((rp.Wp + 255) / 256));
-        stage_rows_kernel<<<grid, 256, 0, s>>>(static_cast<const uint8_t*>(in), static_cast<uint32_t*>(staged), static_cast<int32_t>(rp.Hp), static_cast<int32_t>(rp.Wp),
-                                               static_cast<int32_t>(g.in[1]), static_cast<int32_t>(g.in[2]), static_cast<int32_t>(g.C), static_cast<int32_t>(g.pb[1]),
-                                               static_cast<int32_t>(g.pb[2]), g.data_layout == HIPQ_LAYOUT_NCX ? 1 : 0, zp, zp_t);
+        dim3 grid(static_cast<unsigned>((rows + kStageRows - 1) / kStageRows), static_cast<unsigned>((rp.Wp + 255) / 256));
+        stage_rows_kernel<<<grid, 256, 0, s>>>(static_cast<const uint8_t*>(in), static_cast<uint32_t*>(staged), static_cast<uint32_t>(rows), static_cast<int32_t>(rp.Hp),
+                                               static_cast<int32_t>(rp.Wp), static_cast<int32_t>(g.in[1]), static_cast<int32_t>(g.in[2]), static_cast<int32_t>(g.C),
+                                               static_cast<int32_t>(g.pb[1]), static_cast<int32_t>(g.pb[2]), g.data_layout == HIPQ_LAYOUT_NCX ? 1 : 0, zp, zp_t);
         return check_launch("stage_rows");
     }
 

@@ -28,9 +28,12 @@ from ngraph_amd import synth  # noqa: E402
 
 PEAK_I8_TOPS = 5000.0  # MI355X dense int8 MFMA, published
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published
-# HBM bytes per launch of the headline kernel at batch 128, from the FETCH_SIZE / WRITE_SIZE
-# counter runs summarised in profiles/conv_band_config1_hbm_traffic.md (scaled by a 64 MiB copy)
+# HBM bytes per launch of the headline kernel at batch 128: not measured by this run (counters need
+# a profiler run of their own) but quoted from the FETCH_SIZE / WRITE_SIZE runs summarised in the
+# file below (scaled by a 64 MiB copy in the same run); the JSON line names that file
 MEASURED_TRAFFIC_BYTES = {("conv_band_i8_32x32x32", 128): 52.3e6}
+TRAFFIC_SOURCE = "profiles/conv_band_config1_hbm_traffic.md"
+_DATA_CACHE = {}
 
 
 class Timer:
@@ -70,9 +73,12 @@ def scalar(v, dt):
 def bench_conv(lib, stream, timer, N, steps, warmup, layout, out_layout=None):
     out_layout = layout if out_layout is None else out_layout
     d = H.make_conv_desc(N, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1), data_layout=layout, out_layout=out_layout)
-    one = H.make_conv_desc(1, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1), data_layout=layout, out_layout=out_layout)
-    img = synth.uniform_int(1001, one.data_shape(), 0, 255, np.uint8)
-    data = dev(np.ascontiguousarray(np.broadcast_to(img, d.data_shape())))
+    # every image of the batch has bytes of its own (operand content moves this chip's clock: a
+    # batch of copies of one image would flatter the kernel); the channels-last tensor holds the same
+    # seeded values as the NCHW one, read in its own order
+    if N not in _DATA_CACHE:
+        _DATA_CACHE[N] = synth.uniform_int(1001, (N, 64, 56, 56), 0, 255, np.uint8)
+    data = dev(_DATA_CACHE[N].reshape(d.data_shape()))
     filt = dev(synth.uniform_int(1002, d.filter_shape(), -127, 127, np.int8))
     packed = H.pack_filter(d, filt)
     assert packed is not None
@@ -240,7 +246,7 @@ def bench_fp32_glue(lib, stream, timer, steps, warmup):
     return out
 
 
-def bench_bert(lib, stream, timer, batches=(1, 32)):
+def bench_bert(lib, stream, timer, batches=(1, 32), use_graph=True):
     """synthetic int8 BERT-base-shaped encoder (ngraph_amd/bert.py): 12 layers of QuantizedDotBias projections
     with f32 attention, Softmax, Gelu and LayerNorm between them, sequence 128, every tensor resident in HBM"""
     from ngraph_amd import bert as B
@@ -251,16 +257,18 @@ def bench_bert(lib, stream, timer, batches=(1, 32)):
         plan.set_input(B.embeddings(B.BASE, n))
         steps = 10 if n <= 8 else 5
         _, eager = timer.run(plan.launch, steps, 2)
-        plan.capture()
-        _, graph = timer.run(plan.replay, steps, 2)
-        H.check(lib.hipq_graph_destroy(plan.graph))
-        best = min(eager, graph)
+        graph = None
+        if use_graph:
+            plan.capture()
+            _, graph = timer.run(plan.replay, steps, 2)
+            plan.close()
+        best = eager if graph is None else min(eager, graph)
         out.append(dict(batch=n, ms_eager=eager, ms_graph=graph, sequences_per_s=n / (best * 1e-3), int8_tops=2 * B.BASE.macs_per_sequence() * n / (best * 1e-3) / 1e12, launches=len(plan.calls)))
         del plan
     return out
 
 
-def bench_resnet50(lib, stream, timer, batches=(1, 32, 128)):
+def bench_resnet50(lib, stream, timer, batches=(1, 32, 128), use_graph=True):
     """synthetic int8 ResNet-50 (ngraph_amd/resnet50.py), every tensor resident in HBM, channels-last,
     one forward pass = 53 convolutions, 2 pools, 1 GEMM; replayed as one HIP graph"""
     from ngraph_amd import resnet50 as R
@@ -271,43 +279,113 @@ def bench_resnet50(lib, stream, timer, batches=(1, 32, 128)):
         plan.set_images_nchw(R.synthetic_images(min(n, 4)).repeat((n + 3) // 4, axis=0)[:n])
         steps = 30 if n <= 32 else 10
         _, eager = timer.run(plan.launch, steps, 2)
-        plan.capture()
-        _, graph = timer.run(plan.replay, steps, 2)
-        H.check(lib.hipq_graph_destroy(plan.graph))
-        best = min(eager, graph)
+        graph = None
+        if use_graph:
+            plan.capture()
+            _, graph = timer.run(plan.replay, steps, 2)
+            plan.close()
+        best = eager if graph is None else min(eager, graph)
         out.append(dict(batch=n, ms_eager=eager, ms_graph=graph, images_per_s=n / (best * 1e-3), tops=plan.ops_per_image * n / (best * 1e-3) / 1e12, launches=len(plan.calls)))
         del plan
     return out
 
 
-def cpu_baseline(seconds=12.0):
-    """The reference's own convolution kernel (oracle/_ref, compiled from the nGraph tree) when it
-    was built, else the C restatement; BASELINE config 1 at N=1 on one host core."""
+def host_threads():
+    """threads for the host baselines: this process's share of the machine (OMP_NUM_THREADS when the
+    environment sets it, never more than the CPUs the process may run on)"""
+    try:
+        allowed = len(os.sched_getaffinity(0))
+    except AttributeError:
+        allowed = os.cpu_count() or 1
+    env = os.environ.get("OMP_NUM_THREADS", "")
+    want = int(env) if env.isdigit() and int(env) > 0 else allowed
+    return max(1, min(want, allowed))
+
+
+def cpu_onednn_conv(batch, threads, seconds=6.0):
+    """The headline layer as an int8 convolution through the oneDNN that ships inside PyTorch, all of
+    this process's cores.  A DNNL-class stand-in for the reference's CPU backend (which drives oneDNN
+    1.6.2 and cannot be built offline) -- not nGraph's own code, and its u8 output saturates where the
+    INTERPRETER wraps, so it is timed, not compared."""
+    try:
+        import torch
+
+        if "onednn" not in torch.backends.quantized.supported_engines:
+            return dict(status="unavailable", reason="torch has no onednn quantized engine")
+        torch.set_num_threads(threads)
+        torch.backends.quantized.engine = "onednn"
+        g = torch.Generator().manual_seed(1001)
+        x = torch.randint(0, 256, (batch, 64, 56, 56), dtype=torch.uint8, generator=g)
+        w = torch.randint(-127, 128, (64, 64, 3, 3), dtype=torch.int8, generator=g)
+        qx = torch._make_per_tensor_quantized_tensor(x, 0.02, 0)
+        qw = torch._make_per_tensor_quantized_tensor(w, 0.005, 0)
+        packed = torch.ops.quantized.conv2d_prepack(qw, None, [1, 1], [1, 1], [1, 1], 1)
+        for _ in range(2):
+            torch.ops.quantized.conv2d(qx, packed, 0.1, 0)
+        calls, t0 = 0, time.perf_counter()
+        while True:
+            torch.ops.quantized.conv2d(qx, packed, 0.1, 0)
+            calls += 1
+            el = time.perf_counter() - t0
+            if el >= seconds or calls >= 100000:
+                break
+        ops = 2 * batch * 64 * 64 * 9 * 56 * 56
+        ver = [l.strip() for l in torch.__config__.show().splitlines() if "oneDNN" in l or "MKL-DNN" in l]
+        return dict(value=ops * calls / el / 1e12, unit="TOP/s", cores=threads, kind="oneDNN via torch %s (quantized engine 'onednn'), not nGraph-CPU" % torch.__version__,
+                    library=ver[0] if ver else "", sample="%d calls of quantized.conv2d u8[%d,64,56,56] x i8[64,64,3,3] -> u8, %.1f s" % (calls, batch, el))
+    except Exception as e:  # informative only
+        return dict(status="unavailable", reason=repr(e)[:200])
+
+
+def cpu_baseline(batch, seconds=8.0):
+    """Host baselines, timed on this machine in the same run, each on a bounded sample:
+    * value: the C restatement of the reference kernel (oracle/, OpenMP over output planes) on the
+      headline layer at batch `min(batch, 32)`, all of this process's cores -- "port";
+    * reference_1core: runtime::reference::convolution itself (oracle/_ref, compiled from the nGraph
+      tree) when it was built, config 1 at N=1, one core;
+    * onednn_via_torch: the DNNL-class figure (see cpu_onednn_conv);
+    * resnet50_int8: one image of the synthetic ResNet-50 through the C restatement, all cores."""
     import oracle_lib as O
 
-    d = H.make_conv_desc(1, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1))
+    threads = host_threads()
+    nb = min(batch, 32)
+    d = H.make_conv_desc(nb, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1))
     data = synth.uniform_int(1001, d.data_shape(), 0, 255, np.uint8)
     filt = synth.uniform_int(1002, d.filter_shape(), -127, 127, np.int8)
-    kind = "reference" if O.have_ref() else "port"
-    fn = O.ref_quantized_convolution if kind == "reference" else O.quantized_convolution
-    O.port().orc_set_threads(1)
+    O.port().orc_set_threads(threads)
     calls, t0 = 0, time.perf_counter()
     while True:
-        fn(d, data, filt, 0.02, 0, 0.005, 0, 0.1, 0)
+        O.quantized_convolution(d, data, filt, 0.02, 0, 0.005, 0, 0.1, 0)
         calls += 1
         el = time.perf_counter() - t0
-        if el >= seconds or calls >= 200:
+        if el >= seconds or calls >= 100:
             break
+    O.port().orc_set_threads(1)
     out = dict(
         value=d.ops() * calls / el / 1e12,
         unit="TOP/s",
-        cores=1,
-        kind=kind,
-        sample="%d calls of QuantizedConvolution u8[1,64,56,56] x i8[64,64,3,3] -> i8 (config 1, N=1), %.1f s, %s"
-        % (calls, el, "runtime::reference::convolution compiled from the nGraph tree" if kind == "reference" else "C restatement of it"),
+        cores=threads,
+        host_cpus=os.cpu_count(),
+        kind="port",
+        sample="%d calls of QuantizedConvolution u8[%d,64,56,56] x i8[64,64,3,3] -> i8 (the headline layer at batch %d), %.1f s, C restatement of runtime::reference::convolution with OpenMP"
+        % (calls, nb, nb, el),
     )
+    # the reference's own kernel, one core, config 1 as BASELINE states it (N=1)
+    d1 = H.make_conv_desc(1, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1))
+    kind = "reference" if O.have_ref() else "port"
+    fn = O.ref_quantized_convolution if kind == "reference" else O.quantized_convolution
+    calls, t0 = 0, time.perf_counter()
+    while True:
+        fn(d1, data[:1], filt, 0.02, 0, 0.005, 0, 0.1, 0)
+        calls += 1
+        el = time.perf_counter() - t0
+        if el >= seconds / 2 or calls >= 100:
+            break
+    out["reference_1core"] = dict(value=d1.ops() * calls / el / 1e12, unit="TOP/s", cores=1, kind=kind,
+                                  sample="%d calls of config 1 at N=1, %.1f s, %s" % (calls, el, "runtime::reference::convolution compiled from the nGraph tree" if kind == "reference" else "C restatement of it"))
+    out["onednn_via_torch"] = cpu_onednn_conv(nb, threads)
     # the synthetic ResNet-50 on the host: one image through the C restatement of its ops (the fused
-    # ops exist only in the reference's CPU backend, which does not build here), all of this box's share of cores
+    # ops exist only in the reference's CPU backend, which does not build here)
     try:
         from ngraph_amd import resnet50 as R
 
@@ -316,7 +394,6 @@ def cpu_baseline(seconds=12.0):
             pool = staticmethod(lambda d, x: O.pool(d, x))
             dot_bias = staticmethod(lambda d, f, a, w, bias, sc: O.quantized_dot_bias(d, f, a, w, bias, sc))
 
-        threads = 16
         O.port().orc_set_threads(threads)
         t0 = time.perf_counter()
         R.run(Port, R.synthetic_images(1))
@@ -338,6 +415,7 @@ def main():
     ap.add_argument("--resnet-only", action="store_true", help="only the synthetic int8 ResNet-50 (for profiling); prints its results")
     ap.add_argument("--bert-only", action="store_true", help="only the synthetic int8 BERT-base encoder (for profiling); prints its results")
     ap.add_argument("--skip-models", action="store_true", help="leave out the BERT and ResNet-50 sections (kernel traces of the single operators; the models have runs of their own)")
+    ap.add_argument("--no-graph", action="store_true", help="time the models' eager launch sequences only, no HIP-graph capture or replay (for runs under a profiler)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -353,10 +431,10 @@ def main():
     timer = Timer(lib, stream)
 
     if args.resnet_only:
-        print(json.dumps({"resnet50_int8": bench_resnet50(lib, stream, timer)}))
+        print(json.dumps({"resnet50_int8": bench_resnet50(lib, stream, timer, use_graph=not args.no_graph)}))
         return
     if args.bert_only:
-        print(json.dumps({"bert_base_int8": bench_bert(lib, stream, timer)}))
+        print(json.dumps({"bert_base_int8": bench_bert(lib, stream, timer, use_graph=not args.no_graph)}))
         return
 
     # headline: the reference's NCHW tensors in, NCHW out
@@ -393,9 +471,9 @@ def main():
         results["glue_resnet50_u8"] = bench_glue(lib, stream, timer, small, 5, args.batch)
         results["fp32_glue_bert_base"] = bench_fp32_glue(lib, stream, timer, small, 5)
         if not args.skip_models:
-            results["bert_base_int8"] = bench_bert(lib, stream, timer)
-            results["resnet50_int8"] = bench_resnet50(lib, stream, timer)
-        cpu = cpu_baseline()
+            results["bert_base_int8"] = bench_bert(lib, stream, timer, use_graph=not args.no_graph)
+            results["resnet50_int8"] = bench_resnet50(lib, stream, timer, use_graph=not args.no_graph)
+        cpu = cpu_baseline(args.batch)
 
     derived_peak = info.compute_units * info.clock_mhz * 1e6 * 8192 / 1e12
     line = {
@@ -412,8 +490,8 @@ def main():
         "dtype": "i8",
         "data": "synthetic",
         "config": {
-            "workload": "op::v0::QuantizedConvolution u8[%d,64,56,56] x i8[64,64,3,3] -> i8, stride 1, pad 1 (BASELINE config 1 layer at batch %d), NCHW in / NCHW out through the C ABI, filter prepacked"
-            % (args.batch, args.batch),
+            "workload": "op::v0::QuantizedConvolution u8[%d,64,56,56] x i8[64,64,3,3] -> i8, stride 1, pad 1 (BASELINE config 1 layer at batch %d), NCHW in / NCHW out through the C ABI, filter prepacked; %d distinct seeded images"
+            % (args.batch, args.batch, args.batch),
             "ops_per_step": head["ops"],
             "device": info.name.decode(),
             "compute_units": info.compute_units,
@@ -428,6 +506,7 @@ def main():
             "unit": "TOP/s",
             "frac": kern["tops_event"] / PEAK_I8_TOPS,
             "traffic": MEASURED_TRAFFIC_BYTES.get((kern["kernel"], args.batch)),
+            "traffic_source": TRAFFIC_SOURCE + " (counter runs of this command; not measured by this run)",
             "algorithmic_bytes": 2 * args.batch * 64 * 56 * 56 + 64 * 64 * 9,
             "kernel_ms": kern["ms_event"],
         },

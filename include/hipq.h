@@ -343,8 +343,14 @@ typedef enum
     HIPQ_OP_MULTIPLY = 2,
     HIPQ_OP_DIVIDE = 3,
     HIPQ_OP_MAXIMUM = 4,
-    HIPQ_OP_MINIMUM = 5
+    HIPQ_OP_MINIMUM = 5,
+    HIPQ_OP_DIVIDE_FLOOR = 6
 } hipq_binary_op_t;
+/* HIPQ_OP_DIVIDE is op::v1::Divide with is_pythondiv() false (C++ truncation), HIPQ_OP_DIVIDE_FLOOR
+ * with it true, the op's default (src/ngraph/op/divide.hpp:72,
+ * src/ngraph/runtime/reference/divide.hpp:41-60: quotient less one when the remainder is not zero
+ * and the signs differ); floating types divide the same way under both.  Deviation: the reference
+ * throws std::domain_error on an integer zero divisor; a kernel cannot throw, the element is 0. */
 
 typedef enum
 {

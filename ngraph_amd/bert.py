@@ -164,6 +164,7 @@ class DevicePlan:
 
     def __init__(self, lib, stream, batch, cfg=BASE):
         self.lib, self.stream, self.batch, self.cfg = lib, stream, batch, cfg
+        self._replay = None
         self.calls, self.keep, self.graph = [], [], None
         vp, i64, i32 = C.c_void_p, C.c_int64, C.c_int32
         lib.hipq_softmax_f32.argtypes = [vp, vp, i64, i64, i64, vp]
@@ -249,18 +250,22 @@ class DevicePlan:
                 H.check(rc)
 
     def capture(self):
-        self.launch()  # sizes the library's workspaces before anything is recorded
-        H.check(self.lib.hipq_stream_sync(self.stream))
-        H.check(self.lib.hipq_capture_begin(self.stream))
-        self.launch()
-        g = C.c_void_p()
-        H.check(self.lib.hipq_capture_end(self.stream, C.byref(g)))
-        self.graph = g
+        """records the pass into a HIP graph (after one eager pass that sizes the library's scratch)"""
+        if self._replay is None:
+            self._replay = H.GraphReplay(self.lib, self.stream, self.launch)
+        self._replay.capture()
 
     def replay(self):
-        rc = self.lib.hipq_graph_launch(self.graph, self.stream)
-        if rc:
-            H.check(rc)
+        """launches the recorded graph; records it again first if the library's scratch has moved"""
+        if self._replay is None:
+            self.capture()
+        self._replay.replay()
+
+    def close(self):
+        """destroys the recorded graph (the buffers go with the object)"""
+        if self._replay is not None:
+            self._replay.close()
+            self._replay = None
 
     def read_output(self):
         H.check(self.lib.hipq_stream_sync(self.stream))

@@ -34,13 +34,16 @@ namespace hipq
     inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
     int check_launch(const char* kernel);
 
-    // Grow-only device workspace, one per device, shared by every call on that device (calls that
-    // need it and overlap on different streams would race; the backend serialises per executable).
-    int workspace(size_t bytes, void** ptr);
-    // a second block for reductions split over workgroups: zeroed tile counters (kSplitCounterBytes of
-    // them) followed by `partial_bytes` for partial sums
+    // Grow-only device workspace, one per (device, stream): launches on different streams never
+    // share a block, so callers that run on streams of their own may overlap.  Growing a block waits
+    // for its stream and frees the old one.
+    int workspace(size_t bytes, hipStream_t stream, void** ptr);
+    // a second block per (device, stream) for reductions split over workgroups: zeroed tile counters
+    // (kSplitCounterBytes of them) followed by `partial_bytes` for partial sums
     constexpr size_t kSplitCounterBytes = 64 * 1024;
-    int split_workspace(size_t partial_bytes, uint32_t** counters, void** partials);
+    int split_workspace(size_t partial_bytes, hipStream_t stream, uint32_t** counters, void** partials);
+    // frees the blocks of a stream that is about to be destroyed
+    int release_stream_workspace(hipStream_t stream);
 
     inline size_t dtype_size(int t)
     {

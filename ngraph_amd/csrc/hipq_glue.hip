@@ -3,6 +3,22 @@
 
 namespace hipq
 {
+    // reference::divide with pythondiv (src/ngraph/runtime/reference/divide.hpp:41-60): the truncated
+    // quotient, less one when the remainder is not zero and the signs differ.  Floating types have
+    // no such mode: the reference divides them the same way whatever the flag says.
+    template <typename T>
+    __device__ __forceinline__ T floor_divide(T a, T b)
+    {
+        if constexpr (std::is_integral<T>::value)
+        {
+            const int32_t x = a, y = b; // 8-bit operands promote; int32 has a specialisation
+            const int32_t quot = x / y, rem = x % y;
+            return static_cast<T>((rem != 0 && ((x < 0) != (y < 0))) ? quot - 1 : quot);
+        }
+        else
+            return static_cast<T>(a / b);
+    }
+
     template <typename T>
     __device__ __forceinline__ T binary_apply(int op, T a, T b)
     {
@@ -12,6 +28,7 @@ namespace hipq
         case HIPQ_OP_SUBTRACT: return static_cast<T>(a - b);
         case HIPQ_OP_MULTIPLY: return static_cast<T>(a * b);
         case HIPQ_OP_DIVIDE: return static_cast<T>(a / b);
+        case HIPQ_OP_DIVIDE_FLOOR: return floor_divide(a, b);
         case HIPQ_OP_MAXIMUM: return a > b ? a : b;
         default: return a < b ? a : b;
         }
@@ -24,12 +41,15 @@ namespace hipq
         case HIPQ_OP_ADD: return __fadd_rn(a, b);
         case HIPQ_OP_SUBTRACT: return __fsub_rn(a, b);
         case HIPQ_OP_MULTIPLY: return __fmul_rn(a, b);
-        case HIPQ_OP_DIVIDE: return __fdiv_rn(a, b);
+        case HIPQ_OP_DIVIDE:
+        case HIPQ_OP_DIVIDE_FLOOR: return __fdiv_rn(a, b);
         case HIPQ_OP_MAXIMUM: return a > b ? a : b;
         default: return a < b ? a : b;
         }
     }
-    // integer division by zero has no defined result in the reference either; keep the GPU quiet
+    // Integer division by zero: the reference throws std::domain_error from the host loop; a kernel
+    // cannot, so a zero divisor gives 0 (documented deviation).  INT32_MIN / -1 overflows in C++; the
+    // x86 build of the reference traps on it, here it gives INT32_MIN.
     template <>
     __device__ __forceinline__ int32_t binary_apply<int32_t>(int op, int32_t a, int32_t b)
     {
@@ -39,6 +59,15 @@ namespace hipq
         case HIPQ_OP_SUBTRACT: return static_cast<int32_t>(static_cast<uint32_t>(a) - static_cast<uint32_t>(b));
         case HIPQ_OP_MULTIPLY: return static_cast<int32_t>(static_cast<uint32_t>(a) * static_cast<uint32_t>(b));
         case HIPQ_OP_DIVIDE: return b == 0 ? 0 : (a == INT32_MIN && b == -1 ? INT32_MIN : a / b);
+        case HIPQ_OP_DIVIDE_FLOOR:
+        {
+            if (b == 0)
+                return 0;
+            if (a == INT32_MIN && b == -1)
+                return INT32_MIN;
+            const int32_t quot = a / b, rem = a % b;
+            return (rem != 0 && ((a < 0) != (b < 0))) ? quot - 1 : quot;
+        }
         case HIPQ_OP_MAXIMUM: return a > b ? a : b;
         default: return a < b ? a : b;
         }
@@ -52,7 +81,7 @@ namespace hipq
         for (; i < n; i += step)
         {
             T x = a[an == 1 ? 0 : i], y = b[bn == 1 ? 0 : i];
-            if (sizeof(T) == 1 && op == HIPQ_OP_DIVIDE && y == 0)
+            if (sizeof(T) == 1 && (op == HIPQ_OP_DIVIDE || op == HIPQ_OP_DIVIDE_FLOOR) && y == 0)
                 out[i] = 0;
             else
                 out[i] = binary_apply<T>(op, x, y);
@@ -199,7 +228,7 @@ namespace hipq
 #pragma unroll
             for (int j = 0; j < V; ++j)
             {
-                if (sizeof(T) == 1 && OP == HIPQ_OP_DIVIDE && y.e[j] == 0)
+                if (sizeof(T) == 1 && (OP == HIPQ_OP_DIVIDE || OP == HIPQ_OP_DIVIDE_FLOOR) && y.e[j] == 0)
                     r.e[j] = 0;
                 else
                     r.e[j] = binary_apply<T>(OP, x.e[j], y.e[j]);
@@ -249,7 +278,7 @@ extern "C" {
 
 int hipq_binary(int32_t op, int32_t dtype, const void* a, int64_t an, const void* b, int64_t bn, void* out, int64_t n, void* stream)
 {
-    HIPQ_REQUIRE(op >= HIPQ_OP_ADD && op <= HIPQ_OP_MINIMUM, "binary op %d unknown", op);
+    HIPQ_REQUIRE(op >= HIPQ_OP_ADD && op <= HIPQ_OP_DIVIDE_FLOOR, "binary op %d unknown", op);
     HIPQ_REQUIRE(n >= 0 && (an == n || an == 1) && (bn == n || bn == 1), "operand counts must be the output count or 1");
     if (n == 0)
         return HIPQ_OK;
@@ -270,7 +299,7 @@ int hipq_binary(int32_t op, int32_t dtype, const void* a, int64_t an, const void
     switch (op)                                                                                    \
     {                                                                                              \
         VEC_B(T, HIPQ_OP_ADD) VEC_B(T, HIPQ_OP_SUBTRACT) VEC_B(T, HIPQ_OP_MULTIPLY) VEC_B(T, HIPQ_OP_DIVIDE) VEC_B(T, HIPQ_OP_MAXIMUM)          \
-            VEC_B(T, HIPQ_OP_MINIMUM)                                                              \
+            VEC_B(T, HIPQ_OP_MINIMUM) VEC_B(T, HIPQ_OP_DIVIDE_FLOOR)                               \
     }
         switch (dtype)
         {

@@ -1500,8 +1500,9 @@ namespace hipq
         // returns true: it runs the epilogue.  Every wavefront of the workgroup takes the same path.
         // The sums travel between compute dies, each with an L2 of its own: they are stored and
         // loaded at device scope (sc1: written through to, and fetched from, the memory side), so no
-        // whole-cache write-back or invalidate is needed; the barrier in front of the counter
-        // update waits for the stores.
+        // whole-cache write-back or invalidate is needed.  A workgroup barrier does not wait for
+        // stores in flight, so every wavefront drains its own (vmcnt 0: acknowledged by the memory
+        // side) before the barrier in front of the counter update.
         uint32_t* const arrival = reinterpret_cast<uint32_t*>(params + 3 * BN);
         constexpr int kDeviceScope = 16; // the sc1 bit of a buffer instruction
         auto gather_splits = [&]() {
@@ -1521,7 +1522,8 @@ namespace hipq
                                                                ks * (BM * BN * 4) + lane_off + ((mi * WN + ni) * 4 + g) * 1024,
                                                                0,
                                                                kDeviceScope);
-            __syncthreads(); // every wavefront's stores have been acknowledged
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wavefront's partial sums have reached memory
+            __syncthreads();                                 // ... and so have the other wavefronts'
             if (tid == 0)
             {
                 const uint32_t seen = atomicAdd(counters + tile, 1u);
@@ -1844,7 +1846,7 @@ namespace hipq
         if (splits > 1 && tiles * sizeof(uint32_t) <= kSplitCounterBytes)
         {
             void* p = nullptr;
-            int rc = split_workspace(static_cast<size_t>(tiles) * splits * BM * BN * sizeof(int32_t), &counters, &p);
+            int rc = split_workspace(static_cast<size_t>(tiles) * splits * BM * BN * sizeof(int32_t), s, &counters, &p);
             if (rc != HIPQ_OK)
                 return rc;
             partials = static_cast<int32_t*>(p);

@@ -40,7 +40,7 @@ namespace hipq
             // a first layer's three or four channels: a copy with the padding materialised, whose
             // filter rows are single 32-byte runs, then the tile kernel that loads straight into LDS
             void* ws = nullptr;
-            int rc = workspace(align_up(static_cast<size_t>(g.N * rp.Hp * rp.Wp * 4), 256), &ws);
+            int rc = workspace(align_up(static_cast<size_t>(g.N * rp.Hp * rp.Wp * 4), 256), s, &ws);
             if (rc)
                 return rc;
             rc = launch_stage_rows(g, rp, data, ws, zp.data_zp, zp.data_t, s);
@@ -54,7 +54,7 @@ namespace hipq
             // a first layer's few channels: a 16-channel channels-last copy, then the MFMA kernel
             void* ws = nullptr;
             const int64_t in_sp = g.in[1] * g.in[2];
-            int rc = workspace(align_up(static_cast<size_t>(g.N * in_sp * 16), 256), &ws);
+            int rc = workspace(align_up(static_cast<size_t>(g.N * in_sp * 16), 256), s, &ws);
             if (rc)
                 return rc;
             rc = launch_pad_channels(data, ws, g.N, in_sp, g.C, g.data_layout == HIPQ_LAYOUT_NCX, zp.data_zp, zp.data_t, s);
@@ -85,7 +85,7 @@ namespace hipq
         if (tr_bytes + col_bytes)
         {
             void* p = nullptr;
-            int rc = workspace(tr_bytes + col_bytes, &p);
+            int rc = workspace(tr_bytes + col_bytes, s, &p);
             if (rc)
                 return rc;
             ws = static_cast<uint8_t*>(p);
@@ -173,7 +173,7 @@ namespace hipq
         if (!blob)
         {
             uint8_t* ws = nullptr;
-            int rc = workspace(wbytes + static_cast<size_t>(d.N) * sizeof(int32_t), reinterpret_cast<void**>(&ws));
+            int rc = workspace(wbytes + static_cast<size_t>(d.N) * sizeof(int32_t), s, reinterpret_cast<void**>(&ws));
             if (rc)
                 return rc;
             rc = hipq_dot_pack(&d, b, ws, s);

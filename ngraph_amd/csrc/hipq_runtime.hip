@@ -1,7 +1,9 @@
 // Device plumbing of libhipq.so: errors, memory, streams, events, workspace, byte fill.
 #include "hipq_common.h"
 
+#include <map>
 #include <mutex>
+#include <utility>
 
 namespace hipq
 {
@@ -30,67 +32,103 @@ namespace hipq
 
     static const int kMaxDevices = 16;
     static std::mutex g_ws_mutex;
-    static void* g_ws_ptr[kMaxDevices] = {};
-    static size_t g_ws_bytes[kMaxDevices] = {};
     static uint64_t g_ws_epoch[kMaxDevices] = {};
 
-    int workspace(size_t bytes, void** ptr)
+    struct Block
     {
-        int dev = 0;
-        HIPQ_HIP(hipGetDevice(&dev));
-        if (dev < 0 || dev >= kMaxDevices)
-            return fail(HIPQ_ERR_LIMIT, "device ordinal %d beyond %d", dev, kMaxDevices);
-        std::lock_guard<std::mutex> lock(g_ws_mutex);
-        if (g_ws_bytes[dev] < bytes)
-        {
-            if (g_ws_ptr[dev])
-            {
-                // earlier launches may still read the old block
-                HIPQ_HIP(hipDeviceSynchronize());
-                HIPQ_HIP(hipFree(g_ws_ptr[dev]));
-                g_ws_ptr[dev] = nullptr;
-                g_ws_bytes[dev] = 0;
-            }
-            size_t want = align_up(bytes + bytes / 4, 1 << 20);
-            HIPQ_HIP(hipMalloc(&g_ws_ptr[dev], want));
-            g_ws_bytes[dev] = want;
-            ++g_ws_epoch[dev];
-        }
-        *ptr = g_ws_ptr[dev];
+        void* ptr = nullptr;
+        size_t bytes = 0;
+    };
+    struct StreamBlocks
+    {
+        Block ws;    // layout copies
+        Block split; // tile counters + partial sums
+    };
+    static std::map<std::pair<int, hipStream_t>, StreamBlocks> g_blocks;
+
+    static int current_device(int* dev)
+    {
+        HIPQ_HIP(hipGetDevice(dev));
+        if (*dev < 0 || *dev >= kMaxDevices)
+            return fail(HIPQ_ERR_LIMIT, "device ordinal %d beyond %d", *dev, kMaxDevices);
         return HIPQ_OK;
     }
 
-    // Second grow-only block: partial sums of reductions split over workgroups, with a counter per
-    // output tile at its head.  The counters are zeroed when the block is (re)allocated and every
-    // kernel that uses them leaves them at zero.
-    static void* g_split_ptr[kMaxDevices] = {};
-    static size_t g_split_bytes[kMaxDevices] = {};
-    int split_workspace(size_t partial_bytes, uint32_t** counters, void** partials)
+    static int grow(Block& b, size_t need, hipStream_t stream, int dev, size_t zero_head)
+    {
+        if (b.bytes >= need)
+            return HIPQ_OK;
+        if (b.ptr)
+        {
+            // earlier launches on this stream may still use the old block
+            HIPQ_HIP(hipStreamSynchronize(stream));
+            HIPQ_HIP(hipFree(b.ptr));
+            b.ptr = nullptr;
+            b.bytes = 0;
+        }
+        const size_t want = align_up(need + need / 4, 1 << 20);
+        HIPQ_HIP(hipMalloc(&b.ptr, want));
+        if (zero_head)
+        {
+            HIPQ_HIP(hipMemset(b.ptr, 0, zero_head));
+            HIPQ_HIP(hipDeviceSynchronize());
+        }
+        b.bytes = want;
+        ++g_ws_epoch[dev];
+        return HIPQ_OK;
+    }
+
+    int workspace(size_t bytes, hipStream_t stream, void** ptr)
     {
         int dev = 0;
-        HIPQ_HIP(hipGetDevice(&dev));
-        if (dev < 0 || dev >= kMaxDevices)
-            return fail(HIPQ_ERR_LIMIT, "device ordinal %d beyond %d", dev, kMaxDevices);
+        int rc = current_device(&dev);
+        if (rc)
+            return rc;
         std::lock_guard<std::mutex> lock(g_ws_mutex);
+        Block& b = g_blocks[std::make_pair(dev, stream)].ws;
+        rc = grow(b, bytes, stream, dev, 0);
+        if (rc)
+            return rc;
+        *ptr = b.ptr;
+        return HIPQ_OK;
+    }
+
+    // The counters are zeroed when the block is (re)allocated and every kernel that uses them
+    // leaves them at zero.
+    int split_workspace(size_t partial_bytes, hipStream_t stream, uint32_t** counters, void** partials)
+    {
+        int dev = 0;
+        int rc = current_device(&dev);
+        if (rc)
+            return rc;
         const size_t need = kSplitCounterBytes + partial_bytes;
-        if (g_split_bytes[dev] < need)
-        {
-            if (g_split_ptr[dev])
-            {
-                HIPQ_HIP(hipDeviceSynchronize());
-                HIPQ_HIP(hipFree(g_split_ptr[dev]));
-                g_split_ptr[dev] = nullptr;
-                g_split_bytes[dev] = 0;
-            }
-            size_t want = align_up(need + need / 4, 1 << 20);
-            HIPQ_HIP(hipMalloc(&g_split_ptr[dev], want));
-            HIPQ_HIP(hipMemset(g_split_ptr[dev], 0, kSplitCounterBytes));
-            HIPQ_HIP(hipDeviceSynchronize());
-            g_split_bytes[dev] = want;
-            ++g_ws_epoch[dev];
-        }
-        *counters = static_cast<uint32_t*>(g_split_ptr[dev]);
-        *partials = static_cast<uint8_t*>(g_split_ptr[dev]) + kSplitCounterBytes;
+        std::lock_guard<std::mutex> lock(g_ws_mutex);
+        Block& b = g_blocks[std::make_pair(dev, stream)].split;
+        rc = grow(b, need, stream, dev, kSplitCounterBytes);
+        if (rc)
+            return rc;
+        *counters = static_cast<uint32_t*>(b.ptr);
+        *partials = static_cast<uint8_t*>(b.ptr) + kSplitCounterBytes;
+        return HIPQ_OK;
+    }
+
+    int release_stream_workspace(hipStream_t stream)
+    {
+        int dev = 0;
+        int rc = current_device(&dev);
+        if (rc)
+            return rc;
+        std::lock_guard<std::mutex> lock(g_ws_mutex);
+        auto it = g_blocks.find(std::make_pair(dev, stream));
+        if (it == g_blocks.end())
+            return HIPQ_OK;
+        const StreamBlocks blocks = it->second;
+        g_blocks.erase(it);
+        ++g_ws_epoch[dev];
+        if (blocks.ws.ptr)
+            HIPQ_HIP(hipFree(blocks.ws.ptr));
+        if (blocks.split.ptr)
+            HIPQ_HIP(hipFree(blocks.split.ptr));
         return HIPQ_OK;
     }
 
@@ -238,7 +276,13 @@ int hipq_stream_create(void** stream)
 int hipq_stream_destroy(void* stream)
 {
     if (stream)
+    {
+        HIPQ_HIP(hipStreamSynchronize(as_stream(stream)));
+        int rc = release_stream_workspace(as_stream(stream));
+        if (rc)
+            return rc;
         HIPQ_HIP(hipStreamDestroy(as_stream(stream)));
+    }
     return HIPQ_OK;
 }
 

@@ -542,7 +542,56 @@ def concat(arrays, axis):
     return out.to_numpy(arrays[0].dtype, shape)
 
 
-BINARY_OPS = {"add": 0, "subtract": 1, "multiply": 2, "divide": 3, "maximum": 4, "minimum": 5}
+class GraphReplay:
+    """One fixed launch sequence on a stream, captured into a HIP graph and replayed.
+
+    `launch` issues the sequence on `stream`.  The graph points into the library's scratch blocks:
+    it is captured again whenever hipq_workspace_epoch says a block of the device was reallocated
+    since the capture, and destroyed by close() (or when the object goes away)."""
+
+    def __init__(self, lib, stream, launch):
+        self.lib, self.stream, self._launch = lib, stream, launch
+        self.graph = None
+        self.epoch = None
+
+    def capture(self):
+        self.close()
+        self._launch()  # sizes the library's scratch blocks before anything is recorded
+        check(self.lib.hipq_stream_sync(self.stream))
+        check(self.lib.hipq_capture_begin(self.stream))
+        g = C.c_void_p()
+        try:
+            self._launch()
+        except Exception:
+            self.lib.hipq_capture_end(self.stream, C.byref(g))  # leave the stream usable
+            if g.value:
+                self.lib.hipq_graph_destroy(g)
+            raise
+        check(self.lib.hipq_capture_end(self.stream, C.byref(g)))
+        self.graph = g
+        self.epoch = self.lib.hipq_workspace_epoch()
+
+    def replay(self):
+        if self.graph is None or self.lib.hipq_workspace_epoch() != self.epoch:
+            self.capture()
+        rc = self.lib.hipq_graph_launch(self.graph, self.stream)
+        if rc:
+            check(rc)
+
+    def close(self):
+        if self.graph is not None:
+            g, self.graph = self.graph, None
+            check(self.lib.hipq_stream_sync(self.stream))
+            check(self.lib.hipq_graph_destroy(g))
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+BINARY_OPS = {"add": 0, "subtract": 1, "multiply": 2, "divide": 3, "maximum": 4, "minimum": 5, "divide_floor": 6}
 UNARY_OPS = {"abs": 0, "relu": 1, "copy": 2}
 
 

@@ -486,7 +486,12 @@ namespace
         if (ti == op::v1::Multiply::type_info)
             return HIPQ_OP_MULTIPLY;
         if (ti == op::v1::Divide::type_info)
-            return HIPQ_OP_DIVIDE;
+        {
+            // integer division floors unless the op says otherwise (src/ngraph/op/divide.hpp:72,
+            // src/ngraph/runtime/reference/divide.hpp:41-60); floats divide the same way under both
+            const auto* div = static_cast<const op::v1::Divide*>(&n);
+            return (div->is_pythondiv() && !n.get_output_element_type(0).is_real()) ? HIPQ_OP_DIVIDE_FLOOR : HIPQ_OP_DIVIDE;
+        }
         if (ti == op::v1::Maximum::type_info)
             return HIPQ_OP_MAXIMUM;
         if (ti == op::v1::Minimum::type_info)

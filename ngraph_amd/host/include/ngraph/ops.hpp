@@ -583,7 +583,27 @@ namespace ngraph
             NGRAPH_BINARY_OP(Add)
             NGRAPH_BINARY_OP(Subtract)
             NGRAPH_BINARY_OP(Multiply)
-            NGRAPH_BINARY_OP(Divide)
+            // Divide carries the reference's flag (src/ngraph/op/divide.hpp:35-76): integer division
+            // floors by default ("python division"), truncates with the flag off
+            class NGRAPH_API Divide : public BinaryElementwise
+            {
+            public:
+                NGRAPH_OP_DECL("Divide", 1)
+                Divide(const Output<Node>& a, const Output<Node>& b, bool pythondiv = true) : BinaryElementwise(a, b), m_pythondiv(pythondiv)
+                {
+                    constructor_validate_and_infer_types();
+                }
+                bool is_pythondiv() const { return m_pythondiv; }
+                void set_is_pythondiv(bool pythondiv) { m_pythondiv = pythondiv; }
+                std::shared_ptr<Node> clone_with_new_inputs(const OutputVector& new_args) const override
+                {
+                    check_new_args_count(this, new_args);
+                    return std::make_shared<Divide>(new_args.at(0), new_args.at(1), m_pythondiv);
+                }
+
+            protected:
+                bool m_pythondiv{true};
+            };
             NGRAPH_BINARY_OP(Maximum)
             NGRAPH_BINARY_OP(Minimum)
 #undef NGRAPH_BINARY_OP

@@ -134,6 +134,7 @@ class DevicePlan:
 
     def __init__(self, lib, stream, N, hw=224):
         self.lib, self.stream, self.N = lib, stream, N
+        self._replay = None
         self.calls, self.keep, self.graph = [], [], None
         dev = lambda a: self._keep(H.DeviceBuffer.from_numpy(np.ascontiguousarray(a)))
         buf = {"input": self._keep(H.DeviceBuffer(N * hw * hw * 3))}
@@ -197,18 +198,22 @@ class DevicePlan:
                 H.check(rc)
 
     def capture(self):
-        self.launch()  # sizes the library's workspace before anything is recorded
-        H.check(self.lib.hipq_stream_sync(self.stream))
-        H.check(self.lib.hipq_capture_begin(self.stream))
-        self.launch()
-        g = C.c_void_p()
-        H.check(self.lib.hipq_capture_end(self.stream, C.byref(g)))
-        self.graph = g
+        """records the pass into a HIP graph (after one eager pass that sizes the library's scratch)"""
+        if self._replay is None:
+            self._replay = H.GraphReplay(self.lib, self.stream, self.launch)
+        self._replay.capture()
 
     def replay(self):
-        rc = self.lib.hipq_graph_launch(self.graph, self.stream)
-        if rc:
-            H.check(rc)
+        """launches the recorded graph; records it again first if the library's scratch has moved"""
+        if self._replay is None:
+            self.capture()
+        self._replay.replay()
+
+    def close(self):
+        """destroys the recorded graph (the buffers go with the object)"""
+        if self._replay is not None:
+            self._replay.close()
+            self._replay = None
 
     def read_logits(self):
         H.check(self.lib.hipq_stream_sync(self.stream))

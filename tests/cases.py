@@ -102,3 +102,24 @@ def brute_conv_acc(d, data, filt, dzp=0, fzp=0):
         wt = w[(slice(None), slice(None)) + taps]  # K, C
         out += np.einsum("nc...,kc->nk...", patch, wt)
     return out
+
+
+def dot_bias_closed_form(a, w, bias, scales, out_t, relu):
+    """QuantizedDotBias from first principles, independent of the oracle's loops: the integer sums
+    through float64 BLAS (exact: 255 * 127 * K stays far below 2^53), then the three float32 steps
+    the reference's CPU backend hands oneDNN (src/ngraph/runtime/cpu/builder/quantized_dot.cpp:36-125,
+    dnnl_emitter.hpp:737-761) -- f32(acc) + f32(bias), times scale[n] (or the one scale), relu -- and
+    round-half-to-even with saturation for 8-bit outputs.  a [M,K] u8/i8, w [N,K] i8."""
+    acc = (a.astype(np.float64) @ w.astype(np.float64).T).astype(np.int64)
+    assert np.all(np.abs(acc) < 2**31)
+    v = acc.astype(np.float32)
+    if bias is not None:
+        v = v + np.asarray(bias, np.int32).astype(np.float32)[None, :]
+    sc = np.asarray(scales, np.float32).reshape(-1)
+    v = (v * (sc[None, :] if sc.size > 1 else sc[0])).astype(np.float32)
+    if relu:
+        v = np.maximum(v, np.float32(0))
+    if out_t == "f32":
+        return v
+    lo, hi = (0, 255) if out_t == "u8" else (-128, 127)
+    return np.clip(np.rint(v), lo, hi).astype(np.uint8 if out_t == "u8" else np.int8)

@@ -1,9 +1,9 @@
-// hip_backend_tests [--cpu | --gpu | --all] [substring]
+// hip_backend_tests [--cpu | --gpu | --all] [--list] [--exact] [substring or, with --exact, suite.name]
 #include "mini_test.hpp"
 
 int main(int argc, char** argv)
 {
-    bool want_cpu = true, want_gpu = false;
+    bool want_cpu = true, want_gpu = false, list = false, exact = false;
     std::string filter;
     for (int i = 1; i < argc; ++i)
     {
@@ -14,8 +14,18 @@ int main(int argc, char** argv)
             want_cpu = false, want_gpu = true;
         else if (a == "--all")
             want_cpu = want_gpu = true;
+        else if (a == "--list")
+            list = true;
+        else if (a == "--exact")
+            exact = true;
         else
             filter = a;
+    }
+    if (list)
+    {
+        for (const auto& c : mini_test::registry())
+            std::cout << (c.needs_gpu ? "gpu " : "cpu ") << c.suite << "." << c.name << std::endl;
+        return 0;
     }
     int ran = 0;
     for (const auto& c : mini_test::registry())
@@ -23,7 +33,7 @@ int main(int argc, char** argv)
         if ((c.needs_gpu && !want_gpu) || (!c.needs_gpu && !want_cpu))
             continue;
         std::string full = c.suite + "." + c.name;
-        if (!filter.empty() && full.find(filter) == std::string::npos)
+        if (!filter.empty() && (exact ? full != filter : full.find(filter) == std::string::npos))
             continue;
         std::cout << "[ RUN      ] " << full << std::endl;
         int before = mini_test::failures();

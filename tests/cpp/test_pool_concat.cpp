@@ -158,3 +158,40 @@ CPU_TEST(type_prop, concat_and_pool_shapes)
     auto mp = make_shared<op::v0::MaxPool>(X, Shape{3, 3}, Strides{2, 2}, Shape{1, 1}, Shape{1, 1});
     EXPECT_EQ(mp->get_output_shape(0), (Shape{8, 64, 56, 56}));
 }
+
+// op::v1::Divide on integers: floor division unless the op says otherwise (values of the
+// reference's test/backend/divide.in.cpp:69-133)
+namespace
+{
+    vector<int32_t> run_divide(const vector<int32_t>& x, const vector<int32_t>& y, bool set_flag, bool pythondiv)
+    {
+        Shape shape{2, 2};
+        auto A = make_shared<op::v0::Parameter>(element::i32, shape);
+        auto B = make_shared<op::v0::Parameter>(element::i32, shape);
+        auto div = set_flag ? make_shared<op::v1::Divide>(A, B, pythondiv) : make_shared<op::v1::Divide>(A, B);
+        auto f = make_shared<Function>(OutputVector{div}, ParameterVector{A, B});
+        auto backend = runtime::Backend::create("HIP");
+        auto a = backend->create_tensor(element::i32, shape);
+        copy_data(a, x);
+        auto b = backend->create_tensor(element::i32, shape);
+        copy_data(b, y);
+        auto result = backend->create_tensor(element::i32, shape);
+        backend->compile(f)->call_with_validate({result}, {a, b});
+        return read_vector<int32_t>(result);
+    }
+}
+
+GPU_TEST(HIP, divide_int32)
+{
+    EXPECT_VEC_EQ((vector<int32_t>{536871072, 214748365, 2, 2}), run_divide({0x40000140, 0x40000001, 8, 16}, {2, 5, 4, 8}, false, true));
+}
+
+GPU_TEST(HIP, divide_cpp_rounding_int32)
+{
+    EXPECT_VEC_EQ((vector<int32_t>{3, -3, -3, 3}), run_divide({-10, -10, 10, 10}, {-3, 3, -3, 3}, true, false));
+}
+
+GPU_TEST(HIP, divide_python_rounding_int32)
+{
+    EXPECT_VEC_EQ((vector<int32_t>{3, -4, -4, 3}), run_divide({-10, -10, 10, 10}, {-3, 3, -3, 3}, false, true));
+}

@@ -141,7 +141,7 @@ def test_device_plan_against_oracle_pipeline(gpu_lib):
         H.check(lib.hipq_stream_sync(None))
         plan.replay()
         assert np.array_equal(plan.read_output(), eager)
-    H.check(lib.hipq_graph_destroy(plan.graph))
+    plan.close()
     diff = np.abs(eager - exp)
     print("bert plan vs oracle: max", float(diff.max()), "mean", float(diff.mean()), "beyond 1e-3:", float(np.mean(diff > 1e-3)), flush=True)
     assert np.all(np.isfinite(eager))
@@ -149,3 +149,48 @@ def test_device_plan_against_oracle_pipeline(gpu_lib):
     # the HIP provider's op-at-a-time pass takes the same kernels: identical to the plan
     hp, _ = B.run(B.HipProvider, x, SMALL)
     assert np.array_equal(hp, eager)
+
+
+@pytest.mark.gpu
+def test_benchmarked_batch_base_dims(gpu_lib):
+    """What the benchmark times: BASE dimensions, 12 layers, batch 32.  Kernel choice depends on the
+    row count (tile shapes, split reductions, deep slices), so the batch-32 launches are not the
+    batch-2 ones.  Every op is a function of one sequence alone, and every kernel's arithmetic per
+    output is the same whatever the batch (exact integer sums; f32 rows reduced by one wavefront in a
+    fixed order; products accumulated in double, k ascending): a batch of 16 copies of two sequences
+    must reproduce the batch-2 pass bit for bit, eager and as a HIP graph.  The batch-2 pass itself is
+    held against the oracle's 12-layer pass in distribution (the bar of the small-model test above)."""
+    lib = gpu_lib
+    two = B.embeddings(B.BASE, 2)
+    print("[case] bert base oracle pass, 2 sequences x 12 layers", flush=True)
+    O.port().orc_set_threads(8)
+    exp, _ = B.run(OracleProvider, two, B.BASE)
+    O.port().orc_set_threads(1)
+    sp = H.C.c_void_p()
+    H.check(lib.hipq_stream_create(H.C.byref(sp)))
+    print("[case] bert base plan, batch 2", flush=True)
+    small = B.DevicePlan(lib, sp.value, 2, B.BASE)
+    assert len(small.calls) == 19 * 12
+    small.set_input(two)
+    small.launch()
+    ref = small.read_output()
+    assert np.all(np.isfinite(ref))
+    diff = np.abs(ref - exp)
+    print("bert base batch 2 vs oracle: max", float(diff.max()), "mean", float(diff.mean()), "beyond 0.05:", float(np.mean(diff > 0.05)), flush=True)
+    assert diff.mean() < 2e-3 and np.mean(diff > 0.05) < 0.01
+    print("[case] bert base plan, batch 32", flush=True)
+    x = np.ascontiguousarray(np.tile(two, (16, 1)))
+    plan = B.DevicePlan(lib, sp.value, 32, B.BASE)
+    plan.set_input(x)
+    plan.launch()
+    eager = plan.read_output()
+    assert np.array_equal(eager, np.tile(ref, (16, 1)))
+    plan.capture()
+    for _ in range(2):
+        plan.set_input(x)
+        H.check(lib.hipq_stream_sync(None))
+        plan.replay()
+        assert np.array_equal(plan.read_output(), eager)
+    plan.close()
+    small.close()
+    H.check(lib.hipq_stream_destroy(sp.value))

@@ -43,16 +43,35 @@ def test_binary_ops(gpu_lib, dtype):
 
 @pytest.mark.gpu
 def test_divide(gpu_lib):
+    """op::v1::Divide: floor division for integers by default (is_pythondiv, src/ngraph/op/divide.hpp:72,
+    reference/divide.hpp:41-60 -- numpy's `//`), C++ truncation with the flag off; floats divide the same
+    way under both.  Mixed signs with a remainder are where the two differ by one."""
     for n in SIZES:
         a, b = synth.normal_f32(21, (n,)), synth.normal_f32(22, (n,))
         assert np.array_equal(H.binary("divide", a, b), a / b)
+        assert np.array_equal(H.binary("divide_floor", a, b), a / b)
         ia = synth.uniform_int(23, (n,), -100000, 100000, np.int32)
-        ib = synth.uniform_int(24, (n,), 1, 300, np.int32)
-        # C++ integer division truncates toward zero
-        assert np.array_equal(H.binary("divide", ia, ib), (np.abs(ia) // ib * np.sign(ia)).astype(np.int32))
+        ib = synth.uniform_int(24, (n,), -300, 300, np.int32)
+        ib[ib == 0] = 7
+        trunc = (np.abs(ia) // np.abs(ib) * np.sign(ia) * np.sign(ib)).astype(np.int32)
+        assert np.array_equal(H.binary("divide", ia, ib), trunc)
+        assert np.array_equal(H.binary("divide_floor", ia, ib), ia // ib)
+        if n > 1000:
+            assert np.any(trunc != ia // ib)
+        sa = synth.uniform_int(27, (n,), -128, 127, np.int8)
+        sb = synth.uniform_int(28, (n,), -128, 127, np.int8)
+        sb[sb == 0] = -3
+        wide = sa.astype(np.int32) // sb.astype(np.int32)
+        assert np.array_equal(H.binary("divide_floor", sa, sb), wide.astype(np.int8))  # -128 // -1 wraps like the reference's T quot
         ua = synth.uniform_int(25, (n,), 0, 255, np.uint8)
         ub = synth.uniform_int(26, (n,), 1, 255, np.uint8)
         assert np.array_equal(H.binary("divide", ua, ub), ua // ub)
+        assert np.array_equal(H.binary("divide_floor", ua, ub), ua // ub)
+    # hand-checked corners of the reference's rule: quot - 1 when rem != 0 and the signs differ
+    a = np.array([7, -7, 7, -7, 6, -6, 0, -1], np.int32)
+    b = np.array([2, 2, -2, -2, 3, 3, 5, 5], np.int32)
+    assert H.binary("divide_floor", a, b).tolist() == [3, -4, -4, 3, 2, -2, 0, -1]
+    assert H.binary("divide", a, b).tolist() == [3, -3, -3, 3, 2, -2, 0, 0]
 
 
 @pytest.mark.gpu

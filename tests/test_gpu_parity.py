@@ -821,6 +821,34 @@ def test_dot_config2_full_size_properties(gpu_lib):
         assert np.array_equal(gm, got[:M])
 
 
+@pytest.mark.parametrize("M", [1, 32, 256])
+def test_dot_bias_config2_benchmarked_form(gpu_lib, M):
+    """BASELINE config 2 exactly as bench.py times it: QuantizedDotBias u8 [M,4096] x i8 [4096,4096]
+    ([N,K] weights, prepacked), int32 bias, per-output-channel scales, requantized to i8 -- on the
+    kernel the bench reports for that M -- against the closed form of tests/cases.py (float64 BLAS
+    sums, numpy float32 post-ops, rint + clip), which test_oracle_conv_dot.py also holds the oracle
+    to.  The u8 + relu and f32 forms ride along."""
+    say("config2 benchmarked form, M", M)
+    K = N = 4096
+    a = synth.uniform_int(2001, (M, K), 0, 255, np.uint8)
+    w = synth.uniform_int(2002, (N, K), -127, 127, np.int8)
+    bias = synth.uniform_int(2003, (N,), -(2**15), 2**15, np.int32)
+    scales = synth.uniform_f32(2004, (N,), 0.001, 0.01)
+    # BASELINE's weight scales; the data and output scales fold into the same per-channel factor
+    scales = (scales * np.float32(0.02)).astype(np.float32)
+    for out_t, relu in (("i8", False), ("u8", True), ("f32", False)):
+        d = H.make_dot_desc(M, K, N, out_t=out_t, b_layout=H.B_NK)
+        f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
+        got = H.quantized_dot_bias(d, f, a, w, bias, scales)
+        kernel = H.last_kernel()
+        exp = cases.dot_bias_closed_form(a, w, bias, scales, out_t, relu)
+        assert np.array_equal(got, exp), (out_t, relu, kernel, int(np.sum(got != exp)))
+        if out_t == "i8":
+            # the kernels bench.py's gemm_config2 entries name: weight-streaming up to 64 rows, MFMA tiles above
+            assert kernel == ("dot_skinny_i8_16x16x64" if M <= 64 else "dot_mfma_i8_32x32x32"), kernel
+            assert len(np.unique(exp)) > 100 and (exp == 127).any() and (exp == -128).any()
+
+
 @pytest.mark.parametrize("M", [1, 7, 16, 17, 33, 64, 100, 129, 256])
 def test_dot_skinny(gpu_lib, M):
     """the weight-streaming kernel for a handful of rows: ragged row and column tiles, a reduction

@@ -1,6 +1,7 @@
 """The C++ host side: the nGraph-compatible graph / builder / runtime subset and the "HIP" backend
 plugin.  The C++ test program (tests/cpp, built into ngraph_amd/host/hip_backend_tests) holds the
-reference's own backend tests re-typed; this file runs it."""
+reference's own backend tests re-typed; every C++ test is one pytest item here, so a failure names
+the C++ test that failed."""
 import ctypes
 import os
 import subprocess
@@ -12,19 +13,29 @@ HOST = os.path.join(ROOT, "ngraph_amd", "host")
 TESTS = os.path.join(HOST, "hip_backend_tests")
 
 
-def _run(flag):
+def _listed(kind):
+    """names of the C++ tests of one kind ("cpu" / "gpu"); needs no device"""
+    if not os.path.exists(TESTS):
+        return ["<hip_backend_tests is not built: make -C ngraph_amd/host>"]
+    out = subprocess.run([TESTS, "--list"], capture_output=True, text=True, timeout=60).stdout
+    return [l.split()[1] for l in out.splitlines() if l.startswith(kind + " ")]
+
+
+def _run(flag, name):
     assert os.path.exists(TESTS), "build the host first: make -C ngraph_amd/host"
-    p = subprocess.run([TESTS, flag], capture_output=True, text=True, timeout=600)
+    print("[case] hip_backend_tests", flag, name, flush=True)
+    p = subprocess.run([TESTS, flag, "--exact", name], capture_output=True, text=True, timeout=600)
     print(p.stdout[-6000:])
     print(p.stderr[-2000:])
-    assert p.returncode == 0, "C++ tests failed:\n" + "\n".join(l for l in p.stdout.splitlines() if "FAIL" in l)
-    return p.stdout
+    assert p.returncode == 0, "C++ test %s failed (exit %d):\n%s" % (
+        name, p.returncode, "\n".join(l for l in p.stdout.splitlines() if "FAIL" in l))
+    assert "1 tests ran, 0 failures" in p.stdout
 
 
-def test_cpp_cpu_suite():
+@pytest.mark.parametrize("name", _listed("cpu"))
+def test_cpp_cpu(name):
     """type_prop validation, builders + constant folding, plugin discovery, HostTensor"""
-    out = _run("--cpu")
-    assert "0 failures" in out
+    _run("--cpu", name)
 
 
 def test_plugin_exports_register_symbol():
@@ -34,8 +45,9 @@ def test_plugin_exports_register_symbol():
 
 
 @pytest.mark.gpu
-def test_cpp_gpu_suite():
+@pytest.mark.parametrize("name", _listed("gpu"))
+def test_cpp_gpu(name):
     """api / validate_call / unhandled_op, quantized_convolution, quantized_dot, the 28
-    quantize_dequantize vectors and the builder_quantization tests, on backend "HIP" """
-    out = _run("--gpu")
-    assert "0 failures" in out
+    quantize_dequantize vectors, the builder_quantization tests, fusion, layout, ResNet-50, on
+    backend "HIP" """
+    _run("--gpu", name)

@@ -228,6 +228,37 @@ def test_dot_bias_kat(kats):
         assert np.array_equal(got, exp), key
 
 
+@pytest.mark.parametrize("a_t,lo,hi", [("u8", 0, 255), ("i8", -128, 127)])
+def test_dot_bias_per_channel_closed_form(a_t, lo, hi):
+    """the per-output-channel branch of orc_quantized_dot_bias (BASELINE config 2's form) against a
+    formulation that shares nothing with it: float64 BLAS for the sums, numpy float32 for the three
+    post-ops, np.rint + clip.  A scale indexed by row instead of column, a bias added after the
+    scaling, a truncating round or a missing saturation each fail it (the case saturates on both
+    sides and has exact ties through the scales 0.5 / 0.25)."""
+    M, K, N = 37, 320, 48
+    a = synth.uniform_int(401, (M, K), lo, hi, np.uint8 if a_t == "u8" else np.int8)
+    w = synth.uniform_int(402, (N, K), -127, 127, np.int8)
+    bias = synth.uniform_int(403, (N,), -(2**15), 2**15, np.int32)
+    scales = (synth.uniform_f32(404, (N,), 0.001, 0.01) * np.float32(0.02)).astype(np.float32)
+    scales[3], scales[7] = np.float32(0.5), np.float32(0.25)  # exact halves: ties go to even, and these columns saturate
+    scales[11] = np.float32(2.0**-12)
+    for out_t, relu in (("i8", False), ("u8", True), ("f32", False), ("f32", True)):
+        d = H.make_dot_desc(M, K, N, a_t=a_t, out_t=out_t, b_layout=H.B_NK)
+        f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
+        got = O.quantized_dot_bias(d, f, a, w, bias, scales)
+        exp = cases.dot_bias_closed_form(a, w, bias, scales, out_t, relu)
+        assert got.dtype == exp.dtype
+        assert np.array_equal(got, exp), (out_t, relu)
+        if out_t != "f32":
+            info = np.iinfo(exp.dtype)
+            assert (exp == info.max).any() and (exp == info.min).any() and len(np.unique(exp)) > 30
+    # a bias on the far side of 2^24 (the float add rounds): same closed form
+    bias[5] = 2**26 + 12345
+    d = H.make_dot_desc(M, K, N, a_t=a_t, out_t="f32", b_layout=H.B_NK)
+    f = H.make_fused_desc(has_bias=True, with_relu=False, scale_count=N)
+    assert np.array_equal(O.quantized_dot_bias(d, f, a, w, bias, scales), cases.dot_bias_closed_form(a, w, bias, scales, "f32", False))
+
+
 def test_fused_matches_decomposed_graph():
     """the INTERPRETER-runnable decomposition: conv(i32, unit scales) -> +bias -> f32 -> *scale ->
     [+ sum_scale*sum] -> [relu] -> Quantize(RNE) (whose clamp is the saturation); exact-arithmetic

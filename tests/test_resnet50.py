@@ -113,5 +113,50 @@ def test_resnet50_device_plan_and_graph_replay(gpu_lib):
         plan.set_images_nchw(images)
         plan.replay()
         assert np.array_equal(plan.read_logits(), ref["logits"]), seed
-    H.check(lib.hipq_graph_destroy(plan.graph))
+    plan.close()
+    H.check(lib.hipq_stream_destroy(sp.value))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("N", [32, 128])
+def test_resnet50_benchmarked_batches_against_oracle(gpu_lib, N):
+    """The batches the benchmark times.  Kernel choice depends on the batch (tile shapes, split
+    reductions, grid sizes), so the launches of batch 32 and 128 are not those of batch 1: the plan is
+    fed four distinct images repeated N/4 times, and every image's logits and interior tensors must
+    equal the oracle's for that image, bit for bit -- eager and replayed as a HIP graph.  Image 0 is
+    the image of the committed golden logits."""
+    lib = gpu_lib
+    meta, golden = _golden()
+    four = R.synthetic_images(4, seed=meta["image_seed"])
+    assert np.array_equal(four[:1], R.synthetic_images(1, seed=meta["image_seed"]))
+    print("[case] resnet50 oracle on 4 images", flush=True)
+    O.port().orc_set_threads(8)
+    exp = R.run(OracleProvider, four)
+    O.port().orc_set_threads(1)
+    assert np.array_equal(exp["logits"][:1], golden)
+    images = np.ascontiguousarray(np.tile(four, (N // 4, 1, 1, 1)))
+    sp = C.c_void_p()
+    H.check(lib.hipq_stream_create(C.byref(sp)))
+    plan = R.DevicePlan(lib, sp.value, N)
+    plan.set_images_nchw(images)
+    print("[case] resnet50 plan launch, batch", N, flush=True)
+    plan.launch()
+
+    def check_all(tag):
+        logits = plan.read_logits()
+        assert np.array_equal(logits, np.tile(exp["logits"], (N // 4, 1))), tag
+        for name, ch, hw in (("s2_b0_out", 256, 56), ("s3_b0_out", 512, 28), ("s4_b5_out", 1024, 14), ("s5_b2_out", 2048, 7)):
+            got = plan.read(name, ch, hw)
+            assert got.shape == (N, ch, hw, hw)
+            assert np.array_equal(got, np.tile(exp[name], (N // 4, 1, 1, 1))), (tag, name)
+
+    check_all("eager")
+    print("[case] resnet50 plan capture + replay, batch", N, flush=True)
+    plan.capture()
+    plan.set_images_nchw(images[::-1].copy())  # other bytes in every buffer before the replay that is checked
+    plan.replay()
+    plan.set_images_nchw(images)
+    plan.replay()
+    check_all("replayed")
+    plan.close()
     H.check(lib.hipq_stream_destroy(sp.value))

@@ -45,9 +45,9 @@ namespace
             return make_shared<op::v0::QuantizedConvolutionBias>(data, w, b, Strides{1, 1}, Strides{1, 1}, CoordinateDiff{pad, pad}, CoordinateDiff{pad, pad}, Strides{1, 1},
                                                                  op::v0::Constant::create(element::f32, Shape{}, {s}), relu);
         };
-        auto c1 = conv(x, 256, 256, 3, true, 1.0f / 9000);
-        auto c2 = conv(c1, 512, 256, 3, true, 1.0f / 9000);
-        auto c3 = conv(c2, 64, 512, 1, false, 1.0f / 4000);
+        auto c1 = conv(x, 256, 256, 3, true, 1.0f / 2500);
+        auto c2 = conv(c1, 512, 256, 3, true, 1.0f / 500);
+        auto c3 = conv(c2, 64, 512, 1, false, 1.0f / 200);
         return make_shared<Function>(OutputVector{c3}, ParameterVector{x});
     }
 }

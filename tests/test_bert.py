@@ -158,14 +158,21 @@ def test_benchmarked_batch_base_dims(gpu_lib):
     batch-2 ones.  Every op is a function of one sequence alone, and every kernel's arithmetic per
     output is the same whatever the batch (exact integer sums; f32 rows reduced by one wavefront in a
     fixed order; products accumulated in double, k ascending): a batch of 16 copies of two sequences
-    must reproduce the batch-2 pass bit for bit, eager and as a HIP graph.  The batch-2 pass itself is
-    held against the oracle's 12-layer pass in distribution (the bar of the small-model test above)."""
+    must reproduce the batch-2 pass bit for bit, eager and as a HIP graph.  The batch-2 pass is tied to
+    the oracle op by op: every one of the 12 x 19 ops is run on the oracle's own inputs and held to the
+    bar of its kind.  End to end the two passes agree only in distribution, and less tightly than two
+    layers do: a last-bit difference in an f32 value flips an int8 code, and twelve layers compound
+    the flips (the outputs are layer-normalised, of order one)."""
     lib = gpu_lib
     two = B.embeddings(B.BASE, 2)
     print("[case] bert base oracle pass, 2 sequences x 12 layers", flush=True)
     O.port().orc_set_threads(8)
-    exp, _ = B.run(OracleProvider, two, B.BASE)
+    exp, trace = B.run(OracleProvider, two, B.BASE)
     O.port().orc_set_threads(1)
+    assert len(trace) == 19 * 12
+    print("[case] bert base every op of 12 layers on the oracle's inputs", flush=True)
+    for name, op, args, res in trace:
+        _check(name, op, getattr(B.HipProvider, op)(*args), res)
     sp = H.C.c_void_p()
     H.check(lib.hipq_stream_create(H.C.byref(sp)))
     print("[case] bert base plan, batch 2", flush=True)
@@ -177,7 +184,7 @@ def test_benchmarked_batch_base_dims(gpu_lib):
     assert np.all(np.isfinite(ref))
     diff = np.abs(ref - exp)
     print("bert base batch 2 vs oracle: max", float(diff.max()), "mean", float(diff.mean()), "beyond 0.05:", float(np.mean(diff > 0.05)), flush=True)
-    assert diff.mean() < 2e-3 and np.mean(diff > 0.05) < 0.01
+    assert diff.mean() < 0.05 and np.mean(diff > 0.5) < 0.001
     print("[case] bert base plan, batch 32", flush=True)
     x = np.ascontiguousarray(np.tile(two, (16, 1)))
     plan = B.DevicePlan(lib, sp.value, 32, B.BASE)

@@ -227,6 +227,38 @@ HIPQ_API int hipq_quantized_convolution(const hipq_conv_desc_t* desc,
                                         void* out,
                                         void* stream);
 
+/*
+ * hipq_quantized_convolution for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the nGraph
+ * reference.  Arguments, kernels and results are those of hipq_quantized_convolution; the difference
+ * is where scratch comes from.  That entry point keeps grow-only blocks per stream (hipMalloc on
+ * first use and on growth); this one calls no hipMalloc / hipFree at all and takes its scratch from
+ * a fixed array that every GPU the library runs on holds from load time until the process ends:
+ *   HIPQ_NOALLOC_LAYOUT_BYTES  for the channels-last / padded / unrolled copy of an NCX input
+ *                              (an NCX u8 input of up to that many bytes; channels-last inputs
+ *                              with 64-multiple channel counts need none)
+ *   HIPQ_NOALLOC_SPLIT_BYTES   for tile counters (64 KiB) and partial sums of reductions split over
+ *                              workgroups
+ * A call that would need more returns HIPQ_ERR_LIMIT and launches nothing.  Every call on a GPU
+ * shares that GPU's array: calls of this entry point that overlap on one GPU (two streams, two
+ * threads) race; calls on one stream are ordered by the stream.  The tile counters are cleared by
+ * a kernel on `stream` ahead of every launch that uses them.
+ */
+#define HIPQ_NOALLOC_LAYOUT_BYTES (32u << 20)
+#define HIPQ_NOALLOC_SPLIT_BYTES (16u << 20)
+HIPQ_API int hipq_quantized_convolution_noalloc(const hipq_conv_desc_t* desc,
+                                                const void* data,
+                                                const void* filter,
+                                                const void* packed_filter, /* may be NULL */
+                                                const float* data_scale,
+                                                const void* data_zp,
+                                                const float* filter_scale,
+                                                const void* filter_zp,
+                                                const float* out_scale,
+                                                const void* out_zp,
+                                                void* out,
+                                                void* stream);
+
 /* Post-ops of the fused ops.  The arithmetic is oneDNN's as driven by the nGraph CPU backend:
  *   v = scale[k or 0] * ((float)acc + (float)bias[k]);  v = fmaf(sum_scale, (float)sum_in, v);
  *   v = relu ? max(v, 0) : v;  out = saturate<OUT>(nearbyintf(v))        round-half-to-even

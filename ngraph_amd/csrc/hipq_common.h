@@ -45,6 +45,15 @@ namespace hipq
     // frees the blocks of a stream that is about to be destroyed
     int release_stream_workspace(hipStream_t stream);
 
+    // Between noalloc_begin() and noalloc_end() on a thread, workspace() and split_workspace() hand
+    // out pieces of a fixed per-device array instead of allocating (sizes beyond it: HIPQ_ERR_LIMIT).
+    // noalloc_begin() fails when the array's address cannot be resolved on the current device.
+    constexpr size_t kScratchWorkspaceBytes = HIPQ_NOALLOC_LAYOUT_BYTES; // layout copies (transposed / padded / unrolled input)
+    constexpr size_t kScratchSplitBytes = HIPQ_NOALLOC_SPLIT_BYTES;      // tile counters + partial sums
+    constexpr size_t kScratchBytes = kScratchWorkspaceBytes + kScratchSplitBytes;
+    int noalloc_begin();
+    void noalloc_end();
+
     inline size_t dtype_size(int t)
     {
         switch (t)

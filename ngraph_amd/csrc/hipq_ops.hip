@@ -264,6 +264,28 @@ int hipq_quantized_convolution(const hipq_conv_desc_t* desc,
     return run_conv(g, data, filter, packed_filter, zp, e, out, as_stream(stream));
 }
 
+int hipq_quantized_convolution_noalloc(const hipq_conv_desc_t* desc,
+                                       const void* data,
+                                       const void* filter,
+                                       const void* packed_filter,
+                                       const float* data_scale,
+                                       const void* data_zp,
+                                       const float* filter_scale,
+                                       const void* filter_zp,
+                                       const float* out_scale,
+                                       const void* out_zp,
+                                       void* out,
+                                       void* stream)
+{
+    // same kernels, same choices; whatever scratch they need comes out of the fixed per-device array
+    int rc = noalloc_begin();
+    if (rc)
+        return rc;
+    rc = hipq_quantized_convolution(desc, data, filter, packed_filter, data_scale, data_zp, filter_scale, filter_zp, out_scale, out_zp, out, stream);
+    noalloc_end();
+    return rc;
+}
+
 int hipq_quantized_convolution_fused(const hipq_conv_desc_t* desc,
                                      const hipq_fused_desc_t* fused,
                                      const void* data,

@@ -30,6 +30,8 @@ namespace hipq
         return HIPQ_OK;
     }
 
+    __global__ void fill_bytes_kernel(uint8_t* dst, uint32_t pattern, size_t bytes);
+
     static const int kMaxDevices = 16;
     static std::mutex g_ws_mutex;
     static uint64_t g_ws_epoch[kMaxDevices] = {};
@@ -46,12 +48,46 @@ namespace hipq
     };
     static std::map<std::pair<int, hipStream_t>, StreamBlocks> g_blocks;
 
+    // Scratch of the entry point that allocates nothing: one array per device, resident from the
+    // moment the library's code is loaded until the process ends.  Host code never uses the name
+    // as an address; g_scratch_ptr[dev] is what hipGetSymbolAddress gave on that device.
+    static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+    static unsigned char* g_scratch_ptr[kMaxDevices] = {};
+    static thread_local int t_noalloc = 0;
+
     static int current_device(int* dev)
     {
         HIPQ_HIP(hipGetDevice(dev));
         if (*dev < 0 || *dev >= kMaxDevices)
             return fail(HIPQ_ERR_LIMIT, "device ordinal %d beyond %d", *dev, kMaxDevices);
         return HIPQ_OK;
+    }
+
+    int noalloc_begin()
+    {
+        int dev = 0;
+        int rc = current_device(&dev);
+        if (rc)
+            return rc;
+        {
+            std::lock_guard<std::mutex> lock(g_ws_mutex);
+            if (!g_scratch_ptr[dev])
+            {
+                void* p = nullptr;
+                HIPQ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+                if (!p)
+                    return fail(HIPQ_ERR_HIP, "the scratch array has no address on device %d", dev);
+                g_scratch_ptr[dev] = static_cast<unsigned char*>(p);
+            }
+        }
+        ++t_noalloc;
+        return HIPQ_OK;
+    }
+
+    void noalloc_end()
+    {
+        if (t_noalloc > 0)
+            --t_noalloc;
     }
 
     static int grow(Block& b, size_t need, hipStream_t stream, int dev, size_t zero_head)
@@ -84,6 +120,16 @@ namespace hipq
         int rc = current_device(&dev);
         if (rc)
             return rc;
+        if (t_noalloc)
+        {
+            if (bytes > kScratchWorkspaceBytes)
+                return fail(HIPQ_ERR_LIMIT,
+                            "this call needs a %zu-byte layout copy of its input; the entry point that allocates nothing holds %zu bytes for it",
+                            bytes,
+                            kScratchWorkspaceBytes);
+            *ptr = g_scratch_ptr[dev];
+            return HIPQ_OK;
+        }
         std::lock_guard<std::mutex> lock(g_ws_mutex);
         Block& b = g_blocks[std::make_pair(dev, stream)].ws;
         rc = grow(b, bytes, stream, dev, 0);
@@ -94,7 +140,9 @@ namespace hipq
     }
 
     // The counters are zeroed when the block is (re)allocated and every kernel that uses them
-    // leaves them at zero.
+    // leaves them at zero.  The fixed array of the entry point that allocates nothing keeps whatever
+    // its last call left, so there the counters are cleared (by a kernel: a caller may be capturing
+    // a graph) ahead of every launch that uses them.
     int split_workspace(size_t partial_bytes, hipStream_t stream, uint32_t** counters, void** partials)
     {
         int dev = 0;
@@ -102,6 +150,22 @@ namespace hipq
         if (rc)
             return rc;
         const size_t need = kSplitCounterBytes + partial_bytes;
+        if (t_noalloc)
+        {
+            if (need > kScratchSplitBytes)
+                return fail(HIPQ_ERR_LIMIT,
+                            "this call needs %zu bytes of partial sums; the entry point that allocates nothing holds %zu bytes for them",
+                            partial_bytes,
+                            kScratchSplitBytes - kSplitCounterBytes);
+            unsigned char* base = g_scratch_ptr[dev] + kScratchWorkspaceBytes;
+            fill_bytes_kernel<<<static_cast<unsigned>(kSplitCounterBytes / 16 / 256), 256, 0, stream>>>(base, 0u, kSplitCounterBytes);
+            rc = check_launch("fill_bytes");
+            if (rc)
+                return rc;
+            *counters = reinterpret_cast<uint32_t*>(base);
+            *partials = base + kSplitCounterBytes;
+            return HIPQ_OK;
+        }
         std::lock_guard<std::mutex> lock(g_ws_mutex);
         Block& b = g_blocks[std::make_pair(dev, stream)].split;
         rc = grow(b, need, stream, dev, kSplitCounterBytes);

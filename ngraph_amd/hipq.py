@@ -279,6 +279,7 @@ EXPORTS = [
     "hipq_conv_packed_filter_bytes",
     "hipq_conv_pack_filter",
     "hipq_quantized_convolution",
+    "hipq_quantized_convolution_noalloc",
     "hipq_quantized_convolution_fused",
     "hipq_dot_packed_bytes",
     "hipq_dot_pack",
@@ -347,6 +348,7 @@ def load():
     lib.hipq_conv_infer_output.argtypes = [C.POINTER(ConvDesc)]
     lib.hipq_conv_pack_filter.argtypes = [C.POINTER(ConvDesc), vp, vp, vp]
     lib.hipq_quantized_convolution.argtypes = [C.POINTER(ConvDesc)] + [vp] * 11
+    lib.hipq_quantized_convolution_noalloc.argtypes = [C.POINTER(ConvDesc)] + [vp] * 11
     lib.hipq_quantized_convolution_fused.argtypes = [C.POINTER(ConvDesc), C.POINTER(FusedDesc)] + [vp] * 9
     lib.hipq_dot_packed_bytes.restype = C.c_size_t
     lib.hipq_dot_packed_bytes.argtypes = [C.POINTER(DotDesc)]
@@ -474,7 +476,8 @@ def pack_dot(desc: DotDesc, b_dev: DeviceBuffer):
     return packed
 
 
-def quantized_convolution(desc, data, filt, data_scale, data_zp, filter_scale, filter_zp, out_scale, out_zp, use_packed=True):
+def quantized_convolution(desc, data, filt, data_scale, data_zp, filter_scale, filter_zp, out_scale, out_zp, use_packed=True, noalloc=False):
+    """noalloc=True goes through the entry point that takes its scratch from the library's fixed array"""
     lib = load()
     bd, bf = _dev(data), _dev(filt)
     packed = pack_filter(desc, bf) if use_packed else None
@@ -486,11 +489,8 @@ def quantized_convolution(desc, data, filt, data_scale, data_zp, filter_scale, f
     ]
     oshape = desc.out_shape()
     out = DeviceBuffer(int(np.prod(oshape)) * np.dtype(NP_OF[desc.out_t]).itemsize)
-    check(
-        lib.hipq_quantized_convolution(
-            C.byref(desc), bd.ptr, bf.ptr, _p(packed), s[0].ptr, z[0].ptr, s[1].ptr, z[1].ptr, s[2].ptr, z[2].ptr, out.ptr, None
-        )
-    )
+    entry = lib.hipq_quantized_convolution_noalloc if noalloc else lib.hipq_quantized_convolution
+    check(entry(C.byref(desc), bd.ptr, bf.ptr, _p(packed), s[0].ptr, z[0].ptr, s[1].ptr, z[1].ptr, s[2].ptr, z[2].ptr, out.ptr, None))
     check(lib.hipq_stream_sync(None))
     return out.to_numpy(NP_OF[desc.out_t], oshape)
 

@@ -290,6 +290,22 @@ def bench_resnet50(lib, stream, timer, batches=(1, 32, 128), use_graph=True):
     return out
 
 
+def copy_calibration(lib, stream, timer):
+    """a plain device-to-device copy of known size: the yardstick for the FETCH_SIZE / WRITE_SIZE
+    counters of a profiler run over this same command"""
+    cal_bytes = 64 << 20
+    ca, cb = H.DeviceBuffer(cal_bytes), H.DeviceBuffer(cal_bytes)
+    H.check(lib.hipq_fill_bytes(ca.ptr, 1, cal_bytes, stream))
+
+    def copy():
+        rc = lib.hipq_memcpy_d2d(cb.ptr, ca.ptr, cal_bytes, stream)
+        if rc:
+            H.check(rc)
+
+    _, cev = timer.run(copy, 10, 2)
+    return dict(bytes=cal_bytes, ms_event=cev, gbs=2 * cal_bytes / (cev * 1e-3) / 1e9)
+
+
 def host_threads():
     """threads for the host baselines: this process's share of the machine (OMP_NUM_THREADS when the
     environment sets it, never more than the CPUs the process may run on)"""
@@ -415,6 +431,7 @@ def main():
     ap.add_argument("--resnet-only", action="store_true", help="only the synthetic int8 ResNet-50 (for profiling); prints its results")
     ap.add_argument("--bert-only", action="store_true", help="only the synthetic int8 BERT-base encoder (for profiling); prints its results")
     ap.add_argument("--skip-models", action="store_true", help="leave out the BERT and ResNet-50 sections (kernel traces of the single operators; the models have runs of their own)")
+    ap.add_argument("--only", choices=["gemm", "qdq"], help="only config 2's GEMMs or config 3's Quantize / Dequantize (for counter runs under a profiler); prints their results")
     ap.add_argument("--no-graph", action="store_true", help="time the models' eager launch sequences only, no HIP-graph capture or replay (for runs under a profiler)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -430,6 +447,12 @@ def main():
     stream = sp.value
     timer = Timer(lib, stream)
 
+    if args.only == "gemm":
+        print(json.dumps({"gemm_config2": [bench_gemm(lib, stream, timer, m, args.steps, args.warmup) for m in (1, 32, 256)], "copy_calibration": copy_calibration(lib, stream, timer)}))
+        return
+    if args.only == "qdq":
+        print(json.dumps({"quantize_dequantize_config3": bench_qdq(lib, stream, timer, args.steps, args.warmup), "copy_calibration": copy_calibration(lib, stream, timer)}))
+        return
     if args.resnet_only:
         print(json.dumps({"resnet50_int8": bench_resnet50(lib, stream, timer, use_graph=not args.no_graph)}))
         return
@@ -446,19 +469,7 @@ def main():
     nhwc = bench_conv(lib, stream, timer, args.batch, args.steps, args.warmup, H.NXC)
 
     results = {"conv_nchw": [head], "conv_kernel_nhwc_in_nchw_out": [kern], "conv_nhwc_kernel": [nhwc]}
-    # a plain device-to-device copy of known size: the yardstick for the FETCH_SIZE / WRITE_SIZE
-    # counters of a profiler run over this same command
-    cal_bytes = 64 << 20
-    ca, cb = H.DeviceBuffer(cal_bytes), H.DeviceBuffer(cal_bytes)
-    H.check(lib.hipq_fill_bytes(ca.ptr, 1, cal_bytes, stream))
-
-    def copy():
-        rc = lib.hipq_memcpy_d2d(cb.ptr, ca.ptr, cal_bytes, stream)
-        if rc:
-            H.check(rc)
-
-    _, cev = timer.run(copy, 10, 2)
-    results["copy_calibration"] = dict(bytes=cal_bytes, ms_event=cev, gbs=2 * cal_bytes / (cev * 1e-3) / 1e9)
+    results["copy_calibration"] = copy_calibration(lib, stream, timer)
     cpu = None
     if not args.quick:
         small = max(20, args.steps // 4)

@@ -236,7 +236,9 @@ HIPQ_API int hipq_quantized_convolution(const hipq_conv_desc_t* desc,
  * a fixed array that every GPU the library runs on holds from load time until the process ends:
  *   HIPQ_NOALLOC_LAYOUT_BYTES  for the channels-last / padded / unrolled copy of an NCX input
  *                              (an NCX u8 input of up to that many bytes; channels-last inputs
- *                              with 64-multiple channel counts need none)
+ *                              with 64-multiple channel counts need none, nor do 3x3 stride-1
+ *                              layers over 64 channels with an NCX output, whose kernel reads
+ *                              NCX itself)
  *   HIPQ_NOALLOC_SPLIT_BYTES   for tile counters (64 KiB) and partial sums of reductions split over
  *                              workgroups
  * A call that would need more returns HIPQ_ERR_LIMIT and launches nothing.  Every call on a GPU

@@ -235,6 +235,9 @@ namespace hipq
                          void* out,
                          bool out_ncx,
                          hipStream_t s);
+    // 3x3 over 64 channels, filter in registers; data in the layout g.data_layout names
+    bool conv_regw_eligible(const ConvGeom& g, bool out_ncx);
+    int launch_conv_regw(const ConvGeom& g, const void* data, const void* packed, const ZeroPoints& zp, const Epilogue& epi, void* out, bool out_ncx, hipStream_t s);
     int launch_conv_mfma(const ConvGeom& g,
                          const void* data_nxc,
                          const void* packed,

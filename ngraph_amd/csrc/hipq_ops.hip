@@ -65,7 +65,12 @@ namespace hipq
         if (!packed || !conv_mfma_eligible(g) || (epi.mode == EPI_FUSED && g.out_t == HIPQ_I32))
             return launch_conv_direct(g, data, filter, zp, epi, out, s);
 
-        // The kernels read channels-last data; an NCHW input is transposed through the workspace.
+        // 3x3 layers over 64 channels with an NCHW output keep their filter in registers and read the
+        // input in whichever layout it has: no transposition, no scratch
+        if (conv_regw_eligible(g, g.out_layout == HIPQ_LAYOUT_NCX && g.K > 1))
+            return launch_conv_regw(g, data, packed, zp, epi, out, true, s);
+
+        // The other kernels read channels-last data; an NCHW input is transposed through the workspace.
         // The output is written directly in either layout (sum_in is indexed like the output).
         // A layer with few output pixels in all (M <= 64: the deepest layers of a network at batch 1)
         // is a skinny GEMM over its receptive-field matrix [M][taps * C] -- the data itself for a 1x1

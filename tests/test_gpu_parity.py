@@ -225,7 +225,7 @@ def test_conv_mfma_shapes(gpu_lib, i):
         exp = O.quantized_convolution(d, data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
         O.port().orc_set_threads(1)
         got = H.quantized_convolution(d, data, filt, s[0], z[0], s[1], z[1], s[2], z[2])
-        assert H.last_kernel().startswith(("conv_mfma", "conv_band", "dot_skinny")), H.last_kernel()
+        assert H.last_kernel().startswith(("conv_mfma", "conv_band", "conv_regw", "dot_skinny")), H.last_kernel()
         assert np.array_equal(got, exp), (out_t, z)
     # reference layouts in and out (transposed through the workspace)
     d = H.make_conv_desc(N, Cc, K, in_sp, f_sp, out_t="i8", **kw)
@@ -234,7 +234,7 @@ def test_conv_mfma_shapes(gpu_lib, i):
     exp = O.quantized_convolution(d, data, filt, 0.02, 0, 0.005, 0, 0.9, 0)
     O.port().orc_set_threads(1)
     got = H.quantized_convolution(d, data, filt, 0.02, 0, 0.005, 0, 0.9, 0)
-    assert H.last_kernel().startswith(("conv_mfma", "conv_band", "dot_skinny")), H.last_kernel()
+    assert H.last_kernel().startswith(("conv_mfma", "conv_band", "conv_regw", "dot_skinny")), H.last_kernel()
     assert np.array_equal(got, exp)
 
 
@@ -275,7 +275,7 @@ def test_conv_linearity_at_config1_batch(gpu_lib):
     a = H.quantized_convolution(d, data, f1, 1.0, 0, 1.0, 0, 1.0, 0).astype(np.int64)
     b = H.quantized_convolution(d, data, f2, 1.0, 0, 1.0, 0, 1.0, 0).astype(np.int64)
     c = H.quantized_convolution(d, data, (f1 + f2).astype(np.int8), 1.0, 0, 1.0, 0, 1.0, 0).astype(np.int64)
-    assert H.last_kernel().startswith(("conv_mfma", "conv_band", "dot_skinny"))
+    assert H.last_kernel().startswith(("conv_mfma", "conv_band", "conv_regw", "dot_skinny"))
     assert np.array_equal(a + b, c)
     d1 = H.make_conv_desc(1, 64, 64, (56, 56), (3, 3), **kw)
     O.port().orc_set_threads(8)
@@ -372,9 +372,12 @@ BAND_SHAPES = [
 
 
 @pytest.mark.parametrize("i", range(len(BAND_SHAPES)))
-def test_conv_band(gpu_lib, i):
+def test_conv_band(gpu_lib, i, monkeypatch):
     """the LDS-resident-filter kernel against the oracle: both requantization policies, both output
-    layouts, both fixed-point and float requantization branches, i32 output, zero points"""
+    layouts, both fixed-point and float requantization branches, i32 output, zero points (the
+    filter-in-registers kernel, which would take the 3x3 shapes with an NCHW output, is switched off:
+    tests/test_conv_regw.py is its own)"""
+    monkeypatch.setenv("HIPQ_NO_REGW", "1")
     N, K, in_sp, f_sp, kw = BAND_SHAPES[i]
     say("band conv", BAND_SHAPES[i])
     O.port().orc_set_threads(8)
@@ -632,12 +635,15 @@ def test_conv_band_matches_generic_kernel(gpu_lib, monkeypatch):
     d = H.make_conv_desc(16, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1))
     data = synth.uniform_int(701, d.data_shape(), 0, 255, np.uint8)
     filt = synth.uniform_int(702, d.filter_shape(), -127, 127, np.int8)
+    r = H.quantized_convolution(d, data, filt, 0.02, 0, 0.005, 0, 0.1, 0)
+    assert H.last_kernel().startswith("conv_regw"), H.last_kernel()  # NCHW out, 3x3 over 64 channels: filter in registers
+    monkeypatch.setenv("HIPQ_NO_REGW", "1")
     a = H.quantized_convolution(d, data, filt, 0.02, 0, 0.005, 0, 0.1, 0)
     assert H.last_kernel().startswith("conv_band"), H.last_kernel()
     monkeypatch.setenv("HIPQ_NO_BAND", "1")
     b = H.quantized_convolution(d, data, filt, 0.02, 0, 0.005, 0, 0.1, 0)
     assert H.last_kernel().startswith("conv_mfma"), H.last_kernel()
-    assert np.array_equal(a, b)
+    assert np.array_equal(a, b) and np.array_equal(r, a)
 
 
 # ------------------------------------------------------------------ QuantizedDot

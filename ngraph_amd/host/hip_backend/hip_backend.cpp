@@ -14,7 +14,14 @@
 
 #include "hipq.h"
 #include "ngraph/ngraph.hpp"
+#include "ngraph/pass/constant_folding.hpp"
+#include "ngraph/pass/manager.hpp"
+#include "ngraph/pass/pass_config.hpp"
+#include "ngraph/runtime/backend_manager.hpp"
+#include "ngraph/runtime/executable.hpp"
 #include "ngraph/runtime/hip/pass/hip_quant_fusion.hpp"
+#include "ngraph/runtime/performance_counter.hpp"
+#include "ngraph/runtime/tensor.hpp"
 
 using namespace std;
 using namespace ngraph;
@@ -191,13 +198,35 @@ namespace
         auto c = as_type_ptr<op::v0::Constant>(o.get_node_shared_ptr());
         if (!c)
             return false;
-        for (double v : c->get_values_as_double())
-            if (v != 0.0)
+        // zero in every element type of a zero point (u8, i8, i32) is all bytes zero
+        const auto* bytes = static_cast<const unsigned char*>(c->get_data_ptr());
+        const size_t count = shape_size(c->get_output_shape(0)) * c->get_output_element_type(0).size();
+        for (size_t i = 0; i < count; ++i)
+            if (bytes[i] != 0)
                 return false;
         return true;
     }
 
-    void fill_conv_desc(hipq_conv_desc_t& d, const Node& n, const op::v0::ConvAttributes& a)
+    // the five attributes every quantized convolution op carries, read through the getters each op
+    // class has of its own (src/ngraph/op/quantized_convolution.hpp:72-80,
+    // src/ngraph/op/experimental/quantized_conv_bias.hpp, quantized_conv_relu.hpp)
+    struct ConvAttrs
+    {
+        Strides window_movement_strides, window_dilation_strides, data_dilation_strides;
+        CoordinateDiff padding_below, padding_above;
+        const Strides& get_window_movement_strides() const { return window_movement_strides; }
+        const Strides& get_window_dilation_strides() const { return window_dilation_strides; }
+        const Strides& get_data_dilation_strides() const { return data_dilation_strides; }
+        const CoordinateDiff& get_padding_below() const { return padding_below; }
+        const CoordinateDiff& get_padding_above() const { return padding_above; }
+    };
+    template <typename OP>
+    ConvAttrs conv_attrs(const OP& op)
+    {
+        return ConvAttrs{op.get_window_movement_strides(), op.get_window_dilation_strides(), op.get_data_dilation_strides(), op.get_padding_below(), op.get_padding_above()};
+    }
+
+    void fill_conv_desc(hipq_conv_desc_t& d, const Node& n, const ConvAttrs& a)
     {
         memset(&d, 0, sizeof(d));
         const Shape& ds = n.get_input_shape(0);
@@ -263,12 +292,12 @@ namespace
             return r;
         if (is_type<op::v0::Relu>(n) || is_type<op::v0::Abs>(n) || is_type<op::v0::Convert>(n) || is_type<op::v0::MaxPool>(n) || is_type<op::v0::AvgPool>(n))
             r.push_back(0);
-        else if (auto q = as_type<op::v0::Quantize>(n))
+        else if (auto q = as_type<const op::v0::Quantize>(n))
         {
             if (q->get_axes().empty())
                 r.push_back(0);
         }
-        else if (auto dq = as_type<op::v0::Dequantize>(n))
+        else if (auto dq = as_type<const op::v0::Dequantize>(n))
         {
             if (dq->get_axes().empty())
                 r.push_back(0);
@@ -337,38 +366,38 @@ namespace
 
     void HIPExecutable::lower_conv(const shared_ptr<Node>& n, Step& st)
     {
-        const op::v0::ConvAttributes* attrs = nullptr;
+        ConvAttrs attrs;
         // input positions per op (src/ngraph/op/experimental/quantized_conv_bias.cpp, quantized_conv_relu.cpp)
         int bias_i = -1, sum_i = -1, scale_i = -1, sum_scale_i = -1;
         bool relu = false, plain = false;
         int sum_t = HIPQ_U8;
         if (auto q = as_type_ptr<op::v0::QuantizedConvolution>(n))
         {
-            attrs = q.get();
+            attrs = conv_attrs(*q);
             plain = true;
         }
         else if (auto qb = as_type_ptr<op::v0::QuantizedConvolutionBias>(n))
         {
-            attrs = qb.get();
+            attrs = conv_attrs(*qb);
             bias_i = 2, scale_i = 3, relu = qb->with_relu();
         }
         else if (auto qr = as_type_ptr<op::v0::QuantizedConvolutionRelu>(n))
         {
-            attrs = qr.get();
+            attrs = conv_attrs(*qr);
             scale_i = 2, relu = true;
         }
         else if (auto qa = as_type_ptr<op::v0::QuantizedConvolutionBiasAdd>(n))
         {
-            attrs = qa.get();
+            attrs = conv_attrs(*qa);
             bias_i = 2, sum_i = 3, scale_i = 4, sum_scale_i = 5, relu = qa->with_relu();
         }
         else if (auto qs = as_type_ptr<op::v0::QuantizedConvolutionBiasSignedAdd>(n))
         {
-            attrs = qs.get();
+            attrs = conv_attrs(*qs);
             bias_i = 2, sum_i = 3, scale_i = 4, sum_scale_i = 5, relu = qs->with_relu();
         }
         hipq_conv_desc_t d;
-        fill_conv_desc(d, *n, *attrs);
+        fill_conv_desc(d, *n, attrs);
         d.data_layout = nxc(n->input_value(0).get_node()) ? HIPQ_LAYOUT_NXC : HIPQ_LAYOUT_NCX;
         d.out_layout = nxc(n.get()) ? HIPQ_LAYOUT_NXC : HIPQ_LAYOUT_NCX; // the sum input is in the output's class
         if (sum_i >= 0)
@@ -827,8 +856,13 @@ namespace
         check(hipq_stream_create(&m_stream), "stream creation");
         // work on a private copy: compile must not change the caller's graph
         m_function = clone_function(*func);
+        // a pass named in NGRAPH_PASS_ENABLES with 0 is left out, like the reference CPU backend's
+        // knobbed passes (src/ngraph/runtime/cpu/cpu_external_function.cpp:215-226)
         pass::Manager pm;
-        pm.register_pass<runtime::hip::pass::HIPQuantFusion>();
+        const auto& knobs = pm.get_pass_config().get_enables();
+        const auto fusion = knobs.find("HIPQuantFusion");
+        if (fusion == knobs.end() || fusion->second)
+            pm.register_pass<runtime::hip::pass::HIPQuantFusion>();
         pm.register_pass<pass::ConstantFolding>();
         pm.run_passes(m_function);
         assign_layouts();

@@ -15,6 +15,7 @@
 #include <sstream>
 #include <stdexcept>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #define NGRAPH_API __attribute__((visibility("default")))
@@ -369,10 +370,12 @@ namespace ngraph
     {
         return is_type<T>(n) ? std::static_pointer_cast<T>(n) : std::shared_ptr<T>();
     }
-    template <typename T>
-    const T* as_type(const Node* n)
+    // src/ngraph/type.hpp:80-90: casts a Value* to a Type* if it is of that type, nullptr otherwise
+    // (Type carries the constness: as_type<const op::v0::Quantize>(const Node*))
+    template <typename Type, typename Value>
+    Type* as_type(Value value)
     {
-        return is_type<T>(n) ? static_cast<const T*>(n) : nullptr;
+        return is_type<typename std::remove_const<Type>::type>(value) ? static_cast<Type*>(value) : nullptr;
     }
 
     namespace op

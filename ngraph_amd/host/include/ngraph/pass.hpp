@@ -28,11 +28,13 @@ namespace ngraph
             std::map<std::string, bool> m_pass_attributes;
         };
 
+        // as in src/ngraph/pass/pass.hpp:72-99: a pass has no name of its own; which passes run is the
+        // registering backend's decision (it consults PassConfig the way REGISTER_KNOBBED_PASS does,
+        // src/ngraph/runtime/cpu/cpu_external_function.cpp:215-226)
         class NGRAPH_API PassBase
         {
         public:
             virtual ~PassBase() {}
-            virtual std::string get_name() const = 0;
         };
 
         class NGRAPH_API FunctionPass : public PassBase
@@ -51,9 +53,9 @@ namespace ngraph
             {
                 m_passes.push_back(std::make_shared<T>(std::forward<Args>(args)...));
             }
-            // runs the registered passes in order; a pass named in NGRAPH_PASS_ENABLES with 0 is skipped
+            // runs the registered passes in order
             void run_passes(std::shared_ptr<Function> f);
-            const PassConfig& get_pass_config() const { return m_config; }
+            PassConfig& get_pass_config() { return m_config; }
             void set_pass_config(const PassConfig& c) { m_config = c; }
 
         private:
@@ -67,7 +69,6 @@ namespace ngraph
         class NGRAPH_API ConstantFolding : public FunctionPass
         {
         public:
-            std::string get_name() const override { return "ConstantFolding"; }
             bool run_on_function(std::shared_ptr<Function> f) override;
         };
     }

@@ -4,7 +4,7 @@
 // "HIPQuantFusion:0" switches it off.
 #pragma once
 
-#include "ngraph/pass.hpp"
+#include "ngraph/pass/pass.hpp"
 
 namespace ngraph
 {
@@ -27,7 +27,6 @@ namespace ngraph
                 class NGRAPH_API HIPQuantFusion : public ngraph::pass::FunctionPass
                 {
                 public:
-                    std::string get_name() const override { return "HIPQuantFusion"; }
                     bool run_on_function(std::shared_ptr<Function> f) override;
                 };
             }

@@ -5,7 +5,7 @@
 #include <vector>
 
 #include "ngraph/builder/make_constant.hpp"
-#include "ngraph/ops.hpp"
+#include "ngraph/ngraph.hpp"
 #include "ngraph/runtime/hip/pass/hip_quant_fusion.hpp"
 
 using namespace std;
@@ -45,7 +45,7 @@ namespace
     }
 
     // src/ngraph/graph_util.cpp compare_constants: both Constants, same shape and the same values
-    bool compare_constants(const shared_ptr<Node>& a, const shared_ptr<Node>& b)
+    bool same_constants(const shared_ptr<Node>& a, const shared_ptr<Node>& b)
     {
         if (a == b && a->is_constant())
             return true;
@@ -145,7 +145,7 @@ namespace
                     if (is_type<op::v0::Quantize>(user))
                     {
                         auto q_scale = user->get_argument(1);
-                        if (!compare_constants(q_scale, dq_l->get_argument(1)) && compare_constants(q_scale, dq_r->get_argument(1)))
+                        if (!same_constants(q_scale, dq_l->get_argument(1)) && same_constants(q_scale, dq_r->get_argument(1)))
                             swap(dq_l, dq_r);
                         break;
                     }
@@ -221,7 +221,7 @@ namespace
             auto dq = as_type_ptr<op::v0::Dequantize>(cc->get_argument(i));
             if (!dq || !dq->get_axes().empty() || dq->get_input_element_type(0) != dq0->get_input_element_type(0))
                 return false;
-            if (!compare_constants(dq->get_argument(1), dq0->get_argument(1)) || !compare_constants(dq->get_argument(2), dq0->get_argument(2)))
+            if (!same_constants(dq->get_argument(1), dq0->get_argument(1)) || !same_constants(dq->get_argument(2), dq0->get_argument(2)))
                 return false;
             args.push_back(dq->input_value(0));
         }
@@ -237,7 +237,7 @@ namespace
             return false;
         if (q->get_output_element_type(0) != dq->get_input_element_type(0))
             return false;
-        if (!compare_constants(q->get_argument(1), dq->get_argument(1)))
+        if (!same_constants(q->get_argument(1), dq->get_argument(1)))
             return false;
         f.replace_node(q, dq->get_argument(0));
         return true;

@@ -55,12 +55,7 @@ namespace ngraph
         void Manager::run_passes(shared_ptr<Function> f)
         {
             for (auto& p : m_passes)
-            {
-                auto it = m_config.get_enables().find(p->get_name());
-                if (it != m_config.get_enables().end() && !it->second)
-                    continue;
                 p->run_on_function(f);
-            }
         }
 
         // ---- constant folding ----------------------------------------------------------------

@@ -421,11 +421,11 @@ namespace hipq
         }
     };
 
-    // Out of line, so that its registers do not weigh on the MFMA path, with the descriptors passed
-    // by value: passed by reference the kernel's own arguments would have to live in scratch
-    // memory, and every lane of every launch would store them there on entry.
+    // Inlined: as a call its by-value descriptors travelled on the stack, which gave every kernel 96
+    // bytes of scratch a lane (set up at every launch although only this path touched it); inlined it
+    // costs the MFMA path at most two registers, the branch being uniform and the loops scalar.
     template <class XL>
-    __device__ __noinline__ void slow_tile(const XL xl,
+    __device__ __attribute__((always_inline)) void slow_tile(const XL xl,
                                            const int8_t* __restrict__ w,
                                            int64_t M,
                                            int32_t Kred,

@@ -208,14 +208,76 @@ namespace hipq
         return row - q * v.a;
     }
 
-    constexpr int kUnroll = 4;
+    // Groups a lane handles per launch, one wavefront-contiguous step of 256 groups apart (measured
+    // on f32[64,1024,1024]: 3 is best for Quantize, 2 for Dequantize).
+    constexpr int kQuantUnroll = 3;
+    constexpr int kDequantUnroll = 2;
+
+    // ROW_UNIFORM: inner/4 is a multiple of the 256 groups one step of a workgroup covers (or the
+    // scale is a scalar), so a step lies inside one row of the scale table and its index comes from
+    // the block index alone: scale and zero point arrive through the scalar unit instead of two
+    // vector loads and two 64-bit multiplies per lane.
+    template <bool ROW_UNIFORM>
+    __device__ __forceinline__ uint32_t step_run_index(const RunView& v, uint32_t first_group_of_step, uint32_t g)
+    {
+        return run_index(v, ROW_UNIFORM ? first_group_of_step : g);
+    }
     typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+    // ---- division with the reciprocal shared by the four elements of a group -------------------
+    // The instruction sequence the compiler emits for an IEEE float division is
+    //     r = rcp(s); r = fma(fma(-s, r, 1), r, r);
+    //     q = x * r;  q = fma(fma(-s, q, x), r, q);  q = fma(fma(-s, q, x), r, q);
+    // wrapped in v_div_scale / v_div_fmas / v_div_fixup, which rescale the operands when an
+    // exponent is extreme and patch the special cases (zero, Inf, NaN, denormal).  For a divisor
+    // with 2^-30 <= |s| <= 2^30 and a dividend with 2^-60 <= |x| < 2^30 neither does anything, so
+    // the bare sequence returns the same bits, and the first line depends on s alone.  A dividend
+    // below 2^-60 gives a quotient below 2^-30 in magnitude from either sequence: it rounds to
+    // zero whichever bits it has.  Groups outside these ranges take the compiler's division.
+    __device__ __forceinline__ bool shared_reciprocal_ok(f32x4 x, float s)
+    {
+        const float big = 1073741824.0f;       // 2^30
+        const float small = 9.31322574615478515625e-10f; // 2^-30
+        // the sum is NaN or Inf if any element is, and bounds every |x|
+        float sum = (__builtin_fabsf(x[0]) + __builtin_fabsf(x[1])) + (__builtin_fabsf(x[2]) + __builtin_fabsf(x[3]));
+        float a = __builtin_fabsf(s);
+        return (sum < big) & (__builtin_amdgcn_fmed3f(a, small, big) == a);
+    }
+
+    // Four elements to four bytes, round-half-even, for a group that passed shared_reciprocal_ok.
+    // v_cvt_pk_u8_f32 converts with saturation to 0..255 and places the byte, i.e. the clamp, the
+    // cast and the packing in one instruction; signed outputs are computed 128 higher and flipped
+    // back with one XOR (the sum rint(q) + z is exact wherever it lies near the clamp range).
+    template <typename QUANT>
+    __device__ __forceinline__ uint32_t quantize4_shared_reciprocal(f32x4 x, float s, float z)
+    {
+        const bool is_signed = QLimits<QUANT>::lo < 0.0;
+        float zz = is_signed ? z + 128.0f : z;
+        float r = __builtin_amdgcn_rcpf(s);
+        float e = __builtin_fmaf(-s, r, 1.0f);
+        r = __builtin_fmaf(e, r, r);
+        uint32_t packed = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+        {
+            float q = __fmul_rn(x[k], r);
+            float t = __builtin_fmaf(-s, q, x[k]);
+            q = __builtin_fmaf(t, r, q);
+            t = __builtin_fmaf(-s, q, x[k]);
+            q = __builtin_fmaf(t, r, q);
+            float v = __fadd_rn(__builtin_rintf(q), zz);
+            packed = __builtin_amdgcn_cvt_pk_u8_f32(v, k, packed);
+        }
+        return is_signed ? packed ^ 0x80808080u : packed;
+    }
 
     // For 8-bit outputs the reference's round-half-even formula equals rintf(): the two differ only
     // for |q| >= 2^23, where both lie beyond the clamp range whatever the zero point.
     template <typename QUANT, bool RNE>
     __device__ __forceinline__ uint32_t quantize4(f32x4 x, float s, float z, int mode)
     {
+        if (RNE && shared_reciprocal_ok(x, s))
+            return quantize4_shared_reciprocal<QUANT>(x, s, z);
         const float lo = static_cast<float>(QLimits<QUANT>::lo);
         const float hi = static_cast<float>(QLimits<QUANT>::hi);
         float q[4] = {x[0], x[1], x[2], x[3]};
@@ -234,7 +296,7 @@ namespace hipq
         return packed;
     }
 
-    template <typename QUANT, bool RNE>
+    template <typename QUANT, bool RNE, bool ROW_UNIFORM>
     __global__ __launch_bounds__(256) void quantize_vec4_kernel(const f32x4* __restrict__ in,
                                                                 const float* __restrict__ scale,
                                                                 const QUANT* __restrict__ zp,
@@ -243,7 +305,9 @@ namespace hipq
                                                                 RunView view,
                                                                 int mode)
     {
-        uint32_t base = blockIdx.x * (256u * kUnroll) + threadIdx.x;
+        constexpr int kUnroll = kQuantUnroll;
+        uint32_t first = blockIdx.x * (256u * kUnroll);
+        uint32_t base = first + threadIdx.x;
         f32x4 x[kUnroll];
         float s[kUnroll];
         float z[kUnroll];
@@ -254,7 +318,7 @@ namespace hipq
             if (g < groups)
             {
                 x[u] = __builtin_nontemporal_load(&in[g]);
-                uint32_t j = run_index(view, g);
+                uint32_t j = step_run_index<ROW_UNIFORM>(view, first + u * 256u, g);
                 s[u] = scale[j];
                 z[u] = static_cast<float>(zp[j]);
             }
@@ -268,7 +332,9 @@ namespace hipq
         }
     }
 
-    template <typename QUANT>
+    // The quantized side is read with ordinary loads (4 bytes a lane: streaming hints on so narrow a
+    // load cost a sixth of the rate), the f32 side written with streaming stores.
+    template <typename QUANT, bool ROW_UNIFORM>
     __global__ __launch_bounds__(256) void dequantize_vec4_kernel(const uint32_t* __restrict__ in,
                                                                   const float* __restrict__ scale,
                                                                   const QUANT* __restrict__ zp,
@@ -276,7 +342,9 @@ namespace hipq
                                                                   uint32_t groups,
                                                                   RunView view)
     {
-        uint32_t base = blockIdx.x * (256u * kUnroll) + threadIdx.x;
+        constexpr int kUnroll = kDequantUnroll;
+        uint32_t first = blockIdx.x * (256u * kUnroll);
+        uint32_t base = first + threadIdx.x;
         uint32_t q[kUnroll];
         float s[kUnroll];
         int32_t z[kUnroll];
@@ -286,8 +354,8 @@ namespace hipq
             uint32_t g = base + u * 256u;
             if (g < groups)
             {
-                q[u] = __builtin_nontemporal_load(&in[g]);
-                uint32_t j = run_index(view, g);
+                q[u] = in[g];
+                uint32_t j = step_run_index<ROW_UNIFORM>(view, first + u * 256u, g);
                 s[u] = scale[j];
                 z[u] = static_cast<int32_t>(zp[j]);
             }
@@ -389,6 +457,9 @@ namespace hipq
                (reinterpret_cast<uintptr_t>(f32_ptr) & 15) == 0 && (reinterpret_cast<uintptr_t>(q_ptr) & 3) == 0;
     }
 
+    // every 256-group step of a workgroup lies inside one row of the scale table
+    static bool row_uniform(const Canon& c) { return c.a == 1 || (c.inner / 4) % 256 == 0; }
+
     static RunView make_view(const Canon& c)
     {
         RunView v;
@@ -423,31 +494,35 @@ int hipq_quantize(const hipq_quant_desc_t* d, const void* in, const void* scale,
     if (vec4_ok(*d, c, in, out))
     {
         uint32_t groups = static_cast<uint32_t>(c.count / 4);
-        unsigned blocks = (groups + 256 * kUnroll - 1) / (256 * kUnroll);
+        unsigned blocks = (groups + 256 * kQuantUnroll - 1) / (256 * kQuantUnroll);
         RunView v = make_view(c);
         bool rne = d->round_mode == HIPQ_ROUND_NEAREST_TOWARD_EVEN;
-#define LAUNCH_Q4(QT, RNE)                                                                         \
-    quantize_vec4_kernel<QT, RNE><<<blocks, 256, 0, s>>>(static_cast<const f32x4*>(in),           \
-                                                         static_cast<const float*>(scale),         \
-                                                         static_cast<const QT*>(zp),               \
-                                                         static_cast<uint32_t*>(out),              \
-                                                         groups,                                   \
-                                                         v,                                        \
-                                                         d->round_mode)
+        bool uniform = row_uniform(c);
+#define LAUNCH_Q4(QT, RNE, UNI)                                                                    \
+    quantize_vec4_kernel<QT, RNE, UNI><<<blocks, 256, 0, s>>>(static_cast<const f32x4*>(in),      \
+                                                              static_cast<const float*>(scale),    \
+                                                              static_cast<const QT*>(zp),          \
+                                                              static_cast<uint32_t*>(out),         \
+                                                              groups,                              \
+                                                              v,                                   \
+                                                              d->round_mode)
+#define LAUNCH_Q4_T(QT)                                                                            \
+    do                                                                                             \
+    {                                                                                              \
+        if (rne && uniform)                                                                        \
+            LAUNCH_Q4(QT, true, true);                                                             \
+        else if (rne)                                                                              \
+            LAUNCH_Q4(QT, true, false);                                                            \
+        else if (uniform)                                                                          \
+            LAUNCH_Q4(QT, false, true);                                                            \
+        else                                                                                       \
+            LAUNCH_Q4(QT, false, false);                                                           \
+    } while (0)
         if (d->quant_t == HIPQ_I8)
-        {
-            if (rne)
-                LAUNCH_Q4(int8_t, true);
-            else
-                LAUNCH_Q4(int8_t, false);
-        }
+            LAUNCH_Q4_T(int8_t);
         else
-        {
-            if (rne)
-                LAUNCH_Q4(uint8_t, true);
-            else
-                LAUNCH_Q4(uint8_t, false);
-        }
+            LAUNCH_Q4_T(uint8_t);
+#undef LAUNCH_Q4_T
 #undef LAUNCH_Q4
         return check_launch("quantize_vec4");
     }
@@ -496,22 +571,31 @@ int hipq_dequantize(const hipq_quant_desc_t* d, const void* in, const void* scal
     if (vec4_ok(*d, c, out, in))
     {
         uint32_t groups = static_cast<uint32_t>(c.count / 4);
-        unsigned blocks = (groups + 256 * kUnroll - 1) / (256 * kUnroll);
+        unsigned blocks = (groups + 256 * kDequantUnroll - 1) / (256 * kDequantUnroll);
         RunView v = make_view(c);
+        bool uniform = row_uniform(c);
+#define LAUNCH_D4(QT, UNI)                                                                         \
+    dequantize_vec4_kernel<QT, UNI><<<blocks, 256, 0, s>>>(static_cast<const uint32_t*>(in),       \
+                                                           static_cast<const float*>(scale),       \
+                                                           static_cast<const QT*>(zp),             \
+                                                           static_cast<f32x4*>(out),               \
+                                                           groups,                                 \
+                                                           v)
         if (d->quant_t == HIPQ_I8)
-            dequantize_vec4_kernel<int8_t><<<blocks, 256, 0, s>>>(static_cast<const uint32_t*>(in),
-                                                                  static_cast<const float*>(scale),
-                                                                  static_cast<const int8_t*>(zp),
-                                                                  static_cast<f32x4*>(out),
-                                                                  groups,
-                                                                  v);
+        {
+            if (uniform)
+                LAUNCH_D4(int8_t, true);
+            else
+                LAUNCH_D4(int8_t, false);
+        }
         else
-            dequantize_vec4_kernel<uint8_t><<<blocks, 256, 0, s>>>(static_cast<const uint32_t*>(in),
-                                                                   static_cast<const float*>(scale),
-                                                                   static_cast<const uint8_t*>(zp),
-                                                                   static_cast<f32x4*>(out),
-                                                                   groups,
-                                                                   v);
+        {
+            if (uniform)
+                LAUNCH_D4(uint8_t, true);
+            else
+                LAUNCH_D4(uint8_t, false);
+        }
+#undef LAUNCH_D4
         return check_launch("dequantize_vec4");
     }
     DimInfo di = dim_info(*d);

@@ -140,6 +140,51 @@ def test_quantize_dequantize_config3_full_size_properties(gpu_lib):
     assert np.all(err <= bound)
 
 
+@pytest.mark.parametrize("inner", [1024, 1000])
+@pytest.mark.parametrize("qt", ["i8", "u8"])
+def test_quantize_division_bits_near_ties(gpu_lib, qt, inner):
+    """The vectorised kernel shares one reciprocal among the four elements of a group when the
+    exponents allow it: its quotients must still be the IEEE ones.  Dividends are placed on and a
+    few ulp either side of scale * (k + 1/2), where one wrong last bit of the quotient changes the
+    rounded integer; scales cover the range limits of the shared-reciprocal path (2^-30, 2^30), what
+    lies beyond them (denormal, huge, negative, Inf, NaN, zero), and groups mix special dividends
+    (NaN, Inf, denormals, -0, 1e35) with ordinary ones.  inner = 1024 takes the kernel form whose
+    scale index is uniform over a workgroup step, inner = 1000 the per-lane form; the dequantize
+    kernels have the same two forms and are checked on the result."""
+    rng = np.random.default_rng(2024)
+    chans = 256
+    scale = rng.uniform(0.001, 3.0, chans).astype(np.float32)
+    scale[:24] = np.float32(
+        [2.0**-30, 2.0**-30 * (1 - 2.0**-24), 2.0**30, 2.0**30 * (1 + 2.0**-23), 1e-40, 3e38, -0.37, -(2.0**-31), np.inf, np.nan, 0.0, -0.0,
+         1.0, 0.5, 3.0, 1 / 3, 0.1, 127.0, 1 / 127, 2.0**-29, 2.0**29, 1.9999999, 1.0000001, 0.99999994]
+    )
+    k = rng.integers(-140, 140, (chans, inner)).astype(np.float32) + np.float32(0.5)
+    with np.errstate(all="ignore"):
+        x = (scale[:, None] * k).astype(np.float32)
+        ulps = rng.integers(-3, 4, x.shape).astype(np.int32)
+        x = (x.view(np.int32) + ulps).view(np.float32)
+    special = np.float32([np.nan, np.inf, -np.inf, 1e-42, -1e-42, -0.0, 1e35, -1e35, 2.0**30, 2.0**-60, 2.0**-61, 1e-30])
+    pos = rng.integers(0, inner, (chans, special.size))
+    for c in range(0, chans, 3):
+        x[c, pos[c]] = special
+    zp = rng.integers(-9, 9, chans).astype(np.int8) if qt == "i8" else rng.integers(0, 30, chans).astype(np.uint8)
+    say("ties", qt)
+    got = H.quantize(x, scale, zp, qt, (0,))
+    assert H.last_kernel() == "quantize_vec4"
+    with np.errstate(all="ignore"):
+        exp = O.quantize(x, scale, zp, qt, (0,))
+    assert np.array_equal(got, exp)
+    with np.errstate(all="ignore"):
+        dq = H.dequantize(got, scale, zp, "f32", (0,))
+        assert H.last_kernel() == "dequantize_vec4"
+        assert np.array_equal(dq, O.dequantize(exp, scale, zp, "f32", (0,)), equal_nan=True)
+    # the same through the scalar-scale form, ordinary scales only
+    for c in (12, 13, 15, 16, 40, 41):
+        g1 = H.quantize(x[c], scale[c], zp[c], qt)
+        with np.errstate(all="ignore"):
+            assert np.array_equal(g1, O.quantize(x[c], scale[c], zp[c], qt)), c
+
+
 def test_quantize_empty_and_scalar(gpu_lib):
     say("empty / rank-0")
     assert H.quantize(np.zeros((0, 3), np.float32), 1.0, 0, "i8").shape == (0, 3)

@@ -375,6 +375,9 @@ namespace ngraph
                 void validate_and_infer_types() override;
                 size_t get_reduction_axes_count() const { return m_reduction_axes_count; }
                 const element::Type& get_output_type() const { return m_output_type; }
+                const AxisSet& get_input0_axes() const { return m_input0_axes; }
+                const AxisSet& get_input1_axes() const { return m_input1_axes; }
+                const AxisSet& get_output_axes() const { return m_output_axes; }
                 std::shared_ptr<Node> clone_with_new_inputs(const OutputVector& new_args) const override;
 
             private:

@@ -1,0 +1,174 @@
+"""Model ingress from the command line: `nbench` (nGraph's model benchmark tool: same options,
+data initialisation and timing protocol, src/tools/nbench/nbench.cpp:157-253, benchmark.cpp:87-185)
+and `reserialize` (src/tools/reserialize/reserialize.cpp) over the serialized graphs of
+tests/golden/serialized and, where the nGraph tree is at hand, over its own model files."""
+import glob
+import json
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HOST = os.path.join(ROOT, "ngraph_amd", "host")
+NBENCH = os.path.join(HOST, "nbench")
+RESERIALIZE = os.path.join(HOST, "reserialize")
+GOLDEN = os.path.join(ROOT, "tests", "golden", "serialized")
+SMALL = ["qconv_i32_output.json", "qdot_u8u8.json", "qdot_i32_output.json", "quantize_dequantize.json", "legacy_scale_subgraph.json"]
+
+
+def run(cmd, timeout=300):
+    print("[case]", " ".join(os.path.basename(c) if os.sep in c else c for c in cmd), flush=True)
+    p = subprocess.run(cmd, capture_output=True, text=True, timeout=timeout)
+    print(p.stdout[-4000:])
+    print(p.stderr[-2000:])
+    return p
+
+
+def renumbered(functions):
+    """A document independent of node numbering and of the order of independent ops: every node is
+    described by its op, its attributes and, recursively, its inputs; Parameters by their position in
+    the function's parameter list.  Friendly names (the file's names, added by a reader,
+    serializer.cpp:2594-2601) are dropped."""
+    out = []
+    for fn in functions:
+        nodes = {n["name"]: n for n in fn["ops"]}
+        memo = {}
+
+        def describe(name):
+            if name in memo:
+                return memo[name]
+            n = nodes[name]
+            attrs = {k: v for k, v in n.items() if k not in ("name", "outputs", "inputs", "friendly_name")}
+            if n["op"] == "Parameter":
+                attrs["position"] = fn["parameters"].index(name)
+            ins = []
+            for i in n.get("inputs", []):
+                ins.append(describe(i) if isinstance(i, str) else [describe(i["node"]), i["index"]])
+            memo[name] = json.dumps([attrs, ins], sort_keys=True)
+            return memo[name]
+
+        out.append(
+            {
+                "name": fn["name"],
+                "ops": sorted(describe(n["name"]) for n in fn["ops"]),
+                "result": [describe(r) for r in fn["result"]],
+                "outputs_follow_names": all(n.get("outputs", [n["name"] + "_0"])[0] == n["name"] + "_0" for n in fn["ops"]),
+            }
+        )
+    return out
+
+
+def test_tools_are_built():
+    assert os.path.exists(NBENCH) and os.path.exists(RESERIALIZE), "build the host first: make -C ngraph_amd/host"
+
+
+def test_nbench_usage_and_option_errors():
+    p = run([NBENCH])
+    assert p.returncode == 1 and "Either file or directory must be specified" in p.stdout and "SYNOPSIS" in p.stdout
+    p = run([NBENCH, "--bogus", "-f", os.path.join(GOLDEN, SMALL[0])])
+    assert p.returncode == 1 and "Unknown option: --bogus" in p.stdout
+    p = run([NBENCH, "-f", "/nonexistent/model.json", "-b", "HIP"])
+    assert p.returncode == 1 and "File /nonexistent/model.json not found" in p.stdout
+    p = run([NBENCH, "-f", os.path.join(GOLDEN, SMALL[0]), "-i", "many"])
+    assert p.returncode == 1 and "Invalid Argument" in p.stdout
+    p = run([NBENCH, "-f", os.path.join(GOLDEN, SMALL[0]), "--double_buffer"])
+    assert p.returncode == 1 and "not supported" in p.stdout
+
+
+def test_nbench_statistics_without_backend():
+    """-s alone loads the model and prints the graph statistics (nbench.cpp:343-429); no device"""
+    p = run([NBENCH, "-s", "-f", os.path.join(GOLDEN, "qconv_3x3_64ch_b128.json")])
+    assert p.returncode == 0
+    assert "Total nodes: 10" in p.stdout
+    assert "Total Constant size: 36879 bytes in 7 constants" in p.stdout  # 64*64*9 i8 + 3 f32 + 3 one-byte zero points
+    assert "Total Parameter size: 25690112 bytes in 1 parameters" in p.stdout
+    assert "QuantizedConvolution{128,64,56,56}: 1 ops" in p.stdout
+
+
+def test_nbench_directory_scan_reports_each_model():
+    p = run([NBENCH, "-s", "-d", GOLDEN])
+    assert p.returncode == 0
+    for f in SMALL:
+        assert "---- Processing '%s'" % os.path.join(GOLDEN, f) in p.stdout
+
+
+def test_nbench_unknown_backend_is_reported_not_fatal():
+    p = run([NBENCH, "-f", os.path.join(GOLDEN, SMALL[1]), "-b", "NO_SUCH_BACKEND"])
+    assert p.returncode == 1 and "Exception caught on" in p.stdout
+
+
+@pytest.mark.parametrize("name", SMALL + ["qconv_3x3_64ch_b128.json"])
+def test_reserialize_keeps_the_graph(name, tmp_path):
+    """read -> write gives the same JSON document (keys, values, order of ops) up to node numbering;
+    for the files in nGraph's current layout that is the golden file itself"""
+    src = os.path.join(GOLDEN, name)
+    once, twice = str(tmp_path / "once.json"), str(tmp_path / "twice.json")
+    assert run([RESERIALIZE, "-i", src, "-o", once]).returncode == 0
+    assert run([RESERIALIZE, "-i", once, "-o", twice, "--indent", "3"]).returncode == 0
+    a, b = json.load(open(once)), json.load(open(twice))
+    assert renumbered(a) == renumbered(b)
+    if not name.startswith("legacy"):
+        assert renumbered(json.load(open(src))) == renumbered(a)
+
+
+def test_reserialize_errors():
+    p = run([RESERIALIZE])
+    assert p.returncode == 1 and "input file missing" in p.stdout
+    p = run([RESERIALIZE, "-i", "/nonexistent.json", "-o", "/tmp/x.json"])
+    assert p.returncode == 2 and "failed to open" in p.stdout
+
+
+def test_reference_model_files_parse_or_name_the_op_outside_the_path(tmp_path):
+    """nGraph's own serialized models (float training / inference graphs, several generations of
+    the layout) all pass the JSON parser; each then either loads or stops at the first op that is
+    not part of the int8 path, with nGraph's message.  Runs where the nGraph tree exists."""
+    models = sorted(glob.glob("/root/reference/test/models/**/*.json", recursive=True))
+    if not models:
+        pytest.skip("no nGraph source tree at /root/reference")
+    loaded, stopped = 0, {}
+    for m in models:
+        if os.path.getsize(m) > 600000:
+            continue
+        p = subprocess.run([RESERIALIZE, "-i", m, "-o", str(tmp_path / "out.json")], capture_output=True, text=True, timeout=120)
+        assert "json parse error" not in p.stdout, (m, p.stdout[-300:])
+        if p.returncode == 0:
+            loaded += 1
+            continue
+        assert p.returncode == 3, (m, p.stdout[-300:])
+        hit = re.search(r"Error parsing json at node '([A-Za-z0-9_]+)': unsupported op ([A-Za-z]+):0", p.stdout)
+        assert hit, (m, p.stdout[-300:])
+        stopped[hit.group(2)] = stopped.get(hit.group(2), 0) + 1
+    print("loaded", loaded, "stopped at", stopped)
+    assert loaded + sum(stopped.values()) >= 30
+    # every op that stopped a file is one the int8 path has no use for
+    assert not set(stopped) & {"Parameter", "Constant", "Result", "Add", "Multiply", "Divide", "Broadcast", "Reshape", "Maximum", "Relu", "MaxPool", "AvgPool", "Concat", "Softmax", "Convert", "Abs"}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", SMALL)
+def test_nbench_runs_small_models_on_hip(name):
+    p = run([NBENCH, "-f", os.path.join(GOLDEN, name), "-b", "HIP", "-i", "3", "-w", "1", "--dump_results"])
+    assert p.returncode == 0
+    assert re.search(r"compile time: [0-9.e+-]+ms", p.stdout)
+    assert re.search(r"[0-9.e+-]+ms per iteration", p.stdout)
+    assert "Result 0 (" in p.stdout
+
+
+@pytest.mark.gpu
+def test_nbench_headline_layer_protocol():
+    """the 3x3 / 64-channel layer at batch 128 from its JSON file: with --no_copy_data an iteration
+    is one Executable::call (kernel + synchronisation), with copies it also moves 2 x 25.7 MB over
+    PCIe, so it is slower; --timing_detail lists the one op that does the work"""
+    model = os.path.join(GOLDEN, "qconv_3x3_64ch_b128.json")
+    p = run([NBENCH, "-f", model, "-b", "HIP", "-i", "20", "-w", "5", "--no_copy_data", "--timing_detail"])
+    assert p.returncode == 0
+    resident = float(re.search(r"([0-9.e+-]+)ms per iteration", p.stdout).group(1))
+    assert "QuantizedConvolution" in p.stdout and "---- Aggregate times per op type ----" in p.stdout
+    p = run([NBENCH, "-f", model, "-b", "HIP", "-i", "5", "-w", "2"])
+    assert p.returncode == 0
+    copied = float(re.search(r"([0-9.e+-]+)ms per iteration", p.stdout).group(1))
+    print("ms per iteration: resident %.4f, with copies %.4f" % (resident, copied))
+    assert resident < 1.0, "one call of the layer takes tens of microseconds on the device"
+    assert copied > resident

@@ -31,8 +31,8 @@ PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the headline kernel at batch 128: not measured by this run (counters need
 # a profiler run of their own) but quoted from the FETCH_SIZE / WRITE_SIZE runs summarised in the
 # file below (scaled by a 64 MiB copy in the same run); the JSON line names that file
-MEASURED_TRAFFIC_BYTES = {("conv_band_i8_32x32x32", 128): 52.3e6}
-TRAFFIC_SOURCE = "profiles/conv_band_config1_hbm_traffic.md"
+MEASURED_TRAFFIC_BYTES = {("conv_regw_i8_32x32x32", 128): 52.9e6, ("conv_band_i8_32x32x32", 128): 52.3e6}
+TRAFFIC_SOURCE = {"conv_regw_i8_32x32x32": "profiles/conv_regw_config1_batch128.md", "conv_band_i8_32x32x32": "profiles/conv_band_config1_hbm_traffic.md"}
 _DATA_CACHE = {}
 
 
@@ -531,7 +531,7 @@ def main():
             "unit": "TOP/s",
             "frac": kern["tops_event"] / PEAK_I8_TOPS,
             "traffic": MEASURED_TRAFFIC_BYTES.get((kern["kernel"], args.batch)),
-            "traffic_source": TRAFFIC_SOURCE + " (counter runs of this command; not measured by this run)",
+            "traffic_source": TRAFFIC_SOURCE.get(kern["kernel"], "none") + " (counter runs of this command; not measured by this run)",
             "algorithmic_bytes": 2 * args.batch * 64 * 56 * 56 + 64 * 64 * 9,
             "kernel_ms": kern["ms_event"],
         },

@@ -371,9 +371,16 @@ int hipq_capture_end(void* stream, void** graph_exec)
     HIPQ_HIP(hipStreamEndCapture(as_stream(stream), &graph));
     hipGraphExec_t exec = nullptr;
     hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-    (void)hipGraphDestroy(graph); // the executable graph keeps what it needs
+    hipError_t d = hipGraphDestroy(graph); // the executable graph keeps what it needs
     if (e != hipSuccess)
         return fail(HIPQ_ERR_HIP, "hipGraphInstantiate: %s", hipGetErrorString(e));
+    if (d != hipSuccess)
+    {
+        // a template graph that cannot be destroyed says the runtime's graph state is damaged:
+        // hand back no executable rather than one that may replay wrongly
+        (void)hipGraphExecDestroy(exec);
+        return fail(HIPQ_ERR_HIP, "hipGraphDestroy after instantiation: %s", hipGetErrorString(d));
+    }
     *graph_exec = exec;
     return HIPQ_OK;
 }

@@ -304,6 +304,30 @@ def bench_resnet50(lib, stream, timer, batches=(1, 32, 128), use_graph=True):
     return out
 
 
+def mfma_ceiling(lib, stream, timer, compute_units):
+    """What the matrix cores sustain with nothing in their way: every wavefront of a full-chip launch
+    issues one dependent chain of v_mfma_i32_32x32x32_i8 on operands it holds in registers (no memory,
+    no LDS, no other instructions).  The rate depends on the operand bytes -- the device lowers its
+    clock under the switching activity of dense data -- so it is measured for all-zero operands and
+    for the kind the convolution multiplies (random bytes)."""
+    iters, wgs = 400, int(compute_units)
+    sink = H.DeviceBuffer(wgs * 256 * 4)
+    out = {}
+    rng = np.random.default_rng(4001)
+    for kind, host in (("zero_bytes", np.zeros(8192, np.uint8)), ("random_bytes", rng.integers(0, 256, 8192, dtype=np.uint8))):
+        ops = dev(host)
+
+        def step():
+            rc = lib.hipq_probe_mfma_i8(ops.ptr, sink.ptr, wgs, iters, stream)
+            if rc:
+                H.check(rc)
+
+        _, ev = timer.run(step, 5, 2)
+        total = wgs * 4 * 64 * iters * 65536.0
+        out[kind] = dict(ms_event=ev, tops=total / (ev * 1e-3) / 1e12, frac_of_published_peak=total / (ev * 1e-3) / 1e12 / PEAK_I8_TOPS)
+    return out
+
+
 def copy_calibration(lib, stream, timer):
     """a plain device-to-device copy of known size: the yardstick for the FETCH_SIZE / WRITE_SIZE
     counters of a profiler run over this same command"""
@@ -484,6 +508,7 @@ def main():
 
     results = {"conv_nchw": [head], "conv_kernel_nhwc_in_nchw_out": [kern], "conv_nhwc_kernel": [nhwc]}
     results["copy_calibration"] = copy_calibration(lib, stream, timer)
+    results["mfma_ceiling_i8"] = mfma_ceiling(lib, stream, timer, info.compute_units)
     cpu = None
     if not args.quick:
         small = max(20, args.steps // 4)
@@ -534,6 +559,8 @@ def main():
             "traffic_source": TRAFFIC_SOURCE.get(kern["kernel"], "none") + " (counter runs of this command; not measured by this run)",
             "algorithmic_bytes": 2 * args.batch * 64 * 56 * 56 + 64 * 64 * 9,
             "kernel_ms": kern["ms_event"],
+            "measured_ceiling_random_bytes": results["mfma_ceiling_i8"]["random_bytes"]["tops"],
+            "frac_of_measured_ceiling": kern["tops_event"] / results["mfma_ceiling_i8"]["random_bytes"]["tops"],
         },
         "cpu_baseline": cpu,
         "results": results,

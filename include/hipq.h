@@ -97,6 +97,14 @@ HIPQ_API int hipq_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes, 
 HIPQ_API int hipq_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
 /* byte fill done by a kernel (not a memset node), safe to record into a HIP graph */
 HIPQ_API int hipq_fill_bytes(void* dst_dev, int value, size_t bytes, void* stream);
+/*
+ * Measurement aid with no counterpart in the reference: a full-chip launch of dependent
+ * v_mfma_i32_32x32x32_i8 chains on register-resident operands (`operands_8k`: 8 sets of 64 lanes x
+ * 16 bytes on the device; `sink`: workgroups x 256 ints).  Each of the workgroups' 4 wavefronts
+ * issues 64 x iters MFMAs of 65536 operations.  bench.py times it to report the matrix-core rate
+ * this device sustains for a given kind of operand bytes.
+ */
+HIPQ_API int hipq_probe_mfma_i8(const void* operands_8k, void* sink, int32_t workgroups, int32_t iters, void* stream);
 HIPQ_API int hipq_stream_create(void** stream);
 HIPQ_API int hipq_stream_destroy(void* stream);
 HIPQ_API int hipq_stream_sync(void* stream);

@@ -260,6 +260,7 @@ EXPORTS = [
     "hipq_memcpy_d2h",
     "hipq_memcpy_d2d",
     "hipq_fill_bytes",
+    "hipq_probe_mfma_i8",
     "hipq_stream_create",
     "hipq_stream_destroy",
     "hipq_stream_sync",
@@ -335,6 +336,7 @@ def load():
     for n in ("hipq_memcpy_h2d", "hipq_memcpy_d2h", "hipq_memcpy_d2d"):
         getattr(lib, n).argtypes = [vp, vp, C.c_size_t, vp]
     lib.hipq_fill_bytes.argtypes = [vp, C.c_int, C.c_size_t, vp]
+    lib.hipq_probe_mfma_i8.argtypes = [vp, vp, C.c_int32, C.c_int32, vp]
     lib.hipq_stream_create.argtypes = [C.POINTER(vp)]
     lib.hipq_stream_destroy.argtypes = [vp]
     lib.hipq_stream_sync.argtypes = [vp]

@@ -16,13 +16,28 @@ namespace hipq
     typedef int v4acc __attribute__((ext_vector_type(4)));
 
     // Requantization and store of one lane's finished outputs (column n, rows m[i]), with the
-    // policy and output kind resolved once instead of per element.
-    template <int COUNT, class RowOf, class AccOf>
-    __device__ __forceinline__ void skinny_finish(const Epilogue& epi, int32_t M, int32_t N, int n, RowOf row_of, AccOf acc_of, void* __restrict__ out)
+    // policy and output kind resolved once instead of per element.  The caller brings the scalars
+    // (ec) and its column's bias and scale: it asks memory for them before its main loop.
+    struct SkinnyColumn
     {
-        const EpiConst ec = epi_const(epi);
-        const float bias = (epi.mode == EPI_FUSED && epi.bias) ? static_cast<float>(epi.bias[n]) : 0.0f;
-        const float scale = (epi.mode == EPI_FUSED && epi.per_channel) ? epi.scale[n] : ec.scale;
+        EpiConst ec;
+        float bias, scale;
+        int32_t wsum;
+    };
+    __device__ __forceinline__ SkinnyColumn skinny_column(const Epilogue& epi, const int32_t* __restrict__ wsum, int n, int32_t N)
+    {
+        SkinnyColumn c;
+        c.ec = epi_const(epi);
+        const bool ok = n < N;
+        c.wsum = ok ? wsum[n] : 0;
+        c.bias = (epi.mode == EPI_FUSED && epi.bias && ok) ? static_cast<float>(epi.bias[n]) : 0.0f;
+        c.scale = (epi.mode == EPI_FUSED && epi.per_channel && ok) ? epi.scale[n] : c.ec.scale;
+        return c;
+    }
+    template <int COUNT, class RowOf, class AccOf>
+    __device__ __forceinline__ void skinny_finish(const Epilogue& epi, const EpiConst& ec, float bias, float scale, int32_t M, int32_t N, int n, RowOf row_of, AccOf acc_of,
+                                                  void* __restrict__ out)
+    {
         const bool relu = epi.relu != 0;
         auto run = [&](auto mode_c, auto kind_c) {
             constexpr int MODE = decltype(mode_c)::value;
@@ -82,11 +97,39 @@ namespace hipq
         const int r16 = lane & 15; // A: row within the m-tile, B: column within the n-tile
         const int kc = lane >> 4;  // 16-byte chunk of a 64-byte step
         const int n0 = blockIdx.x * 16;
+        const int xor_mask = x_unsigned ? static_cast<int>(0x80808080u) : 0;
+        const __amdgpu_buffer_rsrc_t ars = make_rsrc(a, static_cast<uint32_t>(M) * static_cast<uint32_t>(K));
+        const __amdgpu_buffer_rsrc_t wrs = make_rsrc(w, static_cast<uint32_t>(N) * static_cast<uint32_t>(K));
+        const int kq = ((K / 64 + 3) / 4) * 64; // bytes of K per wavefront, whole 64-byte steps
+        // (rotated by workgroup: in lockstep all workgroups would queue on the same activation lines in L2)
+        const int k_begin = ((wave + static_cast<int>(blockIdx.x)) & 3) * kq;
+        const int k_end = min(K, k_begin + kq);
+        const int32_t wrow = n0 + r16 < N ? (n0 + r16) * K + kc * 16 : kOob;
+        int32_t arow[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            arow[mt] = mt * 16 + r16 < M ? (mt * 16 + r16) * K + kc * 16 : kOob;
+        v4i bf[STEPS], af[MT][STEPS];
+        auto load = [&](int kb) {
+#pragma unroll
+            for (int st = 0; st < STEPS; ++st)
+            {
+                const int k = kb + st * 64;
+                bf[st] = buffer_load16(wrs, (wrow != kOob && k < k_end) ? wrow + k : kOob);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    af[mt][st] = buffer_load16(ars, (arow[mt] != kOob && k < k_end) ? arow[mt] + k : kOob);
+            }
+        };
+        // the weights and activations of the first steps are asked for before anything else; the
+        // scalars and this lane's column constants (needed at the very end) right behind them
+        load(k_begin);
         const int32_t xzp = load_zp(zp.data_zp, zp.data_t);
         const int32_t wzp = load_zp(zp.filter_zp, zp.filter_t);
-        const EpiRegs er = epi_load(epi);
+        const SkinnyColumn col = skinny_column(epi, wsum, n0 + r16, N);
         if (wzp != 0) // uniform; w - wzp does not fit a signed byte: exact, slow
         {
+            const EpiRegs er = epi_load(epi);
             for (int i = tid; i < 16 * M; i += 256)
             {
                 const int m = i >> 4, n = n0 + (i & 15);
@@ -105,18 +148,6 @@ namespace hipq
             }
             return;
         }
-        const int xor_mask = x_unsigned ? static_cast<int>(0x80808080u) : 0;
-        const __amdgpu_buffer_rsrc_t ars = make_rsrc(a, static_cast<uint32_t>(M) * static_cast<uint32_t>(K));
-        const __amdgpu_buffer_rsrc_t wrs = make_rsrc(w, static_cast<uint32_t>(N) * static_cast<uint32_t>(K));
-        const int kq = ((K / 64 + 3) / 4) * 64; // bytes of K per wavefront, whole 64-byte steps
-        // (rotated by workgroup: in lockstep all workgroups would queue on the same activation lines in L2)
-        const int k_begin = ((wave + static_cast<int>(blockIdx.x)) & 3) * kq;
-        const int k_end = min(K, k_begin + kq);
-        const int32_t wrow = n0 + r16 < N ? (n0 + r16) * K + kc * 16 : kOob;
-        int32_t arow[MT];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-            arow[mt] = mt * 16 + r16 < M ? (mt * 16 + r16) * K + kc * 16 : kOob;
 
         v4acc acc[MT];
 #pragma unroll
@@ -124,16 +155,8 @@ namespace hipq
             acc[mt] = v4acc{0, 0, 0, 0};
         for (int kb = k_begin; kb < k_end; kb += 64 * STEPS)
         {
-            v4i bf[STEPS], af[MT][STEPS];
-#pragma unroll
-            for (int st = 0; st < STEPS; ++st)
-            {
-                const int k = kb + st * 64;
-                bf[st] = buffer_load16(wrs, (wrow != kOob && k < k_end) ? wrow + k : kOob);
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-                    af[mt][st] = buffer_load16(ars, (arow[mt] != kOob && k < k_end) ? arow[mt] + k : kOob);
-            }
+            if (kb != k_begin)
+                load(kb);
 #pragma unroll
             for (int st = 0; st < STEPS; ++st)
 #pragma unroll
@@ -160,10 +183,10 @@ namespace hipq
         const int n = n0 + r16;
         if (n >= N)
             return;
-        const int32_t corr = ((x_unsigned ? 128 : 0) - xzp) * wsum[n];
+        const int32_t corr = ((x_unsigned ? 128 : 0) - xzp) * col.wsum;
         // lane: column lane % 16; accumulator register r is row 4 * (lane / 16) + r of the tile
         skinny_finish<MT * 4>(
-            epi, M, N, n, [&](int i) { return (i >> 2) * 16 + 4 * kc + (i & 3); },
+            epi, col.ec, col.bias, col.scale, M, N, n, [&](int i) { return (i >> 2) * 16 + 4 * kc + (i & 3); },
             [&](int i) { return acc[i >> 2][i & 3] + red[0][i >> 2][i & 3][lane] + red[1][i >> 2][i & 3][lane] + red[2][i >> 2][i & 3][lane] + corr; }, out);
     }
 
@@ -191,29 +214,6 @@ namespace hipq
         const int r16 = lane & 15;
         const int kc = lane >> 4;
         const int n0 = blockIdx.x * 16;
-        const int32_t xzp = load_zp(zp.data_zp, zp.data_t);
-        const int32_t wzp = load_zp(zp.filter_zp, zp.filter_t);
-        const EpiRegs er = epi_load(epi);
-        if (wzp != 0) // uniform; exact, slow
-        {
-            for (int i = tid; i < 16 * M; i += 256)
-            {
-                const int m = i >> 4, n = n0 + (i & 15);
-                if (n < N)
-                {
-                    int32_t acc = 0;
-                    for (int k = 0; k < K; ++k)
-                    {
-                        const int32_t xv = x_unsigned ? static_cast<int32_t>(a[static_cast<int64_t>(m) * K + k])
-                                                      : static_cast<int32_t>(static_cast<int8_t>(a[static_cast<int64_t>(m) * K + k]));
-                        acc += (xv - xzp) * (static_cast<int32_t>(w[static_cast<int64_t>(n) * K + k]) - wzp);
-                    }
-                    const int64_t o = static_cast<int64_t>(m) * N + n;
-                    store_out(out, epi.out_t, o, epi_apply(epi, er, acc, n, o));
-                }
-            }
-            return;
-        }
         const int xor_mask = x_unsigned ? static_cast<int>(0x80808080u) : 0;
         const __amdgpu_buffer_rsrc_t ars = make_rsrc(a, static_cast<uint32_t>(M) * static_cast<uint32_t>(K));
         const __amdgpu_buffer_rsrc_t wrs = make_rsrc(w, static_cast<uint32_t>(N) * static_cast<uint32_t>(K));
@@ -259,6 +259,31 @@ namespace hipq
 #pragma unroll
         for (int d = 0; d < D; ++d)
             load_a(piece_k(0), d, af[d]);
+        // (the scalars and this lane's column constants are asked for behind the first fragments)
+        const int32_t xzp = load_zp(zp.data_zp, zp.data_t);
+        const int32_t wzp = load_zp(zp.filter_zp, zp.filter_t);
+        const SkinnyColumn col = skinny_column(epi, wsum, n0 + r16, N);
+        if (wzp != 0) // uniform; exact, slow
+        {
+            const EpiRegs er = epi_load(epi);
+            for (int i = tid; i < 16 * M; i += 256)
+            {
+                const int m = i >> 4, n = n0 + (i & 15);
+                if (n < N)
+                {
+                    int32_t acc = 0;
+                    for (int k = 0; k < K; ++k)
+                    {
+                        const int32_t xv = x_unsigned ? static_cast<int32_t>(a[static_cast<int64_t>(m) * K + k])
+                                                      : static_cast<int32_t>(static_cast<int8_t>(a[static_cast<int64_t>(m) * K + k]));
+                        acc += (xv - xzp) * (static_cast<int32_t>(w[static_cast<int64_t>(n) * K + k]) - wzp);
+                    }
+                    const int64_t o = static_cast<int64_t>(m) * N + n;
+                    store_out(out, epi.out_t, o, epi_apply(epi, er, acc, n, o));
+                }
+            }
+            return;
+        }
         for (int c = 0; c < pieces; ++c)
         {
             const int kb = piece_k(c), kb_next = piece_k(c + 1);
@@ -298,11 +323,236 @@ namespace hipq
         const int n = n0 + r16;
         if (n >= N)
             return;
-        const int32_t corr = ((x_unsigned ? 128 : 0) - xzp) * wsum[n];
+        const int32_t corr = ((x_unsigned ? 128 : 0) - xzp) * col.wsum;
         // lane: column lane % 16; accumulator register r is row 4 * (lane / 16) + r of the tile
         skinny_finish<MT * 4>(
-            epi, M, N, n, [&](int i) { return (i >> 2) * 16 + 4 * kc + (i & 3); },
+            epi, col.ec, col.bias, col.scale, M, N, n, [&](int i) { return (i >> 2) * 16 + 4 * kc + (i & 3); },
             [&](int i) { return acc[i >> 2][i & 3] + red[0][i >> 2][i & 3][lane] + red[1][i >> 2][i & 3][lane] + red[2][i >> 2][i & 3][lane] + corr; }, out);
+    }
+
+    // Between the skinny kernels and the tile kernels: a few hundred rows against a weight matrix that
+    // must stream from HBM once (config 2 at 256 rows).  The tile kernels would have too few 128 x 128
+    // tiles for the chip and split each reduction over workgroups, which costs a round trip of partial
+    // sums through memory.  Here a workgroup owns a 64 x 64 output tile and the WHOLE reduction: its
+    // eight wavefronts split K eight ways (128-byte pieces dealt round robin).  A wavefront brings
+    // its piece of the 64 activation rows and the 64 weight rows straight into a 16 KB LDS region of
+    // its own -- every load instruction is 8 rows x 128 bytes, eight whole cache lines (loads shaped
+    // like an MFMA fragment, 16 rows x 64 bytes, run at less than half the rate) -- and reads the
+    // v_mfma_i32_16x16x64_i8 fragments back 16 bytes a lane; the next piece is on its way while this
+    // one multiplies.  No barrier in the loop: nothing is shared between wavefronts until the
+    // eight partial tiles meet in LDS (each in its wavefront's region), after which every wavefront
+    // requantizes two 16 x 16 blocks.  Everything the epilogue needs from memory (zero points,
+    // scales, bias, weight sums) is asked for before the loop.  Workgroups of one compute die share
+    // a run of column tiles, so each die's L2 fetches its part of the weights from HBM once.
+    constexpr int kRows64Threads = 512;
+    constexpr size_t kRows64Lds = 8 * 16384;
+
+    __global__ __launch_bounds__(kRows64Threads) void dot_rows64_kernel(const uint8_t* __restrict__ a,
+                                                                        const int8_t* __restrict__ w,
+                                                                        const int32_t* __restrict__ wsum,
+                                                                        int32_t M,
+                                                                        int32_t N,
+                                                                        int32_t K,
+                                                                        int32_t tiles_m,
+                                                                        int32_t x_unsigned,
+                                                                        ZeroPoints zp,
+                                                                        Epilogue epi,
+                                                                        void* __restrict__ out)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int r16 = lane & 15;
+        const int kc = lane >> 4;
+        // workgroups are dealt round robin to the eight compute dies: renumber so that a die's
+        // workgroups are consecutive tiles (row tiles of one column tile next to each other)
+        const int grid = static_cast<int>(gridDim.x);
+        const int id = (grid & 7) == 0 ? (static_cast<int>(blockIdx.x) & 7) * (grid >> 3) + (static_cast<int>(blockIdx.x) >> 3) : static_cast<int>(blockIdx.x);
+        const int ct = id / tiles_m, rt = id - ct * tiles_m;
+        const int m0 = rt * 64, n0 = ct * 64;
+        const v4i arsw = rsrc_words(a, static_cast<uint32_t>(M) * static_cast<uint32_t>(K));
+        const v4i wrsw = rsrc_words(w, static_cast<uint32_t>(N) * static_cast<uint32_t>(K));
+        // One load instruction brings 8 rows x 128 bytes (eight whole cache lines) into a 1 KB block of
+        // this wavefront's 16 KB region: [A, B][block of 8 rows][64 pieces of 16 bytes].  Which piece
+        // (row rho, chunk c of the 128 bytes) a lane fetches decides where it lands (at 16 * lane), so
+        // the block's order is free: piece (rho, c) sits at 16 * (c / 2) + 8 * ((c % 2) ^ (block % 2)) + rho,
+        // which makes the fragment reads below conflict-free (16 lanes of one chunk index read rows of
+        // an even and an odd block from 16 different 16-byte columns).
+        const int rho = lane & 7;
+        int32_t arow[8], wrow[8];
+#pragma unroll
+        for (int blk = 0; blk < 8; ++blk)
+        {
+            const int c = 2 * (lane >> 4) + (((lane >> 3) & 1) ^ (blk & 1));
+            arow[blk] = m0 + blk * 8 + rho < M ? (m0 + blk * 8 + rho) * K + c * 16 : kOob;
+            wrow[blk] = n0 + blk * 8 + rho < N ? (n0 + blk * 8 + rho) * K + c * 16 : kOob;
+        }
+        uint8_t* const mine = lds + wave * 16384;
+        const uint32_t ring = lds_address(mine);
+        auto issue = [&](int pc) {
+            const int k = pc * 128;
+#pragma unroll
+            for (int blk = 0; blk < 8; ++blk)
+            {
+                // (K is a multiple of 64: a chunk of the second half of the last piece may be past the end)
+                const int c16 = (2 * (lane >> 4) + (((lane >> 3) & 1) ^ (blk & 1))) * 16;
+                const bool in_k = k + c16 < K;
+                lds_dma16(wrsw, (in_k && wrow[blk] != kOob) ? wrow[blk] + k : kOob, ring + 8192 + blk * 1024);
+                lds_dma16(arsw, (in_k && arow[blk] != kOob) ? arow[blk] + k : kOob, ring + blk * 1024);
+            }
+        };
+        // fragment (16-row block i, 64-byte half h) of lane (row r16, chunk kc): at frag0 + 2048 i + 512 h
+        const int frag0 = (r16 >> 3) * 1024 + (16 * (kc >> 1) + 8 * ((kc & 1) ^ (r16 >> 3)) + (r16 & 7)) * 16;
+        // wavefront v takes pieces v, v + 8, ... (rotated by workgroup: in lockstep all workgroups of
+        // a row tile would queue on the same activation lines in L2)
+        const int pieces = (K + 127) >> 7;
+        const int first = (wave + id) & 7;
+        if (first < pieces) // uniform
+            issue(first);
+
+        // what the epilogue needs, asked for now: two blocks (i, j) = (blk / 4, blk % 4) a wavefront
+        const int32_t xzp = load_zp(zp.data_zp, zp.data_t);
+        const int32_t wzp = load_zp(zp.filter_zp, zp.filter_t);
+        const EpiConst ec = epi_const(epi);
+        int32_t col_wsum[2];
+        float col_bias[2], col_scale[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+        {
+            const int n = n0 + ((wave * 2 + b) & 3) * 16 + r16;
+            const bool ok = n < N;
+            col_wsum[b] = ok ? wsum[n] : 0;
+            col_bias[b] = (epi.mode == EPI_FUSED && epi.bias && ok) ? static_cast<float>(epi.bias[n]) : 0.0f;
+            col_scale[b] = (epi.mode == EPI_FUSED && epi.per_channel && ok) ? epi.scale[n] : ec.scale;
+        }
+        if (wzp != 0) // uniform; w - wzp does not fit a signed byte: exact, slow
+        {
+            wait_vmcnt<0>(); // nothing may still be on its way into LDS when the wavefront ends
+            const EpiRegs er = epi_load(epi);
+            for (int i = tid; i < 64 * 64; i += kRows64Threads)
+            {
+                const int m = m0 + (i >> 6), n = n0 + (i & 63);
+                if (m < M && n < N)
+                {
+                    int32_t acc = 0;
+                    for (int k = 0; k < K; ++k)
+                    {
+                        const int32_t xv = x_unsigned ? static_cast<int32_t>(a[static_cast<int64_t>(m) * K + k])
+                                                      : static_cast<int32_t>(static_cast<int8_t>(a[static_cast<int64_t>(m) * K + k]));
+                        acc += (xv - xzp) * (static_cast<int32_t>(w[static_cast<int64_t>(n) * K + k]) - wzp);
+                    }
+                    const int64_t o = static_cast<int64_t>(m) * N + n;
+                    store_out(out, epi.out_t, o, epi_apply(epi, er, acc, n, o));
+                }
+            }
+            return;
+        }
+        const int xor_mask = x_unsigned ? static_cast<int>(0x80808080u) : 0;
+        v4acc acc[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[i][j] = v4acc{0, 0, 0, 0};
+        for (int pc = first; pc < pieces; pc += 8)
+        {
+            wait_vmcnt<0>(); // the piece has landed
+            v4i x[2][4], bf[2][4];
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                {
+                    // out-of-range fragments read zeros; a zero weight fragment cancels whatever the
+                    // sign bias makes of a zero activation fragment
+                    const v4i t = *reinterpret_cast<const v4i*>(mine + frag0 + i * 2048 + h * 512);
+                    x[h][i] = v4i{t[0] ^ xor_mask, t[1] ^ xor_mask, t[2] ^ xor_mask, t[3] ^ xor_mask};
+                    bf[h][i] = *reinterpret_cast<const v4i*>(mine + 8192 + frag0 + i * 2048 + h * 512);
+                }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the region is in registers: the next piece may overwrite it
+            if (pc + 8 < pieces) // uniform
+                issue(pc + 8);
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(x[h][i], bf[h][j], acc[i][j], 0, 0, 0);
+        }
+        // ---- the eight partial tiles meet in LDS (each in its wavefront's region); every wavefront
+        // finishes two 16 x 16 blocks --------------------------------------------------------------------
+        v4acc* const red = reinterpret_cast<v4acc*>(lds);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                red[(wave * 16 + i * 4 + j) * 64 + lane] = acc[i][j];
+        __syncthreads();
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+        {
+            const int blk = wave * 2 + b;
+            v4acc sum = red[blk * 64 + lane];
+#pragma unroll
+            for (int v = 1; v < 8; ++v)
+            {
+                const v4acc t = red[(v * 16 + blk) * 64 + lane];
+                sum = v4acc{sum[0] + t[0], sum[1] + t[1], sum[2] + t[2], sum[3] + t[3]};
+            }
+            const int n = n0 + (blk & 3) * 16 + r16;
+            if (n >= N)
+                continue;
+            const int32_t corr = ((x_unsigned ? 128 : 0) - xzp) * col_wsum[b];
+            const int mb = m0 + (blk >> 2) * 16 + 4 * kc;
+            // lane: column lane % 16; accumulator register r is row 4 * (lane / 16) + r of the block
+            skinny_finish<4>(
+                epi, ec, col_bias[b], col_scale[b], M, N, n, [&](int i) { return mb + i; }, [&](int i) { return sum[i] + corr; }, out);
+        }
+    }
+
+    static int rows64_cus()
+    {
+        static int cus[16] = {};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16)
+            return 256;
+        if (cus[dev] == 0)
+        {
+            hipDeviceProp_t prop;
+            cus[dev] = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        }
+        return cus[dev];
+    }
+
+    // More than 64 rows, a long reduction, and too few 128 x 128 tiles to give every compute unit one
+    // without splitting reductions; at most two rounds of 64 x 64 tiles.
+    static bool dot_rows64_eligible(const hipq_dot_desc_t& d)
+    {
+        if (getenv("HIPQ_NO_ROWS64") != nullptr || d.M <= 64 || d.K % 64 != 0 || d.K < 1024)
+            return false;
+        const int64_t tiles64 = ((d.M + 63) / 64) * ((d.N + 63) / 64);
+        const int64_t tiles128 = ((d.M + 127) / 128) * ((d.N + 127) / 128);
+        const int cus = rows64_cus();
+        return tiles128 * 4 < 3 * cus && tiles64 <= 2 * cus && d.M * d.K < (1ll << 31) && d.N * d.K < (1ll << 31);
+    }
+
+    static int launch_rows64(const hipq_dot_desc_t& d, const void* a, const void* w_nk, const int32_t* wsum, const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s)
+    {
+        static bool configured[16] = {};
+        int dev = 0;
+        HIPQ_HIP(hipGetDevice(&dev));
+        if (dev >= 0 && dev < 16 && !configured[dev])
+        {
+            HIPQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dot_rows64_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kRows64Lds)));
+            configured[dev] = true;
+        }
+        const int32_t tiles_m = static_cast<int32_t>((d.M + 63) / 64);
+        const unsigned grid = static_cast<unsigned>(tiles_m * ((d.N + 63) / 64));
+        dot_rows64_kernel<<<grid, kRows64Threads, kRows64Lds, s>>>(static_cast<const uint8_t*>(a), static_cast<const int8_t*>(w_nk), wsum, static_cast<int32_t>(d.M),
+                                                                  static_cast<int32_t>(d.N), static_cast<int32_t>(d.K), tiles_m, d.a_t == HIPQ_U8 ? 1 : 0, zp, epi, out);
+        return check_launch("dot_rows64_i8_16x16x64");
     }
 
     static bool dot_skinny_eligible(const hipq_dot_desc_t& d)
@@ -383,6 +633,8 @@ namespace hipq
                 return launch_skinny<2, 16>(d, a, w_nk, wsum, zp, epi, out, s);
             if (d.M <= 64)
                 return launch_skinny<4, 8>(d, a, w_nk, wsum, zp, epi, out, s);
+            if (dot_rows64_eligible(d))
+                return launch_rows64(d, a, w_nk, wsum, zp, epi, out, s);
             // above 64 rows an 8-bit or (fused policy) float output is faster on the tile kernels,
             // whose reductions are split over workgroups when the tiles are few (config 2, 256 rows:
             // 22 us against 44)

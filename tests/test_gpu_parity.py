@@ -733,7 +733,7 @@ def test_dot_mfma_vs_oracle(gpu_lib, M):
         d = H.make_dot_desc(M, K, N, out_t=out_t)
         exp = O.quantized_dot(d, a, b, s[0], z[0], s[1], z[1], s[2], z[2])
         got = H.quantized_dot(d, a, b, s[0], z[0], s[1], z[1], s[2], z[2])
-        assert H.last_kernel().startswith(("dot_mfma", "dot_skinny")), H.last_kernel()
+        assert H.last_kernel().startswith(("dot_mfma", "dot_skinny", "dot_rows64")), H.last_kernel()
         assert np.array_equal(got, exp), (out_t, z)
     O.port().orc_set_threads(1)
 
@@ -771,14 +771,14 @@ def test_dot_bias_config2_shape(gpu_lib, M):
         f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
         exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
         got = H.quantized_dot_bias(d, f, a, w, bias, scales)
-        assert H.last_kernel().startswith(("dot_mfma", "dot_skinny")), H.last_kernel()
+        assert H.last_kernel().startswith(("dot_mfma", "dot_skinny", "dot_rows64")), H.last_kernel()
         assert np.array_equal(got, exp), (out_t, relu)
         assert len(np.unique(exp)) > 20  # the case is not degenerate (all saturated)
     O.port().orc_set_threads(1)
 
 
 @pytest.mark.parametrize("shape", [(200, 192, 144), (130, 4096, 64), (333, 768, 272), (4096, 64, 128)])
-def test_dot_bias_f32_tiles(gpu_lib, shape):
+def test_dot_bias_f32_tiles(gpu_lib, shape, monkeypatch):
     """float outputs of QuantizedDotBias through the tile kernels: ragged row and column tiles, a
     long reduction that is split over workgroups, a single-slice reduction; small biases (added to
     the accumulators as integers) and one beyond 2^24 (kept as a float add); with and without relu"""
@@ -798,8 +798,16 @@ def test_dot_bias_f32_tiles(gpu_lib, shape):
                 f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
                 exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
                 got = H.quantized_dot_bias(d, f, a, w, bias, scales)
-                assert H.last_kernel().startswith("dot_mfma"), H.last_kernel()
+                # (up to 256 rows with a long reduction and few tiles: one workgroup per 64 x 64 tile, whole reduction)
+                rows64 = 64 < M <= 256 and K >= 1024
+                assert H.last_kernel().startswith("dot_rows64" if rows64 else "dot_mfma"), H.last_kernel()
                 assert np.array_equal(got.view(np.uint32), exp.view(np.uint32)), (a_t, big_bias, relu)
+                if rows64:
+                    monkeypatch.setenv("HIPQ_NO_ROWS64", "1")
+                    got = H.quantized_dot_bias(d, f, a, w, bias, scales)
+                    monkeypatch.delenv("HIPQ_NO_ROWS64")
+                    assert H.last_kernel().startswith("dot_mfma"), H.last_kernel()
+                    assert np.array_equal(got.view(np.uint32), exp.view(np.uint32)), (a_t, big_bias, relu, "tiles")
     O.port().orc_set_threads(1)
 
 
@@ -862,7 +870,7 @@ def test_dot_config2_full_size_properties(gpu_lib):
     w = synth.uniform_int(96, (N, K), -127, 127, np.int8)
     d = H.make_dot_desc(256, K, N, out_t="i32", b_layout=H.B_NK)
     got = H.quantized_dot(d, a, w, 1.0, 0, 1.0, 0, 1.0, 0)
-    assert H.last_kernel().startswith(("dot_mfma", "dot_skinny")), H.last_kernel()
+    assert H.last_kernel().startswith("dot_rows64"), H.last_kernel()
     rows = [0, 1, 31, 32, 127, 128, 255]
     exp = a[rows].astype(np.int64) @ w.astype(np.int64).T
     assert np.array_equal(got[rows].astype(np.int64), exp)
@@ -895,8 +903,8 @@ def test_dot_bias_config2_benchmarked_form(gpu_lib, M):
         exp = cases.dot_bias_closed_form(a, w, bias, scales, out_t, relu)
         assert np.array_equal(got, exp), (out_t, relu, kernel, int(np.sum(got != exp)))
         if out_t == "i8":
-            # the kernels bench.py's gemm_config2 entries name: weight-streaming up to 64 rows, MFMA tiles above
-            assert kernel == ("dot_skinny_i8_16x16x64" if M <= 64 else "dot_mfma_i8_32x32x32"), kernel
+            # the kernels bench.py's gemm_config2 entries name: weight-streaming up to 64 rows, 64 x 64 tiles with the whole reduction above
+            assert kernel == ("dot_skinny_i8_16x16x64" if M <= 64 else "dot_rows64_i8_16x16x64"), kernel
             assert len(np.unique(exp)) > 100 and (exp == 127).any() and (exp == -128).any()
 
 
@@ -917,7 +925,8 @@ def test_dot_skinny(gpu_lib, M):
                 got = H.quantized_dot(d, a, w, s[0], z[0], s[1], z[1], s[2], z[2])
                 # (more than 64 rows with an 8-bit output in whole 16-byte rows go to the tile kernels)
                 tiles = M > 64 and out_t != "i32" and N % 16 == 0
-                assert H.last_kernel().startswith("dot_mfma" if tiles else "dot_skinny"), H.last_kernel()
+                rows64 = M > 64 and K >= 1024
+                assert H.last_kernel().startswith("dot_rows64" if rows64 else "dot_mfma" if tiles else "dot_skinny"), H.last_kernel()
                 assert np.array_equal(got, exp), (K, N, a_t, out_t, z)
             bias = synth.uniform_int(803, (N,), -(2**15), 2**15, np.int32)
             scales = synth.uniform_f32(804, (N,), 0.001, 0.01) * np.float32(0.05)
@@ -927,7 +936,8 @@ def test_dot_skinny(gpu_lib, M):
                 exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
                 got = H.quantized_dot_bias(d, f, a, w, bias, scales)
                 tiles = M > 64 and N % 16 == 0
-                assert H.last_kernel().startswith("dot_mfma" if tiles else "dot_skinny"), H.last_kernel()
+                rows64 = M > 64 and K >= 1024
+                assert H.last_kernel().startswith("dot_rows64" if rows64 else "dot_mfma" if tiles else "dot_skinny"), H.last_kernel()
                 assert np.array_equal(got, exp), (K, N, a_t, out_t, relu)
     O.port().orc_set_threads(1)
 

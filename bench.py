@@ -507,6 +507,10 @@ def main():
     nhwc = bench_conv(lib, stream, timer, args.batch, args.steps, args.warmup, H.NXC)
 
     results = {"conv_nchw": [head], "conv_kernel_nhwc_in_nchw_out": [kern], "conv_nhwc_kernel": [nhwc]}
+    # when the headline call is a single launch (the kernel that reads NCHW itself), its own HIP-event
+    # time per step is the dominant kernel's launch duration
+    if head["kernel"] == kern["kernel"] and head["kernel"].startswith("conv_regw"):
+        kern = head
     results["copy_calibration"] = copy_calibration(lib, stream, timer)
     results["mfma_ceiling_i8"] = mfma_ceiling(lib, stream, timer, info.compute_units)
     cpu = None

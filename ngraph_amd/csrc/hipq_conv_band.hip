@@ -78,6 +78,10 @@ extern "C" HIPQ_API int hipq_debug_band_phases(long long* out32)
 namespace hipq
 {
     constexpr int kBandC = 64;           // input channels (bytes per pixel slot)
+    // Output stores carry the device-scope bit (sc1): written through to the memory side as they are
+    // issued instead of sitting dirty in the compute dies' L2s until the write-back that ends the
+    // kernel (batch 128, channels-last: 26.1 -> 23.1 us).
+    constexpr int kBandStoreScope = 16;
     constexpr int kBandGroupThreads = 256; // a group: four wavefronts, one per SIMD
     constexpr int kBandStagePitch = 144; // NCHW staging: bytes per channel row (128 pixels + pad, 16-byte multiple)
     constexpr int kBandStageWave = 64 * kBandStagePitch; // 9216 bytes per wavefront
@@ -784,7 +788,7 @@ namespace hipq
                             const int part = h * T + id % T;
                             const int band0 = (img * p.K) * static_cast<int>(p.PQ) + p0 * p.Q + gw * (32 * T);
                             const bool ok = (ch < p.K) & (gw * (32 * T) + part * 16 < npix);
-                            __builtin_amdgcn_raw_buffer_store_b128(piece[j], ors, ok ? band0 + ch * static_cast<int>(p.PQ) + part * 16 : kOob, 0, 0);
+                            __builtin_amdgcn_raw_buffer_store_b128(piece[j], ors, ok ? band0 + ch * static_cast<int>(p.PQ) + part * 16 : kOob, 0, kBandStoreScope);
                         }
                         else
                         {
@@ -792,7 +796,7 @@ namespace hipq
                             const int part = id & 3;
                             const int band0 = (img * static_cast<int>(p.PQ) + p0 * p.Q + gw * (32 * T)) * p.K;
                             const bool ok = (gw * (32 * T) + px < npix) & (part * 16 < p.K);
-                            __builtin_amdgcn_raw_buffer_store_b128(piece[j], ors, ok ? band0 + px * p.K + part * 16 : kOob, 0, 0);
+                            __builtin_amdgcn_raw_buffer_store_b128(piece[j], ors, ok ? band0 + px * p.K + part * 16 : kOob, 0, kBandStoreScope);
                         }
                     }
                 };

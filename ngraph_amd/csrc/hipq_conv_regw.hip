@@ -47,9 +47,14 @@ extern "C" HIPQ_API int hipq_debug_regw_clocks(long long* out512)
 namespace hipq
 {
     constexpr int kRwThreads = 512;
-    constexpr int kRwRoundRows = 4; // band rows per load round of the four loader wavefronts
+    constexpr int kRwRoundRows = 4; // band rows per load round
+    // (measured at batch 128: two loaders 21.3 us, four 20.6; 2 / 4 / 8 rounds in flight 20.35 / 20.1 / 21.3 us --
+    // a deeper queue delays the first rounds, which the multiplying wavefronts are waiting for)
+    constexpr int kRwLoaders = 4;               // wavefronts that start as loaders (the last ones of the workgroup)
+    constexpr int kRwGroups = 4 / kRwLoaders;   // 16-channel groups (NCHW) or piece quarters (NHWC) a loader brings per round
+    constexpr int kRwMulThreads = (8 - kRwLoaders) * 64; // lanes of the wavefronts that multiply from the start
     constexpr int kRwMaxRounds = 24;
-    constexpr int kRwDepth = 4;    // rounds of loads a loader keeps in flight
+    constexpr int kRwDepth = 4;     // rounds of loads a loader keeps in flight
     constexpr int kRwAhead = 3;     // pixel fragments on their way from LDS while a tile multiplies and the previous one requantizes
     constexpr int kRwKred = 576;    // 9 taps x 64 channels
     // Output stores carry the device-scope bit (sc1): they are written through to the memory side as
@@ -79,12 +84,17 @@ namespace hipq
     // where (slot / 8) is odd, which spreads 16 consecutive slots over all 64 banks.
     __device__ __forceinline__ int regw_cell(int slot, int chunk) { return slot * 32 + (((chunk ^ (slot >> 3)) & 1) << 4); }
 
+    // bytes of one LDS plane for a band of `rows` output rows of a layer `w` pixels wide
+    // (= 128 mod 256, so that the two planes use different banks)
+    __host__ __device__ constexpr int regw_plane_bytes(int w, int rows) { return ((rows + 2) * ((w + 2) * 32 + 16) + 255) / 256 * 256 + 128; }
+    constexpr int kRwMaxRowsCT = 28; // band rows the compile-time geometry leaves room for (56-wide layers: 2 x 56448 + 36864 bytes)
+
     struct RegwRaw
     {
         int v[16];
     };
 
-    template <int MODE, bool IN_NCX, bool SUM>
+    template <int MODE, bool IN_NCX, bool SUM, int WCT>
     __global__ __launch_bounds__(kRwThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_regw_kernel(RegwParams p,
                                                                                                                const int8_t* __restrict__ w,
                                                                                                                const int32_t* __restrict__ wsum,
@@ -99,6 +109,13 @@ namespace hipq
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const int half = lane >> 5;
         const int l32 = lane & 31;
+        // WCT != 0: a layer WCT pixels wide with the LDS geometry fixed at compile time, so that every
+        // fragment address is a per-lane base plus an immediate offset (no address arithmetic between
+        // the MFMAs); WCT == 0: any width, geometry from the parameters
+        const int W_ = WCT ? WCT : p.W;
+        const int pitch = WCT ? (WCT + 2) * 32 + 16 : p.pitch;
+        const int plane = WCT ? regw_plane_bytes(WCT, kRwMaxRowsCT) : p.plane_bytes;
+        auto div_w = [&](int v) { return WCT ? static_cast<int>(static_cast<uint32_t>(v) / static_cast<uint32_t>(WCT ? WCT : 1)) : static_cast<int>(p.div_w.div(static_cast<uint32_t>(v))); };
 
         // ---- which band ----------------------------------------------------------------------------
         // workgroups are dealt round-robin to the 8 XCDs (an L2 each): renumbered so that the bands of
@@ -109,8 +126,8 @@ namespace hipq
         const int h0 = (item - img * p.bands) * p.TP;
         const int rows = p.TP;
         const int band_rows = rows + 2;
-        const int npix = rows * p.W;
-        const int PQ = p.H * p.W;
+        const int npix = rows * W_;
+        const int PQ = p.H * W_;
 
         HIPQ_RW_MARK(0);
 #ifdef HIPQ_REGW_CLOCKS
@@ -119,8 +136,8 @@ namespace hipq
 #endif
         const __amdgpu_buffer_rsrc_t xrs = make_rsrc(p.x, p.x_bytes);
         const __amdgpu_buffer_rsrc_t ors = make_rsrc(out, p.out_bytes);
-        const bool loader = wave >= 4; // uniform
-        const int lw = wave & 3;
+        const bool loader = wave >= 8 - kRwLoaders; // uniform
+        const int lw0 = (wave - (8 - kRwLoaders)) * kRwGroups; // first group of this loader
         const int nrounds = (band_rows + kRwRoundRows - 1) / kRwRoundRows;
         const int ntiles = (npix + 31) >> 5;
         const int xor_mask = x_unsigned ? static_cast<int>(0x80808080u) : 0;
@@ -137,7 +154,7 @@ namespace hipq
         // writes at step e is rotated by lane / 4, which spreads the 16 lanes of an LDS write over all
         // banks; the rotation rides in the selectors of the first permutation stage.
         // NHWC: a lane takes four 16-byte pieces (pixel, channel quarter) as they lie in memory.
-        const int n4 = p.W >> 2; // 4-pixel groups a row (NCHW)
+        const int n4 = W_ >> 2; // 4-pixel groups a row (NCHW)
         const int rot = (lane >> 2) & 3;
         uint32_t sel_lo, sel_hi;
         {
@@ -145,14 +162,14 @@ namespace hipq
             sel_lo = r0 | ((4 + r0) << 8) | (r1 << 16) | ((4 + r1) << 24);
             sel_hi = r2 | ((4 + r2) << 8) | (r3 << 16) | ((4 + r3) << 24);
         }
-        auto issue = [&](RegwRaw& raw, int k) {
+        auto issue = [&](RegwRaw& raw, int k, int lw) {
             if (IN_NCX)
             {
                 const int j = lane & 15;
                 const int r = k * kRwRoundRows + (lane >> 4);
                 const int y = h0 - 1 + r;
                 const bool ok = (j < n4) & (r < band_rows) & (static_cast<uint32_t>(y) < static_cast<uint32_t>(p.H));
-                const int base = ok ? ((img * 64 + lw * 16) * p.H + y) * p.W + 4 * j : kOob;
+                const int base = ok ? ((img * 64 + lw * 16) * p.H + y) * W_ + 4 * j : kOob;
 #pragma unroll
                 for (int i = 0; i < 16; ++i)
                     raw.v[i] = __builtin_amdgcn_raw_buffer_load_b32(xrs, base, i * PQ, 0);
@@ -164,12 +181,12 @@ namespace hipq
                 {
                     const int id = i * 256 + lw * 64 + lane;
                     const int pl = id >> 2, c4 = id & 3;
-                    const int rr = static_cast<int>(p.div_w.div(static_cast<uint32_t>(pl)));
-                    const int col = pl - rr * p.W;
+                    const int rr = div_w(pl);
+                    const int col = pl - rr * W_;
                     const int r = k * kRwRoundRows + rr;
                     const int y = h0 - 1 + r;
                     const bool ok = (rr < kRwRoundRows) & (r < band_rows) & (static_cast<uint32_t>(y) < static_cast<uint32_t>(p.H));
-                    const v4i t = buffer_load16(xrs, ok ? ((img * p.H + y) * p.W + col) * 64 + c4 * 16 : kOob);
+                    const v4i t = buffer_load16(xrs, ok ? ((img * p.H + y) * W_ + col) * 64 + c4 * 16 : kOob);
                     raw.v[4 * i] = t[0];
                     raw.v[4 * i + 1] = t[1];
                     raw.v[4 * i + 2] = t[2];
@@ -177,7 +194,7 @@ namespace hipq
                 }
             }
         };
-        auto commit = [&](const RegwRaw& raw, int k) {
+        auto commit = [&](const RegwRaw& raw, int k, int lw) {
             if (IN_NCX)
             {
                 const int j = lane & 15;
@@ -198,7 +215,7 @@ namespace hipq
                 }
                 if (ok)
                 {
-                    uint8_t* const row = lds + (lw >> 1) * p.plane_bytes + r * p.pitch;
+                    uint8_t* const row = lds + (lw >> 1) * plane + r * pitch;
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                     {
@@ -214,13 +231,13 @@ namespace hipq
                 {
                     const int id = i * 256 + lw * 64 + lane;
                     const int pl = id >> 2, c4 = id & 3;
-                    const int rr = static_cast<int>(p.div_w.div(static_cast<uint32_t>(pl)));
-                    const int col = pl - rr * p.W;
+                    const int rr = div_w(pl);
+                    const int col = pl - rr * W_;
                     const int r = k * kRwRoundRows + rr;
                     const int y = h0 - 1 + r;
                     const bool ok = (rr < kRwRoundRows) & (r < band_rows) & (static_cast<uint32_t>(y) < static_cast<uint32_t>(p.H));
                     if (ok)
-                        *reinterpret_cast<v4i*>(lds + (c4 >> 1) * p.plane_bytes + r * p.pitch + regw_cell(col + 1, c4 & 1)) =
+                        *reinterpret_cast<v4i*>(lds + (c4 >> 1) * plane + r * pitch + regw_cell(col + 1, c4 & 1)) =
                             v4i{raw.v[4 * i] ^ xor_mask, raw.v[4 * i + 1] ^ xor_mask, raw.v[4 * i + 2] ^ xor_mask, raw.v[4 * i + 3] ^ xor_mask};
                 }
             }
@@ -230,25 +247,41 @@ namespace hipq
         // loaders: the first rounds of the band are asked for before anything else, and nothing the
         // loaders do before the barrier waits for memory.  The others: filter into LDS (fragment order),
         // scalars, the constant parts of the band (horizontal padding, rows outside the image).
-        RegwRaw raw[kRwDepth];
+        RegwRaw raw[kRwDepth][kRwGroups];
         int32_t xzp = 0, wzp = 0;
         if (loader)
         {
 #pragma unroll
             for (int d = 0; d < kRwDepth; ++d)
                 if (d < nrounds)
-                    issue(raw[d], d);
+#pragma unroll
+                    for (int g = 0; g < kRwGroups; ++g)
+                        issue(raw[d][g], d, lw0 + g);
         }
-        else
+        // what the requantization needs from memory is asked for now, behind the band (loaders) or
+        // ahead of the filter (the others), and used long after it has arrived
+        const EpiConst ec = epi_const(epi);
+        int32_t wsum_n[2];
+        float bias[2], scale[2]; // a lane owns channels lane % 32 and 32 + lane % 32
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+        {
+            const int n = ni * 32 + l32;
+            const bool ok = n < p.K;
+            wsum_n[ni] = ok ? wsum[n] : 0;
+            bias[ni] = (MODE == EPI_FUSED && epi.bias && ok) ? static_cast<float>(epi.bias[n]) : 0.0f;
+            scale[ni] = (MODE == EPI_FUSED && epi.per_channel && ok) ? epi.scale[n] : ec.scale;
+        }
+        if (!loader)
         {
             constexpr int kFilterPieces = 64 * kRwKred / 16; // 2304 16-byte pieces
-            constexpr int kFilterLoads = kFilterPieces / 256;
-            static_assert(kFilterPieces % 256 == 0, "filter pieces divide over four wavefronts");
+            constexpr int kFilterLoads = kFilterPieces / kRwMulThreads;
+            static_assert(kFilterPieces % kRwMulThreads == 0, "filter pieces divide over the wavefronts that fetch them");
             v4i fpiece[kFilterLoads];
             const __amdgpu_buffer_rsrc_t wrs = make_rsrc(w, static_cast<uint32_t>(p.K) * kRwKred);
 #pragma unroll
             for (int i = 0; i < kFilterLoads; ++i)
-                fpiece[i] = buffer_load16(wrs, (i * 256 + tid) * 16); // rows beyond K read as zeros
+                fpiece[i] = buffer_load16(wrs, (i * kRwMulThreads + tid) * 16); // rows beyond K read as zeros
             xzp = load_zp(zp.data_zp, zp.data_t);
             wzp = load_zp(zp.filter_zp, zp.filter_t);
             if (tid < kRwMaxRounds + 2)
@@ -256,24 +289,24 @@ namespace hipq
             const int fill = ((xzp & 0xFF) * 0x01010101) ^ xor_mask;
             const v4i f4 = {fill, fill, fill, fill};
             // slots 0 and W + 1 of every row: 2 planes x 2 slots x 2 chunks pieces a row
-            for (int i = tid; i < band_rows * 8; i += 256)
+            for (int i = tid; i < band_rows * 8; i += kRwMulThreads)
             {
-                const int r = i >> 3, pl = (i >> 2) & 1, sl = (i & 2) ? p.W + 1 : 0, c = i & 1;
-                *reinterpret_cast<v4i*>(lds + pl * p.plane_bytes + r * p.pitch + regw_cell(sl, c)) = f4;
+                const int r = i >> 3, pl = (i >> 2) & 1, sl = (i & 2) ? W_ + 1 : 0, c = i & 1;
+                *reinterpret_cast<v4i*>(lds + pl * plane + r * pitch + regw_cell(sl, c)) = f4;
             }
-            const int per_row = (p.W + 2) * 4; // pieces of a whole row in both planes
+            const int per_row = (W_ + 2) * 4; // pieces of a whole row in both planes
             if (h0 == 0)
-                for (int i = tid; i < per_row; i += 256)
-                    *reinterpret_cast<v4i*>(lds + (i & 1) * p.plane_bytes + regw_cell(i >> 2, (i >> 1) & 1)) = f4;
+                for (int i = tid; i < per_row; i += kRwMulThreads)
+                    *reinterpret_cast<v4i*>(lds + (i & 1) * plane + regw_cell(i >> 2, (i >> 1) & 1)) = f4;
             if (h0 + rows == p.H)
-                for (int i = tid; i < per_row; i += 256)
-                    *reinterpret_cast<v4i*>(lds + (i & 1) * p.plane_bytes + (band_rows - 1) * p.pitch + regw_cell(i >> 2, (i >> 1) & 1)) = f4;
+                for (int i = tid; i < per_row; i += kRwMulThreads)
+                    *reinterpret_cast<v4i*>(lds + (i & 1) * plane + (band_rows - 1) * pitch + regw_cell(i >> 2, (i >> 1) & 1)) = f4;
             // the filter in fragment order: piece ((ks * 2 + ni) * 64 + lane) is what `lane` feeds the MFMAs
             // of step ks, channel tile ni: row ni * 32 + lane % 32, bytes ks * 32 + 16 * (lane / 32) ...
 #pragma unroll
             for (int i = 0; i < kFilterLoads; ++i)
             {
-                const int g = i * 256 + tid;
+                const int g = i * kRwMulThreads + tid;
                 const int n = g / 36, r = g - n * 36; // 36 pieces a filter row
                 const int ks = r >> 1, hf = r & 1;
                 *reinterpret_cast<v4i*>(wlds + (((ks * 2 + (n >> 5)) * 2 + hf) * 32 + (n & 31)) * 16) = fpiece[i];
@@ -291,24 +324,24 @@ namespace hipq
             for (int i = tid; i < npix * p.K; i += kRwThreads)
             {
                 const int n = i / npix, pix = i - n * npix;
-                const int py = h0 + static_cast<int>(p.div_w.div(static_cast<uint32_t>(pix)));
-                const int px = pix - (py - h0) * p.W;
+                const int py = h0 + div_w(pix);
+                const int px = pix - (py - h0) * W_;
                 int32_t a = 0;
                 for (int r = 0; r < 3; ++r)
                     for (int sx = 0; sx < 3; ++sx)
                     {
                         const int iy = py + r - 1, ix = px + sx - 1;
-                        if (static_cast<uint32_t>(iy) >= static_cast<uint32_t>(p.H) || static_cast<uint32_t>(ix) >= static_cast<uint32_t>(p.W))
+                        if (static_cast<uint32_t>(iy) >= static_cast<uint32_t>(p.H) || static_cast<uint32_t>(ix) >= static_cast<uint32_t>(W_))
                             continue; // padding is the data zero point: contributes nothing
                         const int8_t* wp = w + n * kRwKred + (r * 3 + sx) * 64;
                         for (int c = 0; c < 64; ++c)
                         {
-                            const int64_t xi = IN_NCX ? (static_cast<int64_t>(img) * 64 + c) * PQ + iy * p.W + ix : (static_cast<int64_t>(img) * PQ + iy * p.W + ix) * 64 + c;
+                            const int64_t xi = IN_NCX ? (static_cast<int64_t>(img) * 64 + c) * PQ + iy * W_ + ix : (static_cast<int64_t>(img) * PQ + iy * W_ + ix) * 64 + c;
                             const int32_t xv = x_unsigned ? static_cast<int32_t>(p.x[xi]) : static_cast<int32_t>(static_cast<int8_t>(p.x[xi]));
                             a += (xv - xzp) * (static_cast<int32_t>(wp[c]) - wzp);
                         }
                     }
-                const int64_t o = (static_cast<int64_t>(img) * p.K + n) * PQ + h0 * p.W + pix;
+                const int64_t o = (static_cast<int64_t>(img) * p.K + n) * PQ + h0 * W_ + pix;
                 store_out(out, epi.out_t, o, epi_apply(epi, er, a, n, o));
             }
             return;
@@ -325,13 +358,17 @@ namespace hipq
                     const int k = base + d;
                     if (k < nrounds) // uniform
                     {
-                        commit(raw[d], k);
-                        // this wavefront's share of round k is in LDS: count it in
+#pragma unroll
+                        for (int g = 0; g < kRwGroups; ++g)
+                            commit(raw[d][g], k, lw0 + g);
+                        // this wavefront's share of round k is in LDS: count it in (a round is complete at 4)
                         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                         if (lane == 0)
-                            __hip_atomic_fetch_add(flags + k, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                            __hip_atomic_fetch_add(flags + k, static_cast<uint32_t>(kRwGroups), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                         if (k + kRwDepth < nrounds)
-                            issue(raw[d], k + kRwDepth);
+#pragma unroll
+                            for (int g = 0; g < kRwGroups; ++g)
+                                issue(raw[d][g], k + kRwDepth, lw0 + g);
                     }
                 }
             }
@@ -340,18 +377,6 @@ namespace hipq
         }
 
         // ---- everyone multiplies from here on ---------------------------------------------------------
-        const EpiConst ec = epi_const(epi);
-        int32_t wsum_n[2];
-        float bias[2], scale[2]; // a lane owns channels lane % 32 and 32 + lane % 32
-#pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-        {
-            const int n = ni * 32 + l32;
-            const bool ok = n < p.K;
-            wsum_n[ni] = ok ? wsum[n] : 0;
-            bias[ni] = (MODE == EPI_FUSED && epi.bias && ok) ? static_cast<float>(epi.bias[n]) : 0.0f;
-            scale[ni] = (MODE == EPI_FUSED && epi.per_channel && ok) ? epi.scale[n] : ec.scale;
-        }
         const int32_t mult = (x_unsigned ? 128 : 0) - xzp;
         const int32_t corr[2] = {mult * wsum_n[0], mult * wsum_n[1]};
         // INTERPRETER requantization in fixed point needs |acc * scale| * 256 < 2^31
@@ -377,7 +402,7 @@ namespace hipq
         auto await_rows = [&](int t) {
             // the tile's last pixel is in band-relative output row ro_max and needs band rows up to ro_max + 2
             const int last = min(t * 32 + 31, npix - 1);
-            const int ro_max = static_cast<int>(p.div_w.div(static_cast<uint32_t>(last)));
+            const int ro_max = div_w(last);
             const int need = min((ro_max + 3 + kRwRoundRows - 1) / kRwRoundRows, nrounds);
             while (ready < need)
             {
@@ -392,16 +417,16 @@ namespace hipq
         auto tile_mfma = [&](int t, v16i (&acc)[2]) {
             // tiles past the end re-read the last pixel; their results are never stored
             const int pix = min(t * 32 + l32, npix - 1);
-            const int ro = static_cast<int>(p.div_w.div(static_cast<uint32_t>(pix)));
-            const int col = pix - ro * p.W;
+            const int ro = div_w(pix);
+            const int col = pix - ro * W_;
             int xb[3];
 #pragma unroll
             for (int sx = 0; sx < 3; ++sx)
-                xb[sx] = ro * p.pitch + regw_cell(col + sx, half);
+                xb[sx] = ro * pitch + regw_cell(col + sx, half);
             const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
             auto frag = [&](int ks) {
                 const int tap = ks >> 1, h = ks & 1, r = tap / 3, sx = tap % 3;
-                return *reinterpret_cast<const v4i*>(lds + xb[sx] + r * p.pitch + h * p.plane_bytes);
+                return *reinterpret_cast<const v4i*>(lds + xb[sx] + r * pitch + h * plane);
             };
             constexpr int kAhead = 6; // no requantization in this stream: registers to spare
             v4i xf[kAhead + 1];
@@ -425,7 +450,7 @@ namespace hipq
         // uniform branch per output would cost more than the arithmetic)
         auto tile_store = [&](int t, const v16i (&acc)[2], auto fast_c) {
             constexpr bool FAST = decltype(fast_c)::value;
-            const int gpix0 = h0 * p.W + t * 32; // first pixel of the tile within the image
+            const int gpix0 = h0 * W_ + t * 32; // first pixel of the tile within the image
 #pragma unroll
             for (int ni = 0; ni < 2; ++ni)
             {
@@ -487,17 +512,17 @@ namespace hipq
         auto tile_both = [&](int t, v16i (&acc)[2], int tp, const v16i (&accp)[2], auto fast_c) {
             constexpr bool FAST = decltype(fast_c)::value;
             const int pix = min(t * 32 + l32, npix - 1);
-            const int ro = static_cast<int>(p.div_w.div(static_cast<uint32_t>(pix)));
-            const int col = pix - ro * p.W;
+            const int ro = div_w(pix);
+            const int col = pix - ro * W_;
             int xb[3];
 #pragma unroll
             for (int sx = 0; sx < 3; ++sx)
-                xb[sx] = ro * p.pitch + regw_cell(col + sx, half);
+                xb[sx] = ro * pitch + regw_cell(col + sx, half);
             const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-            const int gpix0 = h0 * p.W + tp * 32; // first pixel of the previous tile within the image
+            const int gpix0 = h0 * W_ + tp * 32; // first pixel of the previous tile within the image
             auto frag = [&](int ks) {
                 const int tap = ks >> 1, h = ks & 1, r = tap / 3, sx = tap % 3;
-                return *reinterpret_cast<const v4i*>(lds + xb[sx] + r * p.pitch + h * p.plane_bytes);
+                return *reinterpret_cast<const v4i*>(lds + xb[sx] + r * pitch + h * plane);
             };
             int32_t x[4];
             uint32_t d[4];
@@ -657,7 +682,7 @@ namespace hipq
         {
             if (H % tp != 0 || (tp * W) % 16 != 0)
                 continue;
-            const int64_t plane = ((tp + 2) * pitch + 255) / 256 * 256 + 128;
+            const int64_t plane = (W == 56 && tp <= kRwMaxRowsCT) ? regw_plane_bytes(56, kRwMaxRowsCT) : ((tp + 2) * pitch + 255) / 256 * 256 + 128;
             if (2 * plane + (kRwMaxRounds + 8) * 4 + 64 * kRwKred > 160 * 1024 || (tp + 2 + kRwRoundRows - 1) / kRwRoundRows > kRwMaxRounds)
                 break;
             const int64_t items = g.N * (H / tp);
@@ -678,7 +703,7 @@ namespace hipq
         rp->bands = static_cast<int32_t>(H / best);
         rp->items = static_cast<int32_t>(g.N * rp->bands);
         rp->pitch = static_cast<int32_t>(pitch);
-        rp->plane_bytes = static_cast<int32_t>(((best + 2) * pitch + 255) / 256 * 256 + 128);
+        rp->plane_bytes = static_cast<int32_t>((W == 56 && best <= kRwMaxRowsCT) ? regw_plane_bytes(56, kRwMaxRowsCT) : ((best + 2) * pitch + 255) / 256 * 256 + 128);
         rp->flags_lds = 2 * rp->plane_bytes;
         rp->bands_magic = rp->bands > 1 ? static_cast<uint32_t>((1ull << 32) / static_cast<uint64_t>(rp->bands) + 1) : 0u;
         if (static_cast<int64_t>(rp->items) * rp->bands >= (1ll << 32))
@@ -711,10 +736,10 @@ namespace hipq
         return getenv("HIPQ_NO_REGW") == nullptr && regw_plan(g, out_ncx, 256, &rp, &lds_bytes);
     }
 
-    template <int MODE, bool IN_NCX, bool SUM>
+    template <int MODE, bool IN_NCX, bool SUM, int WCT>
     static int launch_regw(const RegwParams& rp, size_t lds_bytes, const int8_t* w, const int32_t* wsum, int xu, const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s)
     {
-        auto kernel = conv_regw_kernel<MODE, IN_NCX, SUM>;
+        auto kernel = conv_regw_kernel<MODE, IN_NCX, SUM, WCT>;
         static bool configured[16] = {};
         int dev = 0;
         HIPQ_HIP(hipGetDevice(&dev));
@@ -741,10 +766,14 @@ namespace hipq
         const bool in_ncx = g.data_layout == HIPQ_LAYOUT_NCX;
         const bool sum = epi.mode == EPI_FUSED && epi.sum_in != nullptr;
         HIPQ_REQUIRE(!sum || (reinterpret_cast<uintptr_t>(epi.sum_in) & 3) == 0, "sum input must be 4-byte aligned");
-#define REGW(MODE, SUM) (in_ncx ? launch_regw<MODE, true, SUM>(rp, lds_bytes, w, wsum, xu, zp, epi, out, s) : launch_regw<MODE, false, SUM>(rp, lds_bytes, w, wsum, xu, zp, epi, out, s))
+        // 56-wide layers (ResNet's first stage, config 1) with the compile-time LDS geometry
+        const bool w56 = rp.W == 56 && rp.TP <= kRwMaxRowsCT && rp.plane_bytes == regw_plane_bytes(56, kRwMaxRowsCT) && getenv("HIPQ_REGW_NO_CT") == nullptr;
+#define REGW_W(MODE, IN, SUM) (w56 ? launch_regw<MODE, IN, SUM, 56>(rp, lds_bytes, w, wsum, xu, zp, epi, out, s) : launch_regw<MODE, IN, SUM, 0>(rp, lds_bytes, w, wsum, xu, zp, epi, out, s))
+#define REGW(MODE, SUM) (in_ncx ? REGW_W(MODE, true, SUM) : REGW_W(MODE, false, SUM))
         if (epi.mode == EPI_INTERP)
             return REGW(EPI_INTERP, false);
         return sum ? REGW(EPI_FUSED, true) : REGW(EPI_FUSED, false);
 #undef REGW
+#undef REGW_W
     }
 }

@@ -528,52 +528,107 @@ namespace hipq
             uint32_t d[4];
             float s4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
             // slot s of 36: output (ni, g, e) = (s / 16, (s / 4) % 4, s % 4) of the previous tile
+            // slot sl of 36 (one behind every MFMA): stage sl % 4 of the four outputs (ni, g) = (sl / 16,
+            // (sl / 4) % 4) of the previous tile.  The four outputs of a group go through each stage
+            // together, so an instruction's input is four instructions old instead of one: a wavefront
+            // that shares its SIMD issues dependent arithmetic a third slower than independent.
             auto requant = [&](int sl) {
                 if (sl >= 32)
                     return;
-                const int ni = sl >> 4, g = (sl >> 2) & 3, e = sl & 3;
+                const int ni = sl >> 4, g = (sl >> 2) & 3, stage = sl & 3;
                 const int n = ni * 32 + l32;
-                if (SUM && e == 0)
+                if (stage == 0)
                 {
-                    const int lp = tp * 32 + 8 * g + 4 * half;
-                    s4[0] = s4[1] = s4[2] = s4[3] = 0.0f;
-                    if (n < p.K && lp < npix)
-                        sum4(epi.sum_in, epi.sum_t, (static_cast<int64_t>(img) * p.K + n) * PQ + gpix0 + 8 * g + 4 * half, true, s4);
-                }
-                const int32_t a = accp[ni][4 * g + e] + corr[ni];
-                if (MODE == EPI_INTERP && FAST)
-                {
-                    // t = trunc(256 v); round-half-away(v) = (t + 128 - (t < 0)) >> 8, exactly
-                    const int32_t tt = static_cast<int32_t>(__fmul_rn(static_cast<float>(a), s256));
-                    x[e] = tt + (tt >> 31) + c256;
-                }
-                else if (MODE == EPI_INTERP)
-                    x[e] = epi_interp<OUT_Q8>(ec, a);
-                else
-                {
-                    float v = __fmul_rn(__fadd_rn(static_cast<float>(a), bias[ni]), scale[ni]);
                     if (SUM)
-                        v = fmaf(ec.sum_scale, s4[e], v);
-                    v = __builtin_amdgcn_fmed3f(v, lo, ec.hi);
-                    // 1.5 * 2^23 + v rounds half-to-even into the low mantissa bits
-                    x[e] = __float_as_int(__fadd_rn(v, 12582912.0f));
+                    {
+                        const int lp = tp * 32 + 8 * g + 4 * half;
+                        s4[0] = s4[1] = s4[2] = s4[3] = 0.0f;
+                        if (n < p.K && lp < npix)
+                            sum4(epi.sum_in, epi.sum_t, (static_cast<int64_t>(img) * p.K + n) * PQ + gpix0 + 8 * g + 4 * half, true, s4);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        x[e] = accp[ni][4 * g + e] + corr[ni];
+                    if (MODE == EPI_FUSED || FAST)
+                    {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            x[e] = __float_as_int(static_cast<float>(x[e]));
+                    }
                 }
-                if (e == 3)
+                else if (stage == 1)
+                {
+                    if (MODE == EPI_INTERP && FAST)
+                    {
+                        // t = trunc(256 v); round-half-away(v) = (t + 128 - (t < 0)) >> 8, exactly
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            x[e] = __float_as_int(__fmul_rn(__int_as_float(x[e]), s256));
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            x[e] = static_cast<int32_t>(__int_as_float(x[e]));
+                    }
+                    else if (MODE == EPI_FUSED)
+                    {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            x[e] = __float_as_int(__fadd_rn(__int_as_float(x[e]), bias[ni]));
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            x[e] = __float_as_int(__fmul_rn(__int_as_float(x[e]), scale[ni]));
+                    }
+                }
+                else if (stage == 2)
+                {
+                    if (MODE == EPI_INTERP && FAST)
+                    {
+                        int32_t sg[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            sg[e] = x[e] >> 31;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            x[e] = x[e] + sg[e] + c256;
+                    }
+                    else if (MODE == EPI_INTERP)
+                    {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            x[e] = epi_interp<OUT_Q8>(ec, x[e]);
+                    }
+                    else
+                    {
+                        if (SUM)
+                        {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                x[e] = __float_as_int(fmaf(ec.sum_scale, s4[e], __int_as_float(x[e])));
+                        }
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            x[e] = __float_as_int(__builtin_amdgcn_fmed3f(__int_as_float(x[e]), lo, ec.hi));
+                        // 1.5 * 2^23 + v rounds half-to-even into the low mantissa bits
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            x[e] = __float_as_int(__fadd_rn(__int_as_float(x[e]), 12582912.0f));
+                    }
+                }
+                else
                 {
                     constexpr uint32_t sel = (MODE == EPI_INTERP && FAST) ? 0x0c0c0501u : 0x0c0c0400u;
                     const uint32_t lo2 = __builtin_amdgcn_perm(x[1], x[0], sel);
                     const uint32_t hi2 = __builtin_amdgcn_perm(x[3], x[2], sel);
                     d[g] = (hi2 << 16) | lo2;
-                }
-                if (e == 3 && g == 3)
-                {
-                    // the lower half of the wavefront holds pixels 8g .. 8g+3, the upper 8g+4 .. 8g+7: after the
-                    // two swaps a lane holds 16 consecutive pixels of its channel (lower: 0..15, upper: 16..31)
-                    const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
-                    const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
-                    const v4i piece = {static_cast<int>(s02[0]), static_cast<int>(s02[1]), static_cast<int>(s13[0]), static_cast<int>(s13[1])};
-                    const bool ok = (n < p.K) & (tp * 32 + 16 * half < npix);
-                    __builtin_amdgcn_raw_buffer_store_b128(piece, ors, ok ? (img * p.K + n) * PQ + gpix0 + 16 * half : kOob, 0, kRwStoreScope);
+                    if (g == 3)
+                    {
+                        // the lower half of the wavefront holds pixels 8g .. 8g+3, the upper 8g+4 .. 8g+7: after the
+                        // two swaps a lane holds 16 consecutive pixels of its channel (lower: 0..15, upper: 16..31)
+                        const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+                        const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+                        const v4i piece = {static_cast<int>(s02[0]), static_cast<int>(s02[1]), static_cast<int>(s13[0]), static_cast<int>(s13[1])};
+                        const bool ok = (n < p.K) & (tp * 32 + 16 * half < npix);
+                        __builtin_amdgcn_raw_buffer_store_b128(piece, ors, ok ? (img * p.K + n) * PQ + gpix0 + 16 * half : kOob, 0, kRwStoreScope);
+                    }
                 }
             };
             // an LDS read takes about three MFMA pairs to come back: kRwAhead fragments are on their way

@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the headline kernel at batch 128: not measured by this run (counters need
 # a profiler run of their own) but quoted from the FETCH_SIZE / WRITE_SIZE runs summarised in the
 # file below (scaled by a 64 MiB copy in the same run); the JSON line names that file
-MEASURED_TRAFFIC_BYTES = {("conv_regw_i8_32x32x32", 128): 52.9e6, ("conv_band_i8_32x32x32", 128): 52.3e6}
+MEASURED_TRAFFIC_BYTES = {("conv_regw_i8_32x32x32", 128): 52.0e6, ("conv_band_i8_32x32x32", 128): 52.3e6}
 TRAFFIC_SOURCE = {"conv_regw_i8_32x32x32": "profiles/conv_regw_config1_batch128.md", "conv_band_i8_32x32x32": "profiles/conv_band_config1_hbm_traffic.md"}
 _DATA_CACHE = {}
 

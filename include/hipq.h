@@ -487,12 +487,35 @@ HIPQ_API int hipq_concat(int32_t elem_bytes,
  * (src/ngraph/runtime/reference/softmax.hpp:31-57). */
 HIPQ_API int hipq_softmax_f32(const float* in, float* out, int64_t outer, int64_t axis, int64_t inner, void* stream);
 
+/* Softmax(Multiply(in, Broadcast(factor))) in one pass: `factor` is a device f32 scalar, every
+ * product is rounded to f32 as op::v1::Multiply rounds it (src/ngraph/runtime/reference/multiply.hpp),
+ * so the result equals hipq_binary(multiply) followed by hipq_softmax_f32 bit for bit.  What an
+ * attention layer's scores / sqrt(head size) -> Softmax chain lowers to. */
+HIPQ_API int hipq_softmax_scaled_f32(const float* in, const float* factor, float* out, int64_t outer, int64_t axis, int64_t inner, void* stream);
+
+/* A Quantize of a kernel's f32 result, written beside it (one scale and zero point for the whole
+ * tensor; arithmetic of hipq_quantize, src/ngraph/runtime/reference/quantize.hpp:29-117, so the bytes
+ * equal a hipq_quantize call on the f32 result).  What a backend passes when the only consumer of an
+ * f32 tensor -- or one of two -- is a Quantize: the tensor is not read back from memory for it. */
+typedef struct hipq_quant_out
+{
+    void* out;              /* [same element count], quant_t */
+    const float* scale;     /* device scalar */
+    const void* zero_point; /* device scalar of quant_t; null: 0 */
+    int32_t quant_t;        /* HIPQ_I8 or HIPQ_U8 */
+    int32_t round_mode;     /* hipq_round_mode_t */
+} hipq_quant_out_t;
+
 /* op::v0::Erf (src/ngraph/runtime/reference/erf.hpp:29-35). */
 HIPQ_API int hipq_erf_f32(const float* in, float* out, int64_t count, void* stream);
 
 /* op::v0::Gelu as FusedOpDecomposition lowers it (src/ngraph/op/gelu.cpp:46-60):
  * (0.5 * x) * (1 + erf(x / sqrt(2))), every step in f32. */
 HIPQ_API int hipq_gelu_f32(const float* in, float* out, int64_t count, void* stream);
+
+/* Gelu with a Quantize of its result: q->out = Quantize(Gelu(in)); `out` (the f32 result) may be null
+ * when the Quantize is its only consumer.  Equals hipq_gelu_f32 + hipq_quantize bit for bit. */
+HIPQ_API int hipq_gelu_quantize_f32(const float* in, float* out, const hipq_quant_out_t* q, int64_t count, void* stream);
 
 /* op::v0::LayerNorm forward as it decomposes (src/ngraph/op/layer_norm.cpp:68-150,
  * src/ngraph/builder/reduce_ops.cpp:68-124): the tensor is [rows][cols] with cols the product of the
@@ -509,6 +532,22 @@ HIPQ_API int hipq_layer_norm_f32(const float* in,
                                  int64_t cols,
                                  double epsilon,
                                  void* stream);
+
+/* LayerNorm(Add(a, b)) in one pass, optionally with a Quantize of the result beside it:
+ * out = LayerNorm(a + b) (b may be null: LayerNorm(a)), the sum rounded to f32 as op::v1::Add rounds
+ * it; q (may be null) as above.  Equals hipq_binary(add) + hipq_layer_norm_f32 (+ hipq_quantize) bit
+ * for bit: the residual-and-normalise step of a transformer layer whose result feeds the next
+ * quantized projection. */
+HIPQ_API int hipq_add_layer_norm_f32(const float* a,
+                                     const float* b,
+                                     const float* scale,
+                                     const float* bias,
+                                     float* out,
+                                     const hipq_quant_out_t* q,
+                                     int64_t rows,
+                                     int64_t cols,
+                                     double epsilon,
+                                     void* stream);
 
 /* op::v0::BatchMatMul (src/ngraph/runtime/reference/batch_mat_mul.hpp:31-57: runtime::reference::dot,
  * dot.hpp:34-167 with one reduction axis, on every pair of the batch), op::v0::Dot of two f32
@@ -528,6 +567,33 @@ HIPQ_API int hipq_batch_matmul_f32(const float* a,
                                    int32_t transpose_b,
                                    void* stream);
 
+/* The same product on views of larger tensors and into one, with an optional Quantize of the result:
+ * batch element e = outer * batch_inner + inner reads a + outer * a_outer + inner * a_inner with
+ * rows lda elements apart (likewise b and out; strides in elements, rows at least as far apart as
+ * they are long).  What BatchMatMul(Reshape / transpose of a slice) lowers to without moving data:
+ * the Q, K and V heads of a fused [tokens, 3 * hidden] projection, and a context written straight
+ * into the [tokens, hidden] layout of the merged heads.  q (may be null): Quantize of the f32 result
+ * at the same element offsets of q->out; `out` may then be null.  Bit-exact like the plain entry point;
+ * no counterpart as a single reference op. */
+typedef struct hipq_matmul_view
+{
+    int64_t batch_inner;
+    int64_t a_outer, a_inner, lda;
+    int64_t b_outer, b_inner, ldb;
+    int64_t o_outer, o_inner, ldo;
+} hipq_matmul_view_t;
+HIPQ_API int hipq_batch_matmul_view_f32(const float* a,
+                                        const float* b,
+                                        float* out,
+                                        const hipq_matmul_view_t* view,
+                                        const hipq_quant_out_t* q,
+                                        int64_t batch,
+                                        int64_t M,
+                                        int64_t K,
+                                        int64_t N,
+                                        int32_t transpose_a,
+                                        int32_t transpose_b,
+                                        void* stream);
 
 /* Which kernel the last hipq_quantized_* call on this thread used: "mfma", "direct", ... (host
  * string, never NULL).  For tests and profiles. */

@@ -160,10 +160,18 @@ class HipProvider:
 
 class DevicePlan:
     """The encoder with every tensor resident in HBM and the weights prepared once: `launch()` issues
-    the 19 kernel launches of every layer on `stream`; `capture()` turns the pass into one HIP graph."""
+    the kernel launches of every layer on `stream`; `capture()` turns the pass into one HIP graph.
 
-    def __init__(self, lib, stream, batch, cfg=BASE):
+    fused=False launches the graph op by op, 19 launches a layer.  fused=True (what a backend's fusion
+    pass makes of the same graph, 10 launches a layer) folds the ops that only re-read and re-write a
+    tensor into their producers, each through an entry point whose result equals the op-by-op one bit
+    for bit: the head split and merge become views of the attention products, Multiply goes into
+    Softmax, the residual Add into LayerNorm, and every Quantize into the kernel that produces its
+    input (the context product, LayerNorm, Gelu)."""
+
+    def __init__(self, lib, stream, batch, cfg=BASE, fused=True):
         self.lib, self.stream, self.batch, self.cfg = lib, stream, batch, cfg
+        self.fused = fused
         self._replay = None
         self.calls, self.keep, self.graph = [], [], None
         vp, i64, i32 = C.c_void_p, C.c_int64, C.c_int32
@@ -199,6 +207,34 @@ class DevicePlan:
         def permute(src, dst, shape, order):
             call(lib.hipq_permute, 4, src, dst, len(shape), self._keep((i64 * len(shape))(*shape)), self._keep((i32 * len(shape))(*order)))
 
+        if fused:
+            lib.hipq_softmax_scaled_f32.argtypes = [vp, vp, vp, i64, i64, i64, vp]
+            lib.hipq_gelu_quantize_f32.argtypes = [vp, vp, vp, i64, vp]
+            lib.hipq_add_layer_norm_f32.argtypes = [vp] * 6 + [i64, i64, C.c_double, vp]
+            lib.hipq_batch_matmul_view_f32.argtypes = [vp] * 5 + [i64] * 4 + [i32] * 2 + [vp]
+            qout = {s: self._keep(H.QuantOut(x8.ptr, scales[s].ptr, zero.ptr, H.I8, H.RNE)) for s in scales}
+            H3 = 3 * h
+            # Q, K, V of batch element (b, head): rows of the [T, 3H] projection, 3H apart, starting at column
+            # {0, H, 2H} + head * hd; scores [B * heads, S, S] dense; the context goes straight into [T, H]
+            v_scores = self._keep(H.MatmulView(nh, S * H3, hd, H3, S * H3, hd, H3, nh * S * S, S * S, S))
+            v_context = self._keep(H.MatmulView(nh, nh * S * S, S * S, S, S * H3, hd, H3, S * h, hd, h))
+            for l in range(cfg.layers):
+                w = layer_weights(cfg, l)
+                if l == 0:
+                    quantize(self.x, h, cfg.s_x)
+                dot(w["qkv"], h, H3, qkv)
+                call(lib.hipq_batch_matmul_view_f32, qkv, (qkv, h * 4), scores, v_scores, None, batch * nh, S, hd, S, 0, 1)
+                call(lib.hipq_softmax_scaled_f32, scores, inv, probs, batch * nh * S, S, 1)
+                call(lib.hipq_batch_matmul_view_f32, probs, (qkv, 2 * h * 4), None, v_context, qout[cfg.s_c], batch * nh, S, S, hd, 0, 0)
+                dot(w["out"], h, h, proj)
+                g1, b1 = dev(w["ln1"][0]), dev(w["ln1"][1])
+                call(lib.hipq_add_layer_norm_f32, self.x, proj, g1, b1, x1, qout[cfg.s_x], T, h, 1e-5)
+                dot(w["ffn1"], h, f, ffn)
+                call(lib.hipq_gelu_quantize_f32, ffn, None, qout[cfg.s_g], T * f)
+                dot(w["ffn2"], f, h, proj)
+                g2, b2 = dev(w["ln2"][0]), dev(w["ln2"][1])
+                call(lib.hipq_add_layer_norm_f32, x1, proj, g2, b2, self.x, qout[cfg.s_x] if l + 1 < cfg.layers else None, T, h, 1e-5)
+            return
         for l in range(cfg.layers):
             w = layer_weights(cfg, l)
             quantize(self.x, h, cfg.s_x)

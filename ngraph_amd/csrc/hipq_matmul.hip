@@ -6,6 +6,7 @@
 // floats is exact in double, hence the fused multiply-add rounds exactly as the reference's separate
 // multiply and add, and the results are the reference's bit for bit.
 #include "hipq_common.h"
+#include "hipq_quant_math.h"
 
 namespace hipq
 {
@@ -14,9 +15,28 @@ namespace hipq
         typedef float f4 __attribute__((ext_vector_type(4)));
         constexpr int TM = 64, TN = 64, TK = 16;
 
+        // where the matrices of batch element (outer, inner) start and how far apart their rows are (in
+        // elements): the plain op has one batch level and dense matrices; views of a larger tensor
+        // (the heads of a fused QKV projection, a context written head-interleaved) have two
+        struct MatView
+        {
+            int64_t batch_inner;
+            int64_t a_outer, a_inner, lda;
+            int64_t b_outer, b_inner, ldb;
+            int64_t o_outer, o_inner, ldo;
+        };
+        struct MatQuant
+        {
+            void* out; // null: none
+            const float* scale;
+            const void* zero_point;
+            int32_t quant_t, mode;
+        };
+
         // out[b] = op(A[b]) * op(B[b]): A is [M][K] (or [K][M] with ta), B is [K][N] (or [N][K] with tb)
-        __global__ __launch_bounds__(256) void batch_matmul_f32_kernel(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ out, int32_t M, int32_t K, int32_t N, int32_t ta,
-                                                                       int32_t tb, int32_t m_tiles, int32_t n_tiles, int32_t vec_a, int32_t vec_b)
+        __global__ __launch_bounds__(256) void batch_matmul_f32_kernel(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ out, MatView view, MatQuant mq, int32_t M,
+                                                                       int32_t K, int32_t N, int32_t ta, int32_t tb, int32_t m_tiles, int32_t n_tiles, int32_t vec_a, int32_t vec_b,
+                                                                       int32_t vec_o)
         {
             __shared__ __attribute__((aligned(16))) float as[TK][TM + 4]; // [k][m]
             __shared__ __attribute__((aligned(16))) float bs[TK][TN + 4]; // [k][n]
@@ -26,9 +46,12 @@ namespace hipq
             t /= n_tiles;
             const int mt = t % m_tiles;
             const int64_t batch = t / m_tiles;
-            const float* A = a + batch * static_cast<int64_t>(M) * K;
-            const float* B = b + batch * static_cast<int64_t>(K) * N;
-            float* O = out + batch * static_cast<int64_t>(M) * N;
+            const int64_t bo = batch / view.batch_inner, bi = batch - bo * view.batch_inner;
+            const float* A = a + bo * view.a_outer + bi * view.a_inner;
+            const float* B = b + bo * view.b_outer + bi * view.b_inner;
+            const int64_t o_base = bo * view.o_outer + bi * view.o_inner;
+            float* O = out ? out + o_base : nullptr;
+            const int64_t lda = view.lda, ldb = view.ldb, ldo = view.ldo;
             const int m0 = mt * TM, n0 = nt * TN;
             const int tm = (tid >> 4) * 4, tn = (tid & 15) * 4; // this lane's 4 x 4 outputs within the tile
             double acc[4][4] = {};
@@ -40,24 +63,24 @@ namespace hipq
                 {
                     const int r = tid >> 2, kq = (tid & 3) * 4; // A[m0 + r][k0 + kq ..]
                     if (vec_a && m0 + r < M && k0 + kq + 3 < K)
-                        v = *reinterpret_cast<const f4*>(A + static_cast<int64_t>(m0 + r) * K + k0 + kq);
+                        v = *reinterpret_cast<const f4*>(A + static_cast<int64_t>(m0 + r) * lda + k0 + kq);
                     else
                     {
 #pragma unroll
                         for (int i = 0; i < 4; ++i)
-                            v[i] = (m0 + r < M && k0 + kq + i < K) ? A[static_cast<int64_t>(m0 + r) * K + k0 + kq + i] : 0.0f;
+                            v[i] = (m0 + r < M && k0 + kq + i < K) ? A[static_cast<int64_t>(m0 + r) * lda + k0 + kq + i] : 0.0f;
                     }
                 }
                 else
                 {
                     const int kk = tid >> 4, mq = (tid & 15) * 4; // A[k0 + kk][m0 + mq ..]
                     if (vec_a && k0 + kk < K && m0 + mq + 3 < M)
-                        v = *reinterpret_cast<const f4*>(A + static_cast<int64_t>(k0 + kk) * M + m0 + mq);
+                        v = *reinterpret_cast<const f4*>(A + static_cast<int64_t>(k0 + kk) * lda + m0 + mq);
                     else
                     {
 #pragma unroll
                         for (int i = 0; i < 4; ++i)
-                            v[i] = (k0 + kk < K && m0 + mq + i < M) ? A[static_cast<int64_t>(k0 + kk) * M + m0 + mq + i] : 0.0f;
+                            v[i] = (k0 + kk < K && m0 + mq + i < M) ? A[static_cast<int64_t>(k0 + kk) * lda + m0 + mq + i] : 0.0f;
                     }
                 }
                 return v;
@@ -82,24 +105,24 @@ namespace hipq
                 {
                     const int kk = tid >> 4, nq = (tid & 15) * 4; // B[k0 + kk][n0 + nq ..]
                     if (vec_b && k0 + kk < K && n0 + nq + 3 < N)
-                        v = *reinterpret_cast<const f4*>(B + static_cast<int64_t>(k0 + kk) * N + n0 + nq);
+                        v = *reinterpret_cast<const f4*>(B + static_cast<int64_t>(k0 + kk) * ldb + n0 + nq);
                     else
                     {
 #pragma unroll
                         for (int i = 0; i < 4; ++i)
-                            v[i] = (k0 + kk < K && n0 + nq + i < N) ? B[static_cast<int64_t>(k0 + kk) * N + n0 + nq + i] : 0.0f;
+                            v[i] = (k0 + kk < K && n0 + nq + i < N) ? B[static_cast<int64_t>(k0 + kk) * ldb + n0 + nq + i] : 0.0f;
                     }
                 }
                 else
                 {
                     const int r = tid >> 2, kq = (tid & 3) * 4; // B[n0 + r][k0 + kq ..]
                     if (vec_b && n0 + r < N && k0 + kq + 3 < K)
-                        v = *reinterpret_cast<const f4*>(B + static_cast<int64_t>(n0 + r) * K + k0 + kq);
+                        v = *reinterpret_cast<const f4*>(B + static_cast<int64_t>(n0 + r) * ldb + k0 + kq);
                     else
                     {
 #pragma unroll
                         for (int i = 0; i < 4; ++i)
-                            v[i] = (n0 + r < N && k0 + kq + i < K) ? B[static_cast<int64_t>(n0 + r) * K + k0 + kq + i] : 0.0f;
+                            v[i] = (n0 + r < N && k0 + kq + i < K) ? B[static_cast<int64_t>(n0 + r) * ldb + k0 + kq + i] : 0.0f;
                     }
                 }
                 return v;
@@ -150,21 +173,39 @@ namespace hipq
                 }
                 __syncthreads();
             }
+            // (the optional quantized copy: Quantize of the f32 result, the arithmetic of hipq_quantize)
+            const float qs = mq.out ? *mq.scale : 1.0f;
+            const int32_t qz = mq.out ? load_zp(mq.zero_point, mq.quant_t) : 0;
+            auto q1 = [&](float v) -> uint32_t {
+                return mq.quant_t == HIPQ_U8 ? static_cast<uint32_t>(quantize_one<float, uint8_t>(v, qs, static_cast<uint8_t>(qz), mq.mode))
+                                             : static_cast<uint32_t>(static_cast<uint8_t>(quantize_one<float, int8_t>(v, qs, static_cast<int8_t>(qz), mq.mode)));
+            };
 #pragma unroll
             for (int i = 0; i < 4; ++i)
             {
                 const int m = m0 + tm + i;
                 if (m >= M)
                     continue;
-                float* row = O + static_cast<int64_t>(m) * N + n0 + tn;
-                if (n0 + tn + 3 < N && (N & 3) == 0)
-                    *reinterpret_cast<f4*>(row) = f4{static_cast<float>(acc[i][0]), static_cast<float>(acc[i][1]), static_cast<float>(acc[i][2]), static_cast<float>(acc[i][3])};
+                const int64_t at = static_cast<int64_t>(m) * ldo + n0 + tn;
+                const f4 r = f4{static_cast<float>(acc[i][0]), static_cast<float>(acc[i][1]), static_cast<float>(acc[i][2]), static_cast<float>(acc[i][3])};
+                if (n0 + tn + 3 < N && vec_o)
+                {
+                    if (O)
+                        *reinterpret_cast<f4*>(O + at) = r;
+                    if (mq.out)
+                        *reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(mq.out) + o_base + at) = q1(r[0]) | (q1(r[1]) << 8) | (q1(r[2]) << 16) | (q1(r[3]) << 24);
+                }
                 else
                 {
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
                         if (n0 + tn + j < N)
-                            row[j] = static_cast<float>(acc[i][j]);
+                        {
+                            if (O)
+                                O[at + j] = r[j];
+                            if (mq.out)
+                                static_cast<uint8_t*>(mq.out)[o_base + at + j] = static_cast<uint8_t>(q1(r[j]));
+                        }
                 }
             }
         }
@@ -173,6 +214,23 @@ namespace hipq
 
 using namespace hipq;
 
+static int launch_batch_matmul(const float* a, const float* b, float* out, const MatView& view, const MatQuant& mq, int64_t batch, int64_t M, int64_t K, int64_t N, int32_t transpose_a,
+                               int32_t transpose_b, void* stream)
+{
+    HIPQ_REQUIRE(M < (1ll << 31) && K < (1ll << 31) && N < (1ll << 31), "extent too large");
+    const int64_t m_tiles = (M + TM - 1) / TM, n_tiles = (N + TN - 1) / TN;
+    // 16-byte accesses along the rows when every row of every matrix starts aligned
+    auto all4 = [](int64_t x, int64_t y, int64_t z) { return x % 4 == 0 && y % 4 == 0 && z % 4 == 0; };
+    const int vec_a = (reinterpret_cast<uintptr_t>(a) & 15) == 0 && all4(view.lda, view.a_outer, view.a_inner);
+    const int vec_b = (reinterpret_cast<uintptr_t>(b) & 15) == 0 && all4(view.ldb, view.b_outer, view.b_inner);
+    const int vec_o = (!out || (reinterpret_cast<uintptr_t>(out) & 15) == 0) && (!mq.out || (reinterpret_cast<uintptr_t>(mq.out) & 3) == 0) && all4(view.ldo, view.o_outer, view.o_inner);
+    HIPQ_REQUIRE(batch * m_tiles * n_tiles < (1ll << 31), "too many tiles for one launch");
+    batch_matmul_f32_kernel<<<static_cast<unsigned>(batch * m_tiles * n_tiles), 256, 0, as_stream(stream)>>>(a, b, out, view, mq, static_cast<int32_t>(M), static_cast<int32_t>(K),
+                                                                                                              static_cast<int32_t>(N), transpose_a ? 1 : 0, transpose_b ? 1 : 0,
+                                                                                                              static_cast<int32_t>(m_tiles), static_cast<int32_t>(n_tiles), vec_a, vec_b, vec_o);
+    return check_launch("batch_matmul_f32");
+}
+
 int hipq_batch_matmul_f32(const float* a, const float* b, float* out, int64_t batch, int64_t M, int64_t K, int64_t N, int32_t transpose_a, int32_t transpose_b, void* stream)
 {
     HIPQ_REQUIRE(batch >= 0 && M >= 0 && K >= 0 && N >= 0, "negative extent");
@@ -180,14 +238,29 @@ int hipq_batch_matmul_f32(const float* a, const float* b, float* out, int64_t ba
         return HIPQ_OK;
     HIPQ_REQUIRE(out && (K == 0 || (a && b)), "null pointer");
     HIPQ_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15) == 0, "the output must be 16-byte aligned");
-    HIPQ_REQUIRE(M < (1ll << 31) && K < (1ll << 31) && N < (1ll << 31), "extent too large");
-    const int64_t m_tiles = (M + TM - 1) / TM, n_tiles = (N + TN - 1) / TN;
-    // 16-byte loads along the operands' rows when every row starts aligned
-    const int vec_a = (reinterpret_cast<uintptr_t>(a) & 15) == 0 && (transpose_a ? M : K) % 4 == 0;
-    const int vec_b = (reinterpret_cast<uintptr_t>(b) & 15) == 0 && (transpose_b ? K : N) % 4 == 0;
-    HIPQ_REQUIRE(batch * m_tiles * n_tiles < (1ll << 31), "too many tiles for one launch");
-    batch_matmul_f32_kernel<<<static_cast<unsigned>(batch * m_tiles * n_tiles), 256, 0, as_stream(stream)>>>(a, b, out, static_cast<int32_t>(M), static_cast<int32_t>(K), static_cast<int32_t>(N),
-                                                                                                              transpose_a ? 1 : 0, transpose_b ? 1 : 0, static_cast<int32_t>(m_tiles),
-                                                                                                              static_cast<int32_t>(n_tiles), vec_a, vec_b);
-    return check_launch("batch_matmul_f32");
+    const MatView view{1, M * K, 0, transpose_a ? M : K, K * N, 0, transpose_b ? K : N, M * N, 0, N};
+    return launch_batch_matmul(a, b, out, view, MatQuant{nullptr, nullptr, nullptr, HIPQ_I8, HIPQ_ROUND_NEAREST_TOWARD_EVEN}, batch, M, K, N, transpose_a, transpose_b, stream);
+}
+
+int hipq_batch_matmul_view_f32(const float* a, const float* b, float* out, const hipq_matmul_view_t* v, const hipq_quant_out_t* q, int64_t batch, int64_t M, int64_t K, int64_t N,
+                               int32_t transpose_a, int32_t transpose_b, void* stream)
+{
+    HIPQ_REQUIRE(v, "null view");
+    HIPQ_REQUIRE(batch >= 0 && M >= 0 && K >= 0 && N >= 0, "negative extent");
+    if (batch == 0 || M == 0 || N == 0)
+        return HIPQ_OK;
+    MatQuant mq{nullptr, nullptr, nullptr, HIPQ_I8, HIPQ_ROUND_NEAREST_TOWARD_EVEN};
+    if (q)
+    {
+        HIPQ_REQUIRE(q->out && q->scale, "quantized output: null pointer");
+        HIPQ_REQUIRE(q->quant_t == HIPQ_I8 || q->quant_t == HIPQ_U8, "quantized output: i8 or u8");
+        HIPQ_REQUIRE(q->round_mode >= HIPQ_ROUND_NEAREST_TOWARD_INFINITY && q->round_mode <= HIPQ_ROUND_DOWN, "quantized output: unknown round mode");
+        mq = MatQuant{q->out, q->scale, q->zero_point, q->quant_t, q->round_mode};
+    }
+    HIPQ_REQUIRE((out || mq.out) && (K == 0 || (a && b)), "null pointer");
+    HIPQ_REQUIRE(v->batch_inner >= 1, "batch_inner must be at least 1");
+    HIPQ_REQUIRE(v->lda >= (transpose_a ? M : K) && v->ldb >= (transpose_b ? K : N) && v->ldo >= N, "a row stride is shorter than the row");
+    HIPQ_REQUIRE(v->a_outer >= 0 && v->a_inner >= 0 && v->b_outer >= 0 && v->b_inner >= 0 && v->o_outer >= 0 && v->o_inner >= 0, "negative batch stride");
+    const MatView view{v->batch_inner, v->a_outer, v->a_inner, v->lda, v->b_outer, v->b_inner, v->ldb, v->o_outer, v->o_inner, v->ldo};
+    return launch_batch_matmul(a, b, out, view, mq, batch, M, K, N, transpose_a, transpose_b, stream);
 }

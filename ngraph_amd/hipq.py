@@ -151,6 +151,18 @@ class PoolDesc(C.Structure):
 POOL_MAX, POOL_AVG = 0, 1
 
 
+class QuantOut(C.Structure):
+    """hipq_quant_out_t: a Quantize of a kernel's f32 result written beside it"""
+
+    _fields_ = [("out", C.c_void_p), ("scale", C.c_void_p), ("zero_point", C.c_void_p), ("quant_t", C.c_int32), ("round_mode", C.c_int32)]
+
+
+class MatmulView(C.Structure):
+    """hipq_matmul_view_t: batch strides (two levels) and row strides of a, b and out, in elements"""
+
+    _fields_ = [(n, C.c_int64) for n in ("batch_inner", "a_outer", "a_inner", "lda", "b_outer", "b_inner", "ldb", "o_outer", "o_inner", "ldo")]
+
+
 class DeviceInfo(C.Structure):
     _fields_ = [
         ("name", C.c_char * 64),
@@ -302,6 +314,10 @@ EXPORTS = [
     "hipq_gelu_f32",
     "hipq_layer_norm_f32",
     "hipq_batch_matmul_f32",
+    "hipq_softmax_scaled_f32",
+    "hipq_gelu_quantize_f32",
+    "hipq_add_layer_norm_f32",
+    "hipq_batch_matmul_view_f32",
 ]
 
 _lib = None
@@ -758,3 +774,72 @@ def batch_matmul(a, b, transpose_a=False, transpose_b=False):
     check(lib.hipq_stream_sync(None))
     r = out.to_numpy(np.float32, (batch, M, N))
     return r[0] if squeeze else r
+
+
+# ---- fused forms: each equals the op-by-op sequence it replaces bit for bit
+
+
+def _quant_out(n, scale, zp, quant_t, round_mode):
+    qt = dtype_code(quant_t)
+    out = DeviceBuffer(max(n, 4))
+    bs, bz = _dev(np.asarray(scale, dtype=np.float32)), _dev(np.asarray(zp, dtype=NP_OF[qt]))
+    return QuantOut(out.ptr, bs.ptr, bz.ptr, qt, round_mode), (out, bs, bz), qt
+
+
+def softmax_scaled(x, factor):
+    """Softmax(x * factor) over the last axis in one launch"""
+    lib = load()
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    src, dst, fac = _dev(x), DeviceBuffer(max(x.nbytes, 4)), _dev(np.asarray(factor, dtype=np.float32))
+    lib.hipq_softmax_scaled_f32.argtypes = [C.c_void_p] * 3 + [C.c_int64] * 3 + [C.c_void_p]
+    check(lib.hipq_softmax_scaled_f32(src.ptr, fac.ptr, dst.ptr, int(np.prod(x.shape[:-1], dtype=np.int64)), x.shape[-1], 1, None))
+    check(lib.hipq_stream_sync(None))
+    return dst.to_numpy(np.float32, x.shape)
+
+
+def add_layer_norm(a, b, scale, bias, epsilon=1e-5, q_scale=None, q_zp=0, quant_t="i8", round_mode=RNE):
+    """LayerNorm(a + b) over the last axis (b may be None); with q_scale also Quantize of the result: returns (norm, q or None)"""
+    lib = load()
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    rows, cols = int(np.prod(a.shape[:-1], dtype=np.int64)), a.shape[-1]
+    ba, bb = _dev(a), (_dev(np.ascontiguousarray(b, dtype=np.float32)) if b is not None else None)
+    sc, bi = _dev(np.ascontiguousarray(scale, dtype=np.float32)), _dev(np.ascontiguousarray(bias, dtype=np.float32))
+    dst = DeviceBuffer(max(a.nbytes, 4))
+    q = keep = qt = None
+    if q_scale is not None:
+        q, keep, qt = _quant_out(a.size, q_scale, q_zp, quant_t, round_mode)
+    lib.hipq_add_layer_norm_f32.argtypes = [C.c_void_p] * 6 + [C.c_int64, C.c_int64, C.c_double, C.c_void_p]
+    check(lib.hipq_add_layer_norm_f32(ba.ptr, bb.ptr if bb else None, sc.ptr, bi.ptr, dst.ptr, C.byref(q) if q else None, rows, cols, float(epsilon), None))
+    check(lib.hipq_stream_sync(None))
+    return dst.to_numpy(np.float32, a.shape), (keep[0].to_numpy(NP_OF[qt], a.shape) if q else None)
+
+
+def gelu_quantize(x, q_scale, q_zp=0, quant_t="i8", round_mode=RNE, keep_f32=True):
+    """Gelu(x) and Quantize(Gelu(x)) in one launch: returns (gelu or None, q)"""
+    lib = load()
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    src = _dev(x)
+    dst = DeviceBuffer(max(x.nbytes, 4)) if keep_f32 else None
+    q, keep, qt = _quant_out(x.size, q_scale, q_zp, quant_t, round_mode)
+    lib.hipq_gelu_quantize_f32.argtypes = [C.c_void_p] * 3 + [C.c_int64, C.c_void_p]
+    check(lib.hipq_gelu_quantize_f32(src.ptr, dst.ptr if dst else None, C.byref(q), x.size, None))
+    check(lib.hipq_stream_sync(None))
+    return (dst.to_numpy(np.float32, x.shape) if dst else None), keep[0].to_numpy(NP_OF[qt], x.shape)
+
+
+def batch_matmul_view(a, a_off, b, b_off, out_elems, out_off, view, batch, M, K, N, transpose_a=False, transpose_b=False, q_scale=None, q_zp=0, quant_t="i8", keep_f32=True):
+    """hipq_batch_matmul_view_f32 on flat f32 buffers a and b (element offsets a_off, b_off) into a flat
+    zero-initialised output of out_elems elements: returns (out or None, q or None)"""
+    lib = load()
+    a, b = np.ascontiguousarray(a, dtype=np.float32).ravel(), np.ascontiguousarray(b, dtype=np.float32).ravel()
+    ba, bb = _dev(a), _dev(b)
+    dst = DeviceBuffer.from_numpy(np.zeros(out_elems, np.float32)) if keep_f32 else None
+    q = keep = qt = None
+    if q_scale is not None:
+        q, keep, qt = _quant_out(out_elems, q_scale, q_zp, quant_t, RNE)
+        check(lib.hipq_fill_bytes(keep[0].ptr, 0, out_elems, None))
+    lib.hipq_batch_matmul_view_f32.argtypes = [C.c_void_p] * 5 + [C.c_int64] * 4 + [C.c_int32] * 2 + [C.c_void_p]
+    check(lib.hipq_batch_matmul_view_f32(ba.ptr + 4 * a_off, bb.ptr + 4 * b_off, (dst.ptr + 4 * out_off) if dst else None, C.byref(view), C.byref(q) if q else None, batch, M, K, N,
+                                         1 if transpose_a else 0, 1 if transpose_b else 0, None))
+    check(lib.hipq_stream_sync(None))
+    return (dst.to_numpy(np.float32, (out_elems,)) if dst else None), (keep[0].to_numpy(NP_OF[qt], (out_elems,)) if q else None)

@@ -130,7 +130,7 @@ def test_device_plan_against_oracle_pipeline(gpu_lib):
     lib = gpu_lib
     sp = H.C.c_void_p()
     H.check(lib.hipq_stream_create(H.C.byref(sp)))
-    plan = B.DevicePlan(lib, sp.value, 4, SMALL)
+    plan = B.DevicePlan(lib, sp.value, 4, SMALL, fused=False)
     assert len(plan.calls) == 19 * SMALL.layers
     plan.set_input(x)
     plan.launch()
@@ -149,6 +149,20 @@ def test_device_plan_against_oracle_pipeline(gpu_lib):
     # the HIP provider's op-at-a-time pass takes the same kernels: identical to the plan
     hp, _ = B.run(B.HipProvider, x, SMALL)
     assert np.array_equal(hp, eager)
+    # the fused plan (10 launches a layer: reshapes as views, Multiply in Softmax, Add in LayerNorm, every
+    # Quantize in its producer) gives the same bits, eager and replayed
+    fused = B.DevicePlan(lib, sp.value, 4, SMALL, fused=True)
+    assert len(fused.calls) == 10 * SMALL.layers + 1
+    fused.set_input(x)
+    fused.launch()
+    assert np.array_equal(fused.read_output(), eager)
+    fused.capture()
+    for _ in range(2):
+        fused.set_input(x)
+        H.check(lib.hipq_stream_sync(None))
+        fused.replay()
+        assert np.array_equal(fused.read_output(), eager)
+    fused.close()
 
 
 @pytest.mark.gpu
@@ -176,7 +190,7 @@ def test_benchmarked_batch_base_dims(gpu_lib):
     sp = H.C.c_void_p()
     H.check(lib.hipq_stream_create(H.C.byref(sp)))
     print("[case] bert base plan, batch 2", flush=True)
-    small = B.DevicePlan(lib, sp.value, 2, B.BASE)
+    small = B.DevicePlan(lib, sp.value, 2, B.BASE, fused=False)
     assert len(small.calls) == 19 * 12
     small.set_input(two)
     small.launch()
@@ -187,7 +201,14 @@ def test_benchmarked_batch_base_dims(gpu_lib):
     assert diff.mean() < 0.05 and np.mean(diff > 0.5) < 0.001
     print("[case] bert base plan, batch 32", flush=True)
     x = np.ascontiguousarray(np.tile(two, (16, 1)))
+    unfused = B.DevicePlan(lib, sp.value, 32, B.BASE, fused=False)
+    unfused.set_input(x)
+    unfused.launch()
+    assert np.array_equal(unfused.read_output(), np.tile(ref, (16, 1)))
+    del unfused
+    # what bench.py times: the fused plan (10 launches a layer), bit for bit the op-by-op result
     plan = B.DevicePlan(lib, sp.value, 32, B.BASE)
+    assert plan.fused and len(plan.calls) == 10 * 12 + 1
     plan.set_input(x)
     plan.launch()
     eager = plan.read_output()

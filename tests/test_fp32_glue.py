@@ -186,3 +186,74 @@ def test_batch_matmul_reference_vectors(gpu_lib):
     # two matrices
     x, y = synth.normal_f32(53, (10, 20)), synth.normal_f32(54, (20, 6))
     assert np.allclose(H.batch_matmul(x, y), x.astype(np.float64) @ y.astype(np.float64), rtol=1e-5, atol=1e-5)
+
+
+# ---- fused forms: equal to the op-by-op sequence they replace, bit for bit ------------------------
+
+
+@pytest.mark.parametrize("shape", [(32 * 12 * 128, 128), (7, 128), (5, 300), (3, 2052), (9, 131), (50, 20)])
+def test_softmax_scaled_equals_multiply_then_softmax(gpu_lib, shape):
+    say("softmax scaled", shape)
+    x = synth.normal_f32(41, shape) * f32(7.0)
+    for c in (0.125, 0.3):
+        got = H.softmax_scaled(x, c)
+        exp = H.softmax(H.binary("multiply", x, np.asarray([c], dtype=f32)), (len(shape) - 1,))
+        assert np.array_equal(got.view(np.uint32), exp.view(np.uint32)), c
+
+
+@pytest.mark.parametrize("shape", [(4096, 768), (9, 768), (5, 30), (3, 2050), (6, 4)])
+def test_add_layer_norm_with_quantized_output(gpu_lib, shape):
+    say("add + layer norm + quantize", shape)
+    a, b = synth.normal_f32(42, shape), synth.normal_f32(43, shape) * f32(0.3)
+    gamma, beta = synth.uniform_f32(44, (shape[-1],), 0.8, 1.2), synth.uniform_f32(45, (shape[-1],), -0.1, 0.1)
+    summed = H.binary("add", a, b)
+    exp = H.layer_norm(summed, gamma, beta, begin_norm_axis=len(shape) - 1, epsilon=1e-5, keep_stats=False)[0]
+    got, q = H.add_layer_norm(a, b, gamma, beta, 1e-5)
+    assert q is None and np.array_equal(got.view(np.uint32), exp.view(np.uint32))
+    for quant_t, zp, s in (("i8", 0, 6.0 / 127.0), ("i8", -3, 0.02), ("u8", 128, 0.03)):
+        got, q = H.add_layer_norm(a, b, gamma, beta, 1e-5, q_scale=s, q_zp=zp, quant_t=quant_t)
+        assert np.array_equal(got.view(np.uint32), exp.view(np.uint32)), quant_t
+        assert np.array_equal(q, H.quantize(exp, f32(s), zp, quant_t)), (quant_t, zp)
+        assert len(np.unique(q)) > 5
+    # without the addend: plain LayerNorm with the quantized copy
+    plain = H.layer_norm(a, gamma, beta, begin_norm_axis=len(shape) - 1, epsilon=1e-5, keep_stats=False)[0]
+    got, q = H.add_layer_norm(a, None, gamma, beta, 1e-5, q_scale=0.05)
+    assert np.array_equal(got.view(np.uint32), plain.view(np.uint32)) and np.array_equal(q, H.quantize(plain, f32(0.05), 0, "i8"))
+
+
+@pytest.mark.parametrize("n", [3, 4096, 4099, 4096 * 3072])
+def test_gelu_with_quantized_output(gpu_lib, n):
+    say("gelu + quantize", n)
+    x = synth.normal_f32(46, (n,)) * f32(2.0)
+    exp = H.gelu(x)
+    for quant_t, zp, s in (("i8", 0, 4.0 * 0.02 * 27.7 / 127.0), ("u8", 7, 0.01)):
+        g, q = H.gelu_quantize(x, s, zp, quant_t)
+        assert np.array_equal(g.view(np.uint32), exp.view(np.uint32))
+        assert np.array_equal(q, H.quantize(exp, f32(s), zp, quant_t)), (quant_t, zp)
+        g, q2 = H.gelu_quantize(x, s, zp, quant_t, keep_f32=False)
+        assert g is None and np.array_equal(q2, q)
+
+
+@pytest.mark.parametrize("B,S,nh,hd", [(2, 128, 12, 64), (3, 9, 2, 8), (2, 7, 3, 5)])
+def test_batch_matmul_views_are_attention_without_the_reshapes(gpu_lib, B, S, nh, hd):
+    """scores and context of an attention layer straight from the fused [tokens, 3 * hidden] projection
+    and into the merged-heads layout, against the same products on permuted copies"""
+    say("matmul views", B, S, nh, hd)
+    h = nh * hd
+    qkv = synth.normal_f32(47, (B * S, 3 * h))
+    heads = np.ascontiguousarray(qkv.reshape(B, S, 3, nh, hd).transpose(2, 0, 3, 1, 4))
+    Q, K, V = (heads[i].reshape(B * nh, S, hd) for i in range(3))
+    exp_scores = H.batch_matmul(Q, K, False, True)
+    v_scores = H.MatmulView(nh, S * 3 * h, hd, 3 * h, S * 3 * h, hd, 3 * h, nh * S * S, S * S, S)
+    got_scores, _ = H.batch_matmul_view(qkv, 0, qkv, h, B * nh * S * S, 0, v_scores, B * nh, S, hd, S, False, True)
+    assert np.array_equal(got_scores.view(np.uint32), exp_scores.ravel().view(np.uint32))
+    probs = H.softmax(exp_scores * f32(0.125), (2,))
+    exp_ctx = H.batch_matmul(probs, V, False, False)
+    exp_merged = np.ascontiguousarray(exp_ctx.reshape(B, nh, S, hd).transpose(0, 2, 1, 3)).reshape(B * S, h)
+    v_ctx = H.MatmulView(nh, nh * S * S, S * S, S, S * 3 * h, hd, 3 * h, S * h, hd, h)
+    s_c = 0.4 / 127.0
+    got_ctx, q = H.batch_matmul_view(probs, 0, qkv, 2 * h, B * S * h, 0, v_ctx, B * nh, S, S, hd, False, False, q_scale=s_c)
+    assert np.array_equal(got_ctx.view(np.uint32), exp_merged.ravel().view(np.uint32))
+    assert np.array_equal(q, H.quantize(exp_merged, f32(s_c), 0, "i8").ravel())
+    _, q_only = H.batch_matmul_view(probs, 0, qkv, 2 * h, B * S * h, 0, v_ctx, B * nh, S, S, hd, False, False, q_scale=s_c, keep_f32=False)
+    assert np.array_equal(q_only, q)

@@ -986,3 +986,33 @@ def test_mfma_requant_ties(gpu_lib):
     for s in (1.5, 3.0e8):
         assert np.array_equal(H.quantized_dot(d32, a, w, s, 0, 1.0, 0, 1.0, 0), O.quantized_dot(d32, a, w, s, 0, 1.0, 0, 1.0, 0)), s
         assert np.array_equal(H.quantized_dot(d, a, w, s, 0, 1.0, 0, 1.0, 5), O.quantized_dot(d, a, w, s, 0, 1.0, 0, 1.0, 5)), s
+
+
+@pytest.mark.parametrize("shape", [(65, 1088, 64), (200, 1152, 130), (256, 2048, 48), (129, 1024, 1000), (192, 3008, 200)])
+def test_dot_rows64(gpu_lib, shape):
+    """the whole-reduction kernel for 65-256 rows: ragged row and column tiles, reductions that end in
+    half a 128-byte piece (K % 128 == 64) or leave wavefronts without a piece, signed and unsigned
+    data with zero points, both requantization policies, every output type, and the exact path for a
+    non-zero weight zero point"""
+    M, K, N = shape
+    say("dot rows64", shape)
+    O.port().orc_set_threads(8)
+    w = synth.uniform_int(1502, (N, K), -128, 127, np.int8)
+    for a_t, lo, hi in (("u8", 0, 255), ("i8", -128, 127)):
+        a = synth.uniform_int(1501, (M, K), lo, hi, H.NP_OF[H.dtype_code(a_t)])
+        for out_t, s, z in (("i32", (1.0, 1.0, 1.0), (0, 0, 0)), ("i8", (0.01, 0.01, 2.5), (5 if a_t == "u8" else -5, 0, 4)), ("u8", (0.01, 0.01, 2.5), (0, 3, 9))):
+            d = H.make_dot_desc(M, K, N, a_t=a_t, out_t=out_t, b_layout=H.B_NK)
+            exp = O.quantized_dot(d, a, w, s[0], z[0], s[1], z[1], s[2], z[2])
+            got = H.quantized_dot(d, a, w, s[0], z[0], s[1], z[1], s[2], z[2])
+            assert H.last_kernel().startswith("dot_rows64"), H.last_kernel()
+            assert np.array_equal(got, exp), (a_t, out_t, z)
+        bias = synth.uniform_int(1503, (N,), -(2**15), 2**15, np.int32)
+        scales = synth.uniform_f32(1504, (N,), 0.001, 0.01) * np.float32(0.05)
+        for out_t, relu in (("i8", False), ("u8", True), ("f32", True)):
+            d = H.make_dot_desc(M, K, N, a_t=a_t, out_t=out_t, b_layout=H.B_NK)
+            f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
+            exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
+            got = H.quantized_dot_bias(d, f, a, w, bias, scales)
+            assert H.last_kernel().startswith("dot_rows64"), H.last_kernel()
+            assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), (a_t, out_t, relu)
+    O.port().orc_set_threads(1)

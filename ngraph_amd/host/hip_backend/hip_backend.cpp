@@ -11,6 +11,7 @@
 #include <map>
 #include <mutex>
 #include <unordered_map>
+#include <unordered_set>
 
 #include "hipq.h"
 #include "ngraph/ngraph.hpp"
@@ -158,6 +159,7 @@ namespace
         void lower_dot(const shared_ptr<Node>& n, Step& st);
         void lower_pool(const shared_ptr<Node>& n, Step& st);
         void assign_layouts();
+        void plan_glue_fusion();
         bool nxc(const Node* n) const { return m_nxc.count(n) != 0; }
         shared_ptr<DeviceBlock> alloc(size_t bytes)
         {
@@ -171,6 +173,25 @@ namespace
         shared_ptr<Function> m_function;
         unordered_map<const Node*, int> m_value_of; // node -> value id of its output 0
         unordered_map<const Node*, bool> m_nxc;     // nodes whose output tensor is kept channels-last
+        // f32 glue folded into its neighbours (plan_glue_fusion): nodes that get no launch of their own ...
+        unordered_set<const Node*> m_folded;
+        // ... a Softmax that multiplies its input by a constant first, a LayerNorm that adds two tensors
+        // first, and a LayerNorm / Gelu that also writes the Quantize of its result
+        struct ScaledInput
+        {
+            Output<Node> x;
+            float factor;
+        };
+        unordered_map<const Node*, ScaledInput> m_softmax_of_product;
+        unordered_map<const Node*, pair<Output<Node>, Output<Node>>> m_layer_norm_of_sum;
+        struct QuantizedCopy
+        {
+            shared_ptr<Node> quantize;
+            float scale;
+            int32_t zero_point;
+            bool only_user; // the f32 result has no other reader
+        };
+        unordered_map<const Node*, QuantizedCopy> m_quantized_copy;
         vector<void*> m_value_ptr;                  // persistent device pointer, or null when bound per call
         vector<size_t> m_value_bytes;
         vector<int> m_value_uses;
@@ -310,6 +331,94 @@ namespace
                 if (n->get_input_shape(i) == n->get_output_shape(0))
                     r.push_back(i);
         return r;
+    }
+
+    // One f32 value shared by every element of a Constant (also behind Broadcasts): what a graph's
+    // "x * c" looks like before and after constant folding.
+    bool uniform_f32_constant(const Output<Node>& o, float* value)
+    {
+        shared_ptr<Node> n = o.get_node_shared_ptr();
+        while (is_type<op::v0::Broadcast>(n))
+            n = n->get_argument(0);
+        auto c = as_type_ptr<op::v0::Constant>(n);
+        if (!c || c->get_output_element_type(0) != element::f32)
+            return false;
+        const size_t count = shape_size(c->get_output_shape(0));
+        if (count == 0)
+            return false;
+        const float* p = static_cast<const float*>(c->get_data_ptr());
+        for (size_t i = 1; i < count; ++i)
+            if (memcmp(p + i, p, sizeof(float)) != 0)
+                return false;
+        *value = p[0];
+        return true;
+    }
+
+    // Launches that only re-read and re-write a tensor are folded into a neighbour (every fused form
+    // of the library equals the op sequence bit for bit): Multiply by a constant into the Softmax it
+    // feeds, Add into the LayerNorm it feeds, Quantize (one scale and zero point) into the LayerNorm
+    // or Gelu that produces its input.  Switch: NGRAPH_PASS_ENABLES "HIPGlueFusion:0".
+    void HIPExecutable::plan_glue_fusion()
+    {
+        pass::PassConfig config;
+        auto en = config.get_enables().find("HIPGlueFusion");
+        if (en != config.get_enables().end() && !en->second)
+            return;
+        unordered_map<const Node*, vector<const Node*>> users;
+        for (const auto& n : m_function->get_ordered_ops())
+            for (size_t i = 0; i < n->get_input_size(); ++i)
+                users[n->input_value(i).get_node()].push_back(n.get());
+        auto single_user = [&](const Node* n) { return users[n].size() == 1; };
+        for (const auto& n : m_function->get_ordered_ops())
+        {
+            if (auto sm = as_type_ptr<op::v0::Softmax>(n))
+            {
+                auto mul = as_type_ptr<op::v1::Multiply>(n->input_value(0).get_node_shared_ptr());
+                if (!mul || !single_user(mul.get()) || n->get_output_element_type(0) != element::f32 || mul->get_output_shape(0) != n->get_output_shape(0))
+                    continue;
+                for (size_t side = 0; side < 2; ++side)
+                {
+                    float c = 0.0f;
+                    if (mul->get_input_shape(1 - side) == n->get_output_shape(0) && uniform_f32_constant(mul->input_value(side), &c))
+                    {
+                        m_softmax_of_product[n.get()] = ScaledInput{mul->input_value(1 - side), c};
+                        m_folded.insert(mul.get());
+                        break;
+                    }
+                }
+            }
+            else if (auto ln = as_type_ptr<op::v0::LayerNorm>(n))
+            {
+                auto add = as_type_ptr<op::v1::Add>(n->input_value(0).get_node_shared_ptr());
+                if (add && single_user(add.get()) && !ln->get_keep_stats() && n->get_output_element_type(0) == element::f32 &&
+                    add->get_input_shape(0) == add->get_output_shape(0) && add->get_input_shape(1) == add->get_output_shape(0))
+                {
+                    m_layer_norm_of_sum[n.get()] = {add->input_value(0), add->input_value(1)};
+                    m_folded.insert(add.get());
+                }
+            }
+        }
+        for (const auto& n : m_function->get_ordered_ops())
+        {
+            auto q = as_type_ptr<op::v0::Quantize>(n);
+            if (!q || !q->get_axes().empty() || n->get_input_element_type(0) != element::f32)
+                continue;
+            const auto qt = n->get_output_element_type(0);
+            if (qt != element::i8 && qt != element::u8)
+                continue;
+            const Node* producer = n->input_value(0).get_node();
+            const bool from_ln = is_type<op::v0::LayerNorm>(producer) && !static_cast<const op::v0::LayerNorm*>(producer)->get_keep_stats();
+            if (!(from_ln || is_type<op::v0::Gelu>(producer)) || m_quantized_copy.count(producer))
+                continue;
+            auto cs = as_type_ptr<op::v0::Constant>(n->input_value(1).get_node_shared_ptr());
+            auto cz = as_type_ptr<op::v0::Constant>(n->input_value(2).get_node_shared_ptr());
+            if (!cs || !cz || shape_size(cs->get_output_shape(0)) != 1 || shape_size(cz->get_output_shape(0)) != 1)
+                continue;
+            const float scale = *static_cast<const float*>(cs->get_data_ptr());
+            const int32_t zp = qt == element::i8 ? static_cast<int32_t>(*static_cast<const int8_t*>(cz->get_data_ptr())) : static_cast<int32_t>(*static_cast<const uint8_t*>(cz->get_data_ptr()));
+            m_quantized_copy[producer] = QuantizedCopy{n, scale, zp, single_user(producer)};
+            m_folded.insert(n.get());
+        }
     }
 
     void HIPExecutable::assign_layouts()
@@ -603,6 +712,10 @@ namespace
         // value ids and reach the launch as pointers after the inputs
         if (n->get_output_size() != 1 && !is_type<op::v0::LayerNorm>(n))
             throw unsupported_op(string("HIP backend: op '") + n->description() + "' with " + to_string(n->get_output_size()) + " outputs");
+        // folded into a neighbour: no launch and (Multiply, Add) no value; a folded Quantize got its
+        // value when its producer was lowered
+        if (m_folded.count(n.get()))
+            return;
         const auto et = n->get_output_element_type(0);
         const size_t bytes = shape_size(n->get_output_shape(0)) * et.size();
         const int id = static_cast<int>(m_value_ptr.size());
@@ -634,7 +747,15 @@ namespace
         st.output = id;
         for (size_t i = 0; i < n->get_input_size(); ++i)
         {
-            st.inputs.push_back(value_of(n->input_value(i)));
+            // (a folded Multiply / Add in front of input 0: the consumer reads the folded node's inputs instead)
+            const auto sp = m_softmax_of_product.find(n.get());
+            const auto ls = m_layer_norm_of_sum.find(n.get());
+            if (i == 0 && sp != m_softmax_of_product.end())
+                st.inputs.push_back(value_of(sp->second.x));
+            else if (i == 0 && ls != m_layer_norm_of_sum.end())
+                st.inputs.push_back(value_of(ls->second.first));
+            else
+                st.inputs.push_back(value_of(n->input_value(i)));
             m_value_uses[st.inputs.back()] += 1;
         }
         for (size_t o = 1; o < n->get_output_size(); ++o)
@@ -644,6 +765,43 @@ namespace
             m_value_bytes.push_back(obytes);
             m_value_uses.push_back(0);
             st.inputs.push_back(id + static_cast<int>(o)); // written, not read: no use counted
+        }
+        // glue fusion: the second addend of a folded Add, then the quantized copy a folded Quantize stands for
+        int addend_at = -1, qcopy_at = -1;
+        hipq_quant_out_t qcopy;
+        memset(&qcopy, 0, sizeof(qcopy));
+        bool qcopy_only = false;
+        {
+            const auto ls = m_layer_norm_of_sum.find(n.get());
+            if (ls != m_layer_norm_of_sum.end())
+            {
+                addend_at = static_cast<int>(st.inputs.size());
+                st.inputs.push_back(value_of(ls->second.second));
+                m_value_uses[st.inputs.back()] += 1;
+            }
+            const auto qc = m_quantized_copy.find(n.get());
+            if (qc != m_quantized_copy.end())
+            {
+                const shared_ptr<Node>& qn = qc->second.quantize;
+                const size_t qbytes = shape_size(qn->get_output_shape(0));
+                const int qid = static_cast<int>(m_value_ptr.size());
+                m_value_of[qn.get()] = qid;
+                m_value_ptr.push_back(alloc(qbytes)->ptr);
+                m_value_bytes.push_back(qbytes);
+                m_value_uses.push_back(0);
+                qcopy_at = static_cast<int>(st.inputs.size());
+                st.inputs.push_back(qid); // written, not read: no use counted
+                auto scalars = alloc(8);
+                unsigned char host[8] = {0};
+                memcpy(host, &qc->second.scale, sizeof(float));
+                host[4] = static_cast<unsigned char>(qc->second.zero_point & 0xFF);
+                check(hipq_memcpy_h2d(scalars->ptr, host, 8, m_stream), "constant upload");
+                qcopy.scale = static_cast<const float*>(scalars->ptr);
+                qcopy.zero_point = static_cast<const unsigned char*>(scalars->ptr) + 4;
+                qcopy.quant_t = dtype_of(qn->get_output_element_type(0));
+                qcopy.round_mode = static_cast<int32_t>(static_cast<const op::v0::Quantize*>(qn.get())->get_round_mode());
+                qcopy_only = qc->second.only_user;
+            }
         }
         const int64_t count = static_cast<int64_t>(shape_size(n->get_output_shape(0)));
         const int dt = dtype_of(et);
@@ -753,9 +911,21 @@ namespace
             int64_t outer = 1, axis = 1, inner = 1;
             for (size_t i = 0; i < s.size(); ++i)
                 (i < first ? outer : (i <= last ? axis : inner)) *= static_cast<int64_t>(s[i]);
-            st.launch = [outer, axis, inner](const vector<void*>& in, void* out, void* stream) {
-                check(hipq_softmax_f32(static_cast<const float*>(in[0]), static_cast<float*>(out), outer, axis, inner, stream), "Softmax");
-            };
+            const auto product = m_softmax_of_product.find(n.get());
+            if (product != m_softmax_of_product.end())
+            {
+                // Softmax(Multiply(x, c)): the factor as a device scalar of this executable
+                auto block = alloc(sizeof(float));
+                check(hipq_memcpy_h2d(block->ptr, &product->second.factor, sizeof(float), m_stream), "constant upload");
+                const float* factor = static_cast<const float*>(block->ptr);
+                st.launch = [outer, axis, inner, factor](const vector<void*>& in, void* out, void* stream) {
+                    check(hipq_softmax_scaled_f32(static_cast<const float*>(in[0]), factor, static_cast<float*>(out), outer, axis, inner, stream), "Softmax of a product");
+                };
+            }
+            else
+                st.launch = [outer, axis, inner](const vector<void*>& in, void* out, void* stream) {
+                    check(hipq_softmax_f32(static_cast<const float*>(in[0]), static_cast<float*>(out), outer, axis, inner, stream), "Softmax");
+                };
         }
         else if (is_type<op::v0::Erf>(n) || is_type<op::v0::Gelu>(n))
         {
@@ -764,12 +934,19 @@ namespace
                 throw unsupported_op("HIP backend: " + n->description() + " on " + et.get_type_name());
             const int64_t count = static_cast<int64_t>(shape_size(n->get_output_shape(0)));
             const bool gelu = is_type<op::v0::Gelu>(n);
-            st.launch = [count, gelu](const vector<void*>& in, void* out, void* stream) {
-                if (gelu)
-                    check(hipq_gelu_f32(static_cast<const float*>(in[0]), static_cast<float*>(out), count, stream), "Gelu");
-                else
-                    check(hipq_erf_f32(static_cast<const float*>(in[0]), static_cast<float*>(out), count, stream), "Erf");
-            };
+            if (gelu && qcopy_at >= 0)
+                st.launch = [count, qcopy, qcopy_at, qcopy_only](const vector<void*>& in, void* out, void* stream) {
+                    hipq_quant_out_t q = qcopy;
+                    q.out = in[qcopy_at];
+                    check(hipq_gelu_quantize_f32(static_cast<const float*>(in[0]), qcopy_only ? nullptr : static_cast<float*>(out), &q, count, stream), "Gelu with its Quantize");
+                };
+            else
+                st.launch = [count, gelu](const vector<void*>& in, void* out, void* stream) {
+                    if (gelu)
+                        check(hipq_gelu_f32(static_cast<const float*>(in[0]), static_cast<float*>(out), count, stream), "Gelu");
+                    else
+                        check(hipq_erf_f32(static_cast<const float*>(in[0]), static_cast<float*>(out), count, stream), "Erf");
+                };
         }
         else if (auto ln = as_type_ptr<op::v0::LayerNorm>(n))
         {
@@ -788,12 +965,23 @@ namespace
             const double eps = ln->get_epsilon();
             const bool stats = ln->get_keep_stats();
             const size_t first_stat = affine ? 3 : 1;
-            st.launch = [rows, cols, affine, eps, stats, first_stat](const vector<void*>& in, void* out, void* stream) {
-                check(hipq_layer_norm_f32(static_cast<const float*>(in[0]), affine ? static_cast<const float*>(in[1]) : nullptr, affine ? static_cast<const float*>(in[2]) : nullptr,
-                                          static_cast<float*>(out), stats ? static_cast<float*>(in[first_stat]) : nullptr, stats ? static_cast<float*>(in[first_stat + 1]) : nullptr, rows,
-                                          cols, eps, stream),
-                      "LayerNorm");
-            };
+            if (addend_at >= 0 || qcopy_at >= 0)
+                st.launch = [rows, cols, affine, eps, addend_at, qcopy, qcopy_at](const vector<void*>& in, void* out, void* stream) {
+                    hipq_quant_out_t q = qcopy;
+                    if (qcopy_at >= 0)
+                        q.out = in[qcopy_at];
+                    check(hipq_add_layer_norm_f32(static_cast<const float*>(in[0]), addend_at >= 0 ? static_cast<const float*>(in[addend_at]) : nullptr,
+                                                  affine ? static_cast<const float*>(in[1]) : nullptr, affine ? static_cast<const float*>(in[2]) : nullptr, static_cast<float*>(out),
+                                                  qcopy_at >= 0 ? &q : nullptr, rows, cols, eps, stream),
+                          "LayerNorm with its Add / Quantize");
+                };
+            else
+                st.launch = [rows, cols, affine, eps, stats, first_stat](const vector<void*>& in, void* out, void* stream) {
+                    check(hipq_layer_norm_f32(static_cast<const float*>(in[0]), affine ? static_cast<const float*>(in[1]) : nullptr, affine ? static_cast<const float*>(in[2]) : nullptr,
+                                              static_cast<float*>(out), stats ? static_cast<float*>(in[first_stat]) : nullptr, stats ? static_cast<float*>(in[first_stat + 1]) : nullptr,
+                                              rows, cols, eps, stream),
+                          "LayerNorm");
+                };
         }
         else if (is_type<op::v0::BatchMatMul>(n) || is_type<op::v0::BatchMatMulTranspose>(n))
         {
@@ -866,6 +1054,7 @@ namespace
         pm.register_pass<pass::ConstantFolding>();
         pm.run_passes(m_function);
         assign_layouts();
+        plan_glue_fusion();
         for (const auto& n : m_function->get_ordered_ops())
             lower(n);
         for (const auto& p : m_function->get_parameters())

@@ -3,6 +3,8 @@
 // gelu.in.cpp:49-108, layer_norm.in.cpp:48-91 and batch_mat_mul.in.cpp:51-102; type propagation
 // after src/ngraph/op/{softmax,gelu,layer_norm}.cpp and op/experimental/batch_mat_mul.cpp.
 #include <cmath>
+#include <cstdlib>
+#include <set>
 
 #include "test_util.hpp"
 
@@ -216,4 +218,117 @@ CPU_TEST(type_prop, fp32_glue_shapes_and_failures)
     EXPECT_THROW(make_shared<op::v0::BatchMatMul>(a, c), NodeValidationFailure);
     auto m = make_shared<op::v0::Parameter>(element::f32, Shape{3, 7});
     EXPECT_THROW(make_shared<op::v0::BatchMatMul>(a, m), NodeValidationFailure);
+}
+
+// ---- glue fusion of the backend: Multiply into Softmax, Add into LayerNorm, Quantize into the
+// LayerNorm / Gelu that feeds it.  Every fused launch equals the op sequence bit for bit, so the
+// results with NGRAPH_PASS_ENABLES "HIPGlueFusion:0" and with the default must be identical, and the
+// fused executable runs fewer launches (one performance counter a launch).
+namespace
+{
+    struct GlueRun
+    {
+        vector<vector<uint8_t>> bytes; // every result, raw
+        size_t launches;
+    };
+
+    GlueRun run_glue(const shared_ptr<Function>& f, const vector<vector<float>>& args, bool fuse)
+    {
+        setenv("NGRAPH_PASS_ENABLES", fuse ? "HIPGlueFusion:1" : "HIPGlueFusion:0", 1);
+        auto backend = runtime::Backend::create("HIP");
+        vector<shared_ptr<runtime::Tensor>> in, out;
+        for (size_t i = 0; i < args.size(); ++i)
+        {
+            auto t = backend->create_tensor(element::f32, f->get_parameters()[i]->get_output_shape(0));
+            copy_data(t, args[i]);
+            in.push_back(t);
+        }
+        for (size_t i = 0; i < f->get_output_size(); ++i)
+            out.push_back(backend->create_tensor(f->get_output_element_type(i), f->get_output_shape(i)));
+        auto exec = backend->compile(f, true);
+        exec->call_with_validate(out, in);
+        unsetenv("NGRAPH_PASS_ENABLES");
+        GlueRun r;
+        r.launches = exec->get_performance_data().size();
+        for (auto& t : out)
+        {
+            vector<uint8_t> b(shape_size(t->get_shape()) * t->get_element_type().size());
+            t->read(b.data(), b.size());
+            r.bytes.push_back(b);
+        }
+        return r;
+    }
+
+    vector<float> wave(size_t n, float amplitude, float step)
+    {
+        vector<float> v(n);
+        for (size_t i = 0; i < n; ++i)
+            v[i] = amplitude * sinf(step * static_cast<float>(i)) + 0.01f * static_cast<float>(i % 7);
+        return v;
+    }
+}
+
+GPU_TEST(HIP, glue_fusion_softmax_of_a_product)
+{
+    Shape shape{6, 4, 128};
+    auto A = make_shared<op::v0::Parameter>(element::f32, shape);
+    auto c = op::v0::Constant::create(element::f32, Shape{}, {0.125f});
+    auto scaled = make_shared<op::v1::Multiply>(A, make_shared<op::v0::Broadcast>(c, shape, AxisSet{0, 1, 2}));
+    auto f = make_shared<Function>(OutputVector{make_shared<op::v0::Softmax>(scaled, AxisSet{2})}, ParameterVector{A});
+    const auto x = wave(shape_size(shape), 9.0f, 0.37f);
+    const auto plain = run_glue(f, {x}, false), fused = run_glue(f, {x}, true);
+    EXPECT_TRUE(plain.bytes == fused.bytes);
+    EXPECT_TRUE(fused.launches < plain.launches);
+}
+
+GPU_TEST(HIP, glue_fusion_residual_layer_norm_with_quantize)
+{
+    // x1 = LayerNorm(a + b) feeds a Quantize (the next projection) and stays live (the next residual)
+    Shape shape{9, 768};
+    auto a = make_shared<op::v0::Parameter>(element::f32, shape);
+    auto b = make_shared<op::v0::Parameter>(element::f32, shape);
+    auto g = make_shared<op::v0::Parameter>(element::f32, Shape{768});
+    auto be = make_shared<op::v0::Parameter>(element::f32, Shape{768});
+    auto sum = make_shared<op::v1::Add>(a, b);
+    auto ln = make_shared<op::v0::LayerNorm>(sum, g, be, false, 1, 1e-5);
+    auto scale = op::v0::Constant::create(element::f32, Shape{}, {6.0f / 127.0f});
+    auto zp = op::v0::Constant::create(element::i8, Shape{}, {-3});
+    auto q = make_shared<op::v0::Quantize>(ln, scale, zp, element::i8, AxisSet{}, op::v0::Quantize::RoundMode::ROUND_NEAREST_TOWARD_EVEN);
+    auto f = make_shared<Function>(OutputVector{ln, q}, ParameterVector{a, b, g, be});
+    vector<float> gamma(768), beta(768);
+    for (size_t i = 0; i < 768; ++i)
+    {
+        gamma[i] = 0.8f + 0.0005f * static_cast<float>(i);
+        beta[i] = -0.1f + 0.0002f * static_cast<float>(i);
+    }
+    const vector<vector<float>> args{wave(shape_size(shape), 1.0f, 0.11f), wave(shape_size(shape), 0.3f, 0.53f), gamma, beta};
+    const auto plain = run_glue(f, args, false), fused = run_glue(f, args, true);
+    EXPECT_TRUE(plain.bytes == fused.bytes);
+    EXPECT_TRUE(fused.launches + 2 == plain.launches); // Add and Quantize are gone
+    // the quantized copy is not degenerate
+    set<uint8_t> codes(fused.bytes[1].begin(), fused.bytes[1].end());
+    EXPECT_TRUE(codes.size() > 40);
+}
+
+GPU_TEST(HIP, glue_fusion_gelu_with_quantize)
+{
+    Shape shape{5, 3072};
+    auto A = make_shared<op::v0::Parameter>(element::f32, shape);
+    auto gelu = make_shared<op::v0::Gelu>(A);
+    auto scale = op::v0::Constant::create(element::f32, Shape{}, {0.0175f});
+    auto zp = op::v0::Constant::create(element::u8, Shape{}, {16});
+    auto q = make_shared<op::v0::Quantize>(gelu, scale, zp, element::u8, AxisSet{}, op::v0::Quantize::RoundMode::ROUND_NEAREST_TOWARD_EVEN);
+    const auto x = wave(shape_size(shape), 2.5f, 0.071f);
+    {
+        auto f = make_shared<Function>(OutputVector{q}, ParameterVector{A}); // the Quantize is Gelu's only reader
+        const auto plain = run_glue(f, {x}, false), fused = run_glue(f, {x}, true);
+        EXPECT_TRUE(plain.bytes == fused.bytes);
+        EXPECT_TRUE(fused.launches + 1 == plain.launches);
+    }
+    {
+        auto f = make_shared<Function>(OutputVector{q, gelu}, ParameterVector{A}); // ... and with the f32 result live as well
+        const auto plain = run_glue(f, {x}, false), fused = run_glue(f, {x}, true);
+        EXPECT_TRUE(plain.bytes == fused.bytes);
+        EXPECT_TRUE(fused.launches + 1 == plain.launches);
+    }
 }

@@ -33,6 +33,7 @@ namespace hipq
 
     inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
     int check_launch(const char* kernel);
+    int device_compute_units(); // compute units of the current device (cached per device; 256 when the query fails)
 
     // Grow-only device workspace, one per (device, stream): launches on different streams never
     // share a block, so callers that run on streams of their own may overlap.  Growing a block waits

@@ -770,20 +770,6 @@ namespace hipq
         return true;
     }
 
-    static int regw_slots()
-    {
-        static int cus[16] = {};
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16)
-            return 256;
-        if (cus[dev] == 0)
-        {
-            hipDeviceProp_t prop;
-            cus[dev] = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-        }
-        return cus[dev];
-    }
-
     bool conv_regw_eligible(const ConvGeom& g, bool out_ncx)
     {
         RegwParams rp;
@@ -811,7 +797,7 @@ namespace hipq
     {
         RegwParams rp;
         size_t lds_bytes = 0;
-        HIPQ_REQUIRE(regw_plan(g, out_ncx, regw_slots(), &rp, &lds_bytes), "layer does not fit the filter-in-registers convolution");
+        HIPQ_REQUIRE(regw_plan(g, out_ncx, device_compute_units(), &rp, &lds_bytes), "layer does not fit the filter-in-registers convolution");
         HIPQ_REQUIRE((reinterpret_cast<uintptr_t>(data) & 15) == 0 && (reinterpret_cast<uintptr_t>(packed) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0,
                      "convolution needs 16-byte aligned tensors");
         rp.x = static_cast<const uint8_t*>(data);

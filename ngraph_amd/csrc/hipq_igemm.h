@@ -1758,21 +1758,6 @@ namespace hipq
         return check_launch(name);
     }
 
-    // compute units of the current device (cached per device)
-    static inline int device_compute_units()
-    {
-        static int cus[16] = {};
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16)
-            return 256;
-        if (cus[dev] == 0)
-        {
-            hipDeviceProp_t prop;
-            cus[dev] = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-        }
-        return cus[dev];
-    }
-
     template <class XL, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM, int KIND = OUT_Q8, int BKT = BK>
     static int launch_pipe(const XL& xl,
                            const int8_t* w,

@@ -1,10 +1,18 @@
 // f32 batched matrix product (attention scores and contexts of a transformer encoder; op::v0::Dot on
-// two matrices is the batch of one).  64 x 64 output tiles, 16-deep steps through LDS, 4 x 4 outputs a
-// lane in registers.  The reference accumulates f32 products in double, k ascending
-// (src/ngraph/runtime/reference/dot.hpp:34-37 with widen<float> = double,
-// convolution.hpp:34-44), and rounds the sum to f32 once; so does this kernel: a product of two
-// floats is exact in double, hence the fused multiply-add rounds exactly as the reference's separate
-// multiply and add, and the results are the reference's bit for bit.
+// two matrices is the batch of one).  64 x 64 output tiles, 16-deep steps through LDS (f32), every
+// wavefront a 32 x 32 quarter as 2 x 2 blocks of v_mfma_f64_16x16x4_f64.  The reference accumulates
+// f32 products in double, k ascending (src/ngraph/runtime/reference/dot.hpp:34-37 with widen<float> =
+// double, convolution.hpp:34-44), and rounds the sum to f32 once.  A product of two floats is exact
+// in double, so a fused multiply-add rounds exactly as the reference's separate multiply and add;
+// and the f64 matrix instruction accumulates its four products as a chain of such multiply-adds in
+// k order (checked on the device against the chain: a million outputs over uniform, wide-range,
+// integer-valued and cancelling operands, no bit differed -- and every parity test of this kernel
+// is bit-exact against the oracle's sequential sum): the results are the reference's bit for bit.
+// Operands are converted to double as fragments, one element a lane and matrix instruction, which
+// is what makes the matrix instruction pay: the vector form converts eight operands for sixteen
+// multiply-adds and is bound by the conversions.
+#include <algorithm>
+
 #include "hipq_common.h"
 #include "hipq_quant_math.h"
 
@@ -13,7 +21,8 @@ namespace hipq
     namespace
     {
         typedef float f4 __attribute__((ext_vector_type(4)));
-        constexpr int TM = 64, TN = 64, TK = 16;
+        typedef double d4 __attribute__((ext_vector_type(4)));
+        constexpr int TM = 64, TN = 64, TK = 64, TKS = 16; // a stage is TK of the reduction, fetched and laid into LDS in pieces of TKS
 
         // where the matrices of batch element (outer, inner) start and how far apart their rows are (in
         // elements): the plain op has one batch level and dense matrices; views of a larger tensor
@@ -33,146 +42,137 @@ namespace hipq
             int32_t quant_t, mode;
         };
 
-        // out[b] = op(A[b]) * op(B[b]): A is [M][K] (or [K][M] with ta), B is [K][N] (or [N][K] with tb)
-        __global__ __launch_bounds__(256) void batch_matmul_f32_kernel(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ out, MatView view, MatQuant mq, int32_t M,
-                                                                       int32_t K, int32_t N, int32_t ta, int32_t tb, int32_t m_tiles, int32_t n_tiles, int32_t vec_a, int32_t vec_b,
-                                                                       int32_t vec_o)
+        // out[b] = op(A[b]) * op(B[b]): A is [M][K] (or [K][M] with ta), B is [K][N] (or [N][K] with tb).
+        // A workgroup walks tiles item, item + grid, ...; the operands of the next stage -- the next
+        // tile's first one after a tile's last -- are on their way into registers while this stage
+        // multiplies, and a tile's stores drain under the next tile's products.  (One tile a workgroup,
+        // all resident at once, runs the whole grid in lockstep: everyone loads, then everyone
+        // multiplies, then everyone stores, and the three times add up.)
+#ifndef BMM_PER_CU
+#define BMM_PER_CU 3
+#endif
+#ifndef BMM_OCC
+#define BMM_OCC __attribute__((amdgpu_waves_per_eu(3, 3)))
+#endif
+        struct TileAt
+        {
+            const float* A;
+            const float* B;
+            int64_t o_base;
+            int m0, n0;
+        };
+
+        // WHOLE: every tile is full (M, N multiples of 64, K of TK) and every row 16-byte aligned, so
+        // fetches and stores carry no bounds checks or scalar alternatives (uniform, chosen by the host)
+        template <bool WHOLE, bool ta, bool tb>
+        __global__ __launch_bounds__(256) BMM_OCC void batch_matmul_f32_kernel(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ out, MatView view, MatQuant mq, int32_t M,
+                                                                       int32_t K, int32_t N, int32_t m_tiles, int32_t n_tiles, int32_t tiles, int32_t vec_a, int32_t vec_b)
         {
             __shared__ __attribute__((aligned(16))) float as[TK][TM + 4]; // [k][m]
             __shared__ __attribute__((aligned(16))) float bs[TK][TN + 4]; // [k][n]
             const int tid = threadIdx.x;
-            int t = blockIdx.x;
-            const int nt = t % n_tiles;
-            t /= n_tiles;
-            const int mt = t % m_tiles;
-            const int64_t batch = t / m_tiles;
-            const int64_t bo = batch / view.batch_inner, bi = batch - bo * view.batch_inner;
-            const float* A = a + bo * view.a_outer + bi * view.a_inner;
-            const float* B = b + bo * view.b_outer + bi * view.b_inner;
-            const int64_t o_base = bo * view.o_outer + bi * view.o_inner;
-            float* O = out ? out + o_base : nullptr;
             const int64_t lda = view.lda, ldb = view.ldb, ldo = view.ldo;
-            const int m0 = mt * TM, n0 = nt * TN;
-            const int tm = (tid >> 4) * 4, tn = (tid & 15) * 4; // this lane's 4 x 4 outputs within the tile
-            double acc[4][4] = {};
-            // 64 x 16 elements of each operand, four a lane, contiguous along the operand's rows in
-            // memory; the next step's elements are fetched into registers while this step multiplies
-            auto fetch_a = [&](int k0) -> f4 {
+            const int lane = tid & 63, wave = tid >> 6;
+            const int r16 = lane & 15, kq = lane >> 4;          // fragment element: row / column r16 of a block, k = 4 * step + kq
+            const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32; // this wavefront's quarter of the tile
+            // workgroups are dealt round-robin to the 8 XCDs (an L2 each): renumbered so that
+            // neighbouring tiles, which share operand rows, meet in one L2
+            const int grid = static_cast<int>(gridDim.x);
+            const int item = (grid & 7) == 0 ? (static_cast<int>(blockIdx.x) & 7) * (grid >> 3) + (static_cast<int>(blockIdx.x) >> 3) : static_cast<int>(blockIdx.x);
+            const uint32_t batch_inner = static_cast<uint32_t>(view.batch_inner < (1ll << 31) ? view.batch_inner : (1ll << 31)); // (there are fewer than 2^31 tiles)
+            auto tile_at = [&](int t) -> TileAt {
+                const int nt = t % n_tiles;
+                t /= n_tiles;
+                const int mt = t % m_tiles;
+                const uint32_t batch = static_cast<uint32_t>(t / m_tiles);
+                const int64_t bo = batch / batch_inner, bi = batch - bo * batch_inner; // (32-bit division)
+                return TileAt{a + bo * view.a_outer + bi * view.a_inner, b + bo * view.b_outer + bi * view.b_inner, bo * view.o_outer + bi * view.o_inner, mt * TM, nt * TN};
+            };
+            // 64 x 16 elements of each operand a piece, four a lane, contiguous along the operand's rows in memory
+            auto fetch_a = [&](const TileAt& w, int k0) -> f4 {
                 f4 v = f4{0.0f, 0.0f, 0.0f, 0.0f};
                 if (!ta)
                 {
                     const int r = tid >> 2, kq = (tid & 3) * 4; // A[m0 + r][k0 + kq ..]
-                    if (vec_a && m0 + r < M && k0 + kq + 3 < K)
-                        v = *reinterpret_cast<const f4*>(A + static_cast<int64_t>(m0 + r) * lda + k0 + kq);
+                    if (WHOLE || (vec_a && w.m0 + r < M && k0 + kq + 3 < K))
+                        v = *reinterpret_cast<const f4*>(w.A + static_cast<int64_t>(w.m0 + r) * lda + k0 + kq);
                     else
                     {
 #pragma unroll
                         for (int i = 0; i < 4; ++i)
-                            v[i] = (m0 + r < M && k0 + kq + i < K) ? A[static_cast<int64_t>(m0 + r) * lda + k0 + kq + i] : 0.0f;
+                            v[i] = (w.m0 + r < M && k0 + kq + i < K) ? w.A[static_cast<int64_t>(w.m0 + r) * lda + k0 + kq + i] : 0.0f;
                     }
                 }
                 else
                 {
                     const int kk = tid >> 4, mq = (tid & 15) * 4; // A[k0 + kk][m0 + mq ..]
-                    if (vec_a && k0 + kk < K && m0 + mq + 3 < M)
-                        v = *reinterpret_cast<const f4*>(A + static_cast<int64_t>(k0 + kk) * lda + m0 + mq);
+                    if (WHOLE || (vec_a && k0 + kk < K && w.m0 + mq + 3 < M))
+                        v = *reinterpret_cast<const f4*>(w.A + static_cast<int64_t>(k0 + kk) * lda + w.m0 + mq);
                     else
                     {
 #pragma unroll
                         for (int i = 0; i < 4; ++i)
-                            v[i] = (k0 + kk < K && m0 + mq + i < M) ? A[static_cast<int64_t>(k0 + kk) * lda + m0 + mq + i] : 0.0f;
+                            v[i] = (k0 + kk < K && w.m0 + mq + i < M) ? w.A[static_cast<int64_t>(k0 + kk) * lda + w.m0 + mq + i] : 0.0f;
                     }
                 }
                 return v;
             };
-            auto put_a = [&](f4 v) {
+            auto put_a = [&](f4 v, int kbase) {
                 if (!ta)
                 {
                     const int r = tid >> 2, kq = (tid & 3) * 4;
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
-                        as[kq + i][r] = v[i];
+                        as[kbase + kq + i][r] = v[i];
                 }
                 else
                 {
                     const int kk = tid >> 4, mq = (tid & 15) * 4;
-                    *reinterpret_cast<f4*>(&as[kk][mq]) = v;
+                    *reinterpret_cast<f4*>(&as[kbase + kk][mq]) = v;
                 }
             };
-            auto fetch_b = [&](int k0) -> f4 {
+            auto fetch_b = [&](const TileAt& w, int k0) -> f4 {
                 f4 v = f4{0.0f, 0.0f, 0.0f, 0.0f};
                 if (!tb)
                 {
                     const int kk = tid >> 4, nq = (tid & 15) * 4; // B[k0 + kk][n0 + nq ..]
-                    if (vec_b && k0 + kk < K && n0 + nq + 3 < N)
-                        v = *reinterpret_cast<const f4*>(B + static_cast<int64_t>(k0 + kk) * ldb + n0 + nq);
+                    if (WHOLE || (vec_b && k0 + kk < K && w.n0 + nq + 3 < N))
+                        v = *reinterpret_cast<const f4*>(w.B + static_cast<int64_t>(k0 + kk) * ldb + w.n0 + nq);
                     else
                     {
 #pragma unroll
                         for (int i = 0; i < 4; ++i)
-                            v[i] = (k0 + kk < K && n0 + nq + i < N) ? B[static_cast<int64_t>(k0 + kk) * ldb + n0 + nq + i] : 0.0f;
+                            v[i] = (k0 + kk < K && w.n0 + nq + i < N) ? w.B[static_cast<int64_t>(k0 + kk) * ldb + w.n0 + nq + i] : 0.0f;
                     }
                 }
                 else
                 {
                     const int r = tid >> 2, kq = (tid & 3) * 4; // B[n0 + r][k0 + kq ..]
-                    if (vec_b && n0 + r < N && k0 + kq + 3 < K)
-                        v = *reinterpret_cast<const f4*>(B + static_cast<int64_t>(n0 + r) * ldb + k0 + kq);
+                    if (WHOLE || (vec_b && w.n0 + r < N && k0 + kq + 3 < K))
+                        v = *reinterpret_cast<const f4*>(w.B + static_cast<int64_t>(w.n0 + r) * ldb + k0 + kq);
                     else
                     {
 #pragma unroll
                         for (int i = 0; i < 4; ++i)
-                            v[i] = (n0 + r < N && k0 + kq + i < K) ? B[static_cast<int64_t>(n0 + r) * ldb + k0 + kq + i] : 0.0f;
+                            v[i] = (w.n0 + r < N && k0 + kq + i < K) ? w.B[static_cast<int64_t>(w.n0 + r) * ldb + k0 + kq + i] : 0.0f;
                     }
                 }
                 return v;
             };
-            auto put_b = [&](f4 v) {
+            auto put_b = [&](f4 v, int kbase) {
                 if (!tb)
                 {
                     const int kk = tid >> 4, nq = (tid & 15) * 4;
-                    *reinterpret_cast<f4*>(&bs[kk][nq]) = v;
+                    *reinterpret_cast<f4*>(&bs[kbase + kk][nq]) = v;
                 }
                 else
                 {
                     const int r = tid >> 2, kq = (tid & 3) * 4;
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
-                        bs[kq + i][r] = v[i];
+                        bs[kbase + kq + i][r] = v[i];
                 }
             };
-            f4 va = fetch_a(0), vb = fetch_b(0);
-            for (int k0 = 0; k0 < K; k0 += TK)
-            {
-                put_a(va);
-                put_b(vb);
-                __syncthreads();
-                if (k0 + TK < K) // uniform
-                {
-                    va = fetch_a(k0 + TK);
-                    vb = fetch_b(k0 + TK);
-                }
-#pragma unroll
-                for (int k = 0; k < TK; ++k)
-                {
-                    // (past K both operands hold zeros: + 0 * 0 leaves a sum as it is -- a sum that started from +0 is never -0)
-                    const f4 av = *reinterpret_cast<const f4*>(&as[k][tm]);
-                    const f4 bv = *reinterpret_cast<const f4*>(&bs[k][tn]);
-                    double ad[4], bd[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                    {
-                        ad[i] = static_cast<double>(av[i]);
-                        bd[i] = static_cast<double>(bv[i]);
-                    }
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-#pragma unroll
-                        for (int j = 0; j < 4; ++j)
-                            acc[i][j] = fma(ad[i], bd[j], acc[i][j]);
-                }
-                __syncthreads();
-            }
             // (the optional quantized copy: Quantize of the f32 result, the arithmetic of hipq_quantize)
             const float qs = mq.out ? *mq.scale : 1.0f;
             const int32_t qz = mq.out ? load_zp(mq.zero_point, mq.quant_t) : 0;
@@ -180,34 +180,137 @@ namespace hipq
                 return mq.quant_t == HIPQ_U8 ? static_cast<uint32_t>(quantize_one<float, uint8_t>(v, qs, static_cast<uint8_t>(qz), mq.mode))
                                              : static_cast<uint32_t>(static_cast<uint8_t>(quantize_one<float, int8_t>(v, qs, static_cast<int8_t>(qz), mq.mode)));
             };
+            d4 acc[2][2];
+            auto clear = [&]() {
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-            {
-                const int m = m0 + tm + i;
-                if (m >= M)
-                    continue;
-                const int64_t at = static_cast<int64_t>(m) * ldo + n0 + tn;
-                const f4 r = f4{static_cast<float>(acc[i][0]), static_cast<float>(acc[i][1]), static_cast<float>(acc[i][2]), static_cast<float>(acc[i][3])};
-                if (n0 + tn + 3 < N && vec_o)
-                {
-                    if (O)
-                        *reinterpret_cast<f4*>(O + at) = r;
-                    if (mq.out)
-                        *reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(mq.out) + o_base + at) = q1(r[0]) | (q1(r[1]) << 8) | (q1(r[2]) << 16) | (q1(r[3]) << 24);
-                }
-                else
-                {
+                for (int i = 0; i < 2; ++i)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        if (n0 + tn + j < N)
+                    for (int j = 0; j < 2; ++j)
+                        acc[i][j] = d4{0.0, 0.0, 0.0, 0.0};
+            };
+            // block (i, j), register e of lane (r16, kq): row wm + 16 i + 4 e + kq, column wn + 16 j + r16.
+            // A finished tile is rounded to f32 into `res` and stored one stage later, after the next
+            // tile's operands have arrived: loads and stores share one counter, so stores issued just
+            // before that wait would have to be acknowledged before the next tile could start.
+            float res[2][2][4];
+            auto round_tile = [&]() {
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            res[i][j][e] = static_cast<float>(acc[i][j][e]);
+            };
+            auto each_result = [&](const TileAt& w, auto&& f) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                    {
+                        const int m = w.m0 + wm + i * 16 + 4 * e + kq;
+                        if (!WHOLE && m >= M)
+                            continue;
+#pragma unroll
+                        for (int j = 0; j < 2; ++j)
                         {
-                            if (O)
-                                O[at + j] = r[j];
-                            if (mq.out)
-                                static_cast<uint8_t*>(mq.out)[o_base + at + j] = static_cast<uint8_t>(q1(r[j]));
+                            const int n = w.n0 + wn + j * 16 + r16;
+                            if (!WHOLE && n >= N)
+                                continue;
+                            f(w.o_base + static_cast<int64_t>(m) * ldo + n, res[i][j][e]);
                         }
+                    }
+            };
+            auto store_tile = [&](const TileAt& w) {
+                if (out) // uniform
+                    each_result(w, [&](int64_t at, float r) { out[at] = r; });
+                if (mq.out) // uniform
+                    each_result(w, [&](int64_t at, float r) { static_cast<uint8_t*>(mq.out)[at] = static_cast<uint8_t>(q1(r)); });
+            };
+
+            if (item >= tiles) // uniform
+                return;
+            // a stage is TK of the reduction (the whole reduction of an attention score), asked for at once
+            constexpr int PIECES = TK / TKS;
+            int t_fetch = item, k_fetch = 0, k_done = 0;
+            TileAt ft = tile_at(t_fetch); // the tile whose operands are being fetched
+            TileAt ct = ft;               // the tile being multiplied
+            TileAt st = ft;               // the finished tile waiting in `res`
+            bool unsaved = false;         // uniform
+            f4 va[PIECES], vb[PIECES];
+#pragma unroll
+            for (int q = 0; q < PIECES; ++q)
+            {
+                va[q] = fetch_a(ft, q * TKS);
+                vb[q] = fetch_b(ft, q * TKS);
+            }
+            clear();
+            for (;;)
+            {
+#pragma unroll
+                for (int q = 0; q < PIECES; ++q)
+                {
+                    put_a(va[q], q * TKS);
+                    put_b(vb[q], q * TKS);
+                }
+                __syncthreads();
+                // the stage after this one: of this tile, or the first of the workgroup's next tile
+                bool more = true; // uniform
+                k_fetch += TK;
+                if (k_fetch >= K)
+                {
+                    k_fetch = 0;
+                    t_fetch += grid;
+                    more = t_fetch < tiles;
+                    if (more)
+                        ft = tile_at(t_fetch);
+                }
+                if (more)
+                {
+#pragma unroll
+                    for (int q = 0; q < PIECES; ++q)
+                    {
+                        va[q] = fetch_a(ft, k_fetch + q * TKS);
+                        vb[q] = fetch_b(ft, k_fetch + q * TKS);
+                    }
+                }
+                if (unsaved)
+                {
+                    store_tile(st);
+                    unsaved = false;
+                }
+#pragma unroll
+                for (int k = 0; k < TK; k += 4)
+                {
+                    // (past K both operands hold zeros: + 0 * 0 leaves a sum as it is -- a sum that started from +0 is never -0)
+                    double ad[2], bd[2];
+#pragma unroll
+                    for (int i = 0; i < 2; ++i)
+                    {
+                        ad[i] = static_cast<double>(as[k + kq][wm + i * 16 + r16]);
+                        bd[i] = static_cast<double>(bs[k + kq][wn + i * 16 + r16]);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 2; ++i)
+#pragma unroll
+                        for (int j = 0; j < 2; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(ad[i], bd[j], acc[i][j], 0, 0, 0);
+                }
+                __syncthreads();
+                k_done += TK;
+                if (k_done >= K) // the tile's last stage: the fetch cursor stands on the next tile
+                {
+                    round_tile();
+                    st = ct;
+                    if (!more)
+                        break;
+                    unsaved = true;
+                    clear();
+                    k_done = 0;
+                    ct = ft;
                 }
             }
+            store_tile(st);
         }
     }
 }
@@ -223,11 +326,21 @@ static int launch_batch_matmul(const float* a, const float* b, float* out, const
     auto all4 = [](int64_t x, int64_t y, int64_t z) { return x % 4 == 0 && y % 4 == 0 && z % 4 == 0; };
     const int vec_a = (reinterpret_cast<uintptr_t>(a) & 15) == 0 && all4(view.lda, view.a_outer, view.a_inner);
     const int vec_b = (reinterpret_cast<uintptr_t>(b) & 15) == 0 && all4(view.ldb, view.b_outer, view.b_inner);
-    const int vec_o = (!out || (reinterpret_cast<uintptr_t>(out) & 15) == 0) && (!mq.out || (reinterpret_cast<uintptr_t>(mq.out) & 3) == 0) && all4(view.ldo, view.o_outer, view.o_inner);
-    HIPQ_REQUIRE(batch * m_tiles * n_tiles < (1ll << 31), "too many tiles for one launch");
-    batch_matmul_f32_kernel<<<static_cast<unsigned>(batch * m_tiles * n_tiles), 256, 0, as_stream(stream)>>>(a, b, out, view, mq, static_cast<int32_t>(M), static_cast<int32_t>(K),
-                                                                                                              static_cast<int32_t>(N), transpose_a ? 1 : 0, transpose_b ? 1 : 0,
-                                                                                                              static_cast<int32_t>(m_tiles), static_cast<int32_t>(n_tiles), vec_a, vec_b, vec_o);
+    HIPQ_REQUIRE(batch * m_tiles * n_tiles < (1ll << 31) - (1 << 20), "too many tiles for one launch");
+    const int64_t tiles = batch * m_tiles * n_tiles;
+    // three workgroups a compute unit (their LDS and the 12 wavefronts they make fit), each walking its share of the tiles
+    const int64_t grid = std::min<int64_t>(tiles, static_cast<int64_t>(BMM_PER_CU) * device_compute_units());
+    const bool whole = M % TM == 0 && N % TN == 0 && K % TK == 0 && K > 0 && vec_a && vec_b;
+#define BMM_LAUNCH(W, TA, TB)                                                                                                                                                            \
+    batch_matmul_f32_kernel<W, TA, TB><<<static_cast<unsigned>(grid), 256, 0, as_stream(stream)>>>(a, b, out, view, mq, static_cast<int32_t>(M), static_cast<int32_t>(K), static_cast<int32_t>(N), \
+                                                                                                     static_cast<int32_t>(m_tiles), static_cast<int32_t>(n_tiles), static_cast<int32_t>(tiles), vec_a, vec_b)
+#define BMM_T(W) (transpose_a ? (transpose_b ? BMM_LAUNCH(W, true, true) : BMM_LAUNCH(W, true, false)) : (transpose_b ? BMM_LAUNCH(W, false, true) : BMM_LAUNCH(W, false, false)))
+    if (whole)
+        BMM_T(true);
+    else
+        BMM_T(false);
+#undef BMM_T
+#undef BMM_LAUNCH
     return check_launch("batch_matmul_f32");
 }
 

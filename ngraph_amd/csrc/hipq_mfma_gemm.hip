@@ -512,20 +512,6 @@ namespace hipq
         }
     }
 
-    static int rows64_cus()
-    {
-        static int cus[16] = {};
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16)
-            return 256;
-        if (cus[dev] == 0)
-        {
-            hipDeviceProp_t prop;
-            cus[dev] = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-        }
-        return cus[dev];
-    }
-
     // More than 64 rows, a long reduction, and too few 128 x 128 tiles to give every compute unit one
     // without splitting reductions; at most two rounds of 64 x 64 tiles.
     static bool dot_rows64_eligible(const hipq_dot_desc_t& d)
@@ -534,7 +520,7 @@ namespace hipq
             return false;
         const int64_t tiles64 = ((d.M + 63) / 64) * ((d.N + 63) / 64);
         const int64_t tiles128 = ((d.M + 127) / 128) * ((d.N + 127) / 128);
-        const int cus = rows64_cus();
+        const int cus = device_compute_units();
         return tiles128 * 4 < 3 * cus && tiles64 <= 2 * cus && d.M * d.K < (1ll << 31) && d.N * d.K < (1ll << 31);
     }
 

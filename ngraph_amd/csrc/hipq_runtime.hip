@@ -30,6 +30,20 @@ namespace hipq
         return HIPQ_OK;
     }
 
+    int device_compute_units()
+    {
+        static int cus[16] = {};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16)
+            return 256;
+        if (cus[dev] == 0)
+        {
+            hipDeviceProp_t prop;
+            cus[dev] = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        }
+        return cus[dev];
+    }
+
     __global__ void fill_bytes_kernel(uint8_t* dst, uint32_t pattern, size_t bytes);
 
     static const int kMaxDevices = 16;

@@ -1,6 +1,6 @@
 // f32 batched matrix product (attention scores and contexts of a transformer encoder; op::v0::Dot on
-// two matrices is the batch of one).  64 x 64 output tiles, 16-deep steps through LDS (f32), every
-// wavefront a 32 x 32 quarter as 2 x 2 blocks of v_mfma_f64_16x16x4_f64.  The reference accumulates
+// two matrices is the batch of one).  64 x 64 output tiles, the reduction in stages of 64 through
+// LDS (f32), every wavefront a 32 x 32 quarter as 2 x 2 blocks of v_mfma_f64_16x16x4_f64.  The reference accumulates
 // f32 products in double, k ascending (src/ngraph/runtime/reference/dot.hpp:34-37 with widen<float> =
 // double, convolution.hpp:34-44), and rounds the sum to f32 once.  A product of two floats is exact
 // in double, so a fused multiply-add rounds exactly as the reference's separate multiply and add;
@@ -68,8 +68,16 @@ namespace hipq
         __global__ __launch_bounds__(256) BMM_OCC void batch_matmul_f32_kernel(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ out, MatView view, MatQuant mq, int32_t M,
                                                                        int32_t K, int32_t N, int32_t m_tiles, int32_t n_tiles, int32_t tiles, int32_t vec_a, int32_t vec_b)
         {
-            __shared__ __attribute__((aligned(16))) float as[TK][TM + 4]; // [k][m]
-            __shared__ __attribute__((aligned(16))) float bs[TK][TN + 4]; // [k][n]
+            // An operand lies in LDS the way it lies in memory, so that every piece goes in as one 16-byte
+            // write: [row][k] when its rows run along the reduction (A as given, B transposed), [k][row]
+            // otherwise.  The pitches spread a fragment read (16 rows x 4 consecutive k a wavefront)
+            // over all 64 banks: 68 floats a row ([row][k]: bank 4 row + k), 80 floats a k ([k][row]: bank 16 k + row).
+            constexpr int PR = TK + 4, PK = TM + 16;
+            constexpr int OPERAND = TM * PR > TK * PK ? TM * PR : TK * PK;
+            __shared__ __attribute__((aligned(16))) float as[OPERAND];
+            __shared__ __attribute__((aligned(16))) float bs[OPERAND];
+            auto a_at = [](int k, int m) { return ta ? k * PK + m : m * PR + k; };
+            auto b_at = [](int k, int n) { return tb ? n * PR + k : k * PK + n; };
             const int tid = threadIdx.x;
             const int64_t lda = view.lda, ldb = view.ldb, ldo = view.ldo;
             const int lane = tid & 63, wave = tid >> 6;
@@ -121,14 +129,12 @@ namespace hipq
                 if (!ta)
                 {
                     const int r = tid >> 2, kq = (tid & 3) * 4;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        as[kbase + kq + i][r] = v[i];
+                    *reinterpret_cast<f4*>(&as[a_at(kbase + kq, r)]) = v;
                 }
                 else
                 {
                     const int kk = tid >> 4, mq = (tid & 15) * 4;
-                    *reinterpret_cast<f4*>(&as[kbase + kk][mq]) = v;
+                    *reinterpret_cast<f4*>(&as[a_at(kbase + kk, mq)]) = v;
                 }
             };
             auto fetch_b = [&](const TileAt& w, int k0) -> f4 {
@@ -163,14 +169,12 @@ namespace hipq
                 if (!tb)
                 {
                     const int kk = tid >> 4, nq = (tid & 15) * 4;
-                    *reinterpret_cast<f4*>(&bs[kbase + kk][nq]) = v;
+                    *reinterpret_cast<f4*>(&bs[b_at(kbase + kk, nq)]) = v;
                 }
                 else
                 {
                     const int r = tid >> 2, kq = (tid & 3) * 4;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        bs[kbase + kq + i][r] = v[i];
+                    *reinterpret_cast<f4*>(&bs[b_at(kbase + kq, r)]) = v;
                 }
             };
             // (the optional quantized copy: Quantize of the f32 result, the arithmetic of hipq_quantize)
@@ -287,8 +291,8 @@ namespace hipq
 #pragma unroll
                     for (int i = 0; i < 2; ++i)
                     {
-                        ad[i] = static_cast<double>(as[k + kq][wm + i * 16 + r16]);
-                        bd[i] = static_cast<double>(bs[k + kq][wn + i * 16 + r16]);
+                        ad[i] = static_cast<double>(as[a_at(k + kq, wm + i * 16 + r16)]);
+                        bd[i] = static_cast<double>(bs[b_at(k + kq, wn + i * 16 + r16)]);
                     }
 #pragma unroll
                     for (int i = 0; i < 2; ++i)

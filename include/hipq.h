@@ -595,6 +595,37 @@ HIPQ_API int hipq_batch_matmul_view_f32(const float* a,
                                         int32_t transpose_b,
                                         void* stream);
 
+/* Attention of a batch of heads in one launch:
+ *   out = BatchMatMul(Softmax(Multiply(BatchMatMulTranspose(Q, K), *factor)), V)
+ * -- the sub-graph between the QKV projection and the output projection of a transformer encoder
+ * (src/ngraph/runtime/reference/batch_mat_mul.hpp:31-57, softmax.hpp:31-57, multiply.hpp), with
+ * an optional Quantize of the result.  Equal, bit for bit, to hipq_batch_matmul_view_f32 (transpose_b),
+ * hipq_softmax_scaled_f32 and hipq_batch_matmul_view_f32 in sequence; the [queries, keys] scores stay
+ * on the compute unit.  Q is [queries, depth], K and V are [keys, depth] per batch element, addressed
+ * like the views above (strides in elements); factor may be null (no Multiply); out may be null when
+ * quant is given.  Returns HIPQ_ERR_UNSUPPORTED (nothing launched) unless keys == 128, depth == 64 and
+ * queries is a multiple of 32: callers then run the three ops.  No counterpart as a single reference op. */
+typedef struct hipq_attention_view
+{
+    int64_t batch_inner;
+    int64_t q_outer, q_inner, ldq;
+    int64_t k_outer, k_inner, ldk;
+    int64_t v_outer, v_inner, ldv;
+    int64_t o_outer, o_inner, ldo;
+} hipq_attention_view_t;
+HIPQ_API int hipq_attention_f32(const float* q,
+                                const float* k,
+                                const float* v,
+                                const float* factor,
+                                float* out,
+                                const hipq_attention_view_t* view,
+                                const hipq_quant_out_t* quant,
+                                int64_t batch,
+                                int64_t queries,
+                                int64_t keys,
+                                int64_t depth,
+                                void* stream);
+
 /* Which kernel the last hipq_quantized_* call on this thread used: "mfma", "direct", ... (host
  * string, never NULL).  For tests and profiles. */
 HIPQ_API const char* hipq_last_kernel(void);

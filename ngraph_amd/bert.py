@@ -163,10 +163,10 @@ class DevicePlan:
     the kernel launches of every layer on `stream`; `capture()` turns the pass into one HIP graph.
 
     fused=False launches the graph op by op, 19 launches a layer.  fused=True (what a backend's fusion
-    pass makes of the same graph, 10 launches a layer) folds the ops that only re-read and re-write a
+    pass makes of the same graph, 10 launches a layer, 8 where a head has 128 keys of depth 64) folds the ops that only re-read and re-write a
     tensor into their producers, each through an entry point whose result equals the op-by-op one bit
-    for bit: the head split and merge become views of the attention products, Multiply goes into
-    Softmax, the residual Add into LayerNorm, and every Quantize into the kernel that produces its
+    for bit: the head split and merge become views of the attention products (scores, Softmax and
+    context of a head are one kernel at 128 keys of depth 64), Multiply goes into Softmax, the residual Add into LayerNorm, and every Quantize into the kernel that produces its
     input (the context product, LayerNorm, Gelu)."""
 
     def __init__(self, lib, stream, batch, cfg=BASE, fused=True):
@@ -212,20 +212,27 @@ class DevicePlan:
             lib.hipq_gelu_quantize_f32.argtypes = [vp, vp, vp, i64, vp]
             lib.hipq_add_layer_norm_f32.argtypes = [vp] * 6 + [i64, i64, C.c_double, vp]
             lib.hipq_batch_matmul_view_f32.argtypes = [vp] * 5 + [i64] * 4 + [i32] * 2 + [vp]
+            lib.hipq_attention_f32.argtypes = [vp] * 7 + [i64] * 4 + [vp]
             qout = {s: self._keep(H.QuantOut(x8.ptr, scales[s].ptr, zero.ptr, H.I8, H.RNE)) for s in scales}
             H3 = 3 * h
             # Q, K, V of batch element (b, head): rows of the [T, 3H] projection, 3H apart, starting at column
             # {0, H, 2H} + head * hd; scores [B * heads, S, S] dense; the context goes straight into [T, H]
             v_scores = self._keep(H.MatmulView(nh, S * H3, hd, H3, S * H3, hd, H3, nh * S * S, S * S, S))
             v_context = self._keep(H.MatmulView(nh, nh * S * S, S * S, S, S * H3, hd, H3, S * h, hd, h))
+            # 128 keys of depth 64: scores, Softmax and context of a head in one kernel
+            self.one_kernel_attention = S == 128 and hd == 64
+            v_attention = self._keep(H.AttentionView(nh, S * H3, hd, H3, S * H3, hd, H3, S * H3, hd, H3, S * h, hd, h))
             for l in range(cfg.layers):
                 w = layer_weights(cfg, l)
                 if l == 0:
                     quantize(self.x, h, cfg.s_x)
                 dot(w["qkv"], h, H3, qkv)
-                call(lib.hipq_batch_matmul_view_f32, qkv, (qkv, h * 4), scores, v_scores, None, batch * nh, S, hd, S, 0, 1)
-                call(lib.hipq_softmax_scaled_f32, scores, inv, probs, batch * nh * S, S, 1)
-                call(lib.hipq_batch_matmul_view_f32, probs, (qkv, 2 * h * 4), None, v_context, qout[cfg.s_c], batch * nh, S, S, hd, 0, 0)
+                if self.one_kernel_attention:
+                    call(lib.hipq_attention_f32, qkv, (qkv, h * 4), (qkv, 2 * h * 4), inv, None, v_attention, qout[cfg.s_c], batch * nh, S, S, hd)
+                else:
+                    call(lib.hipq_batch_matmul_view_f32, qkv, (qkv, h * 4), scores, v_scores, None, batch * nh, S, hd, S, 0, 1)
+                    call(lib.hipq_softmax_scaled_f32, scores, inv, probs, batch * nh * S, S, 1)
+                    call(lib.hipq_batch_matmul_view_f32, probs, (qkv, 2 * h * 4), None, v_context, qout[cfg.s_c], batch * nh, S, S, hd, 0, 0)
                 dot(w["out"], h, h, proj)
                 g1, b1 = dev(w["ln1"][0]), dev(w["ln1"][1])
                 call(lib.hipq_add_layer_norm_f32, self.x, proj, g1, b1, x1, qout[cfg.s_x], T, h, 1e-5)

@@ -15,6 +15,7 @@
 
 #include "hipq_common.h"
 #include "hipq_quant_math.h"
+#include "hipq_row_math.h"
 
 namespace hipq
 {
@@ -316,6 +317,227 @@ namespace hipq
             }
             store_tile(st);
         }
+
+        // ---- attention of one head in one kernel -------------------------------------------------------
+        // out = BatchMatMul(Softmax(Multiply(BatchMatMulTranspose(Q, K), factor)), V), every op rounding
+        // as the separate kernels round (the products through the same matrix instruction chain, the
+        // Softmax through softmax_piece with the same lanes on the same pieces), so the result equals
+        // the three launches bit for bit while the scores never leave the compute unit.
+        // A work item is 32 query rows of one head against its 128 keys of depth 64.  LDS: Q [32][64],
+        // K [128][64], V [128][64] as f32; the scores and probabilities [32][132] take K's place once K
+        // has been multiplied.  Rows of Q and K are swizzled by k ^ 4 (row % 16), rows of V by
+        // n ^ 16 (key % 4): fragment reads (16 rows x 4 consecutive k a wavefront) and the 16-byte
+        // writes touch every bank once, without padding, which is what lets two workgroups share a
+        // compute unit's 160 KB.
+        // A workgroup walks items: V is asked for when the item starts and laid into LDS after the
+        // scores, the next item's Q and K are asked for before the second product, and an item's
+        // results wait in registers until the next item's operands have arrived (loads and stores
+        // share one counter).
+        constexpr int AQ = 32, AKEYS = 128, AD = 64, ASP = AKEYS + 4;
+        constexpr size_t kAttnLdsBytes = static_cast<size_t>(AQ * AD + 2 * AKEYS * AD) * sizeof(float);
+        static_assert(AQ * ASP <= AKEYS * AD, "the scores must fit K's region");
+        struct AttnView
+        {
+            int64_t batch_inner;
+            int64_t q_outer, q_inner, ldq;
+            int64_t k_outer, k_inner, ldk;
+            int64_t v_outer, v_inner, ldv;
+            int64_t o_outer, o_inner, ldo;
+        };
+        struct AttnItem
+        {
+            const float* Q;
+            const float* K;
+            const float* V;
+            int64_t o_base;
+        };
+
+        __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attention_f32_kernel(const float* __restrict__ q, const float* __restrict__ k,
+                                                                                                                 const float* __restrict__ v, const float* __restrict__ factor,
+                                                                                                                 float* __restrict__ out, AttnView view, MatQuant mq, int32_t row_blocks,
+                                                                                                                 int32_t items)
+        {
+            extern __shared__ __attribute__((aligned(16))) float attn_lds[];
+            float* const Qs = attn_lds;
+            float* const Ks = Qs + AQ * AD;
+            float* const Vs = Ks + AKEYS * AD;
+            float* const Ss = Ks;
+            const int tid = threadIdx.x;
+            const int lane = tid & 63, wave = tid >> 6;
+            const int r16 = lane & 15, kq = lane >> 4;
+            const int64_t ldq = view.ldq, ldk = view.ldk, ldv = view.ldv, ldo = view.ldo;
+            const bool scaled = factor != nullptr;
+            const float c = scaled ? *factor : 1.0f;
+            const int grid = static_cast<int>(gridDim.x);
+            // (workgroups are dealt round-robin to the 8 XCDs: renumbered so that the row blocks of a head meet in one L2)
+            const int first = (grid & 7) == 0 ? (static_cast<int>(blockIdx.x) & 7) * (grid >> 3) + (static_cast<int>(blockIdx.x) >> 3) : static_cast<int>(blockIdx.x);
+            if (first >= items) // uniform
+                return;
+            const uint32_t batch_inner = static_cast<uint32_t>(view.batch_inner < (1ll << 31) ? view.batch_inner : (1ll << 31));
+            auto item_at = [&](int t) -> AttnItem {
+                const int rb = t % row_blocks;
+                const uint32_t batch = static_cast<uint32_t>(t / row_blocks);
+                const int64_t bo = batch / batch_inner, bi = batch - bo * batch_inner;
+                return AttnItem{q + bo * view.q_outer + bi * view.q_inner + static_cast<int64_t>(rb) * AQ * ldq, k + bo * view.k_outer + bi * view.k_inner,
+                                v + bo * view.v_outer + bi * view.v_inner, bo * view.o_outer + bi * view.o_inner + static_cast<int64_t>(rb) * AQ * ldo};
+            };
+            // a thread's 16-byte pieces: row tid / 16 (+ 16 a piece), columns 4 (tid % 16) ..
+            const int prow = tid >> 4, pcol = (tid & 15) * 4;
+            f4 rq[2], rk[8], rv[8];
+            auto fetch_qk = [&](const AttnItem& w) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    rq[i] = *reinterpret_cast<const f4*>(w.Q + static_cast<int64_t>(prow + 16 * i) * ldq + pcol);
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    rk[i] = *reinterpret_cast<const f4*>(w.K + static_cast<int64_t>(prow + 16 * i) * ldk + pcol);
+            };
+            auto fetch_v = [&](const AttnItem& w) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    rv[i] = *reinterpret_cast<const f4*>(w.V + static_cast<int64_t>(prow + 16 * i) * ldv + pcol);
+            };
+            auto put_qk = [&]() {
+                const int at = prow * AD + (pcol ^ (4 * prow)); // (row % 16 = tid / 16 for every piece of the thread)
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    *reinterpret_cast<f4*>(Qs + at + i * 16 * AD) = rq[i];
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    *reinterpret_cast<f4*>(Ks + at + i * 16 * AD) = rk[i];
+            };
+            auto put_v = [&]() {
+                const int at = prow * AD + (pcol ^ (16 * (prow & 3))); // (key % 4 = (tid / 16) % 4 for every piece)
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    *reinterpret_cast<f4*>(Vs + at + i * 16 * AD) = rv[i];
+            };
+            const float qs = mq.out ? *mq.scale : 1.0f;
+            const int32_t qz = mq.out ? load_zp(mq.zero_point, mq.quant_t) : 0;
+            auto q1 = [&](float x) -> uint32_t {
+                return mq.quant_t == HIPQ_U8 ? static_cast<uint32_t>(quantize_one<float, uint8_t>(x, qs, static_cast<uint8_t>(qz), mq.mode))
+                                             : static_cast<uint32_t>(static_cast<uint8_t>(quantize_one<float, int8_t>(x, qs, static_cast<int8_t>(qz), mq.mode)));
+            };
+            // second product: block i, register e of lane (r16, kq) = row 16 i + 4 e + kq, column 16 wave + r16
+            float res[2][4];
+            auto store_item = [&](const AttnItem& w) {
+                if (out) // uniform
+                {
+#pragma unroll
+                    for (int i = 0; i < 2; ++i)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            out[w.o_base + static_cast<int64_t>(16 * i + 4 * e + kq) * ldo + 16 * wave + r16] = res[i][e];
+                }
+                if (mq.out) // uniform
+                {
+#pragma unroll
+                    for (int i = 0; i < 2; ++i)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            static_cast<uint8_t*>(mq.out)[w.o_base + static_cast<int64_t>(16 * i + 4 * e + kq) * ldo + 16 * wave + r16] = static_cast<uint8_t>(q1(res[i][e]));
+                }
+            };
+
+            int t = first;
+            AttnItem cur = item_at(t);
+            AttnItem done = cur;
+            bool unsaved = false; // uniform
+            fetch_qk(cur);
+            for (;;)
+            {
+                put_qk();
+                __syncthreads();
+                fetch_v(cur);
+                if (unsaved)
+                {
+                    store_item(done);
+                    unsaved = false;
+                }
+                // ---- scores: 32 x 128 over depth 64; this wavefront the 32 keys 32 wave .. as 2 x 2 blocks
+                d4 acc[2][2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc[i][j] = d4{0.0, 0.0, 0.0, 0.0};
+                {
+                    const float* const qa = Qs + r16 * AD + kq;
+                    const float* const kb = Ks + (32 * wave + r16) * AD + kq;
+#pragma unroll
+                    for (int s = 0; s < AD / 4; ++s)
+                    {
+                        const int off = (4 * s) ^ (4 * r16);
+                        double ad[2], bd[2];
+#pragma unroll
+                        for (int i = 0; i < 2; ++i)
+                        {
+                            ad[i] = static_cast<double>(qa[off + i * 16 * AD]);
+                            bd[i] = static_cast<double>(kb[off + i * 16 * AD]);
+                        }
+#pragma unroll
+                        for (int i = 0; i < 2; ++i)
+#pragma unroll
+                            for (int j = 0; j < 2; ++j)
+                                acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(ad[i], bd[j], acc[i][j], 0, 0, 0);
+                    }
+                }
+                __syncthreads(); // every wavefront has read K: the scores take its place
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            Ss[(16 * i + 4 * e + kq) * ASP + 32 * wave + 16 * j + r16] = static_cast<float>(acc[i][j][e]);
+                put_v();
+                __syncthreads();
+                // ---- Softmax of the rows: this wavefront rows 8 wave .., two at a time, 32 lanes a row
+#pragma unroll
+                for (int it = 0; it < 4; ++it)
+                {
+                    f4* const piece = reinterpret_cast<f4*>(Ss + (8 * wave + 2 * it + (lane >> 5)) * ASP) + (lane & 31);
+                    *piece = softmax_piece<32>(*piece, true, scaled, c);
+                }
+                __syncthreads();
+                // the next item's Q and K
+                const int t_next = t + grid;
+                const bool more = t_next < items; // uniform
+                AttnItem next = cur;
+                if (more)
+                {
+                    next = item_at(t_next);
+                    fetch_qk(next);
+                }
+                // ---- context: 32 x 64 over the 128 keys; this wavefront columns 16 wave .. as 2 x 1 blocks
+                d4 ctx[2] = {d4{0.0, 0.0, 0.0, 0.0}, d4{0.0, 0.0, 0.0, 0.0}};
+                {
+                    const float* const pa = Ss + r16 * ASP + kq;
+                    const float* const vb = Vs + kq * AD + ((16 * wave + r16) ^ (16 * kq));
+#pragma unroll
+                    for (int s = 0; s < AKEYS / 4; ++s)
+                    {
+                        const double bd = static_cast<double>(vb[4 * s * AD]);
+#pragma unroll
+                        for (int i = 0; i < 2; ++i)
+                            ctx[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(static_cast<double>(pa[4 * s + i * 16 * ASP]), bd, ctx[i], 0, 0, 0);
+                    }
+                }
+                __syncthreads(); // every wavefront has read Q's, the probabilities' and V's regions
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        res[i][e] = static_cast<float>(ctx[i][e]);
+                done = cur;
+                if (!more)
+                    break;
+                unsaved = true;
+                cur = next;
+                t = t_next;
+            }
+            store_item(done);
+        }
     }
 }
 
@@ -380,4 +602,48 @@ int hipq_batch_matmul_view_f32(const float* a, const float* b, float* out, const
     HIPQ_REQUIRE(v->a_outer >= 0 && v->a_inner >= 0 && v->b_outer >= 0 && v->b_inner >= 0 && v->o_outer >= 0 && v->o_inner >= 0, "negative batch stride");
     const MatView view{v->batch_inner, v->a_outer, v->a_inner, v->lda, v->b_outer, v->b_inner, v->ldb, v->o_outer, v->o_inner, v->ldo};
     return launch_batch_matmul(a, b, out, view, mq, batch, M, K, N, transpose_a, transpose_b, stream);
+}
+
+int hipq_attention_f32(const float* q, const float* k, const float* v, const float* factor, float* out, const hipq_attention_view_t* view, const hipq_quant_out_t* quant, int64_t batch,
+                       int64_t queries, int64_t keys, int64_t depth, void* stream)
+{
+    HIPQ_REQUIRE(view, "null view");
+    HIPQ_REQUIRE(batch >= 0 && queries >= 0 && keys >= 0 && depth >= 0, "negative extent");
+    if (keys != AKEYS || depth != AD || queries % AQ != 0)
+        return fail(HIPQ_ERR_UNSUPPORTED, "the one-kernel attention takes 128 keys of depth 64 and query rows in multiples of 32 (run the three ops otherwise)");
+    if (batch == 0 || queries == 0)
+        return HIPQ_OK;
+    MatQuant mq{nullptr, nullptr, nullptr, HIPQ_I8, HIPQ_ROUND_NEAREST_TOWARD_EVEN};
+    if (quant)
+    {
+        HIPQ_REQUIRE(quant->out && quant->scale, "quantized output: null pointer");
+        HIPQ_REQUIRE(quant->quant_t == HIPQ_I8 || quant->quant_t == HIPQ_U8, "quantized output: i8 or u8");
+        HIPQ_REQUIRE(quant->round_mode >= HIPQ_ROUND_NEAREST_TOWARD_INFINITY && quant->round_mode <= HIPQ_ROUND_DOWN, "quantized output: unknown round mode");
+        mq = MatQuant{quant->out, quant->scale, quant->zero_point, quant->quant_t, quant->round_mode};
+    }
+    HIPQ_REQUIRE(q && k && v && (out || mq.out), "null pointer");
+    HIPQ_REQUIRE(view->batch_inner >= 1, "batch_inner must be at least 1");
+    HIPQ_REQUIRE(view->ldq >= depth && view->ldk >= depth && view->ldv >= depth && view->ldo >= depth, "a row stride is shorter than the row");
+    HIPQ_REQUIRE(view->q_outer >= 0 && view->q_inner >= 0 && view->k_outer >= 0 && view->k_inner >= 0 && view->v_outer >= 0 && view->v_inner >= 0 && view->o_outer >= 0 && view->o_inner >= 0,
+                 "negative batch stride");
+    auto rows16 = [](const float* p, int64_t ld, int64_t outer, int64_t inner) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0 && ld % 4 == 0 && outer % 4 == 0 && inner % 4 == 0; };
+    HIPQ_REQUIRE(rows16(q, view->ldq, view->q_outer, view->q_inner) && rows16(k, view->ldk, view->k_outer, view->k_inner) && rows16(v, view->ldv, view->v_outer, view->v_inner),
+                 "rows of Q, K and V must start 16-byte aligned");
+    const int64_t row_blocks = queries / AQ;
+    HIPQ_REQUIRE(batch * row_blocks < (1ll << 31) - (1 << 20), "too many work items for one launch");
+    static bool configured[16] = {};
+    int dev = 0;
+    HIPQ_HIP(hipGetDevice(&dev));
+    if (dev >= 0 && dev < 16 && !configured[dev])
+    {
+        HIPQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_f32_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kAttnLdsBytes)));
+        configured[dev] = true;
+    }
+    const AttnView av{view->batch_inner, view->q_outer, view->q_inner, view->ldq, view->k_outer, view->k_inner, view->ldk,
+                      view->v_outer, view->v_inner, view->ldv, view->o_outer, view->o_inner, view->ldo};
+    const int64_t items = batch * row_blocks;
+    // two workgroups a compute unit (their LDS fits twice), each walking its share of the items
+    const int64_t grid = std::min<int64_t>(items, 2ll * device_compute_units());
+    attention_f32_kernel<<<static_cast<unsigned>(grid), 256, kAttnLdsBytes, as_stream(stream)>>>(q, k, v, factor, out, av, mq, static_cast<int32_t>(row_blocks), static_cast<int32_t>(items));
+    return check_launch("attention_f32");
 }

@@ -5,30 +5,13 @@
 
 #include "hipq_common.h"
 #include "hipq_quant_math.h"
+#include "hipq_row_math.h"
 
 namespace hipq
 {
     namespace
     {
         typedef float f4 __attribute__((ext_vector_type(4)));
-
-        // reductions over aligned groups of W lanes of a wavefront
-        template <int W = 64>
-        __device__ __forceinline__ float wave_max(float v)
-        {
-#pragma unroll
-            for (int o = W / 2; o > 0; o >>= 1)
-                v = fmaxf(v, __shfl_xor(v, o));
-            return v;
-        }
-        template <int W = 64>
-        __device__ __forceinline__ float wave_sum(float v)
-        {
-#pragma unroll
-            for (int o = W / 2; o > 0; o >>= 1)
-                v += __shfl_xor(v, o);
-            return v;
-        }
 
         // the optional quantized copy of an output: Quantize with one scale and zero point for the whole
         // tensor, computed from the f32 value as it is stored (same arithmetic as hipq_quantize)
@@ -147,19 +130,9 @@ namespace hipq
             f4 v = f4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
             if (live)
                 v = reinterpret_cast<const f4*>(in + row * cols)[sub];
-            if (live && scaled)
-                v = f4{__fmul_rn(v[0], c), __fmul_rn(v[1], c), __fmul_rn(v[2], c), __fmul_rn(v[3], c)};
-            const float m = wave_max<W>(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
-            float s = 0.0f;
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-            {
-                v[e] = live ? expf(v[e] - m) : 0.0f;
-                s += v[e];
-            }
-            s = wave_sum<W>(s);
+            v = softmax_piece<W>(v, live, scaled, c);
             if (live)
-                reinterpret_cast<f4*>(out + row * cols)[sub] = f4{v[0] / s, v[1] / s, v[2] / s, v[3] / s};
+                reinterpret_cast<f4*>(out + row * cols)[sub] = v;
         }
 
         // the same over a strided axis: the tensor is [outer][axis][inner], one lane a column (o, i)

@@ -1,0 +1,54 @@
+// Row reductions over groups of lanes and the Softmax arithmetic of one row piece, shared by the
+// Softmax kernels and by the attention kernel that applies Softmax to scores it has just computed:
+// both must round alike, sums included, so both call these.
+#pragma once
+#include <cmath>
+
+#include "hipq_common.h"
+
+namespace hipq
+{
+    typedef float row_f4 __attribute__((ext_vector_type(4)));
+
+    // reductions over aligned groups of W lanes of a wavefront
+    template <int W = 64>
+    __device__ __forceinline__ float wave_max(float v)
+    {
+#pragma unroll
+        for (int o = W / 2; o > 0; o >>= 1)
+            v = fmaxf(v, __shfl_xor(v, o));
+        return v;
+    }
+    template <int W = 64>
+    __device__ __forceinline__ float wave_sum(float v)
+    {
+#pragma unroll
+        for (int o = W / 2; o > 0; o >>= 1)
+            v += __shfl_xor(v, o);
+        return v;
+    }
+
+    // Softmax of a row of at most 4 W elements held one 16-byte piece a lane by W neighbouring lanes
+    // (src/ngraph/runtime/reference/softmax.hpp:31-57): exp(x - max) / sum(exp(x - max)); with `scaled`
+    // the input is Multiply(x, c), the product rounded to f32 as the Multiply op rounds it.  Lanes
+    // past the row's end pass live = false.  The sum: a lane's four terms in order, then the lanes'
+    // sums through the butterfly of wave_sum.
+    template <int W>
+    __device__ __forceinline__ row_f4 softmax_piece(row_f4 v, bool live, bool scaled, float c)
+    {
+        if (!live)
+            v = row_f4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+        else if (scaled)
+            v = row_f4{__fmul_rn(v[0], c), __fmul_rn(v[1], c), __fmul_rn(v[2], c), __fmul_rn(v[3], c)};
+        const float m = wave_max<W>(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
+        float s = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+        {
+            v[e] = live ? expf(v[e] - m) : 0.0f;
+            s += v[e];
+        }
+        s = wave_sum<W>(s);
+        return row_f4{v[0] / s, v[1] / s, v[2] / s, v[3] / s};
+    }
+}

@@ -163,6 +163,12 @@ class MatmulView(C.Structure):
     _fields_ = [(n, C.c_int64) for n in ("batch_inner", "a_outer", "a_inner", "lda", "b_outer", "b_inner", "ldb", "o_outer", "o_inner", "ldo")]
 
 
+class AttentionView(C.Structure):
+    """hipq_attention_view_t: batch strides (two levels) and row strides of Q, K, V and out, in elements"""
+
+    _fields_ = [(n, C.c_int64) for n in ("batch_inner", "q_outer", "q_inner", "ldq", "k_outer", "k_inner", "ldk", "v_outer", "v_inner", "ldv", "o_outer", "o_inner", "ldo")]
+
+
 class DeviceInfo(C.Structure):
     _fields_ = [
         ("name", C.c_char * 64),
@@ -318,6 +324,7 @@ EXPORTS = [
     "hipq_gelu_quantize_f32",
     "hipq_add_layer_norm_f32",
     "hipq_batch_matmul_view_f32",
+    "hipq_attention_f32",
 ]
 
 _lib = None
@@ -825,6 +832,25 @@ def gelu_quantize(x, q_scale, q_zp=0, quant_t="i8", round_mode=RNE, keep_f32=Tru
     check(lib.hipq_gelu_quantize_f32(src.ptr, dst.ptr if dst else None, C.byref(q), x.size, None))
     check(lib.hipq_stream_sync(None))
     return (dst.to_numpy(np.float32, x.shape) if dst else None), keep[0].to_numpy(NP_OF[qt], x.shape)
+
+
+def attention(qkv, q_off, k_off, v_off, out_elems, view, batch, queries, keys, depth, factor=None, q_scale=None, q_zp=0, quant_t="i8", keep_f32=True):
+    """hipq_attention_f32 on one flat f32 buffer holding Q, K and V (element offsets) into a flat zero-initialised
+    output of out_elems elements: returns (out or None, q or None); raises HipqError (UNSUPPORTED) for shapes the
+    one-kernel form does not take"""
+    lib = load()
+    buf = _dev(np.ascontiguousarray(qkv, dtype=np.float32).ravel())
+    dst = DeviceBuffer.from_numpy(np.zeros(out_elems, np.float32)) if keep_f32 else None
+    fac = _dev(np.asarray([factor], dtype=np.float32)) if factor is not None else None
+    q = keep = qt = None
+    if q_scale is not None:
+        q, keep, qt = _quant_out(out_elems, q_scale, q_zp, quant_t, RNE)
+        check(lib.hipq_fill_bytes(keep[0].ptr, 0, out_elems, None))
+    lib.hipq_attention_f32.argtypes = [C.c_void_p] * 7 + [C.c_int64] * 4 + [C.c_void_p]
+    check(lib.hipq_attention_f32(buf.ptr + 4 * q_off, buf.ptr + 4 * k_off, buf.ptr + 4 * v_off, fac.ptr if fac else None, dst.ptr if dst else None, C.byref(view),
+                                 C.byref(q) if q else None, batch, queries, keys, depth, None))
+    check(lib.hipq_stream_sync(None))
+    return (dst.to_numpy(np.float32, (out_elems,)) if dst else None), (keep[0].to_numpy(NP_OF[qt], (out_elems,)) if q else None)
 
 
 def batch_matmul_view(a, a_off, b, b_off, out_elems, out_off, view, batch, M, K, N, transpose_a=False, transpose_b=False, q_scale=None, q_zp=0, quant_t="i8", keep_f32=True):

@@ -257,3 +257,40 @@ def test_batch_matmul_views_are_attention_without_the_reshapes(gpu_lib, B, S, nh
     assert np.array_equal(q, H.quantize(exp_merged, f32(s_c), 0, "i8").ravel())
     _, q_only = H.batch_matmul_view(probs, 0, qkv, 2 * h, B * S * h, 0, v_ctx, B * nh, S, S, hd, False, False, q_scale=s_c, keep_f32=False)
     assert np.array_equal(q_only, q)
+
+
+@pytest.mark.parametrize("B,S,nh", [(2, 128, 12), (1, 128, 1), (5, 128, 3)])
+def test_attention_in_one_kernel_equals_the_three_ops(gpu_lib, B, S, nh):
+    """scores, scaled Softmax and context of every head in one launch, against the three launches it
+    replaces (bit for bit: the same product chains, the same Softmax lanes), with and without the
+    Multiply, the f32 result and the quantized copy"""
+    say("attention", B, S, nh)
+    hd = 64
+    h = nh * hd
+    qkv = synth.normal_f32(48, (B * S, 3 * h)) * f32(1.5)
+    v_scores = H.MatmulView(nh, S * 3 * h, hd, 3 * h, S * 3 * h, hd, 3 * h, nh * S * S, S * S, S)
+    v_ctx = H.MatmulView(nh, nh * S * S, S * S, S, S * 3 * h, hd, 3 * h, S * h, hd, h)
+    v_att = H.AttentionView(nh, S * 3 * h, hd, 3 * h, S * 3 * h, hd, 3 * h, S * 3 * h, hd, 3 * h, S * h, hd, h)
+    scores, _ = H.batch_matmul_view(qkv, 0, qkv, h, B * nh * S * S, 0, v_scores, B * nh, S, hd, S, False, True)
+    s_c = 0.4 / 127.0
+    for factor in (0.125, None):
+        probs = H.softmax_scaled(scores.reshape(B * nh * S, S), factor) if factor is not None else H.softmax(scores.reshape(B * nh * S, S), (1,))
+        exp, exp_q = H.batch_matmul_view(probs, 0, qkv, 2 * h, B * S * h, 0, v_ctx, B * nh, S, S, hd, False, False, q_scale=s_c)
+        got, q = H.attention(qkv, 0, h, 2 * h, B * S * h, v_att, B * nh, S, S, hd, factor=factor, q_scale=s_c)
+        assert np.array_equal(got.view(np.uint32), exp.view(np.uint32)), factor
+        assert np.array_equal(q, exp_q) and len(np.unique(q)) > 5
+        assert H.last_kernel() == "attention_f32"
+    got, q = H.attention(qkv, 0, h, 2 * h, B * S * h, v_att, B * nh, S, S, hd, factor=0.125)
+    assert q is None
+    _, q_only = H.attention(qkv, 0, h, 2 * h, B * S * h, v_att, B * nh, S, S, hd, factor=0.125, q_scale=s_c, quant_t="u8", q_zp=128, keep_f32=False)
+    assert np.array_equal(q_only, H.quantize(got, f32(s_c), 128, "u8"))
+
+
+def test_attention_in_one_kernel_rejects_other_shapes(gpu_lib):
+    say("attention shapes")
+    qkv = synth.normal_f32(49, (2 * 64, 3 * 64))
+    view = H.AttentionView(1, 64 * 192, 64, 192, 64 * 192, 64, 192, 64 * 192, 64, 192, 64 * 64, 64, 64)
+    for queries, keys, depth in ((64, 64, 64), (128, 128, 32), (100, 128, 64)):
+        with pytest.raises(H.HipqError) as e:
+            H.attention(qkv, 0, 64, 128, 2 * 64 * 64, view, 2, queries, keys, depth)
+        assert e.value.code == H.ERR_UNSUPPORTED

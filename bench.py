@@ -257,6 +257,23 @@ def bench_fp32_glue(lib, stream, timer, steps, warmup):
         nbytes = 4 * heads * (m * k + k * n + m * n)
         out.append(dict(op=name, elements=heads * m * n, ms_event=ev, gbs=nbytes / (ev * 1e-3) / 1e9, frac_hbm=nbytes / (ev * 1e-3) / 1e9 / PEAK_HBM_GBS,
                         tflops=2.0 * heads * m * k * n / (ev * 1e-3) / 1e12, kernel=H.last_kernel()))
+    # ... and the whole attention of those heads in one launch: scores, scaled Softmax, context + Quantize,
+    # Q, K, V read as views of a [4096, 2304] projection, the context written head-interleaved as i8
+    lib.hipq_attention_f32.argtypes = [vp] * 7 + [i64] * 4 + [vp]
+    S, nh, hd, h = 128, 12, 64, 768
+    view = H.AttentionView(nh, S * 3 * h, hd, 3 * h, S * 3 * h, hd, 3 * h, S * 3 * h, hd, 3 * h, S * h, hd, h)
+    inv, qscale, zero = dev(np.asarray([0.125], np.float32)), dev(np.asarray([0.4 / 127.0], np.float32)), dev(np.zeros(1, np.int8))
+    qout = H.QuantOut(dst.ptr, qscale.ptr, zero.ptr, H.I8, H.RNE)
+
+    def attention_step():
+        rc = lib.hipq_attention_f32(src.ptr, src.ptr + 4 * h, src.ptr + 8 * h, inv.ptr, None, C.byref(view), C.byref(qout), heads, S, S, hd, stream)
+        if rc:
+            H.check(rc)
+
+    _, ev = timer.run(attention_step, steps, warmup)
+    nbytes = 4 * 4096 * 3 * h + 4096 * h
+    out.append(dict(op="attention_f32[384x128x64]", elements=4096 * h, ms_event=ev, gbs=nbytes / (ev * 1e-3) / 1e9, frac_hbm=nbytes / (ev * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                    tflops=4.0 * heads * S * S * hd / (ev * 1e-3) / 1e12, kernel=H.last_kernel()))
     return out
 
 

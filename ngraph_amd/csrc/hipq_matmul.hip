@@ -431,11 +431,21 @@ namespace hipq
                 }
                 if (mq.out) // uniform
                 {
+                    const bool rne = mq.mode == HIPQ_ROUND_NEAREST_TOWARD_EVEN; // uniform: the Quantize kernels' four-at-a-time arithmetic
 #pragma unroll
                     for (int i = 0; i < 2; ++i)
+                    {
+                        uint32_t four = 0;
+                        if (rne)
+                        {
+                            const f4 x = f4{res[i][0], res[i][1], res[i][2], res[i][3]};
+                            four = mq.quant_t == HIPQ_U8 ? quantize4<uint8_t, true>(x, qs, static_cast<float>(qz), mq.mode) : quantize4<int8_t, true>(x, qs, static_cast<float>(qz), mq.mode);
+                        }
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
-                            static_cast<uint8_t*>(mq.out)[w.o_base + static_cast<int64_t>(16 * i + 4 * e + kq) * ldo + 16 * wave + r16] = static_cast<uint8_t>(q1(res[i][e]));
+                            static_cast<uint8_t*>(mq.out)[w.o_base + static_cast<int64_t>(16 * i + 4 * e + kq) * ldo + 16 * wave + r16] =
+                                static_cast<uint8_t>(rne ? (four >> (8 * e)) & 0xFFu : q1(res[i][e]));
+                    }
                 }
             };
 

@@ -24,6 +24,9 @@ namespace hipq
         };
         __device__ __forceinline__ uint32_t quant4(const QuantOut& q, float s, int32_t zp, f4 v)
         {
+            // round half to even (uniform): the Quantize kernels' own four-at-a-time arithmetic
+            if (q.mode == HIPQ_ROUND_NEAREST_TOWARD_EVEN)
+                return q.quant_t == HIPQ_U8 ? quantize4<uint8_t, true>(v, s, static_cast<float>(zp), q.mode) : quantize4<int8_t, true>(v, s, static_cast<float>(zp), q.mode);
             uint32_t w = 0;
 #pragma unroll
             for (int e = 0; e < 4; ++e)

@@ -137,80 +137,6 @@ namespace hipq
     {
         return run_index(v, ROW_UNIFORM ? first_group_of_step : g);
     }
-    typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-    // ---- division with the reciprocal shared by the four elements of a group -------------------
-    // The instruction sequence the compiler emits for an IEEE float division is
-    //     r = rcp(s); r = fma(fma(-s, r, 1), r, r);
-    //     q = x * r;  q = fma(fma(-s, q, x), r, q);  q = fma(fma(-s, q, x), r, q);
-    // wrapped in v_div_scale / v_div_fmas / v_div_fixup, which rescale the operands when an
-    // exponent is extreme and patch the special cases (zero, Inf, NaN, denormal).  For a divisor
-    // with 2^-30 <= |s| <= 2^30 and a dividend with 2^-60 <= |x| < 2^30 neither does anything, so
-    // the bare sequence returns the same bits, and the first line depends on s alone.  A dividend
-    // below 2^-60 gives a quotient below 2^-30 in magnitude from either sequence: it rounds to
-    // zero whichever bits it has.  Groups outside these ranges take the compiler's division.
-    __device__ __forceinline__ bool shared_reciprocal_ok(f32x4 x, float s)
-    {
-        const float big = 1073741824.0f;       // 2^30
-        const float small = 9.31322574615478515625e-10f; // 2^-30
-        // the sum is NaN or Inf if any element is, and bounds every |x|
-        float sum = (__builtin_fabsf(x[0]) + __builtin_fabsf(x[1])) + (__builtin_fabsf(x[2]) + __builtin_fabsf(x[3]));
-        float a = __builtin_fabsf(s);
-        return (sum < big) & (__builtin_amdgcn_fmed3f(a, small, big) == a);
-    }
-
-    // Four elements to four bytes, round-half-even, for a group that passed shared_reciprocal_ok.
-    // v_cvt_pk_u8_f32 converts with saturation to 0..255 and places the byte, i.e. the clamp, the
-    // cast and the packing in one instruction; signed outputs are computed 128 higher and flipped
-    // back with one XOR (the sum rint(q) + z is exact wherever it lies near the clamp range).
-    template <typename QUANT>
-    __device__ __forceinline__ uint32_t quantize4_shared_reciprocal(f32x4 x, float s, float z)
-    {
-        const bool is_signed = QLimits<QUANT>::lo < 0.0;
-        float zz = is_signed ? z + 128.0f : z;
-        float r = __builtin_amdgcn_rcpf(s);
-        float e = __builtin_fmaf(-s, r, 1.0f);
-        r = __builtin_fmaf(e, r, r);
-        uint32_t packed = 0;
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-        {
-            float q = __fmul_rn(x[k], r);
-            float t = __builtin_fmaf(-s, q, x[k]);
-            q = __builtin_fmaf(t, r, q);
-            t = __builtin_fmaf(-s, q, x[k]);
-            q = __builtin_fmaf(t, r, q);
-            float v = __fadd_rn(__builtin_rintf(q), zz);
-            packed = __builtin_amdgcn_cvt_pk_u8_f32(v, k, packed);
-        }
-        return is_signed ? packed ^ 0x80808080u : packed;
-    }
-
-    // For 8-bit outputs the reference's round-half-even formula equals rintf(): the two differ only
-    // for |q| >= 2^23, where both lie beyond the clamp range whatever the zero point.
-    template <typename QUANT, bool RNE>
-    __device__ __forceinline__ uint32_t quantize4(f32x4 x, float s, float z, int mode)
-    {
-        if (RNE && shared_reciprocal_ok(x, s))
-            return quantize4_shared_reciprocal<QUANT>(x, s, z);
-        const float lo = static_cast<float>(QLimits<QUANT>::lo);
-        const float hi = static_cast<float>(QLimits<QUANT>::hi);
-        float q[4] = {x[0], x[1], x[2], x[3]};
-        uint32_t packed = 0;
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-        {
-            float v = __fdiv_rn(q[e], s);
-            v = RNE ? rintf(v) : round_by_mode<float>(v, mode);
-            v = __fadd_rn(v, z);
-            v = (v < lo) ? lo : v;
-            v = (hi < v) ? hi : v;
-            int32_t iv = static_cast<int32_t>(v); // in range after the clamp (NaN aside)
-            packed |= (static_cast<uint32_t>(iv) & 0xFFu) << (8 * e);
-        }
-        return packed;
-    }
-
     template <typename QUANT, bool RNE, bool ROW_UNIFORM>
     __global__ __launch_bounds__(256) void quantize_vec4_kernel(const f32x4* __restrict__ in,
                                                                 const float* __restrict__ scale,

@@ -1,11 +1,14 @@
 // reserialize: read a serialized model and write it back (nGraph's tool of the same name,
 // src/tools/reserialize/reserialize.cpp:34-126; its constant-to-broadcast option is not offered).
-// An indent of 0 (the default, as in nGraph) writes the compact form.
+// An indent of 0 (the default, as in nGraph) writes the compact form.  An input named *.onnx or
+// *.prototxt is read as an ONNX model instead (binary or text), which makes this the converter from
+// ONNX to the serialized form nbench takes.
 #include <chrono>
 #include <fstream>
 #include <iostream>
 #include <string>
 
+#include "ngraph/frontend/onnx_import/onnx.hpp"
 #include "ngraph/serializer.hpp"
 
 using namespace std;
@@ -20,7 +23,7 @@ SYNOPSIS
         reserialize [-i|--input <input file>] [-o|--output <output file>] [--indent <n>]
 
 OPTIONS
-        -i or --input  input serialized model
+        -i or --input  input serialized model (or an ONNX model: *.onnx, *.prototxt)
         -o or --output output serialized model
         --indent       pretty-print with this many blanks per level
 )###";
@@ -72,9 +75,11 @@ int main(int argc, char** argv)
     try
     {
         auto t0 = chrono::steady_clock::now();
-        shared_ptr<ngraph::Function> function = ngraph::deserialize(f);
+        auto ends_with = [&](const string& tail) { return input.size() >= tail.size() && input.compare(input.size() - tail.size(), tail.size(), tail) == 0; };
+        const bool onnx = ends_with(".onnx") || ends_with(".prototxt");
+        shared_ptr<ngraph::Function> function = onnx ? ngraph::onnx_import::import_onnx_model(f) : ngraph::deserialize(f);
         auto t1 = chrono::steady_clock::now();
-        cout << "deserialize took " << chrono::duration<double, milli>(t1 - t0).count() << "ms\n";
+        cout << (onnx ? "onnx import took " : "deserialize took ") << chrono::duration<double, milli>(t1 - t0).count() << "ms\n";
         ngraph::serialize(output, function, indent);
         auto t2 = chrono::steady_clock::now();
         cout << "serialize took   " << chrono::duration<double, milli>(t2 - t1).count() << "ms\n";

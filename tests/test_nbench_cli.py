@@ -113,6 +113,28 @@ def test_reserialize_keeps_the_graph(name, tmp_path):
         assert renumbered(json.load(open(src))) == renumbered(a)
 
 
+@pytest.mark.parametrize("ext", [".onnx", ".prototxt"])
+def test_reserialize_converts_onnx_models(ext, tmp_path):
+    """an ONNX file (binary or text) in, the serialized graph nbench takes out: the QLinearConv of
+    tests/golden/onnx/qlinear_conv_3d with its strides and paddings, and the same document from
+    either file format"""
+    src = os.path.join(os.path.dirname(GOLDEN), "onnx", "qlinear_conv_3d" + ext)
+    out = str(tmp_path / "model.json")
+    p = run([RESERIALIZE, "-i", src, "-o", out])
+    assert p.returncode == 0 and "onnx import took" in p.stdout, p.stdout
+    doc = json.load(open(out))
+    ops = doc[0]["ops"]
+    conv = [o for o in ops if o["op"] == "QuantizedConvolution"]
+    assert len(conv) == 1 and conv[0]["window_movement_strides"] == [2, 2, 2] and conv[0]["padding_below"] == [2, 2, 2]
+    assert sum(o["op"] == "Parameter" for o in ops) == 8
+    other = str(tmp_path / "other.json")
+    twin = os.path.join(os.path.dirname(GOLDEN), "onnx", "qlinear_conv_3d" + (".prototxt" if ext == ".onnx" else ".onnx"))
+    assert run([RESERIALIZE, "-i", twin, "-o", other]).returncode == 0
+    assert renumbered(doc) == renumbered(json.load(open(other)))
+    p = run([RESERIALIZE, "-i", os.path.join(os.path.dirname(GOLDEN), "onnx", "unsupported_operator" + ext), "-o", out])
+    assert p.returncode != 0 and "unsupported operator Softplus" in p.stdout
+
+
 def test_reserialize_errors():
     p = run([RESERIALIZE])
     assert p.returncode == 1 and "input file missing" in p.stdout

@@ -263,6 +263,62 @@ CPU_TEST(onnx_import, errors_and_operator_queries)
         EXPECT_TRUE(ops.count(op) == 1);
 }
 
+CPU_TEST(onnx_import, qlinear_conv_with_bias_builds_the_reference_subgraph)
+{
+    // builder/quantization/quantized_linear_convolution.cpp:38-77: QuantizedConvolutionBias whose scale
+    // input is (x_scale * w_scale) / y_scale as graph nodes; an int32 bias goes in as it is
+    for (const char* format : kFormats)
+    {
+        auto f = load("qlinear_conv_bias", format);
+        EXPECT_EQ(f->get_parameters().size(), size_t(1));
+        auto cb = only<op::v0::QuantizedConvolutionBias>(f);
+        EXPECT_TRUE(!cb->with_relu());
+        EXPECT_EQ(cb->get_output_element_type(0), element::i8);
+        EXPECT_EQ(cb->get_argument(2)->get_output_element_type(0), element::i32);
+        EXPECT_TRUE(cb->get_argument(2)->is_constant());
+        auto div = as_type_ptr<op::v1::Divide>(cb->get_argument(3));
+        EXPECT_TRUE(div != nullptr);
+        EXPECT_TRUE(as_type_ptr<op::v1::Multiply>(div->get_argument(0)) != nullptr);
+        EXPECT_VEC_EQ((vector<float>{0.125f}), as_type_ptr<op::v0::Constant>(div->get_argument(1))->get_vector<float>());
+    }
+}
+
+CPU_TEST(onnx_import, damaged_files_are_refused_not_crashed_on)
+{
+    // every prefix of a binary and of a text model, and both with single bytes flipped: the reader
+    // either builds a graph or throws -- no reads past the end, no unbounded recursion or allocation
+    size_t built = 0, refused = 0;
+    auto attempt = [&](const string& bytes) {
+        stringstream ss(bytes);
+        try
+        {
+            onnx_import::import_onnx_model(ss);
+            ++built;
+        }
+        catch (const exception&)
+        {
+            ++refused;
+        }
+    };
+    for (const char* format : kFormats)
+    {
+        const auto raw = file_bytes(golden(string("onnx/qlinear_conv_initializers") + format));
+        const string whole(raw.begin(), raw.end());
+        for (size_t n = 0; n < whole.size(); n += (whole.size() > 2000 ? 7 : 1))
+            attempt(whole.substr(0, n));
+        uint32_t state = 12345;
+        for (int round = 0; round < 3000; ++round)
+        {
+            state = state * 1664525u + 1013904223u;
+            string damaged = whole;
+            damaged[(state >> 8) % damaged.size()] = static_cast<char>(state >> 24);
+            attempt(damaged);
+        }
+    }
+    EXPECT_TRUE(refused > 100);
+    EXPECT_TRUE(built > 0); // (a flipped byte inside a name or a number still gives a model)
+}
+
 // ---------------------------------------------------------------------------------- on the device
 // test/onnx/onnx_import_quant.in.cpp:44-108
 GPU_TEST(onnx_import, quantize_linear_vectors)
@@ -362,4 +418,6 @@ GPU_TEST(onnx_import, automatic_padding_and_glue_chain)
     expect_output<int32_t>("conv_integer_same_lower", {in(ramp), in(ones)}, Shape{1, 1, 2, 2}, {10, 24, 51, 90});
     // Dequantize (scale 0.5) -> Relu -> Quantize (scale 0.5): negatives to zero, everything else unchanged
     expect_output<int8_t>("dequantize_relu_quantize", {in<int8_t>({-4, -1, 0, 1, 5, 127})}, Shape{2, 3}, {0, 0, 0, 1, 5, 127});
+    // QLinearConv with an int32 bias: 1 x 1 filter 2, requantization scale 1: 2 x + 10, saturated to i8
+    expect_output<int8_t>("qlinear_conv_bias", {in<uint8_t>({1, 2, 3, 100})}, Shape{1, 1, 2, 2}, {12, 14, 16, 127});
 }

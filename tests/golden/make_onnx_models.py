@@ -159,8 +159,8 @@ def dequantize_linear(x_type, x_shape, scale_shape, initializers=(), opset=10, *
                  [("x", x_type, x_shape), ("x_scale", FLOAT, scale_shape), ("x_zero_point", x_type, scale_shape)], [("y", FLOAT, x_shape)], initializers, opset)
 
 
-def qlinear_conv(x_shape, w_shape, y_shape, w_type=UINT8, y_type=UINT8, initializers=(), opset=10, **attrs):
-    names = ["x", "x_scale", "x_zero_point", "w", "w_scale", "w_zero_point", "y_scale", "y_zero_point"]
+def qlinear_conv(x_shape, w_shape, y_shape, w_type=UINT8, y_type=UINT8, initializers=(), opset=10, bias=False, **attrs):
+    names = ["x", "x_scale", "x_zero_point", "w", "w_scale", "w_zero_point", "y_scale", "y_zero_point"] + (["bias"] if bias else [])
     inputs = [("x", UINT8, x_shape), ("x_scale", FLOAT, []), ("x_zero_point", UINT8, []), ("w", w_type, w_shape), ("w_scale", FLOAT, []), ("w_zero_point", w_type, []),
               ("y_scale", FLOAT, []), ("y_zero_point", y_type, [])]
     return model([node("QLinearConv", names, ["y"], "node1", **attrs)], inputs, [("y", y_type, y_shape)], initializers, opset)
@@ -234,6 +234,12 @@ MODELS = {
         [("x", INT8, [2, 3])],
         [("y", INT8, [2, 3])],
     ),
+    # QLinearConv with the optional ninth input: an int32 bias (requantization scale 0.5 * 0.25 / 0.125 = 1)
+    "qlinear_conv_bias": qlinear_conv(
+        [1, 1, 2, 2], [1, 1, 1, 1], [1, 1, 2, 2], w_type=INT8, y_type=INT8,
+        initializers=[tensor("x_scale", FLOAT, [], [0.5]), tensor("x_zero_point", UINT8, [], raw=b"\x00"), tensor("w", INT8, [1, 1, 1, 1], [2]), tensor("w_scale", FLOAT, [], [0.25]),
+                      tensor("w_zero_point", INT8, [], raw=b"\x00"), tensor("y_scale", FLOAT, [], [0.125]), tensor("y_zero_point", INT8, [], raw=b"\x00"), tensor("bias", INT32, [1], [10])],
+        bias=True),
     "unsupported_operator": model([node("Softplus", ["x"], ["y"], "node1")], [("x", FLOAT, [2])], [("y", FLOAT, [2])]),
 }
 

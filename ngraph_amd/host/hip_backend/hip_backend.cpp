@@ -183,6 +183,15 @@ namespace
             float factor;
         };
         unordered_map<const Node*, ScaledInput> m_softmax_of_product;
+        // ... a BatchMatMul that stands for the attention of a batch of heads:
+        // BatchMatMul(Softmax(Multiply(BatchMatMulTranspose(q, k), factor)), v), one launch
+        struct Attention
+        {
+            Output<Node> q, k, v;
+            bool scaled;
+            float factor;
+        };
+        unordered_map<const Node*, Attention> m_attention;
         unordered_map<const Node*, pair<Output<Node>, Output<Node>>> m_layer_norm_of_sum;
         struct QuantizedCopy
         {
@@ -397,6 +406,33 @@ namespace
                     m_folded.insert(add.get());
                 }
             }
+        }
+        // attention: context = BatchMatMul(Softmax over the keys of [Multiply(] BatchMatMulTranspose(q, k) [, c)], v)
+        // with 128 keys of depth 64 and query rows in multiples of 32 (what hipq_attention_f32 takes);
+        // scores, product and probabilities must have no other reader
+        for (const auto& n : m_function->get_ordered_ops())
+        {
+            const bool plain = is_type<op::v0::BatchMatMul>(n);
+            auto bt = as_type_ptr<op::v0::BatchMatMulTranspose>(n);
+            if (!plain && !(bt && !bt->get_transpose_arg0() && !bt->get_transpose_arg1()))
+                continue;
+            auto sm = as_type_ptr<op::v0::Softmax>(n->input_value(0).get_node_shared_ptr());
+            if (!sm || !single_user(sm.get()) || n->get_output_element_type(0) != element::f32 || sm->get_output_shape(0).size() != 3 || sm->get_axes() != AxisSet{2})
+                continue;
+            const auto product = m_softmax_of_product.find(sm.get());
+            const Output<Node> scores_out = product != m_softmax_of_product.end() ? product->second.x : sm->input_value(0);
+            auto scores = as_type_ptr<op::v0::BatchMatMulTranspose>(scores_out.get_node_shared_ptr());
+            if (!scores || scores->get_transpose_arg0() || !scores->get_transpose_arg1() || !single_user(scores.get()))
+                continue;
+            const Shape& qs = scores->get_input_shape(0);
+            const Shape& ks = scores->get_input_shape(1);
+            const Shape& vs = n->get_input_shape(1);
+            if (ks[1] != 128 || ks[2] != 64 || qs[1] % 32 != 0 || vs != ks)
+                continue;
+            m_attention[n.get()] = Attention{scores->input_value(0), scores->input_value(1), n->input_value(1), product != m_softmax_of_product.end(),
+                                             product != m_softmax_of_product.end() ? product->second.factor : 1.0f};
+            m_folded.insert(scores.get());
+            m_folded.insert(sm.get()); // (a Multiply in between is folded already)
         }
         for (const auto& n : m_function->get_ordered_ops())
         {
@@ -745,7 +781,17 @@ namespace
         Step st;
         st.node = n;
         st.output = id;
-        for (size_t i = 0; i < n->get_input_size(); ++i)
+        const auto attention = m_attention.find(n.get());
+        if (attention != m_attention.end())
+        {
+            // the folded scores / Softmax chain in front of input 0: the launch reads q, k and v
+            for (const Output<Node>& o : {attention->second.q, attention->second.k, attention->second.v})
+            {
+                st.inputs.push_back(value_of(o));
+                m_value_uses[st.inputs.back()] += 1;
+            }
+        }
+        for (size_t i = 0; attention == m_attention.end() && i < n->get_input_size(); ++i)
         {
             // (a folded Multiply / Add in front of input 0: the consumer reads the folded node's inputs instead)
             const auto sp = m_softmax_of_product.find(n.get());
@@ -997,10 +1043,29 @@ namespace
             const Shape& a = n->get_input_shape(0);
             const Shape& o = n->get_output_shape(0);
             const int64_t batch = static_cast<int64_t>(o[0]), M = static_cast<int64_t>(o[1]), N = static_cast<int64_t>(o[2]), K = static_cast<int64_t>(t0 ? a[1] : a[2]);
-            st.launch = [batch, M, K, N, t0, t1](const vector<void*>& in, void* out, void* stream) {
-                check(hipq_batch_matmul_f32(static_cast<const float*>(in[0]), static_cast<const float*>(in[1]), static_cast<float*>(out), batch, M, K, N, t0 ? 1 : 0, t1 ? 1 : 0, stream),
-                      "BatchMatMul");
-            };
+            if (attention != m_attention.end())
+            {
+                // dense [batch][rows][64] operands and result: one batch level, rows 64 apart
+                const float* factor = nullptr;
+                if (attention->second.scaled)
+                {
+                    auto block = alloc(sizeof(float));
+                    check(hipq_memcpy_h2d(block->ptr, &attention->second.factor, sizeof(float), m_stream), "constant upload");
+                    factor = static_cast<const float*>(block->ptr);
+                }
+                const int64_t keys = K, depth = N;
+                const hipq_attention_view_t view{1, M * depth, 0, depth, keys * depth, 0, depth, keys * depth, 0, depth, M * depth, 0, depth};
+                st.launch = [batch, M, keys, depth, factor, view](const vector<void*>& in, void* out, void* stream) {
+                    check(hipq_attention_f32(static_cast<const float*>(in[0]), static_cast<const float*>(in[1]), static_cast<const float*>(in[2]), factor, static_cast<float*>(out), &view, nullptr,
+                                             batch, M, keys, depth, stream),
+                          "attention");
+                };
+            }
+            else
+                st.launch = [batch, M, K, N, t0, t1](const vector<void*>& in, void* out, void* stream) {
+                    check(hipq_batch_matmul_f32(static_cast<const float*>(in[0]), static_cast<const float*>(in[1]), static_cast<float*>(out), batch, M, K, N, t0 ? 1 : 0, t1 ? 1 : 0, stream),
+                          "BatchMatMul");
+                };
         }
         else if (auto cc = as_type_ptr<op::v0::Concat>(n))
         {

@@ -332,3 +332,51 @@ GPU_TEST(HIP, glue_fusion_gelu_with_quantize)
         EXPECT_TRUE(fused.launches + 1 == plain.launches);
     }
 }
+
+GPU_TEST(HIP, glue_fusion_attention_of_a_batch_of_heads)
+{
+    // BatchMatMul(Softmax(Multiply(BatchMatMulTranspose(q, k), 1/8)), v) with 128 keys of depth 64: one
+    // launch instead of three, the same bits; and the same chain without the Multiply
+    const size_t heads = 6, rows = 64, keys = 128, depth = 64;
+    for (const bool scaled : {true, false})
+    {
+        auto q = make_shared<op::v0::Parameter>(element::f32, Shape{heads, rows, depth});
+        auto k = make_shared<op::v0::Parameter>(element::f32, Shape{heads, keys, depth});
+        auto v = make_shared<op::v0::Parameter>(element::f32, Shape{heads, keys, depth});
+        shared_ptr<Node> scores = make_shared<op::v0::BatchMatMulTranspose>(q, k, false, true);
+        if (scaled)
+            scores = make_shared<op::v1::Multiply>(scores, op::v0::Constant::create(element::f32, Shape{heads, rows, keys}, vector<float>{0.125f}));
+        auto probs = make_shared<op::v0::Softmax>(scores, AxisSet{2});
+        auto context = make_shared<op::v0::BatchMatMul>(probs, v);
+        auto f = make_shared<Function>(NodeVector{context}, ParameterVector{q, k, v});
+        const vector<vector<float>> args{wave(heads * rows * depth, 1.5f, 0.37f), wave(heads * keys * depth, 1.2f, 0.11f), wave(heads * keys * depth, 0.8f, 0.23f)};
+        const GlueRun fused = run_glue(f, args, true), plain = run_glue(f, args, false);
+        EXPECT_TRUE(fused.bytes == plain.bytes);
+        EXPECT_EQ(fused.launches, size_t(1));
+        EXPECT_EQ(plain.launches, size_t(scaled ? 4 : 3));
+    }
+    // probabilities with a second reader keep their own launch: nothing is folded past the Multiply
+    {
+        auto q = make_shared<op::v0::Parameter>(element::f32, Shape{2, 32, depth});
+        auto k = make_shared<op::v0::Parameter>(element::f32, Shape{2, keys, depth});
+        auto v = make_shared<op::v0::Parameter>(element::f32, Shape{2, keys, depth});
+        auto probs = make_shared<op::v0::Softmax>(make_shared<op::v0::BatchMatMulTranspose>(q, k, false, true), AxisSet{2});
+        auto context = make_shared<op::v0::BatchMatMul>(probs, v);
+        auto f = make_shared<Function>(NodeVector{context, probs}, ParameterVector{q, k, v});
+        const vector<vector<float>> args{wave(2 * 32 * depth, 1.0f, 0.3f), wave(2 * keys * depth, 1.0f, 0.7f), wave(2 * keys * depth, 1.0f, 0.9f)};
+        const GlueRun fused = run_glue(f, args, true), plain = run_glue(f, args, false);
+        EXPECT_TRUE(fused.bytes == plain.bytes);
+        EXPECT_EQ(fused.launches, size_t(3));
+    }
+    // other head shapes stay three launches
+    {
+        auto q = make_shared<op::v0::Parameter>(element::f32, Shape{3, 16, 8});
+        auto k = make_shared<op::v0::Parameter>(element::f32, Shape{3, 16, 8});
+        auto probs = make_shared<op::v0::Softmax>(make_shared<op::v0::BatchMatMulTranspose>(q, k, false, true), AxisSet{2});
+        auto f = make_shared<Function>(NodeVector{make_shared<op::v0::BatchMatMul>(probs, k)}, ParameterVector{q, k});
+        const vector<vector<float>> args{wave(3 * 16 * 8, 1.0f, 0.3f), wave(3 * 16 * 8, 1.0f, 0.7f)};
+        const GlueRun fused = run_glue(f, args, true), plain = run_glue(f, args, false);
+        EXPECT_TRUE(fused.bytes == plain.bytes);
+        EXPECT_EQ(fused.launches, size_t(3));
+    }
+}

@@ -431,6 +431,18 @@ HIPQ_API int hipq_permute(int32_t elem_bytes,
                           const int32_t* order,    /* host */
                           void* stream);
 
+/* op::v0::Slice (src/ngraph/runtime/reference/slice.hpp:30-66): out[c] = in[lower + c * strides] along
+ * every axis, out extent ceil((upper - lower) / strides); 0 <= lower <= upper <= extent. */
+HIPQ_API int hipq_slice(int32_t elem_bytes,
+                        const void* in,
+                        void* out,
+                        int32_t rank,
+                        const int64_t* in_shape, /* host */
+                        const int64_t* lower,    /* host */
+                        const int64_t* upper,    /* host */
+                        const int64_t* strides,  /* host */
+                        void* stream);
+
 /* ---- pooling and concatenation: the integer glue between the quantized convolutions of a network ----
  * MaxPool / AvgPool replace runtime::reference::max_pool<T> (src/ngraph/runtime/reference/
  * max_pool.hpp:127-222) and avg_pool<T> (src/ngraph/runtime/reference/avg_pool.hpp:128-250):

@@ -159,6 +159,32 @@ namespace hipq
         }
     }
 
+    // out[c] = in[lower + c * stride] along every axis (src/ngraph/runtime/reference/slice.hpp:30-66)
+    struct SliceInfo
+    {
+        int32_t rank;
+        int64_t out_shape[HIPQ_MAX_RANK];
+        int64_t in_step[HIPQ_MAX_RANK]; // elements of `in` one output step along the axis skips
+        int64_t in_first;               // element of `in` at output coordinate 0
+    };
+
+    template <typename T>
+    __global__ __launch_bounds__(256) void slice_kernel(const T* in, T* out, int64_t n, SliceInfo si)
+    {
+        int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+        const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+        for (; i < n; i += step)
+        {
+            int64_t r = i, j = si.in_first;
+            for (int a = si.rank - 1; a >= 0; --a)
+            {
+                j += (r % si.out_shape[a]) * si.in_step[a];
+                r /= si.out_shape[a];
+            }
+            out[i] = in[j];
+        }
+    }
+
     struct PermuteInfo
     {
         int32_t rank;
@@ -444,6 +470,44 @@ int hipq_broadcast(int32_t elem_bytes, const void* in, void* out, int32_t rank, 
     default: return fail(HIPQ_ERR_UNSUPPORTED, "%d-byte elements", elem_bytes);
     }
     return check_launch("broadcast");
+}
+
+int hipq_slice(int32_t elem_bytes, const void* in, void* out, int32_t rank, const int64_t* in_shape, const int64_t* lower, const int64_t* upper, const int64_t* strides, void* stream)
+{
+    HIPQ_REQUIRE(rank >= 0 && rank <= HIPQ_MAX_RANK, "rank %d out of range", rank);
+    HIPQ_REQUIRE(rank == 0 || (in_shape && lower && upper && strides), "shape, bounds or strides are null");
+    SliceInfo si;
+    si.rank = rank;
+    si.in_first = 0;
+    int64_t n = 1, in_stride = 1;
+    for (int i = 0; i < HIPQ_MAX_RANK; ++i)
+    {
+        si.out_shape[i] = 1;
+        si.in_step[i] = 0;
+    }
+    for (int i = rank - 1; i >= 0; --i)
+    {
+        HIPQ_REQUIRE(in_shape[i] >= 0 && strides[i] >= 1, "negative extent or non-positive stride on axis %d", i);
+        HIPQ_REQUIRE(lower[i] >= 0 && lower[i] <= upper[i] && upper[i] <= in_shape[i], "bounds [%lld, %lld) outside axis %d of extent %lld", static_cast<long long>(lower[i]),
+                     static_cast<long long>(upper[i]), i, static_cast<long long>(in_shape[i]));
+        si.out_shape[i] = (upper[i] - lower[i] + strides[i] - 1) / strides[i]; // ceil
+        si.in_step[i] = in_stride * strides[i];
+        si.in_first += in_stride * lower[i];
+        n *= si.out_shape[i];
+        in_stride *= in_shape[i];
+    }
+    if (n == 0)
+        return HIPQ_OK;
+    HIPQ_REQUIRE(in && out, "null tensor pointer");
+    hipStream_t s = as_stream(stream);
+    switch (elem_bytes)
+    {
+    case 1: slice_kernel<uint8_t><<<blocks_for(n), 256, 0, s>>>(static_cast<const uint8_t*>(in), static_cast<uint8_t*>(out), n, si); break;
+    case 4: slice_kernel<uint32_t><<<blocks_for(n), 256, 0, s>>>(static_cast<const uint32_t*>(in), static_cast<uint32_t*>(out), n, si); break;
+    case 8: slice_kernel<uint64_t><<<blocks_for(n), 256, 0, s>>>(static_cast<const uint64_t*>(in), static_cast<uint64_t*>(out), n, si); break;
+    default: return fail(HIPQ_ERR_UNSUPPORTED, "%d-byte elements", elem_bytes);
+    }
+    return check_launch("slice");
 }
 
 int hipq_permute(int32_t elem_bytes, const void* in, void* out, int32_t rank, const int64_t* in_shape, const int32_t* order, void* stream)

@@ -311,6 +311,7 @@ EXPORTS = [
     "hipq_convert",
     "hipq_broadcast",
     "hipq_permute",
+    "hipq_slice",
     "hipq_pool_infer_output",
     "hipq_pool",
     "hipq_concat",
@@ -664,6 +665,21 @@ def permute(x, order):
     check(lib.hipq_permute(x.dtype.itemsize, bx.ptr, out.ptr, x.ndim, shape, ordr, None))
     check(lib.hipq_stream_sync(None))
     return out.to_numpy(x.dtype, [x.shape[i] for i in order])
+
+
+def slice_(x, lower, upper, strides=None):
+    """x[lower:upper:strides] along every axis (op::v0::Slice)"""
+    lib = load()
+    x = np.ascontiguousarray(x)
+    strides = list(strides) if strides is not None else [1] * x.ndim
+    bx = _dev(x)
+    out = DeviceBuffer(max(x.nbytes, 1))  # (a slice is never larger than its input)
+    i64 = C.c_int64 * x.ndim
+    lib.hipq_slice.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_int32] + [C.c_void_p] * 5
+    check(lib.hipq_slice(x.dtype.itemsize, bx.ptr, out.ptr, x.ndim, i64(*x.shape), i64(*lower), i64(*upper), i64(*strides), None))
+    check(lib.hipq_stream_sync(None))
+    out_shape = [(u - l + s - 1) // s for l, u, s in zip(lower, upper, strides)]
+    return out.to_numpy(x.dtype, out_shape)
 
 
 def quantized_dot(desc, a, b, a_scale, a_zp, b_scale, b_zp, out_scale, out_zp, prepare=True):

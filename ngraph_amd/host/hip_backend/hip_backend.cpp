@@ -732,7 +732,7 @@ namespace
             op::v0::Abs::type_info, op::v0::Relu::type_info, op::v0::Convert::type_info, op::v0::Broadcast::type_info,
             op::v0::Reshape::type_info, op::v1::Add::type_info, op::v1::Subtract::type_info, op::v1::Multiply::type_info,
             op::v1::Divide::type_info, op::v1::Maximum::type_info, op::v1::Minimum::type_info, op::v0::MaxPool::type_info,
-            op::v0::AvgPool::type_info, op::v0::Concat::type_info, op::v0::Softmax::type_info, op::v0::Erf::type_info,
+            op::v0::AvgPool::type_info, op::v0::Concat::type_info, op::v0::Slice::type_info, op::v0::Softmax::type_info, op::v0::Erf::type_info,
             op::v0::Gelu::type_info, op::v0::LayerNorm::type_info, op::v0::BatchMatMul::type_info, op::v0::BatchMatMulTranspose::type_info};
         for (const auto& ti : ops)
             if (n.get_type_info() == ti)
@@ -1066,6 +1066,19 @@ namespace
                     check(hipq_batch_matmul_f32(static_cast<const float*>(in[0]), static_cast<const float*>(in[1]), static_cast<float*>(out), batch, M, K, N, t0 ? 1 : 0, t1 ? 1 : 0, stream),
                           "BatchMatMul");
                 };
+        }
+        else if (auto sl = as_type_ptr<op::v0::Slice>(n))
+        {
+            // src/ngraph/runtime/reference/slice.hpp:30-66
+            const int32_t eb = static_cast<int32_t>(et.size());
+            const Shape& is = n->get_input_shape(0);
+            if (is.size() > HIPQ_MAX_RANK)
+                throw unsupported_op("HIP backend: Slice of rank " + to_string(is.size()));
+            const vector<int64_t> shape(is.begin(), is.end()), lower(sl->get_lower_bounds().begin(), sl->get_lower_bounds().end()),
+                upper(sl->get_upper_bounds().begin(), sl->get_upper_bounds().end()), strides(sl->get_strides().begin(), sl->get_strides().end());
+            st.launch = [eb, shape, lower, upper, strides](const vector<void*>& in, void* out, void* stream) {
+                check(hipq_slice(eb, in[0], out, static_cast<int32_t>(shape.size()), shape.data(), lower.data(), upper.data(), strides.data(), stream), "Slice");
+            };
         }
         else if (auto cc = as_type_ptr<op::v0::Concat>(n))
         {

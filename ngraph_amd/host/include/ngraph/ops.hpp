@@ -471,6 +471,24 @@ namespace ngraph
                 int64_t m_concat_axis = -1;
             };
 
+            // src/ngraph/op/slice.hpp:28-76: the elements lower_bounds + i * strides < upper_bounds of every axis
+            class NGRAPH_API Slice : public Op
+            {
+            public:
+                NGRAPH_OP_DECL("Slice", 0)
+                Slice(const Output<Node>& arg, const Coordinate& lower_bounds, const Coordinate& upper_bounds, const Strides& strides);
+                Slice(const Output<Node>& arg, const Coordinate& lower_bounds, const Coordinate& upper_bounds);
+                void validate_and_infer_types() override;
+                const Coordinate& get_lower_bounds() const { return m_lower_bounds; }
+                const Coordinate& get_upper_bounds() const { return m_upper_bounds; }
+                const Strides& get_strides() const { return m_strides; }
+                std::shared_ptr<Node> clone_with_new_inputs(const OutputVector& new_args) const override;
+
+            private:
+                Coordinate m_lower_bounds, m_upper_bounds;
+                Strides m_strides;
+            };
+
             // ---- fp32 glue of a transformer encoder --------------------------------------------------
             // src/ngraph/op/softmax.hpp:28-60 (static axes)
             class NGRAPH_API Softmax : public Op
@@ -638,6 +656,7 @@ namespace ngraph
         using v0::Relu;
         using v0::Reshape;
         using v0::Result;
+        using v0::Slice;
         using v0::Softmax;
     }
 

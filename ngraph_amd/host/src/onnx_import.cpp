@@ -818,7 +818,7 @@ namespace ngraph
                 return {make_shared<op::v0::Dequantize>(x, x_scale, zero_point, x_scale.get_element_type(), axes)};
             }
 
-            // op/quant_conv.cpp:57-270 (one group; grouped convolutions need Slice, which this host subset leaves out)
+            // op/quant_conv.cpp:57-270
             OutputVector qlinear_conv(const OnnxNode& node)
             {
                 const Output<Node>& data = node.input(0);
@@ -829,9 +829,50 @@ namespace ngraph
                              node.description(),
                              ": incorrect value of 'group' attribute: ",
                              groups);
-                if (groups != 1)
-                    throw ngraph_error(node.description() + ": only group = 1 is supported for QLinearConv here (given: " + to_string(groups) + ")");
+                NGRAPH_CHECK(groups >= 1 && data.get_shape().at(1) % static_cast<size_t>(groups) == 0 && filters.get_shape().at(0) % static_cast<size_t>(groups) == 0,
+                             node.description(),
+                             ": the channels of data and filters must be multiples of 'group' (",
+                             groups,
+                             ")");
                 const ConvGeometry g = conv_geometry(node, data, filters);
+                if (groups > 1)
+                {
+                    // quant_conv.cpp:80-138: one convolution a group over slices of the data's channels and of
+                    // the filters, concatenated along the channel axis
+                    if (node.has_input(8))
+                        throw ngraph_error(node.description() + ": Groups != 1 not supported for Quantized Convolution with bias.");
+                    const size_t data_group = data.get_shape().at(1) / static_cast<size_t>(groups), filters_group = filters.get_shape().at(0) / static_cast<size_t>(groups);
+                    OutputVector pieces;
+                    for (size_t group = 0; group < static_cast<size_t>(groups); ++group)
+                    {
+                        Coordinate data_lower(data.get_shape().size(), 0), data_upper(data.get_shape().begin(), data.get_shape().end());
+                        data_lower[1] = group * data_group;
+                        data_upper[1] = (group + 1) * data_group;
+                        Coordinate filters_lower(filters.get_shape().size(), 0), filters_upper(filters.get_shape().begin(), filters.get_shape().end());
+                        filters_lower[0] = group * filters_group;
+                        filters_upper[0] = (group + 1) * filters_group;
+                        const Output<Node> sliced_data = make_shared<op::v0::Slice>(data, data_lower, data_upper);
+                        const Output<Node> sliced_filters = make_shared<op::v0::Slice>(filters, filters_lower, filters_upper);
+                        pieces.push_back(make_shared<op::v0::QuantizedConvolution>(sliced_data,
+                                                                                   sliced_filters,
+                                                                                   g.strides,
+                                                                                   g.dilations,
+                                                                                   g.pads_below,
+                                                                                   g.pads_above,
+                                                                                   g.data_dilations,
+                                                                                   node.input(1),
+                                                                                   node.input(2),
+                                                                                   node.input(4),
+                                                                                   node.input(5),
+                                                                                   node.input(6),
+                                                                                   node.input(7),
+                                                                                   quantized_result_type(node, data, filters),
+                                                                                   AxisSet{},
+                                                                                   AxisSet{},
+                                                                                   AxisSet{}));
+                    }
+                    return {make_shared<op::v0::Concat>(pieces, 1)};
+                }
                 if (node.has_input(8))
                 {
                     // builder/quantization/quantized_linear_convolution.cpp:38-77
@@ -897,47 +938,89 @@ namespace ngraph
                                                                   AxisSet{})};
             }
 
-            void check_matrix_operands(const OnnxNode& node, const Output<Node>& left, const Output<Node>& right)
+            // builder/matmul_factory.cpp:71-150: operands of rank <= 2 are one dot; stacks of matrices are
+            // collapsed to rank 3, multiplied matrix by matrix (Slice, squeeze, dot, expand) and
+            // concatenated, then given their stack axes back.  Both operands must carry the same stack
+            // here: the reference also broadcasts the stack axes numpy-style.
+            OutputVector matmul_of(const OnnxNode& node, Output<Node> left, Output<Node> right, const function<Output<Node>(const Output<Node>&, const Output<Node>&)>& make_dot)
             {
-                // builder/matmul_factory.cpp:71-86: operands of rank <= 2 are one Dot; stacks of matrices
-                // are sliced, multiplied one by one and concatenated there (Slice is outside this subset)
-                if (left.get_shape().size() > 2 || right.get_shape().size() > 2)
-                    throw ngraph_error(node.description() + ": operands of rank above 2 are not supported here");
+                const Shape left_shape = left.get_shape(), right_shape = right.get_shape();
+                if (left_shape.size() <= 2 && right_shape.size() <= 2)
+                    return {make_dot(left, right)};
+                if (left_shape.size() != right_shape.size() || !equal(left_shape.begin(), left_shape.end() - 2, right_shape.begin()))
+                    throw ngraph_error(node.description() + ": stacks of matrices of different stack shapes (numpy broadcasting) are not supported here");
+                auto reshape = [](const Output<Node>& x, const Shape& to) {
+                    AxisVector order(x.get_shape().size());
+                    for (size_t i = 0; i < order.size(); ++i)
+                        order[i] = i;
+                    return Output<Node>(make_shared<op::v0::Reshape>(x, order, to));
+                };
+                auto collapse = [&](const Output<Node>& x) {
+                    const Shape& s = x.get_shape();
+                    if (s.size() <= 3)
+                        return x;
+                    size_t stack = 1;
+                    for (size_t i = 0; i + 2 < s.size(); ++i)
+                        stack *= s[i];
+                    return reshape(x, Shape{stack, s[s.size() - 2], s[s.size() - 1]});
+                };
+                left = collapse(left);
+                right = collapse(right);
+                const size_t groups = left.get_shape().at(0);
+                auto sub_matrix = [&](const Output<Node>& x, size_t idx) {
+                    const Shape& s = x.get_shape();
+                    Coordinate lower(s.size(), 0), upper(s.begin(), s.end());
+                    lower[0] = idx;
+                    upper[0] = idx + 1;
+                    return reshape(make_shared<op::v0::Slice>(x, lower, upper), Shape{s[1], s[2]});
+                };
+                OutputVector small_dots;
+                for (size_t g = 0; g < groups; ++g)
+                {
+                    const Output<Node> sub_dot = make_dot(sub_matrix(left, g), sub_matrix(right, g));
+                    const Shape& ds = sub_dot.get_shape();
+                    small_dots.push_back(reshape(sub_dot, Shape{1, ds.at(0), ds.at(1)}));
+                }
+                const Output<Node> result = make_shared<op::v0::Concat>(small_dots, 0);
+                if (left_shape.size() <= 3)
+                    return {result};
+                Shape result_shape(left_shape.begin(), left_shape.end() - 2);
+                result_shape.push_back(result.get_shape().at(1));
+                result_shape.push_back(result.get_shape().at(2));
+                return {reshape(result, result_shape)};
             }
 
             // op/qlinear_matmul.cpp:30-47 with builder/matmul_factory.cpp:159-193
             OutputVector qlinear_matmul(const OnnxNode& node)
             {
-                const Output<Node>& left = node.input(0);
-                const Output<Node>& right = node.input(3);
-                check_matrix_operands(node, left, right);
-                return {make_shared<op::v0::QuantizedDot>(left,
-                                                          right,
-                                                          1,
-                                                          node.input(1),
-                                                          node.input(2),
-                                                          node.input(4),
-                                                          node.input(5),
-                                                          node.input(6),
-                                                          node.input(7),
-                                                          quantized_result_type(node, left, right),
-                                                          AxisSet{},
-                                                          AxisSet{},
-                                                          AxisSet{})};
+                return matmul_of(node, node.input(0), node.input(3), [&](const Output<Node>& left, const Output<Node>& right) {
+                    return Output<Node>(make_shared<op::v0::QuantizedDot>(left,
+                                                                         right,
+                                                                         1,
+                                                                         node.input(1),
+                                                                         node.input(2),
+                                                                         node.input(4),
+                                                                         node.input(5),
+                                                                         node.input(6),
+                                                                         node.input(7),
+                                                                         quantized_result_type(node, left, right),
+                                                                         AxisSet{},
+                                                                         AxisSet{},
+                                                                         AxisSet{}));
+                });
             }
 
             // op/matmul_integer.cpp with builder/matmul_factory.cpp:195-243
             OutputVector matmul_integer(const OnnxNode& node)
             {
-                const Output<Node>& left = node.input(0);
-                const Output<Node>& right = node.input(1);
-                check_matrix_operands(node, left, right);
                 const Output<Node> scale_one = builder::make_constant(element::f32, Shape{}, 1);
                 const Output<Node> output_zero_point = builder::make_constant(element::i32, Shape{}, 0);
-                const Output<Node> left_zero_point = node.has_input(2) ? node.input(2) : Output<Node>(builder::make_constant(left.get_element_type(), Shape{}, 0));
-                const Output<Node> right_zero_point = node.has_input(3) ? node.input(3) : Output<Node>(builder::make_constant(right.get_element_type(), Shape{}, 0));
-                return {make_shared<op::v0::QuantizedDot>(
-                    left, right, 1, scale_one, left_zero_point, scale_one, right_zero_point, scale_one, output_zero_point, element::i32, AxisSet{}, AxisSet{}, AxisSet{})};
+                const Output<Node> left_zero_point = node.has_input(2) ? node.input(2) : Output<Node>(builder::make_constant(node.input(0).get_element_type(), Shape{}, 0));
+                const Output<Node> right_zero_point = node.has_input(3) ? node.input(3) : Output<Node>(builder::make_constant(node.input(1).get_element_type(), Shape{}, 0));
+                return matmul_of(node, node.input(0), node.input(1), [&](const Output<Node>& left, const Output<Node>& right) {
+                    return Output<Node>(make_shared<op::v0::QuantizedDot>(
+                        left, right, 1, scale_one, left_zero_point, scale_one, right_zero_point, scale_one, output_zero_point, element::i32, AxisSet{}, AxisSet{}, AxisSet{}));
+                });
             }
 
             // op/constant.cpp: the `value` tensor

@@ -947,6 +947,79 @@ namespace ngraph
                 set_output_type(0, get_input_element_type(0), out);
             }
             shared_ptr<Node> Concat::clone_with_new_inputs(const OutputVector& a) const { return make_shared<Concat>(a, m_axis); }
+
+            // src/ngraph/op/slice.cpp:25-128
+            constexpr NodeTypeInfo Slice::type_info;
+            Slice::Slice(const Output<Node>& arg, const Coordinate& lower_bounds, const Coordinate& upper_bounds, const Strides& strides)
+                : Op({arg}), m_lower_bounds(lower_bounds), m_upper_bounds(upper_bounds), m_strides(strides)
+            {
+                constructor_validate_and_infer_types();
+            }
+            Slice::Slice(const Output<Node>& arg, const Coordinate& lower_bounds, const Coordinate& upper_bounds)
+                : Op({arg}), m_lower_bounds(lower_bounds), m_upper_bounds(upper_bounds), m_strides(Strides())
+            {
+                constructor_validate_and_infer_types();
+            }
+            void Slice::validate_and_infer_types()
+            {
+                if (m_strides.size() == 0) // no strides given: ones
+                    m_strides = Strides(m_lower_bounds.size(), 1);
+                NODE_VALIDATION_CHECK(this,
+                                      m_lower_bounds.size() == m_upper_bounds.size() && m_lower_bounds.size() == m_strides.size(),
+                                      "Ranks of lower bounds (",
+                                      m_lower_bounds,
+                                      "), upper bounds (",
+                                      m_upper_bounds,
+                                      ") and strides (",
+                                      m_strides,
+                                      ") do not match.");
+                const size_t output_rank = m_upper_bounds.size();
+                for (size_t i = 0; i < output_rank; i++)
+                {
+                    NODE_VALIDATION_CHECK(this,
+                                          m_lower_bounds[i] <= m_upper_bounds[i],
+                                          "Lower bound for slice is greater than upper bound at axis ",
+                                          i,
+                                          " (lower bounds: ",
+                                          m_lower_bounds,
+                                          ", upper bounds: ",
+                                          m_upper_bounds,
+                                          ").");
+                    NODE_VALIDATION_CHECK(this, m_strides[i] != 0, "Stride for slice is zero at axis ", i, " (strides: ", m_strides, ").");
+                }
+                const Shape& input_shape = get_input_shape(0);
+                NODE_VALIDATION_CHECK(this,
+                                      input_shape.size() == output_rank,
+                                      "Input rank does not match the rank of the lower bounds (",
+                                      m_lower_bounds,
+                                      "), upper bounds (",
+                                      m_upper_bounds,
+                                      "), and strides (",
+                                      m_strides,
+                                      ").");
+                Shape result(output_rank);
+                for (size_t i = 0; i < output_rank; i++)
+                {
+                    NODE_VALIDATION_CHECK(this,
+                                          m_upper_bounds[i] <= input_shape[i],
+                                          "Upper bound for slice at axis ",
+                                          i,
+                                          " is out of range ",
+                                          "(upper bounds: ",
+                                          m_upper_bounds,
+                                          ", argument shape: ",
+                                          input_shape,
+                                          ").");
+                    const size_t extent = m_upper_bounds[i] - m_lower_bounds[i];
+                    result[i] = extent / m_strides[i] + ((extent % m_strides[i] == 0) ? 0 : 1);
+                }
+                set_output_type(0, get_input_element_type(0), result);
+            }
+            shared_ptr<Node> Slice::clone_with_new_inputs(const OutputVector& a) const
+            {
+                check_new_args_count(this, a);
+                return make_shared<Slice>(a.at(0), m_lower_bounds, m_upper_bounds, m_strides);
+            }
         }
 
         namespace v1

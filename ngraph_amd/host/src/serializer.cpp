@@ -948,6 +948,11 @@ namespace
                 }
                 if (op_name == "Concat")
                     return std::make_shared<v0::Concat>(args, static_cast<int64_t>(node_js.at("axis").get_size()));
+                if (op_name == "Slice") // serializer.cpp:2387-2394
+                    return std::make_shared<v0::Slice>(arg(0),
+                                                       node_js.at("lower_bounds").get_size_vector<Coordinate>(),
+                                                       node_js.at("upper_bounds").get_size_vector<Coordinate>(),
+                                                       node_js.at("strides").get_size_vector<Strides>());
                 if (op_name == "Softmax")
                 {
                     if (node_js.has("softmax_axes"))
@@ -1149,6 +1154,12 @@ namespace
         }
         else if (auto c = as_type<const v0::Concat>(p))
             node["axis"] = Json(c->get_concatenation_axis());
+        else if (auto c = as_type<const v0::Slice>(p))
+        {
+            node["lower_bounds"] = Json::array_of(c->get_lower_bounds());
+            node["upper_bounds"] = Json::array_of(c->get_upper_bounds());
+            node["strides"] = Json::array_of(c->get_strides());
+        }
         else if (auto c = as_type<const v0::Softmax>(p))
             node["softmax_axes"] = write_axis_set(c->get_axes()); // the form with the axes as an attribute (serializer.cpp:2397-2401)
         else if (auto c = as_type<const v0::LayerNorm>(p))

@@ -217,6 +217,14 @@ MODELS = {
     "matmul_integer_no_zero_point": matmul_integer([4, 3], [3, 2], [4, 2], zero_points=False),
     "matmul_integer_scalar": matmul_integer([1, 1], [1, 1], [1, 1]),
     "matmul_integer_4d": matmul_integer([1, 2, 3, 4], [1, 2, 4, 3], [1, 2, 3, 3]),
+    "matmul_integer_4d_no_zero_point": matmul_integer([1, 2, 3, 4], [1, 2, 4, 3], [1, 2, 3, 3], zero_points=False),
+    "matmul_integer_stacks_differ": matmul_integer([2, 3, 4], [1, 4, 3], [2, 3, 3]),
+    # QLinearConv in two groups: a 1 x 1 filter a channel (unit scales, zero zero points)
+    "qlinear_conv_groups": qlinear_conv(
+        [1, 2, 2, 2], [2, 1, 1, 1], [1, 2, 2, 2], w_type=INT8, y_type=INT8,
+        initializers=[tensor("x_scale", FLOAT, [], [1.0]), tensor("x_zero_point", UINT8, [], raw=b"\x00"), tensor("w", INT8, [2, 1, 1, 1], [2, 3]), tensor("w_scale", FLOAT, [], [1.0]),
+                      tensor("w_zero_point", INT8, [], raw=b"\x00"), tensor("y_scale", FLOAT, [], [1.0]), tensor("y_zero_point", INT8, [], raw=b"\x00")],
+        group=2),
     # automatic padding: a 3 x 3 window over 4 x 4 at stride 2 needs one more row and column, below the data (SAME_LOWER) or above it (SAME_UPPER)
     "conv_integer_same_upper": model([node("ConvInteger", ["x", "w"], ["y"], "node1", auto_pad="SAME_UPPER", strides=[2, 2])], [("x", UINT8, [1, 1, 4, 4]), ("w", UINT8, [1, 1, 3, 3])],
                                      [("y", INT32, [1, 1, 2, 2])]),

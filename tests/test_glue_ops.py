@@ -128,3 +128,36 @@ def test_permute(gpu_lib, case, dtype):
     x = _rand(50 + case, int(np.prod(shape)), dtype).reshape(shape)
     got = H.permute(x, order)
     assert np.array_equal(got, np.ascontiguousarray(np.transpose(x, order)))
+
+
+# op::v0::Slice (src/ngraph/runtime/reference/slice.hpp:30-66): (shape, lower, upper, strides); the first
+# three are the shapes of test/backend/slice.in.cpp (matrix, vector, strided 3-D)
+SLICES = [
+    ((4, 4), (0, 1), (3, 3), (1, 1)),
+    ((16,), (2,), (14,), (1,)),
+    ((4, 4, 4), (0, 0, 0), (4, 4, 4), (2, 2, 3)),
+    ((2, 8, 5, 5), (0, 4, 0, 0), (2, 8, 5, 5), (1, 1, 1, 1)),
+    ((3, 7, 9), (1, 2, 3), (3, 7, 8), (1, 3, 2)),
+    ((5, 6), (2, 3), (2, 6), (1, 1)),
+    ((1, 2, 3, 4, 5, 2), (0, 1, 0, 1, 2, 0), (1, 2, 3, 4, 5, 2), (1, 1, 2, 2, 1, 1)),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", range(len(SLICES)))
+@pytest.mark.parametrize("dtype", [np.uint8, np.float32, np.float64])
+def test_slice(gpu_lib, case, dtype):
+    shape, lower, upper, strides = SLICES[case]
+    x = (_rand(70 + case, int(np.prod(shape)), np.float32).astype(np.float64) if dtype == np.float64 else _rand(70 + case, int(np.prod(shape)), dtype)).reshape(shape)
+    got = H.slice_(x, lower, upper, strides)
+    exp = x[tuple(slice(l, u, s) for l, u, s in zip(lower, upper, strides))]
+    assert got.shape == exp.shape and np.array_equal(got, exp)
+
+
+@pytest.mark.gpu
+def test_slice_rejects_bounds_outside_the_tensor(gpu_lib):
+    x = np.zeros((4, 4), np.float32)
+    for lower, upper, strides in (((0, 0), (5, 4), (1, 1)), ((3, 0), (2, 4), (1, 1)), ((0, 0), (4, 4), (0, 1)), ((-1, 0), (4, 4), (1, 1))):
+        with pytest.raises(H.HipqError) as e:
+            H.slice_(x, lower, upper, strides)
+        assert e.value.code == H.ERR_INVALID

@@ -294,3 +294,36 @@ def test_attention_in_one_kernel_rejects_other_shapes(gpu_lib):
         with pytest.raises(H.HipqError) as e:
             H.attention(qkv, 0, 64, 128, 2 * 64 * 64, view, 2, queries, keys, depth)
         assert e.value.code == H.ERR_UNSUPPORTED
+
+
+def test_attention_in_one_kernel_rejects_bad_arguments(gpu_lib):
+    """nothing is launched on operands the kernel's 16-byte fetches and its views could not honour"""
+    say("attention arguments")
+    lib = H.load()
+    import ctypes as C
+
+    S, hd = 128, 64
+    buf = H.DeviceBuffer(4 * (3 * S * hd + 8))
+    out = H.DeviceBuffer(4 * S * hd)
+    lib.hipq_attention_f32.argtypes = [C.c_void_p] * 7 + [C.c_int64] * 4 + [C.c_void_p]
+
+    def call(q_off=0, view=None, out_ptr=out.ptr, quant=None, view_ptr=True):
+        v = view or H.AttentionView(1, S * hd, 0, hd, S * hd, 0, hd, S * hd, 0, hd, S * hd, 0, hd)
+        return lib.hipq_attention_f32(buf.ptr + q_off, buf.ptr + 4 * S * hd, buf.ptr + 8 * S * hd, None, out_ptr, C.byref(v) if view_ptr else None, quant, 1, S, S, hd, None)
+
+    class _H:  # (the library's last error text)
+        @staticmethod
+        def last_error():
+            return lib.hipq_last_error().decode()
+
+    assert call() == H.OK
+    assert call(q_off=4) == H.ERR_INVALID and "16-byte aligned" in _H.last_error()
+    assert call(view=H.AttentionView(1, S * hd, 0, hd - 4, S * hd, 0, hd, S * hd, 0, hd, S * hd, 0, hd)) == H.ERR_INVALID and "shorter than the row" in _H.last_error()
+    assert call(view=H.AttentionView(1, S * hd, 0, hd + 2, S * hd, 0, hd, S * hd, 0, hd, S * hd, 0, hd)) == H.ERR_INVALID
+    assert call(view=H.AttentionView(1, -1, 0, hd, S * hd, 0, hd, S * hd, 0, hd, S * hd, 0, hd)) == H.ERR_INVALID and "negative batch stride" in _H.last_error()
+    assert call(view=H.AttentionView(0, S * hd, 0, hd, S * hd, 0, hd, S * hd, 0, hd, S * hd, 0, hd)) == H.ERR_INVALID
+    assert call(out_ptr=None) == H.ERR_INVALID and "null pointer" in _H.last_error()
+    assert call(view_ptr=False) == H.ERR_INVALID and "null view" in _H.last_error()
+    bad_quant = H.QuantOut(out.ptr, None, None, H.I8, H.RNE)
+    assert call(quant=C.byref(bad_quant)) == H.ERR_INVALID
+    H.check(lib.hipq_stream_sync(None))

@@ -486,7 +486,8 @@ def main():
     ap.add_argument("--resnet-only", action="store_true", help="only the synthetic int8 ResNet-50 (for profiling); prints its results")
     ap.add_argument("--bert-only", action="store_true", help="only the synthetic int8 BERT-base encoder (for profiling); prints its results")
     ap.add_argument("--skip-models", action="store_true", help="leave out the BERT and ResNet-50 sections (kernel traces of the single operators; the models have runs of their own)")
-    ap.add_argument("--only", choices=["gemm", "qdq"], help="only config 2's GEMMs or config 3's Quantize / Dequantize (for counter runs under a profiler); prints their results")
+    ap.add_argument("--only", choices=["gemm", "qdq", "glue"],
+                    help="only config 2's GEMMs, config 3's Quantize / Dequantize, or the encoder's fp32 glue and attention (for counter runs under a profiler); prints their results")
     ap.add_argument("--no-graph", action="store_true", help="time the models' eager launch sequences only, no HIP-graph capture or replay (for runs under a profiler)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -507,6 +508,9 @@ def main():
         return
     if args.only == "qdq":
         print(json.dumps({"quantize_dequantize_config3": bench_qdq(lib, stream, timer, args.steps, args.warmup), "copy_calibration": copy_calibration(lib, stream, timer)}))
+        return
+    if args.only == "glue":
+        print(json.dumps({"fp32_glue": bench_fp32_glue(lib, stream, timer, args.steps, args.warmup), "copy_calibration": copy_calibration(lib, stream, timer)}))
         return
     if args.resnet_only:
         print(json.dumps({"resnet50_int8": bench_resnet50(lib, stream, timer, use_graph=not args.no_graph)}))

@@ -364,6 +364,28 @@ HIPQ_API int hipq_quantized_dot_bias(const hipq_dot_desc_t* desc,
                                      void* out,
                                      void* stream);
 
+/*
+ * Quantize(Gelu(QuantizedDotBias(...) as f32)): the first projection of a transformer encoder's feed-forward
+ * block with the activation and the Quantize that follow it, one launch where the kernels that load
+ * straight into LDS take the product (more than 256 rows, more than 64 outputs in multiples of 16),
+ * the product into the library's workspace and hipq_gelu_quantize_f32 otherwise.  desc->out_t must be
+ * HIPQ_F32 (the form of the product); only quant->out ([M,N] bytes, 16-byte aligned, not overlapping a) is written, equal
+ * bit for bit to hipq_quantized_dot_bias followed by hipq_gelu_quantize_f32.  hipq_quant_out_t is declared
+ * with the fp32 glue below.  No counterpart as a single reference op
+ * (src/ngraph/op/experimental/quantized_dot_bias.cpp:27-56, src/ngraph/op/gelu.cpp:46-60,
+ * src/ngraph/runtime/reference/quantize.hpp:29-117).
+ */
+struct hipq_quant_out;
+HIPQ_API int hipq_quantized_dot_bias_gelu_quantize(const hipq_dot_desc_t* desc,
+                                                   const hipq_fused_desc_t* fused,
+                                                   const void* a,
+                                                   const void* w,
+                                                   const void* packed_w, /* may be NULL where the fused kernels apply; needed otherwise */
+                                                   const int32_t* bias,
+                                                   const float* scale,
+                                                   const struct hipq_quant_out* quant,
+                                                   void* stream);
+
 /* ---------------------------------------------------------------- layout helpers */
 
 /* [N,C,X] -> [N,X,C] and back for elem_bytes in {1,4}; X = product of spatial extents. */

@@ -163,11 +163,11 @@ class DevicePlan:
     the kernel launches of every layer on `stream`; `capture()` turns the pass into one HIP graph.
 
     fused=False launches the graph op by op, 19 launches a layer.  fused=True (what a backend's fusion
-    pass makes of the same graph, 10 launches a layer, 8 where a head has 128 keys of depth 64) folds the ops that only re-read and re-write a
+    pass makes of the same graph, 9 calls a layer, 7 where a head has 128 keys of depth 64) folds the ops that only re-read and re-write a
     tensor into their producers, each through an entry point whose result equals the op-by-op one bit
     for bit: the head split and merge become views of the attention products (scores, Softmax and
-    context of a head are one kernel at 128 keys of depth 64), Multiply goes into Softmax, the residual Add into LayerNorm, and every Quantize into the kernel that produces its
-    input (the context product, LayerNorm, Gelu)."""
+    context of a head are one kernel at 128 keys of depth 64), Multiply goes into Softmax, the residual Add into LayerNorm, Gelu into the projection in front of it, and every
+    Quantize into the kernel that produces its input (the context product, LayerNorm, that projection)."""
 
     def __init__(self, lib, stream, batch, cfg=BASE, fused=True):
         self.lib, self.stream, self.batch, self.cfg = lib, stream, batch, cfg
@@ -197,12 +197,22 @@ class DevicePlan:
             d = self._keep(H.make_quant_desc((T, n_cols), (), np.float32, "i8"))
             call(lib.hipq_quantize, d, src, scales[s], zero, x8)
 
-        def dot(wts, K, N, out):
+        def dot(wts, K, N, out, src=None):
+            wq, bias, scale = wts
+            src = x8 if src is None else src
+            d = self._keep(H.make_dot_desc(T, K, N, a_t="i8", out_t="f32", b_layout=H.B_NK))
+            fd = self._keep(H.make_fused_desc(has_bias=True, with_relu=False, scale_count=N))
+            bw = dev(wq)
+            call(lib.hipq_quantized_dot_bias, d, fd, src, bw, self._keep(H.pack_dot(d, bw)), dev(bias), dev(scale), out)
+
+        def dot_gelu_quantize(wts, K, N, quant):
+            # the projection with Gelu and the Quantize behind it in one call (in the product's epilogue where
+            # the library's tile kernels take it, through its workspace otherwise)
             wq, bias, scale = wts
             d = self._keep(H.make_dot_desc(T, K, N, a_t="i8", out_t="f32", b_layout=H.B_NK))
             fd = self._keep(H.make_fused_desc(has_bias=True, with_relu=False, scale_count=N))
             bw = dev(wq)
-            call(lib.hipq_quantized_dot_bias, d, fd, x8, bw, self._keep(H.pack_dot(d, bw)), dev(bias), dev(scale), out)
+            call(lib.hipq_quantized_dot_bias_gelu_quantize, d, fd, x8, bw, self._keep(H.pack_dot(d, bw)), dev(bias), dev(scale), quant)
 
         def permute(src, dst, shape, order):
             call(lib.hipq_permute, 4, src, dst, len(shape), self._keep((i64 * len(shape))(*shape)), self._keep((i32 * len(shape))(*order)))
@@ -213,7 +223,10 @@ class DevicePlan:
             lib.hipq_add_layer_norm_f32.argtypes = [vp] * 6 + [i64, i64, C.c_double, vp]
             lib.hipq_batch_matmul_view_f32.argtypes = [vp] * 5 + [i64] * 4 + [i32] * 2 + [vp]
             lib.hipq_attention_f32.argtypes = [vp] * 7 + [i64] * 4 + [vp]
+            lib.hipq_quantized_dot_bias_gelu_quantize.argtypes = [vp] * 9
             qout = {s: self._keep(H.QuantOut(x8.ptr, scales[s].ptr, zero.ptr, H.I8, H.RNE)) for s in scales}
+            g8 = new(T * f)
+            gelu_out = self._keep(H.QuantOut(g8.ptr, scales[cfg.s_g].ptr, zero.ptr, H.I8, H.RNE))
             H3 = 3 * h
             # Q, K, V of batch element (b, head): rows of the [T, 3H] projection, 3H apart, starting at column
             # {0, H, 2H} + head * hd; scores [B * heads, S, S] dense; the context goes straight into [T, H]
@@ -236,9 +249,8 @@ class DevicePlan:
                 dot(w["out"], h, h, proj)
                 g1, b1 = dev(w["ln1"][0]), dev(w["ln1"][1])
                 call(lib.hipq_add_layer_norm_f32, self.x, proj, g1, b1, x1, qout[cfg.s_x], T, h, 1e-5)
-                dot(w["ffn1"], h, f, ffn)
-                call(lib.hipq_gelu_quantize_f32, ffn, None, qout[cfg.s_g], T * f)
-                dot(w["ffn2"], f, h, proj)
+                dot_gelu_quantize(w["ffn1"], h, f, gelu_out)  # (reads x8: its bytes go to a tensor of their own)
+                dot(w["ffn2"], f, h, proj, src=g8)
                 g2, b2 = dev(w["ln2"][0]), dev(w["ln2"][1])
                 call(lib.hipq_add_layer_norm_f32, x1, proj, g2, b2, self.x, qout[cfg.s_x] if l + 1 < cfg.layers else None, T, h, 1e-5)
             return

@@ -106,6 +106,12 @@ namespace hipq
         int sum_t;
         int relu;
         int per_channel; // scale_count > 1
+        // EPI_FUSED with out_t F32, optional: the result goes through Gelu and Quantize (one scale and
+        // zero point, device scalars) and only the quantized tensor is written
+        const float* post_scale; // null: none
+        const void* post_zp;
+        int post_t;    // HIPQ_I8 / HIPQ_U8
+        int post_mode; // round mode of the Quantize
     };
 
     // zero points of the accumulation, device scalars typed like their tensors (null = 0)
@@ -259,6 +265,9 @@ namespace hipq
 
     int launch_rows_mfma(const void* a, bool a_unsigned, const int8_t* w_nk, const int32_t* wsum, int64_t M, int32_t N, int32_t K,
                          const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s, const char* name);
+
+    int launch_rows_gelu_q8(const void* a, bool a_unsigned, const int8_t* w_nk, const int32_t* wsum, int64_t M, int32_t N, int32_t K, const ZeroPoints& zp, const Epilogue& epi,
+                            void* out, hipStream_t s);
 
     int launch_transpose(const void* in, void* out, int64_t N, int64_t R, int64_t Cc, int elem_bytes, hipStream_t s);
     int launch_pad_channels(const void* in, void* out, int64_t N, int64_t X, int64_t Cc, bool in_ncx, const void* zp, int zp_t, hipStream_t s);

@@ -30,6 +30,8 @@
 #include <type_traits>
 
 #include "hipq_common.h"
+#include "hipq_quant_math.h"
+#include "hipq_row_math.h"
 
 namespace hipq
 {
@@ -460,7 +462,8 @@ namespace hipq
     {
         OUT_Q8 = 0, // u8 or i8, packed four to a dword by the caller
         OUT_I32 = 1,
-        OUT_F32 = 2
+        OUT_F32 = 2,
+        OUT_GELU_Q8 = 3 // the float result through Gelu and Quantize: only the 8-bit tensor is written
     };
 
     struct EpiConst
@@ -1052,7 +1055,8 @@ namespace hipq
         const EpiConst ec = epi_const(epi);
         constexpr bool has_sum = HAS_SUM; // residual input (fused policy only)
         static_assert(!HAS_SUM || MODE == EPI_FUSED, "only the fused policy adds a residual");
-        static_assert(KIND == OUT_Q8 || (KIND == OUT_F32 && DMA && MODE == EPI_FUSED && !HAS_SUM), "float outputs: fused policy, no residual, loads straight into LDS");
+        static_assert(KIND == OUT_Q8 || ((KIND == OUT_F32 || KIND == OUT_GELU_Q8) && DMA && MODE == EPI_FUSED && !HAS_SUM),
+                      "float outputs: fused policy, no residual, loads straight into LDS");
 
         // ---- loader --------------------------------------------------------------------------
         const int lrow = tid / LPR;
@@ -1289,6 +1293,10 @@ namespace hipq
         const float magic = 12582912.0f; // 1.5 * 2^23: adding it rounds half to even into the low mantissa bits
         const float s256 = __fmul_rn(ec.scale, 256.0f);
         const int32_t c256 = 128 + 256 * ec.ozp;
+        // (Gelu + Quantize of a float result: the Quantize's scale and zero point)
+        const float post_scale = KIND == OUT_GELU_Q8 ? *epi.post_scale : 1.0f;
+        const int32_t post_zp_i = KIND == OUT_GELU_Q8 ? load_zp(epi.post_zp, epi.post_t) : 0;
+        const float post_zp = static_cast<float>(post_zp_i);
         // the fixed-point form needs |acc * scale| * 256 < 2^31 with room to spare
         const bool fast_interp = fabsf(ec.scale) * (static_cast<float>(Kred) * (255.0f * 128.0f)) < 4194304.0f;
         constexpr int SUM_LOADS = TM * TN / 16 / 64;
@@ -1423,6 +1431,32 @@ namespace hipq
                         // round-half-away(v) = (t + 128 - (t < 0)) >> 8 exactly
                         int32_t x[4];
                         uint32_t packed = 0;
+                        if constexpr (KIND == OUT_GELU_Q8)
+                        {
+                            // the float result exactly as the float kernel computes it, then Gelu and
+                            // Quantize with the arithmetic of their own kernels (gelu1, quantize4 /
+                            // quantize_one): the bytes equal the three launches'
+                            v4f r4;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                            {
+                                const float a = static_cast<float>(acc[mi][ni][4 * g + e]);
+                                const float y = __fmul_rn(FOLD ? a : __fadd_rn(a, bias4[e]), scale4[e]);
+                                r4[e] = gelu1(epi.relu ? ((y > 0.0f) ? y : __fmul_rn(y, -0.0f)) : y);
+                            }
+                            if (epi.post_mode == HIPQ_ROUND_NEAREST_TOWARD_EVEN) // uniform
+                                packed = epi.post_t == HIPQ_U8 ? quantize4<uint8_t, true>(r4, post_scale, post_zp, epi.post_mode) : quantize4<int8_t, true>(r4, post_scale, post_zp, epi.post_mode);
+                            else
+                            {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e)
+                                    packed |= (epi.post_t == HIPQ_U8 ? static_cast<uint32_t>(quantize_one<float, uint8_t>(r4[e], post_scale, static_cast<uint8_t>(post_zp_i), epi.post_mode))
+                                                                     : static_cast<uint32_t>(static_cast<uint8_t>(quantize_one<float, int8_t>(r4[e], post_scale, static_cast<int8_t>(post_zp_i), epi.post_mode))))
+                                              << (8 * e);
+                            }
+                            *cell = packed;
+                            continue;
+                        }
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
                         {
@@ -1876,6 +1910,10 @@ namespace hipq
             return HIPQ_ERR_UNSUPPORTED;
         if (f32 && !XL::kFloatOut)
             return HIPQ_ERR_UNSUPPORTED;
+        // Gelu + Quantize in the epilogue: the wide float-output kernels only
+        const bool gelu_q8 = epi.post_scale != nullptr;
+        if (gelu_q8 && (!f32 || N <= 64))
+            return HIPQ_ERR_UNSUPPORTED;
         // row matrices with reductions in whole 128-byte pieces, no residual, wide outputs: deep slices
         bool deep = false;
         if constexpr (XL::kDeep)
@@ -1897,6 +1935,12 @@ namespace hipq
         if constexpr (XL::kFloatOut)
             if (f32)
             {
+                if (gelu_q8)
+                {
+                    if (deep)
+                        return launch_pipe<XL, 2, 2, EPI_FUSED, false, OUT_GELU_Q8, 2 * BK>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+                    return launch_pipe<XL, 2, 2, EPI_FUSED, false, OUT_GELU_Q8>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+                }
                 if (N <= 64)
                     return launch_pipe<XL, 4, 1, EPI_FUSED, false, OUT_F32>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
                 if (deep)

@@ -587,6 +587,20 @@ namespace hipq
         return launch_epilogue<GemmX, false>(xl, w_nk, wsum, M, N, K, a_unsigned ? 1 : 0, zp, epi, om, out, s, name);
     }
 
+    // Quantize(Gelu(rows x weights -> f32)) with Gelu and Quantize in the epilogue of the kernels that
+    // load straight into LDS; HIPQ_ERR_UNSUPPORTED (nothing launched, no error text) when the call is
+    // not of their kind.  epi carries the Quantize in its post_* fields; out is the 8-bit tensor.
+    int launch_rows_gelu_q8(const void* a, bool a_unsigned, const int8_t* w_nk, const int32_t* wsum, int64_t M, int32_t N, int32_t K, const ZeroPoints& zp, const Epilogue& epi,
+                            void* out, hipStream_t s)
+    {
+        OutMap om{0, N, 1};
+        RowsU xu;
+        xu.x = static_cast<const uint8_t*>(a);
+        xu.K = K;
+        xu.bytes = static_cast<uint32_t>(M * K);
+        return launch_uniform(xu, w_nk, wsum, M, N, K, a_unsigned ? 1 : 0, zp, epi, om, out, s, "dot_gelu_q8_mfma_i8_32x32x32");
+    }
+
     bool dot_mfma_eligible(const hipq_dot_desc_t& d)
     {
         if (d.b_t != HIPQ_I8 || (d.a_t != HIPQ_U8 && d.a_t != HIPQ_I8))

@@ -160,14 +160,6 @@ namespace hipq
                 y[a * inner] = expf(at(a) - m) / s;
         }
 
-        // Gelu as the reference decomposes it (src/ngraph/op/gelu.cpp:46-60):
-        // (0.5 * x) * (1 + erf(x / float(sqrt(2.0)))), every step rounded to f32
-        __device__ __forceinline__ float gelu1(float x)
-        {
-            const float sqrt_two = 1.41421354f; // float(std::sqrt(2.0))
-            return __fmul_rn(__fmul_rn(0.5f, x), __fadd_rn(1.0f, erff(__fdiv_rn(x, sqrt_two))));
-        }
-
         template <bool GELU>
         __global__ __launch_bounds__(256) void erf_kernel(const float* __restrict__ in, float* __restrict__ out, QuantOut q, int64_t count, int32_t vec_ok)
         {

@@ -401,4 +401,70 @@ int hipq_quantized_dot_bias(const hipq_dot_desc_t* d,
     ZeroPoints zp{nullptr, nullptr, d->a_t, d->b_t};
     return run_dot(*d, a, w, packed_w, zp, e, out, as_stream(stream));
 }
+
+int hipq_quantized_dot_bias_gelu_quantize(const hipq_dot_desc_t* d,
+                                          const hipq_fused_desc_t* fused,
+                                          const void* a,
+                                          const void* w,
+                                          const void* packed_w,
+                                          const int32_t* bias,
+                                          const float* scale,
+                                          const hipq_quant_out_t* quant,
+                                          void* stream)
+{
+    HIPQ_REQUIRE(d, "descriptor is null");
+    HIPQ_REQUIRE(d->M >= 0 && d->N >= 0 && d->K >= 0, "negative extent");
+    HIPQ_REQUIRE(d->b_layout == HIPQ_B_KN || d->b_layout == HIPQ_B_NK, "bad b_layout");
+    if (!is_quant8(d->a_t) || d->b_t != HIPQ_I8 || d->out_t != HIPQ_F32)
+        return fail(HIPQ_ERR_UNSUPPORTED, "QuantizedDotBias + Gelu + Quantize takes u8/i8 data, i8 weights and the f32 form of the product (out_t F32)");
+    HIPQ_REQUIRE(fused && !fused->has_sum, "QuantizedDotBias has no sum input");
+    HIPQ_REQUIRE(quant && quant->out && quant->scale, "quantized output: null pointer");
+    HIPQ_REQUIRE(quant->quant_t == HIPQ_I8 || quant->quant_t == HIPQ_U8, "quantized output: i8 or u8");
+    HIPQ_REQUIRE(quant->round_mode >= HIPQ_ROUND_NEAREST_TOWARD_INFINITY && quant->round_mode <= HIPQ_ROUND_DOWN, "quantized output: unknown round mode");
+    if (d->M == 0 || d->N == 0)
+        return HIPQ_OK;
+    HIPQ_REQUIRE(d->K == 0 || (a && w), "null tensor pointer");
+    {
+        // workgroups write their output bytes while others still read rows of `a`
+        const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), a1 = a0 + static_cast<size_t>(d->M * d->K);
+        const uintptr_t o0 = reinterpret_cast<uintptr_t>(quant->out), o1 = o0 + static_cast<size_t>(d->M * d->N);
+        HIPQ_REQUIRE(a1 <= o0 || o1 <= a0, "the quantized output must not overlap the input rows");
+    }
+    Epilogue e;
+    int rc = fused_epilogue(fused, HIPQ_F32, d->N, bias, nullptr, scale, nullptr, &e);
+    if (rc)
+        return rc;
+    hipStream_t s = as_stream(stream);
+    // in the epilogue of the product, where the kernels that take it apply
+    if (dot_mfma_eligible(*d) && d->M > 256 && (reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0 && (reinterpret_cast<uintptr_t>(quant->out) & 15) == 0)
+    {
+        const void* wn = nullptr;
+        const int32_t* wsum = nullptr;
+        rc = dot_operands(*d, w, packed_w, &wn, &wsum, s);
+        if (rc)
+            return rc;
+        Epilogue post = e;
+        post.post_scale = quant->scale;
+        post.post_zp = quant->zero_point;
+        post.post_t = quant->quant_t;
+        post.post_mode = quant->round_mode;
+        ZeroPoints zp{nullptr, nullptr, d->a_t, d->b_t};
+        rc = launch_rows_gelu_q8(a, d->a_t == HIPQ_U8, static_cast<const int8_t*>(wn), wsum, d->M, static_cast<int32_t>(d->N), static_cast<int32_t>(d->K), zp, post, quant->out, s);
+        if (rc != HIPQ_ERR_UNSUPPORTED)
+            return rc;
+    }
+    // otherwise the product into the workspace, then Gelu + Quantize from there (prepacked weights only:
+    // weights packed on the fly live in the same workspace)
+    if (!packed_w)
+        return fail(HIPQ_ERR_UNSUPPORTED, "QuantizedDotBias + Gelu + Quantize outside the fused kernels needs prepacked weights (hipq_dot_pack)");
+    float* product = nullptr;
+    rc = workspace(static_cast<size_t>(d->M) * static_cast<size_t>(d->N) * sizeof(float), s, reinterpret_cast<void**>(&product));
+    if (rc)
+        return rc;
+    ZeroPoints zp{nullptr, nullptr, d->a_t, d->b_t};
+    rc = run_dot(*d, a, w, packed_w, zp, e, product, s);
+    if (rc)
+        return rc;
+    return hipq_gelu_quantize_f32(product, nullptr, quant, d->M * d->N, stream);
+}
 }

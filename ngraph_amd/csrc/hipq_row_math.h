@@ -51,4 +51,13 @@ namespace hipq
         s = wave_sum<W>(s);
         return row_f4{v[0] / s, v[1] / s, v[2] / s, v[3] / s};
     }
+    // Gelu as the reference decomposes it (src/ngraph/op/gelu.cpp:46-60):
+    // (0.5 * x) * (1 + erf(x / float(sqrt(2.0)))), every step rounded to f32.  Shared by the Gelu
+    // kernel and by the GEMM epilogue that applies Gelu to what it has just computed.
+    __device__ __forceinline__ float gelu1(float x)
+    {
+        const float sqrt_two = 1.41421354f; // float(std::sqrt(2.0))
+        return __fmul_rn(__fmul_rn(0.5f, x), __fadd_rn(1.0f, erff(__fdiv_rn(x, sqrt_two))));
+    }
+
 }

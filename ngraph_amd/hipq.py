@@ -304,6 +304,7 @@ EXPORTS = [
     "hipq_dot_pack",
     "hipq_quantized_dot",
     "hipq_quantized_dot_bias",
+    "hipq_quantized_dot_bias_gelu_quantize",
     "hipq_transpose_ncx_to_nxc",
     "hipq_transpose_nxc_to_ncx",
     "hipq_binary",
@@ -714,6 +715,20 @@ def quantized_dot_bias(desc, fused, a, w, bias, scale, prepare=True):
     )
     check(lib.hipq_stream_sync(None))
     return out.to_numpy(NP_OF[desc.out_t], (int(desc.M), int(desc.N)))
+
+
+def quantized_dot_bias_gelu_quantize(desc, fused, a, w, bias, scale, q_scale, q_zp=0, quant_t="i8", round_mode=RNE, prepare=True):
+    """Quantize(Gelu(QuantizedDotBias(...) as f32)) through hipq_quantized_dot_bias_gelu_quantize: the [M, N] bytes"""
+    lib = load()
+    ba, bw = _dev(a), _dev(w)
+    wsum = pack_dot(desc, bw) if prepare else None
+    bb = _dev(None if bias is None else np.asarray(bias, dtype=np.int32))
+    bsc = _dev(np.asarray(scale, dtype=np.float32))
+    q, keep, qt = _quant_out(int(desc.M * desc.N), q_scale, q_zp, quant_t, round_mode)
+    lib.hipq_quantized_dot_bias_gelu_quantize.argtypes = [C.c_void_p] * 9
+    check(lib.hipq_quantized_dot_bias_gelu_quantize(C.byref(desc), C.byref(fused), ba.ptr, bw.ptr, _p(wsum), _p(bb), bsc.ptr, C.byref(q), None))
+    check(lib.hipq_stream_sync(None))
+    return keep[0].to_numpy(NP_OF[qt], (int(desc.M), int(desc.N)))
 
 
 # ---- fp32 glue of a transformer encoder -----------------------------------------------------------

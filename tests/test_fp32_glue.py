@@ -327,3 +327,55 @@ def test_attention_in_one_kernel_rejects_bad_arguments(gpu_lib):
     bad_quant = H.QuantOut(out.ptr, None, None, H.I8, H.RNE)
     assert call(quant=C.byref(bad_quant)) == H.ERR_INVALID
     H.check(lib.hipq_stream_sync(None))
+
+
+@pytest.mark.parametrize("M,K,N,kernel", [(4096, 768, 3072, "dot_gelu_q8"), (512, 256, 80, "dot_gelu_q8"), (1000, 320, 144, "dot_gelu_q8"), (4096, 768, 3000, "gelu_vec"), (128, 768, 3072, "gelu_vec"),
+                                          (300, 64, 64, "gelu_vec"), (2048, 1024, 1024, "dot_gelu_q8")])
+def test_dot_bias_gelu_quantize_equals_the_three_ops(gpu_lib, M, K, N, kernel):
+    """the feed-forward block's first projection with Gelu and Quantize in its epilogue (or, where those
+    kernels do not apply, through the workspace) against QuantizedDotBias -> Gelu -> Quantize, bit for bit"""
+    say("dot + gelu + quantize", M, K, N)
+    a = synth.uniform_int(60, (M, K), -127, 127, np.int8)
+    w = synth.uniform_int(61, (N, K), -127, 127, np.int8)
+    bias = synth.uniform_int(62, (N,), -3000, 3000, np.int32)
+    scale = synth.uniform_f32(63, (N,), 0.5, 1.5) * f32(4.0 / (127.0 * 127.0 * np.sqrt(K)))
+    d = H.make_dot_desc(M, K, N, a_t="i8", out_t="f32", b_layout=H.B_NK)
+    fd = H.make_fused_desc(has_bias=True, with_relu=False, scale_count=N)
+    product = H.quantized_dot_bias(d, fd, a, w, bias, scale)
+    for quant_t, zp, s, mode in (("i8", 0, 3.0 / 127.0, H.RNE), ("u8", 9, 0.02, H.RNE), ("i8", -5, 0.03, H.ROUND_MODES.index("ROUND_NEAREST_TOWARD_INFINITY"))):
+        _, exp = H.gelu_quantize(product, s, zp, quant_t, round_mode=mode, keep_f32=False)
+        got = H.quantized_dot_bias_gelu_quantize(d, fd, a, w, bias, scale, s, zp, quant_t, round_mode=mode)
+        assert np.array_equal(got, exp), (quant_t, zp)
+        assert kernel in H.last_kernel(), H.last_kernel()
+        assert len(np.unique(got)) > 20
+    # one scale for all channels, ReLU in front of the Gelu, u8 data
+    au = synth.uniform_int(64, (M, K), 0, 255, np.uint8)
+    du = H.make_dot_desc(M, K, N, a_t="u8", out_t="f32", b_layout=H.B_NK)
+    f1 = H.make_fused_desc(has_bias=True, with_relu=True, scale_count=1)
+    product = H.quantized_dot_bias(du, f1, au, w, bias, scale[:1])
+    _, exp = H.gelu_quantize(product, 0.05, 0, "u8", keep_f32=False)
+    assert np.array_equal(H.quantized_dot_bias_gelu_quantize(du, f1, au, w, bias, scale[:1], 0.05, 0, "u8"), exp)
+
+
+def test_dot_bias_gelu_quantize_refuses_output_over_its_input(gpu_lib):
+    """workgroups write output bytes while others still read rows of the data: an output that overlaps
+    the data is refused before any launch"""
+    say("dot + gelu + quantize in place")
+    import ctypes as C
+
+    lib = H.load()
+    M, K, N = 512, 256, 128
+    d = H.make_dot_desc(M, K, N, a_t="i8", out_t="f32", b_layout=H.B_NK)
+    fd = H.make_fused_desc(has_bias=False, with_relu=False, scale_count=1)
+    buf = H.DeviceBuffer(M * max(K, N) + M * N)
+    w = H.DeviceBuffer.from_numpy(synth.uniform_int(65, (N, K), -127, 127, np.int8))
+    scale = H.DeviceBuffer.from_numpy(np.asarray([0.001], np.float32))
+    qs = H.DeviceBuffer.from_numpy(np.asarray([0.05], np.float32))
+    lib.hipq_quantized_dot_bias_gelu_quantize.argtypes = [C.c_void_p] * 9
+    for out_ptr, ok in ((buf.ptr, False), (buf.ptr + M * K - 16, False), (buf.ptr + M * K, True)):
+        q = H.QuantOut(out_ptr, qs.ptr, None, H.I8, H.RNE)
+        rc = lib.hipq_quantized_dot_bias_gelu_quantize(C.byref(d), C.byref(fd), buf.ptr, w.ptr, None, None, scale.ptr, C.byref(q), None)
+        assert (rc == H.OK) == ok, (out_ptr - buf.ptr, rc)
+        if not ok:
+            assert rc == H.ERR_INVALID and "overlap" in lib.hipq_last_error().decode()
+    H.check(lib.hipq_stream_sync(None))

@@ -156,7 +156,7 @@ namespace
         void* constant_ptr(const Output<Node>& o) const;
         void lower(const shared_ptr<Node>& n);
         void lower_conv(const shared_ptr<Node>& n, Step& st);
-        void lower_dot(const shared_ptr<Node>& n, Step& st);
+        void lower_dot(const shared_ptr<Node>& n, Step& st, const hipq_quant_out_t* gelu_quantize = nullptr, int gelu_quantize_at = -1);
         void lower_pool(const shared_ptr<Node>& n, Step& st);
         void assign_layouts();
         void plan_glue_fusion();
@@ -199,6 +199,7 @@ namespace
             float scale;
             int32_t zero_point;
             bool only_user; // the f32 result has no other reader
+            bool through_gelu = false; // keyed by a QuantizedDotBias: a folded Gelu stands between it and the Quantize
         };
         unordered_map<const Node*, QuantizedCopy> m_quantized_copy;
         vector<void*> m_value_ptr;                  // persistent device pointer, or null when bound per call
@@ -455,6 +456,24 @@ namespace
             m_quantized_copy[producer] = QuantizedCopy{n, scale, zp, single_user(producer)};
             m_folded.insert(n.get());
         }
+        // Quantize(Gelu(QuantizedDotBias -> f32)) with nothing else reading the product or the Gelu, and
+        // constant (prepacked) weights: Gelu and Quantize ride in the product's epilogue
+        for (const auto& n : m_function->get_ordered_ops())
+        {
+            if (!is_type<op::v0::Gelu>(n))
+                continue;
+            const auto qc = m_quantized_copy.find(n.get());
+            if (qc == m_quantized_copy.end() || !qc->second.only_user)
+                continue;
+            const Node* dot = n->input_value(0).get_node();
+            if (!is_type<op::v0::QuantizedDotBias>(dot) || !single_user(dot) || dot->get_output_element_type(0) != element::f32 || !dot->get_argument(1)->is_constant())
+                continue;
+            QuantizedCopy copy = qc->second;
+            copy.through_gelu = true;
+            m_quantized_copy.erase(qc);
+            m_quantized_copy[dot] = copy;
+            m_folded.insert(n.get());
+        }
     }
 
     void HIPExecutable::assign_layouts()
@@ -591,7 +610,7 @@ namespace
         };
     }
 
-    void HIPExecutable::lower_dot(const shared_ptr<Node>& n, Step& st)
+    void HIPExecutable::lower_dot(const shared_ptr<Node>& n, Step& st, const hipq_quant_out_t* gelu_quantize, int gelu_quantize_at)
     {
         hipq_dot_desc_t d;
         memset(&d, 0, sizeof(d));
@@ -642,6 +661,18 @@ namespace
         {
             packed = alloc(pb);
             check(hipq_dot_pack(&d, constant_ptr(n->input_value(1)), packed->ptr, m_stream), "QuantizedDotBias weight packing");
+        }
+        if (gelu_quantize)
+        {
+            // Quantize(Gelu(product)): the bytes go to the folded Quantize's value; the product's own value stays unwritten
+            const hipq_quant_out_t q0 = *gelu_quantize;
+            st.launch = [d, f, packed, q0, gelu_quantize_at](const vector<void*>& in, void*, void* stream) {
+                hipq_quant_out_t q = q0;
+                q.out = in[gelu_quantize_at];
+                check(hipq_quantized_dot_bias_gelu_quantize(&d, &f, in[0], in[1], packed ? packed->ptr : nullptr, static_cast<const int32_t*>(in[2]), static_cast<const float*>(in[3]), &q, stream),
+                      "QuantizedDotBias with Gelu and Quantize");
+            };
+            return;
         }
         st.launch = [d, f, packed](const vector<void*>& in, void* out, void* stream) {
             check(hipq_quantized_dot_bias(&d, &f, in[0], in[1], packed ? packed->ptr : nullptr, static_cast<const int32_t*>(in[2]),
@@ -893,7 +924,7 @@ namespace
         }
         else if (is_type<op::v0::QuantizedDot>(n) || is_type<op::v0::QuantizedDotBias>(n))
         {
-            lower_dot(n, st);
+            lower_dot(n, st, qcopy_at >= 0 ? &qcopy : nullptr, qcopy_at);
         }
         else if (binary_code(*n) >= 0)
         {

@@ -380,3 +380,55 @@ GPU_TEST(HIP, glue_fusion_attention_of_a_batch_of_heads)
         EXPECT_EQ(fused.launches, size_t(3));
     }
 }
+
+GPU_TEST(HIP, glue_fusion_dot_bias_with_gelu_and_quantize)
+{
+    // Quantize(Gelu(QuantizedDotBias(Quantize(x), W, b, s) as f32)): Gelu and the Quantize behind it ride
+    // in the product's epilogue (512 rows: the tile kernels' own epilogue; 40 rows: through the
+    // library's workspace) -- two launches fewer, the same bytes
+    for (const size_t rows : {size_t(512), size_t(40)})
+    {
+        const size_t K = 256, N = 128;
+        auto x = make_shared<op::v0::Parameter>(element::f32, Shape{rows, K});
+        auto xs = op::v0::Constant::create(element::f32, Shape{}, {0.02f});
+        auto xz = op::v0::Constant::create(element::i8, Shape{}, {0});
+        auto x8 = make_shared<op::v0::Quantize>(x, xs, xz, element::i8, AxisSet{}, op::v0::Quantize::RoundMode::ROUND_NEAREST_TOWARD_EVEN);
+        vector<int8_t> w(N * K);
+        for (size_t i = 0; i < w.size(); ++i)
+            w[i] = static_cast<int8_t>(static_cast<int>((i * 37 + i / K * 11) % 255) - 127);
+        vector<int32_t> b(N);
+        vector<float> s(N);
+        for (size_t i = 0; i < N; ++i)
+        {
+            b[i] = static_cast<int32_t>(i * 13) - 700;
+            s[i] = 0.0002f + 0.000001f * static_cast<float>(i);
+        }
+        auto W = op::v0::Constant::create(element::i8, Shape{N, K}, w);
+        auto B = op::v0::Constant::create(element::i32, Shape{N}, b);
+        auto S = op::v0::Constant::create(element::f32, Shape{N}, s);
+        auto dot = make_shared<op::v0::QuantizedDotBias>(x8, W, B, S, false, false);
+        auto gelu = make_shared<op::v0::Gelu>(dot);
+        auto qs = op::v0::Constant::create(element::f32, Shape{}, {0.03f});
+        auto qz = op::v0::Constant::create(element::i8, Shape{}, {-3});
+        auto q = make_shared<op::v0::Quantize>(gelu, qs, qz, element::i8, AxisSet{}, op::v0::Quantize::RoundMode::ROUND_NEAREST_TOWARD_EVEN);
+        const auto data = wave(rows * K, 1.8f, 0.013f);
+        {
+            auto f = make_shared<Function>(OutputVector{q}, ParameterVector{x});
+            const auto plain = run_glue(f, {data}, false), fused = run_glue(f, {data}, true);
+            EXPECT_TRUE(plain.bytes == fused.bytes);
+            EXPECT_EQ(plain.launches, size_t(4)); // Quantize, product, Gelu, Quantize
+            EXPECT_EQ(fused.launches, size_t(2)); // Quantize, product with Gelu and Quantize
+            size_t distinct[256] = {0}, kinds = 0;
+            for (uint8_t v : fused.bytes.at(0))
+                kinds += distinct[v]++ == 0;
+            EXPECT_TRUE(kinds > 20);
+        }
+        {
+            // the product has a second reader: only the Quantize goes into the Gelu
+            auto f = make_shared<Function>(OutputVector{q, dot}, ParameterVector{x});
+            const auto plain = run_glue(f, {data}, false), fused = run_glue(f, {data}, true);
+            EXPECT_TRUE(plain.bytes == fused.bytes);
+            EXPECT_EQ(fused.launches, size_t(3));
+        }
+    }
+}

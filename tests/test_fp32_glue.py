@@ -330,7 +330,7 @@ def test_attention_in_one_kernel_rejects_bad_arguments(gpu_lib):
 
 
 @pytest.mark.parametrize("M,K,N,kernel", [(4096, 768, 3072, "dot_gelu_q8"), (512, 256, 80, "dot_gelu_q8"), (1000, 320, 144, "dot_gelu_q8"), (4096, 768, 3000, "gelu_vec"), (128, 768, 3072, "gelu_vec"),
-                                          (300, 64, 64, "gelu_vec"), (2048, 1024, 1024, "dot_gelu_q8")])
+                                          (300, 64, 64, "gelu_vec"), (2048, 1024, 1024, "dot_gelu_q8"), (512, 4096, 128, "dot_gelu_q8"), (384, 8192, 256, "dot_gelu_q8")])
 def test_dot_bias_gelu_quantize_equals_the_three_ops(gpu_lib, M, K, N, kernel):
     """the feed-forward block's first projection with Gelu and Quantize in its epilogue (or, where those
     kernels do not apply, through the workspace) against QuantizedDotBias -> Gelu -> Quantize, bit for bit"""

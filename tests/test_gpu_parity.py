@@ -1016,3 +1016,105 @@ def test_dot_rows64(gpu_lib, shape):
             assert H.last_kernel().startswith("dot_rows64"), H.last_kernel()
             assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), (a_t, out_t, relu)
     O.port().orc_set_threads(1)
+
+
+def _random_conv_case(rng):
+    """a random geometry the reference accepts: 1 to 3 spatial axes, strides, filter and data dilation,
+    positive and negative padding, channel counts on and off the matrix kernels' multiples"""
+    ns = int(rng.integers(1, 4))
+    N = int(rng.integers(1, 4))
+    Cc = int(rng.choice([1, 3, 4, 7, 16, 32, 48, 64, 96, 128]))
+    K = int(rng.choice([1, 5, 16, 24, 32, 64, 80, 128]))
+    limit = {1: 40, 2: 14, 3: 6}[ns]
+    for _ in range(100):
+        in_sp = [int(rng.integers(1, limit + 1)) for _ in range(ns)]
+        f_sp = [int(rng.integers(1, 4)) for _ in range(ns)]
+        kw = dict(
+            stride=[int(rng.integers(1, 3)) for _ in range(ns)],
+            dilation=[int(rng.integers(1, 3)) for _ in range(ns)],
+            pad_below=[int(rng.integers(-1, 3)) for _ in range(ns)],
+            pad_above=[int(rng.integers(-1, 3)) for _ in range(ns)],
+            data_dilation=[int(rng.choice([1, 1, 1, 2])) for _ in range(ns)],
+        )
+        ok = True
+        for i in range(ns):
+            padded = (in_sp[i] - 1) * kw["data_dilation"][i] + 1 + kw["pad_below"][i] + kw["pad_above"][i]
+            window = (f_sp[i] - 1) * kw["dilation"][i] + 1
+            ok = ok and padded >= window and padded >= 1
+        if ok:
+            return N, Cc, K, in_sp, f_sp, kw
+    return N, Cc, K, [4] * ns, [1] * ns, dict()
+
+
+@pytest.mark.parametrize("block", range(6))
+def test_conv_random_geometries(gpu_lib, block):
+    """seeded sweep: every case against the oracle, bit for bit, in the reference's layouts and (2-D and
+    below) channels-last; INTERPRETER arithmetic with zero points on all three tensors"""
+    rng = np.random.default_rng(9000 + block)
+    kernels = set()
+    for case in range(12):
+        N, Cc, K, in_sp, f_sp, kw = _random_conv_case(rng)
+        data_t = "u8" if rng.integers(0, 4) else "i8"
+        out_t = str(rng.choice(["i8", "u8", "i32"])) if data_t == "u8" else "i32"
+        filter_t = "i8" if out_t != "u8" else "u8"
+        zps = (int(rng.integers(0, 200)) if data_t == "u8" else int(rng.integers(-100, 100)), int(rng.choice([0, 0, 3])) if filter_t == "i8" else int(rng.choice([0, 130])),
+               int(rng.integers(-20, 20)) if out_t != "u8" else int(rng.integers(0, 30)))
+        scales = (1.0, 1.0, 1.0) if out_t == "i32" else (0.02, 0.005, float(rng.choice([0.9, 0.05, 2.5])))
+        if out_t == "i32":
+            zps = (zps[0], zps[1], 0)
+        say("random conv", block, case, N, Cc, K, in_sp, f_sp, kw, data_t, filter_t, out_t, zps)
+        layouts = [(H.NCX, H.NCX)] + ([(H.NXC, H.NXC), (H.NCX, H.NXC)] if K > 1 else [])
+        d0 = H.make_conv_desc(N, Cc, K, in_sp, f_sp, data_t=data_t, filter_t=filter_t, out_t=out_t, **kw)
+        data = synth.uniform_int(int(rng.integers(1 << 30)), d0.data_shape(), 0 if data_t == "u8" else -128, 255 if data_t == "u8" else 127, np.uint8 if data_t == "u8" else np.int8)
+        filt = synth.uniform_int(int(rng.integers(1 << 30)), d0.filter_shape(), -128 if filter_t == "i8" else 0, 127 if filter_t == "i8" else 255, np.int8 if filter_t == "i8" else np.uint8)
+        exp = O.quantized_convolution(d0, data, filt, scales[0], zps[0], scales[1], zps[1], scales[2], zps[2])
+        for dl, ol in layouts:
+            d = H.make_conv_desc(N, Cc, K, in_sp, f_sp, data_t=data_t, filter_t=filter_t, out_t=out_t, data_layout=dl, out_layout=ol, **kw)
+            x = cases.to_nxc(data) if dl == H.NXC else data
+            got = H.quantized_convolution(d, x, filt, scales[0], zps[0], scales[1], zps[1], scales[2], zps[2])
+            kernels.add(H.last_kernel())
+            got = cases.to_ncx(got) if ol == H.NXC else got
+            assert np.array_equal(got, exp), (block, case, dl, ol, H.last_kernel())
+    print("kernels:", sorted(kernels), flush=True)
+
+
+@pytest.mark.parametrize("block", range(3))
+def test_dot_random_shapes(gpu_lib, block):
+    """seeded sweep of QuantizedDot (INTERPRETER arithmetic, [K, N] weights, zero points) and
+    QuantizedDotBias (fused arithmetic, [N, K] weights, per-channel scales) against the oracle"""
+    rng = np.random.default_rng(9100 + block)
+    kernels = set()
+    for case in range(10):
+        M = int(rng.choice([1, 2, 7, 16, 31, 64, 65, 100, 128, 200, 257, 384]))
+        K = int(rng.choice([1, 5, 16, 48, 64, 100, 256, 512, 1024]))
+        N = int(rng.choice([1, 3, 16, 40, 64, 100, 128, 208, 512]))
+        say("random dot", block, case, M, K, N)
+        a_t = "u8"
+        b_t = str(rng.choice(["i8", "u8"]))
+        out_t = str(rng.choice(["i8", "i32"])) if b_t == "i8" else str(rng.choice(["u8", "i32"]))
+        d = H.make_dot_desc(M, K, N, a_t=a_t, b_t=b_t, out_t=out_t)
+        a = synth.uniform_int(int(rng.integers(1 << 30)), (M, K), 0, 255, np.uint8)
+        b = synth.uniform_int(int(rng.integers(1 << 30)), (K, N), -128 if b_t == "i8" else 0, 127 if b_t == "i8" else 255, np.int8 if b_t == "i8" else np.uint8)
+        zps = (int(rng.integers(0, 200)), int(rng.choice([0, 0, 5])) if b_t == "i8" else int(rng.choice([0, 120])), 0 if out_t == "i32" else int(rng.integers(0, 20)))
+        sc = (1.0, 1.0, 1.0) if out_t == "i32" else (0.01, 0.02, float(rng.choice([0.5, 4.0, 40.0])))
+        exp = O.quantized_dot(d, a, b, sc[0], zps[0], sc[1], zps[1], sc[2], zps[2])
+        got = H.quantized_dot(d, a, b, sc[0], zps[0], sc[1], zps[1], sc[2], zps[2])
+        kernels.add(H.last_kernel())
+        assert np.array_equal(got, exp), (block, case, "dot", H.last_kernel())
+        # the fused op on the same extents
+        fo = str(rng.choice(["i8", "u8", "f32"]))
+        relu = fo == "u8" or bool(rng.integers(0, 2))
+        db = H.make_dot_desc(M, K, N, a_t="u8", out_t=fo, b_layout=H.B_NK)
+        per_channel = bool(rng.integers(0, 2))
+        fd = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N if per_channel else 1)
+        w = synth.uniform_int(int(rng.integers(1 << 30)), (N, K), -127, 127, np.int8)
+        bias = synth.uniform_int(int(rng.integers(1 << 30)), (N,), -5000, 5000, np.int32)
+        scale = synth.uniform_f32(int(rng.integers(1 << 30)), (N if per_channel else 1,), 0.5, 1.5) * np.float32(1.0 / (40.0 * np.sqrt(K)))
+        exp = O.quantized_dot_bias(db, fd, a, w, bias, scale)
+        got = H.quantized_dot_bias(db, fd, a, w, bias, scale)
+        kernels.add(H.last_kernel())
+        if fo == "f32":
+            assert np.array_equal(got.view(np.uint32), exp.view(np.uint32)), (block, case, "dot bias f32", H.last_kernel())
+        else:
+            assert np.array_equal(got, exp), (block, case, "dot bias", fo, H.last_kernel())
+    print("kernels:", sorted(kernels), flush=True)

@@ -82,11 +82,118 @@ namespace hipq
         }
     }
 
+    // The same copy for data whose rows are whole aligned dwords: a lane takes four consecutive
+    // pixels of one row -- one dword from each channel plane of [N][C][H][W] data, the 4 C contiguous
+    // bytes of [N][H][W][C] data, instead of single bytes -- and writes their four staged pixels as
+    // one 16-byte piece; kQuadRows rows a lane, every load issued
+    // before the first store.  Quad j of a staged row covers input pixels 4j .. 4j + 3, that is
+    // staged pixels 4j + pad_w .. 4j + pad_w + 3; quads run from -ceil(pad_w / 4) so that the left
+    // padding is written too (pixels outside the staged row are dropped, outside the image filled).
+    constexpr int kQuadRows = 4;
+    struct __attribute__((packed, aligned(4))) Quad
+    {
+        uint32_t px[4];
+    };
+    template <int CC, bool NCX>
+    __global__ __launch_bounds__(256) void stage_rows_quads_kernel(const uint8_t* __restrict__ in, uint32_t* __restrict__ out, uint32_t rows, int32_t Hp, int32_t Wp, int32_t H, int32_t W,
+                                                                   int32_t pbh, int32_t pbw, int32_t first_quad, int32_t quads, const void* zp, int32_t zp_t)
+    {
+        const int32_t q = static_cast<int32_t>(blockIdx.y) * 64 + static_cast<int32_t>(threadIdx.x & 63);
+        if (q >= quads)
+            return;
+        const int32_t x = (q + first_quad) * 4; // first input pixel of the quad; W is a multiple of 4, so a quad is inside the row or outside
+        const bool x_in = x >= 0 && x < W;
+        const uint32_t fill = (static_cast<uint32_t>(load_zp(zp, zp_t)) & 0xffu) * 0x01010101u;
+        const int64_t X = static_cast<int64_t>(H) * W;
+        const uint32_t row0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * kQuadRows;
+        uint32_t word[kQuadRows][CC]; // NCX: the four pixels' bytes of channel c; NXC: bytes 4 c .. 4 c + 3 of the four pixels' run
+        bool live[kQuadRows];
+#pragma unroll
+        for (int i = 0; i < kQuadRows; ++i)
+        {
+            const uint32_t row = row0 + i; // image * Hp + yp
+#pragma unroll
+            for (int c = 0; c < CC; ++c)
+                word[i][c] = fill;
+            live[i] = false;
+            if (row >= rows || !x_in)
+                continue;
+            const uint32_t n = row / static_cast<uint32_t>(Hp);
+            const int32_t y = static_cast<int32_t>(row - n * static_cast<uint32_t>(Hp)) - pbh;
+            if (static_cast<uint32_t>(y) >= static_cast<uint32_t>(H))
+                continue;
+            live[i] = true;
+            const uint8_t* p = NCX ? in + static_cast<int64_t>(n) * CC * X + static_cast<int64_t>(y) * W + x : in + (static_cast<int64_t>(n) * X + static_cast<int64_t>(y) * W + x) * CC;
+#pragma unroll
+            for (int c = 0; c < CC; ++c)
+                word[i][c] = *reinterpret_cast<const uint32_t*>(p + (NCX ? c * X : static_cast<int64_t>(4 * c)));
+        }
+        const int32_t xp = x + pbw;
+#pragma unroll
+        for (int i = 0; i < kQuadRows; ++i)
+        {
+            const uint32_t row = row0 + i;
+            if (row >= rows)
+                continue;
+            Quad v;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+            {
+                v.px[t] = fill;
+                if (!live[i])
+                    continue;
+#pragma unroll
+                for (int c = 0; c < CC; ++c)
+                {
+                    const int k = t * CC + c; // byte of the run in [N][H][W][C] data
+                    const uint32_t b = NCX ? (word[i][c] >> (8 * t)) & 0xffu : (word[i][k >> 2] >> (8 * (k & 3))) & 0xffu;
+                    v.px[t] = (v.px[t] & ~(0xffu << (8 * c))) | (b << (8 * c));
+                }
+            }
+            uint32_t* o = out + static_cast<int64_t>(row) * Wp + xp;
+            if (xp >= 0 && xp + 3 < Wp)
+                *reinterpret_cast<Quad*>(o) = v;
+            else
+            {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    if (xp + t >= 0 && xp + t < Wp)
+                        o[t] = v.px[t];
+            }
+        }
+    }
+
     int launch_stage_rows(const ConvGeom& g, const RowPack& rp, const void* in, void* staged, const void* zp, int zp_t, hipStream_t s)
     {
         const int64_t rows = g.N * rp.Hp;
         if (rows == 0 || rp.Wp == 0)
             return HIPQ_OK;
+        if (g.in[2] % 4 == 0 && (reinterpret_cast<uintptr_t>(in) & 3) == 0 && rows < (1ll << 31) - 64 && getenv("HIPQ_NO_STAGE_QUADS") == nullptr)
+        {
+            const int64_t first_quad = -((g.pb[2] + 3) / 4);
+            const int64_t span = rp.Wp - g.pb[2];                                 // staged pixels from the image's first column on
+            const int64_t end_quad = span >= 0 ? (span + 3) / 4 : -((-span) / 4); // ceil(span / 4)
+            const int64_t quads = end_quad - first_quad;
+            if (quads >= 1 && (quads + 63) / 64 <= 65535 && fits_i32(g.pb[2] + 4 * end_quad))
+            {
+                const int rows_a_block = 4 * kQuadRows;
+                dim3 grid(static_cast<unsigned>((rows + rows_a_block - 1) / rows_a_block), static_cast<unsigned>((quads + 63) / 64));
+                const bool ncx = g.data_layout == HIPQ_LAYOUT_NCX;
+                auto go = [&](auto kernel) {
+                    kernel<<<grid, 256, 0, s>>>(static_cast<const uint8_t*>(in), static_cast<uint32_t*>(staged), static_cast<uint32_t>(rows), static_cast<int32_t>(rp.Hp), static_cast<int32_t>(rp.Wp),
+                                                static_cast<int32_t>(g.in[1]), static_cast<int32_t>(g.in[2]), static_cast<int32_t>(g.pb[1]), static_cast<int32_t>(g.pb[2]),
+                                                static_cast<int32_t>(first_quad), static_cast<int32_t>(quads), zp, zp_t);
+                };
+                switch (g.C)
+                {
+                case 1: ncx ? go(stage_rows_quads_kernel<1, true>) : go(stage_rows_quads_kernel<1, false>); break;
+                case 2: ncx ? go(stage_rows_quads_kernel<2, true>) : go(stage_rows_quads_kernel<2, false>); break;
+                case 3: ncx ? go(stage_rows_quads_kernel<3, true>) : go(stage_rows_quads_kernel<3, false>); break;
+                default: ncx ? go(stage_rows_quads_kernel<4, true>) : go(stage_rows_quads_kernel<4, false>); break;
+                }
+                return check_launch("stage_rows");
+            }
+        }
         HIPQ_REQUIRE(rows < (1ll << 31) && (rp.Wp + 255) / 256 <= 65535, "tensor too large for one launch");
         dim3 grid(static_cast<unsigned>((rows + kStageRows - 1) / kStageRows), static_cast<unsigned>((rp.Wp + 255) / 256));
         stage_rows_kernel<<<grid, 256, 0, s>>>(static_cast<const uint8_t*>(in), static_cast<uint32_t*>(staged), static_cast<uint32_t>(rows), static_cast<int32_t>(rp.Hp),

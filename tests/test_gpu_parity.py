@@ -639,28 +639,31 @@ def test_conv_split_reduction(gpu_lib, i):
     O.port().orc_set_threads(1)
 
 
+@pytest.mark.parametrize("image,pads", [((30, 26), ((3, 3), (3, 3))), ((30, 28), ((3, 3), (3, 3))), ((19, 32), ((2, 5), (4, 0)))], ids=["rows26", "rows28", "rows32_uneven_pads"])
 @pytest.mark.parametrize("K", [24, 32])
 @pytest.mark.parametrize("Cc", [1, 3, 4, 15])
-def test_conv_few_input_channels(gpu_lib, Cc, K):
+def test_conv_few_input_channels(gpu_lib, Cc, K, image, pads):
     """a network's first layer (3 input channels, 7x7 stride 2): the data is padded to 16 channels on
     the way into the MFMA kernel, or -- at most four channels, channels-last 8-bit output in whole
     16-byte pixels (K = 32 here) -- staged with its padding so that a filter row is one 32-byte run;
-    both policies, both layouts, zero points on every operand (a filter zero point takes the exact path)"""
-    say("first-layer conv", Cc, K)
+    both policies, both layouts, zero points on every operand (a filter zero point takes the exact path);
+    image rows of 28 and 32 bytes in NCHW take the staging kernel that moves whole dwords, rows of 26 the
+    one that moves bytes"""
+    say("first-layer conv", Cc, K, image, pads)
     O.port().orc_set_threads(8)
-    kw = dict(stride=(2, 2), pad_below=(3, 3), pad_above=(3, 3))
+    kw = dict(stride=(2, 2), pad_below=pads[0], pad_above=pads[1])
     for dl, ol in ((H.NCX, H.NCX), (H.NXC, H.NXC), (H.NCX, H.NXC)):
         for out_t, z in (("i8", (0, 0, 0)), ("u8", (119, 0, 3)), ("i8", (7, -5, 0))):
-            d = H.make_conv_desc(2, Cc, K, (30, 26), (7, 7), out_t=out_t, data_layout=dl, out_layout=ol, **kw)
-            dn = H.make_conv_desc(2, Cc, K, (30, 26), (7, 7), out_t=out_t, **kw)
+            d = H.make_conv_desc(2, Cc, K, image, (7, 7), out_t=out_t, data_layout=dl, out_layout=ol, **kw)
+            dn = H.make_conv_desc(2, Cc, K, image, (7, 7), out_t=out_t, **kw)
             data = synth.uniform_int(700 + Cc, dn.data_shape(), 0, 255, np.uint8)
             filt = synth.uniform_int(800 + Cc, dn.filter_shape(), -128, 127, np.int8)
             exp = O.quantized_convolution(dn, data, filt, 0.02, z[0], 0.01, z[1], 0.8, z[2])
             got = H.quantized_convolution(d, cases.to_nxc(data) if dl == H.NXC else data, filt, 0.02, z[0], 0.01, z[1], 0.8, z[2])
             assert H.last_kernel().startswith("conv_mfma"), H.last_kernel()
             assert np.array_equal(cases.to_ncx(got) if ol == H.NXC else got, exp), (dl, ol, out_t, z)
-        d = H.make_conv_desc(2, Cc, K, (30, 26), (7, 7), out_t="u8", data_layout=dl, out_layout=ol, **kw)
-        dn = H.make_conv_desc(2, Cc, K, (30, 26), (7, 7), out_t="u8", **kw)
+        d = H.make_conv_desc(2, Cc, K, image, (7, 7), out_t="u8", data_layout=dl, out_layout=ol, **kw)
+        dn = H.make_conv_desc(2, Cc, K, image, (7, 7), out_t="u8", **kw)
         data = synth.uniform_int(900 + Cc, dn.data_shape(), 0, 255, np.uint8)
         filt = synth.uniform_int(901 + Cc, dn.filter_shape(), -127, 127, np.int8)
         bias = synth.uniform_int(902, (K,), -5000, 5000, np.int32)

@@ -676,6 +676,26 @@ def test_conv_few_input_channels(gpu_lib, Cc, K, image, pads):
     O.port().orc_set_threads(1)
 
 
+def test_first_layer_staging_kernels_agree(gpu_lib, monkeypatch):
+    """the padded copy of a first layer written four pixels a lane (image rows of whole dwords) and
+    pixel by pixel: same convolution, both data layouts, at ResNet-50's stem geometry (batch 2)"""
+    say("first-layer staging, dwords vs bytes")
+    kw = dict(stride=(2, 2), pad_below=(3, 3), pad_above=(3, 3))
+    for dl in (H.NCX, H.NXC):
+        d = H.make_conv_desc(2, 3, 64, (224, 224), (7, 7), out_t="u8", data_layout=dl, out_layout=H.NXC, **kw)
+        dn = H.make_conv_desc(2, 3, 64, (224, 224), (7, 7), out_t="u8", **kw)
+        data = synth.uniform_int(910, dn.data_shape(), 0, 255, np.uint8)
+        filt = synth.uniform_int(911, dn.filter_shape(), -127, 127, np.int8)
+        x = cases.to_nxc(data) if dl == H.NXC else data
+        monkeypatch.delenv("HIPQ_NO_STAGE_QUADS", raising=False)
+        a = H.quantized_convolution(d, x, filt, 0.02, 5, 0.01, 0, 0.9, 128)
+        monkeypatch.setenv("HIPQ_NO_STAGE_QUADS", "1")
+        b = H.quantized_convolution(d, x, filt, 0.02, 5, 0.01, 0, 0.9, 128)
+        monkeypatch.delenv("HIPQ_NO_STAGE_QUADS")
+        assert np.array_equal(a, b), dl
+        assert len(np.unique(a)) > 50  # a real spread of outputs, not a saturated tensor
+
+
 def test_conv_band_matches_generic_kernel(gpu_lib, monkeypatch):
     """the band kernel and the generic implicit-GEMM kernel agree byte for byte at a size the oracle
     does not reach (BASELINE config 1 at batch 16, wrapping requantization included)"""

@@ -31,8 +31,8 @@ PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the headline kernel at batch 128: not measured by this run (counters need
 # a profiler run of their own) but quoted from the FETCH_SIZE / WRITE_SIZE runs summarised in the
 # file below (scaled by a 64 MiB copy in the same run); the JSON line names that file
-MEASURED_TRAFFIC_BYTES = {("conv_regw_i8_32x32x32", 128): 52.0e6, ("conv_band_i8_32x32x32", 128): 52.3e6}
-TRAFFIC_SOURCE = {"conv_regw_i8_32x32x32": "profiles/conv_regw_config1_batch128.md", "conv_band_i8_32x32x32": "profiles/conv_band_config1_hbm_traffic.md"}
+MEASURED_TRAFFIC_BYTES = {("conv_regw_i8_32x32x32", 128): 52.0e6}
+TRAFFIC_SOURCE = {"conv_regw_i8_32x32x32": "profiles/conv_regw_config1_batch128.md"}
 _DATA_CACHE = {}
 
 
@@ -70,7 +70,7 @@ def scalar(v, dt):
     return dev(np.asarray(v, dtype=dt))
 
 
-def bench_conv(lib, stream, timer, N, steps, warmup, layout, out_layout=None):
+def bench_conv(lib, stream, timer, N, steps, warmup, layout, out_layout=None, sustained=False):
     out_layout = layout if out_layout is None else out_layout
     d = H.make_conv_desc(N, 64, 64, (56, 56), (3, 3), pad_below=(1, 1), pad_above=(1, 1), data_layout=layout, out_layout=out_layout)
     # every image of the batch has bytes of its own (operand content moves this chip's clock: a
@@ -95,7 +95,14 @@ def bench_conv(lib, stream, timer, N, steps, warmup, layout, out_layout=None):
     kern = H.last_kernel()
     ops = d.ops()
     name = lambda l: "NCHW" if l == H.NCX else "NHWC"
-    return dict(N=N, layout=name(layout), out_layout=name(out_layout), ops=ops, ms_wall=wall, ms_event=ev, tops=ops / (wall * 1e-3) / 1e12, tops_event=ops / (ev * 1e-3) / 1e12, kernel=kern)
+    out_d = dict(N=N, layout=name(layout), out_layout=name(out_layout), ops=ops, ms_wall=wall, ms_event=ev, tops=ops / (wall * 1e-3) / 1e12, tops_event=ops / (ev * 1e-3) / 1e12, kernel=kern)
+    if sustained:
+        # the rate the device settles at once its clock has come down under the load: 2000 calls in a
+        # row, the last 1000 of them timed, in this same process
+        swall, sev = timer.run(step, 1000, 1000)
+        out_d["sustained"] = dict(steps=1000, warmup=1000, ms_wall=swall, ms_event=sev, tops=ops / (swall * 1e-3) / 1e12, tops_event=ops / (sev * 1e-3) / 1e12,
+                                  frac_of_peak=ops / (sev * 1e-3) / 1e12 / PEAK_I8_TOPS)
+    return out_d
 
 
 def bench_gemm(lib, stream, timer, M, steps, warmup):
@@ -327,6 +334,7 @@ def mfma_ceiling(lib, stream, timer, compute_units):
     no LDS, no other instructions).  The rate depends on the operand bytes -- the device lowers its
     clock under the switching activity of dense data -- so it is measured for all-zero operands and
     for the kind the convolution multiplies (random bytes)."""
+    probe = H.load_probe()
     iters, wgs = 400, int(compute_units)
     sink = H.DeviceBuffer(wgs * 256 * 4)
     out = {}
@@ -335,14 +343,96 @@ def mfma_ceiling(lib, stream, timer, compute_units):
         ops = dev(host)
 
         def step():
-            rc = lib.hipq_probe_mfma_i8(ops.ptr, sink.ptr, wgs, iters, stream)
-            if rc:
-                H.check(rc)
+            H.check_probe(probe.hipq_probe_mfma_i8(ops.ptr, sink.ptr, wgs, iters, stream))
 
         _, ev = timer.run(step, 5, 2)
         total = wgs * 4 * 64 * iters * 65536.0
         out[kind] = dict(ms_event=ev, tops=total / (ev * 1e-3) / 1e12, frac_of_published_peak=total / (ev * 1e-3) / 1e12 / PEAK_I8_TOPS)
     return out
+
+
+def bench_intake(lib, stream, timer, compute_units):
+    """What a compute unit takes in: 1 / 2 / 4 workgroups of four wavefronts a compute unit (by their LDS
+    allocation) each read 8 MiB in 16-byte pieces -- a wavefront instruction covering 1 KiB contiguous,
+    8 rows x 128 bytes or 16 rows x 64 bytes (rows 4096 bytes apart) -- into registers or straight into
+    LDS, out of a 2 MiB window (served by the L2s after the first pass) or out of 2 GiB with a region
+    per workgroup (served by HBM).  No division in the address stream; the launch is below 2 % of a sample."""
+    probe = H.load_probe()
+    cus = int(compute_units)
+    total = 2 << 30
+    buf = H.DeviceBuffer(total)
+    H.check(lib.hipq_fill_bytes(buf.ptr, 5, total, stream))
+    sink = H.DeviceBuffer(4 * cus * 256 * 4)
+    steps = 256  # x 32 KiB = 8 MiB a workgroup
+    out = []
+    shapes = {0: "1024 B contiguous", 1: "8 rows x 128 B", 2: "16 rows x 64 B"}
+    for source, window, spread in (("l2", 2 << 20, 0), ("hbm", total, 1)):
+        for to_lds in (0, 1):
+            for shape in (0, 1, 2):
+                for per_cu in (1, 2, 4):
+                    wgs = cus * per_cu
+                    lds_bytes = {1: 160 * 1024, 2: 80 * 1024, 4: 40 * 1024}[per_cu]
+
+                    def step():
+                        H.check_probe(probe.hipq_probe_intake(buf.ptr, total, window, spread, shape, to_lds, wgs, lds_bytes, steps, sink.ptr, stream))
+
+                    _, ev = timer.run(step, 3, 1)
+                    per_cu_gbs = per_cu * steps * 32768 / (ev * 1e-3) / 1e9
+                    out.append(dict(source=source, dest="lds" if to_lds else "registers", shape=shapes[shape], workgroups_per_cu=per_cu, ms_event=ev,
+                                    gbs_per_cu=per_cu_gbs, tbs_chip=per_cu_gbs * cus / 1e3))
+    return out
+
+
+def bench_atomic_tiles(lib, stream, timer, compute_units):
+    """int32 atomic adds of whole 128 x 128 accumulator tiles into L2 (no return value): 256 workgroups,
+    8 rounds each, 1 / 4 / 8 workgroups adding to the same tile, on one compute die or across the eight"""
+    probe = H.load_probe()
+    wgs, rounds = 256, 8
+    dst = H.DeviceBuffer(wgs * rounds * 65536)
+    H.check(lib.hipq_fill_bytes(dst.ptr, 0, wgs * rounds * 65536, stream))
+    out = []
+    for share in (1, 4, 8):
+        for same_die in (1, 0):
+            def step():
+                H.check_probe(probe.hipq_probe_atomic_tiles(dst.ptr, wgs * rounds * 65536, wgs, share, same_die, rounds, stream))
+
+            _, ev = timer.run(step, 5, 2)
+            n = wgs * rounds * 16384
+            out.append(dict(share=share, same_die=bool(same_die), ms_event=ev, giga_atomics_per_s=n / (ev * 1e-3) / 1e9, us_per_tile_per_workgroup=ev * 1e3 / rounds))
+    return out
+
+
+def bench_backend(calls=100, warmup=10):
+    """The same workloads through the product boundary: ngraph_amd/host/hip_backend_tests --bench builds the
+    graphs with the nGraph API and times Backend::create("HIP") -> compile -> Executable::call with nbench's
+    protocol (inputs written once, `warmup` calls, `calls` timed calls, outputs not copied back).  Runs as a
+    child process of its own, before this process touches the GPU."""
+    import subprocess
+
+    exe = os.path.join(ROOT, "ngraph_amd", "host", "hip_backend_tests")
+    if not os.path.exists(exe):
+        return dict(status="unavailable", reason="%s is not built" % exe)
+    try:
+        p = subprocess.run([exe, "--bench", "--calls", str(calls), "--warmup", str(warmup)], capture_output=True, text=True, timeout=600)
+    except subprocess.TimeoutExpired:
+        return dict(status="unavailable", reason="backend benchmark timed out")
+    rows = []
+    for line in p.stdout.splitlines():
+        if line.startswith("{"):
+            try:
+                rows.append(json.loads(line))
+            except ValueError:
+                pass
+    if p.returncode != 0 or not rows:
+        return dict(status="failed", returncode=p.returncode, stderr=p.stderr[-400:])
+    return dict(protocol="Backend::create(\"HIP\") -> compile -> Executable::call; nbench --no_copy_data protocol (src/tools/nbench/benchmark.cpp:141-176): %d warm-up, %d timed calls, "
+                         "host stopwatch around the calls; a call returns when its results are in the output tensors" % (warmup, calls), rows=rows)
+
+
+def under_profiler():
+    """rocprofv3 (and its predecessors) announce themselves in the environment of the program they run"""
+    pre = os.environ.get("LD_PRELOAD", "")
+    return "rocprof" in pre or any(k.startswith(("ROCPROF", "ROCP_", "ROCPROFILER_")) for k in os.environ)
 
 
 def copy_calibration(lib, stream, timer):
@@ -461,6 +551,8 @@ def cpu_baseline(batch, seconds=8.0):
         from ngraph_amd import resnet50 as R
 
         class Port:
+            quantize = staticmethod(lambda x, s, z, t: O.quantize(x, s, z, t))
+            dequantize = staticmethod(lambda q, s, z: O.dequantize(q, s, z, "f32"))
             conv = staticmethod(lambda d, f, x, filt, bias, s, sc, ss: O.quantized_convolution_fused(d, f, x, filt, bias, s, sc, ss))
             pool = staticmethod(lambda d, x: O.pool(d, x))
             dot_bias = staticmethod(lambda d, f, a, w, bias, sc: O.quantized_dot_bias(d, f, a, w, bias, sc))
@@ -486,13 +578,22 @@ def main():
     ap.add_argument("--resnet-only", action="store_true", help="only the synthetic int8 ResNet-50 (for profiling); prints its results")
     ap.add_argument("--bert-only", action="store_true", help="only the synthetic int8 BERT-base encoder (for profiling); prints its results")
     ap.add_argument("--skip-models", action="store_true", help="leave out the BERT and ResNet-50 sections (kernel traces of the single operators; the models have runs of their own)")
-    ap.add_argument("--only", choices=["gemm", "qdq", "glue"],
+    ap.add_argument("--only", choices=["gemm", "qdq", "glue", "intake"],
                     help="only config 2's GEMMs, config 3's Quantize / Dequantize, or the encoder's fp32 glue and attention (for counter runs under a profiler); prints their results")
     ap.add_argument("--no-graph", action="store_true", help="time the models' eager launch sequences only, no HIP-graph capture or replay (for runs under a profiler)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
+    if under_profiler() and not args.no_graph:
+        # graph replays of the models under a profiler's interception of graph launches once ended in a
+        # crash whose cause was never established: profiled runs launch eagerly
+        print("bench.py: running under a profiler -- models are launched eagerly (--no-graph)", file=sys.stderr)
+        args.no_graph = True
+
+    backend = None
+    if not (args.quick or args.only or args.resnet_only or args.bert_only or args.skip_models or under_profiler()):
+        backend = bench_backend()  # a child process with the GPU to itself: before this process opens the device
 
     lib = H.load()
     H.check(lib.hipq_set_device(0))
@@ -509,6 +610,9 @@ def main():
     if args.only == "qdq":
         print(json.dumps({"quantize_dequantize_config3": bench_qdq(lib, stream, timer, args.steps, args.warmup), "copy_calibration": copy_calibration(lib, stream, timer)}))
         return
+    if args.only == "intake":
+        print(json.dumps({"l2_intake_per_cu": bench_intake(lib, stream, timer, info.compute_units), "atomic_tiles": bench_atomic_tiles(lib, stream, timer, info.compute_units)}))
+        return
     if args.only == "glue":
         print(json.dumps({"fp32_glue": bench_fp32_glue(lib, stream, timer, args.steps, args.warmup), "copy_calibration": copy_calibration(lib, stream, timer)}))
         return
@@ -520,7 +624,7 @@ def main():
         return
 
     # headline: the reference's NCHW tensors in, NCHW out
-    head = bench_conv(lib, stream, timer, args.batch, args.steps, args.warmup, H.NCX)
+    head = bench_conv(lib, stream, timer, args.batch, args.steps, args.warmup, H.NCX, sustained=True)
     # the dominant kernel of that call alone: channels-last data in (what the call's transpose
     # hands it), NCHW out -- such a call launches only the MFMA kernel
     kern = bench_conv(lib, stream, timer, args.batch, args.steps, args.warmup, H.NXC, H.NCX)
@@ -549,6 +653,22 @@ def main():
             results["bert_base_int8"] = bench_bert(lib, stream, timer, use_graph=not args.no_graph)
             results["resnet50_int8"] = bench_resnet50(lib, stream, timer, use_graph=not args.no_graph)
         cpu = cpu_baseline(args.batch)
+    if backend is not None:
+        # next to each boundary figure, the same workload as this process timed it over the C ABI
+        if "rows" in backend:
+            for row in backend["rows"]:
+                if row["workload"].startswith("QuantizedConvolution"):
+                    row["c_abi_ms"] = head["ms_wall"]
+                elif "resnet50_int8" in results:
+                    match = [r for r in results["resnet50_int8"] if r["batch"] == row["batch"]]
+                    if match:
+                        row["c_abi_ms"] = min(v for v in (match[0]["ms_eager"], match[0]["ms_graph"]) if v is not None)
+                if "c_abi_ms" in row:
+                    row["boundary_over_c_abi"] = row["ms_per_call"] / row["c_abi_ms"]
+            backend["gap"] = ("Executable::call replays one captured HIP graph and then waits for the stream (hipStreamSynchronize) before it returns, once per call; the C-ABI loop "
+                              "of this process enqueues all its steps and waits once at the end.  The per-call wait and graph launch cost about the same few tens of microseconds at "
+                              "every size: a large part of a 20 us convolution, a few per cent of a ResNet-50 pass.")
+        results["backend"] = backend
 
     derived_peak = info.compute_units * info.clock_mhz * 1e6 * 8192 / 1e12
     line = {

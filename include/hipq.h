@@ -97,16 +97,14 @@ HIPQ_API int hipq_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes, 
 HIPQ_API int hipq_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
 /* byte fill done by a kernel (not a memset node), safe to record into a HIP graph */
 HIPQ_API int hipq_fill_bytes(void* dst_dev, int value, size_t bytes, void* stream);
-/*
- * Measurement aid with no counterpart in the reference: a full-chip launch of dependent
- * v_mfma_i32_32x32x32_i8 chains on register-resident operands (`operands_8k`: 8 sets of 64 lanes x
- * 16 bytes on the device; `sink`: workgroups x 256 ints).  Each of the workgroups' 4 wavefronts
- * issues 64 x iters MFMAs of 65536 operations.  bench.py times it to report the matrix-core rate
- * this device sustains for a given kind of operand bytes.
- */
-HIPQ_API int hipq_probe_mfma_i8(const void* operands_8k, void* sink, int32_t workgroups, int32_t iters, void* stream);
 HIPQ_API int hipq_stream_create(void** stream);
 HIPQ_API int hipq_stream_destroy(void* stream);
+/* The library keeps grow-only scratch blocks per (device, stream) for every stream it has seen in a
+ * call, its own or the caller's.  hipq_stream_destroy releases the blocks of a stream the library
+ * created; a caller that passes streams of its own calls hipq_stream_release_scratch(stream) before
+ * hipStreamDestroy (waits for the stream, frees its blocks, moves hipq_workspace_epoch): otherwise
+ * the blocks stay until the process ends and a later stream with the same handle inherits them. */
+HIPQ_API int hipq_stream_release_scratch(void* stream);
 HIPQ_API int hipq_stream_sync(void* stream);
 /* Stream capture into a HIP graph, for callers that replay one fixed launch sequence (what
  * runtime::Executable::call does, src/ngraph/runtime/executable.hpp:44-52): begin, issue the launches
@@ -253,6 +251,9 @@ HIPQ_API int hipq_quantized_convolution(const hipq_conv_desc_t* desc,
  * shares that GPU's array: calls of this entry point that overlap on one GPU (two streams, two
  * threads) race; calls on one stream are ordered by the stream.  The tile counters are cleared by
  * a kernel on `stream` ahead of every launch that uses them.
+ * Set-up: hipq_set_device resolves the array's address on that device.  A caller that selects its
+ * device some other way makes one call of this entry point outside any graph capture first (the
+ * first call on a device resolves the address itself, which is not a step to record into a graph).
  */
 #define HIPQ_NOALLOC_LAYOUT_BYTES (32u << 20)
 #define HIPQ_NOALLOC_SPLIT_BYTES (16u << 20)

@@ -12,38 +12,11 @@
 //   *_generic every other case (f64, i32, ragged inner extent, scattered axes): one element per
 //             lane, coordinates recovered with 64-bit div/mod.
 #include "hipq_common.h"
+#include "hipq_index_div.h"
 #include "hipq_quant_math.h"
 
 namespace hipq
 {
-    // ---- division of a 31-bit index by a run-time constant -----------------------------------
-    // q = (n * magic) >> (31 + shift) with shift = ceil(log2 d), magic = ceil(2^(31+shift) / d)
-    // is exact for every 0 <= n < 2^31 (Granlund & Montgomery, N = 31).
-    struct FastDiv
-    {
-        uint32_t magic;
-        uint32_t shift;
-        uint32_t d;
-    };
-
-    FastDiv make_fastdiv(uint32_t d)
-    {
-        FastDiv f;
-        f.d = d;
-        uint32_t s = 0;
-        while ((1ull << s) < d)
-            ++s;
-        f.shift = s;
-        unsigned __int128 num = static_cast<unsigned __int128>(1) << (31 + s);
-        f.magic = static_cast<uint32_t>((num + d - 1) / d);
-        return f;
-    }
-
-    __host__ __device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDiv& f)
-    {
-        return static_cast<uint32_t>((static_cast<uint64_t>(n) * f.magic) >> (31 + f.shift));
-    }
-
     struct DimInfo
     {
         int32_t rank;
@@ -109,8 +82,8 @@ namespace hipq
     // (A == 1: scalar scale).  groups = count / 4; group g covers elements 4g .. 4g+3.
     struct RunView
     {
-        FastDiv div_inner4; // divides a group index by inner/4
-        FastDiv div_a;
+        IndexDiv div_inner4; // divides a group index by inner/4
+        IndexDiv div_a;
         uint32_t a;         // extent of the scale table
     };
 
@@ -314,12 +287,6 @@ namespace hipq
 using namespace hipq;
 
 extern "C" {
-
-// host-only helper used by the CPU tests of the index arithmetic
-HIPQ_API uint32_t hipq_debug_fastdiv(uint32_t n, uint32_t d)
-{
-    return fastdiv(n, make_fastdiv(d));
-}
 
 int hipq_quantize(const hipq_quant_desc_t* d, const void* in, const void* scale, const void* zp, void* out, void* stream)
 {

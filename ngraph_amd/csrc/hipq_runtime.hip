@@ -77,23 +77,32 @@ namespace hipq
         return HIPQ_OK;
     }
 
+    // resolves the scratch array's address on the current device (once per device)
+    static int resolve_scratch(int dev)
+    {
+        std::lock_guard<std::mutex> lock(g_ws_mutex);
+        if (!g_scratch_ptr[dev])
+        {
+            void* p = nullptr;
+            HIPQ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+            if (!p)
+                return fail(HIPQ_ERR_HIP, "the scratch array has no address on device %d", dev);
+            g_scratch_ptr[dev] = static_cast<unsigned char*>(p);
+        }
+        return HIPQ_OK;
+    }
+
+    // hipq_set_device resolves the address, so a caller that selected its device through the library
+    // never meets this step inside a graph capture; the check here serves callers that did not.
     int noalloc_begin()
     {
         int dev = 0;
         int rc = current_device(&dev);
         if (rc)
             return rc;
-        {
-            std::lock_guard<std::mutex> lock(g_ws_mutex);
-            if (!g_scratch_ptr[dev])
-            {
-                void* p = nullptr;
-                HIPQ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
-                if (!p)
-                    return fail(HIPQ_ERR_HIP, "the scratch array has no address on device %d", dev);
-                g_scratch_ptr[dev] = static_cast<unsigned char*>(p);
-            }
-        }
+        rc = resolve_scratch(dev);
+        if (rc)
+            return rc;
         ++t_noalloc;
         return HIPQ_OK;
     }
@@ -263,7 +272,8 @@ int hipq_set_device(int ordinal)
     if (ordinal < 0 || ordinal >= n)
         return fail(HIPQ_ERR_INVALID, "device ordinal %d out of range (%d devices)", ordinal, n);
     HIPQ_HIP(hipSetDevice(ordinal));
-    return HIPQ_OK;
+    // set-up of the entry point that allocates nothing: the scratch array's address on this device
+    return ordinal < kMaxDevices ? resolve_scratch(ordinal) : HIPQ_OK;
 }
 
 int hipq_get_device_info(hipq_device_info_t* info)
@@ -362,6 +372,12 @@ int hipq_stream_destroy(void* stream)
         HIPQ_HIP(hipStreamDestroy(as_stream(stream)));
     }
     return HIPQ_OK;
+}
+
+int hipq_stream_release_scratch(void* stream)
+{
+    HIPQ_HIP(hipStreamSynchronize(as_stream(stream)));
+    return release_stream_workspace(as_stream(stream));
 }
 
 int hipq_stream_sync(void* stream)

@@ -1,0 +1,253 @@
+// Measurement aids (libhipq_probe.so): device ceilings that the kernels of libhipq.so are judged
+// against.  Nothing here is on the product path; see hipq_probe.h.
+//   * probe_mfma_i8_kernel: how fast the matrix cores run when nothing else limits them.  Every
+//     wavefront of a full-chip launch issues one dependent chain of v_mfma_i32_32x32x32_i8 on
+//     operands it holds in registers -- no memory traffic, no LDS, no other instructions.  The rate
+//     depends on the operand bytes (the chip lowers its clock under the switching activity of
+//     dense data).
+//   * probe_intake_kernel: bytes a second a compute unit takes in from L2 / HBM, by load shape
+//     and destination (registers or LDS).
+//   * probe_atomic_tiles_kernel: integer atomic adds of whole accumulator tiles into L2.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "../hipq_index_div.h"
+#include "hipq_probe.h"
+
+namespace
+{
+    thread_local char t_error[256] = "";
+
+    int fail(const char* fmt, ...)
+    {
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(t_error, sizeof(t_error), fmt, ap);
+        va_end(ap);
+        return 1;
+    }
+
+    int check_launch(const char* what)
+    {
+        hipError_t e = hipGetLastError();
+        return e == hipSuccess ? 0 : fail("launch of %s failed: %s", what, hipGetErrorString(e));
+    }
+
+    typedef int pv4i __attribute__((ext_vector_type(4)));
+    typedef int pv16i __attribute__((ext_vector_type(16)));
+
+    // ops: 8 operand sets of 64 lanes x 16 bytes (4 for the A side, 4 for the B side)
+    __global__ __launch_bounds__(256) void probe_mfma_i8_kernel(const pv4i* __restrict__ ops, int* __restrict__ sink, int iters)
+    {
+        pv16i acc[2];
+        for (int i = 0; i < 2; ++i)
+            for (int r = 0; r < 16; ++r)
+                acc[i][r] = i;
+        pv4i a[4], b[4];
+        for (int i = 0; i < 4; ++i)
+        {
+            a[i] = ops[(i * 2) * 64 + (threadIdx.x & 63)];
+            b[i] = ops[(i * 2 + 1) * 64 + (threadIdx.x & 63)];
+        }
+        for (int it = 0; it < iters; ++it)
+        {
+#pragma unroll
+            for (int i = 0; i < 64; ++i)
+                acc[i & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i & 3], b[(i >> 2) & 3], acc[i & 1], 0, 0, 0);
+        }
+        int s = 0;
+        for (int i = 0; i < 2; ++i)
+            for (int r = 0; r < 16; ++r)
+                s += acc[i][r];
+        sink[blockIdx.x * 256 + threadIdx.x] = s;
+    }
+
+    constexpr int kIntakeLoads = 8;       // 16-byte loads a lane and step
+    constexpr int kIntakeStepBytes = 32768; // 4 wavefronts x 8 instructions x 1 KiB
+
+    // byte offset (before wrapping) of load u of step `step` for this lane
+    template <int SHAPE>
+    __device__ __forceinline__ uint32_t intake_offset(uint32_t base, uint32_t step, int wave, int lane, int u)
+    {
+        if (SHAPE == 0) // 1 KiB contiguous an instruction, a step is 32 KiB contiguous
+            return base + step * kIntakeStepBytes + static_cast<uint32_t>((wave * kIntakeLoads + u) * 1024 + lane * 16);
+        // row pieces out of rows 4096 bytes apart: a workgroup's step is a block of 256 (128-byte
+        // pieces) or 512 (64-byte pieces) rows at one column; 32 (64) steps sweep the 4096 columns,
+        // then the block moves on by its rows
+        constexpr int PIECE = SHAPE == 1 ? 128 : 64;
+        constexpr int LANES = PIECE / 16;      // lanes a row piece
+        constexpr int ROWS = 64 / LANES;       // rows an instruction
+        constexpr int BLOCK_ROWS = 4 * kIntakeLoads * ROWS;
+        constexpr int SWEEP = 4096 / PIECE;    // steps until the columns wrap (a power of two)
+        const uint32_t row = static_cast<uint32_t>((wave * kIntakeLoads + u) * ROWS + lane / LANES);
+        const uint32_t col = (step & (SWEEP - 1)) * PIECE + static_cast<uint32_t>(lane % LANES) * 16;
+        return base + (step / SWEEP) * (BLOCK_ROWS * 4096u) + row * 4096u + col;
+    }
+
+    template <int SHAPE, bool TO_LDS>
+    __global__ __launch_bounds__(256) void probe_intake_kernel(const uint8_t* __restrict__ buf, uint32_t buf_bytes, uint32_t window_mask, uint32_t spread_bytes, int steps, int* __restrict__ sink)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+        const int lane = threadIdx.x & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(buf), 0, static_cast<int>(buf_bytes), 0x00020000);
+        // spread: every workgroup has a region of its own; else a start of its own inside the shared
+        // window (4 KiB-aligned, scattered), so that the compute units do not walk the same L2
+        // channel in step
+        const uint32_t base = spread_bytes ? static_cast<uint32_t>(blockIdx.x) * spread_bytes : (static_cast<uint32_t>(blockIdx.x) * 0x9E3779B1u) & ~0xFFFu;
+        pv4i acc = {0, 0, 0, 0};
+        if (TO_LDS)
+        {
+            // wavefront w lands its 8 KiB of a step at lds + w * 8 KiB (the same place every step: nothing reads it)
+            const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + static_cast<uint32_t>(wave) * 8192u;
+            for (int s = 0; s < steps; ++s)
+            {
+#pragma unroll
+                for (int u = 0; u < kIntakeLoads; ++u)
+                {
+                    const uint32_t off = intake_offset<SHAPE>(base, static_cast<uint32_t>(s), wave, lane, u) & window_mask;
+                    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base + static_cast<uint32_t>(u) * 1024u), "v"(off), "s"(rs) : "memory");
+                }
+                // the step before this one has landed; this one stays in flight
+                asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            acc[0] = *reinterpret_cast<const int*>(lds + threadIdx.x * 4);
+        }
+        else
+        {
+            pv4i cur[kIntakeLoads], nxt[kIntakeLoads];
+#pragma unroll
+            for (int u = 0; u < kIntakeLoads; ++u)
+                cur[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, intake_offset<SHAPE>(base, 0u, wave, lane, u) & window_mask, 0, 0);
+            for (int s = 1; s <= steps; ++s)
+            {
+                // (one step past the end: a harmless re-read inside the window)
+#pragma unroll
+                for (int u = 0; u < kIntakeLoads; ++u)
+                    nxt[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, intake_offset<SHAPE>(base, static_cast<uint32_t>(s), wave, lane, u) & window_mask, 0, 0);
+#pragma unroll
+                for (int u = 0; u < kIntakeLoads; ++u)
+                    acc ^= cur[u];
+#pragma unroll
+                for (int u = 0; u < kIntakeLoads; ++u)
+                    cur[u] = nxt[u];
+            }
+        }
+        sink[blockIdx.x * 256 + threadIdx.x] = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+    }
+
+    // a workgroup of 256 lanes holds a 128 x 128 int32 tile as 64 values a lane; value j of lane t is
+    // element j * 256 + t of the tile (a wavefront instruction covers 256 contiguous bytes)
+    __global__ __launch_bounds__(256) void probe_atomic_tiles_kernel(int* __restrict__ dst, int share, int same_die, int rounds, int groups)
+    {
+        const int wg = static_cast<int>(blockIdx.x);
+        // same die: workgroups g, g + 8, ... (ids congruent modulo 8) share; else consecutive ids share
+        int group;
+        if (same_die)
+        {
+            const int die = wg & 7, k = wg >> 3; // k-th workgroup of its die
+            group = (k / share) * 8 + die;
+        }
+        else
+            group = wg / share;
+        if (group >= groups)
+            return;
+        for (int r = 0; r < rounds; ++r)
+        {
+            int* tile = dst + (static_cast<size_t>(group) * rounds + r) * 16384;
+#pragma unroll 16
+            for (int j = 0; j < 64; ++j)
+                __hip_atomic_fetch_add(tile + j * 256 + threadIdx.x, wg + j + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+extern "C" {
+
+const char* hipq_probe_last_error(void)
+{
+    return t_error;
+}
+
+int hipq_probe_mfma_i8(const void* operands_8k, void* sink, int32_t workgroups, int32_t iters, void* stream)
+{
+    if (!operands_8k || !sink)
+        return fail("null pointer");
+    if (workgroups <= 0 || workgroups > 65535 || iters <= 0 || iters > 100000)
+        return fail("workgroups / iterations out of range");
+    if (reinterpret_cast<uintptr_t>(operands_8k) & 15)
+        return fail("operands must be 16-byte aligned");
+    probe_mfma_i8_kernel<<<static_cast<unsigned>(workgroups), 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const pv4i*>(operands_8k), static_cast<int*>(sink), iters);
+    return check_launch("probe_mfma_i8");
+}
+
+int hipq_probe_intake(const void* buf, size_t buf_bytes, size_t window_bytes, int32_t spread, int32_t shape, int32_t to_lds, int32_t workgroups, int32_t lds_bytes, int32_t steps,
+                      void* sink, void* stream)
+{
+    if (!buf || !sink)
+        return fail("null pointer");
+    if (reinterpret_cast<uintptr_t>(buf) & 15)
+        return fail("buffer must be 16-byte aligned");
+    if (window_bytes < (1u << 20) || (window_bytes & (window_bytes - 1)) != 0 || window_bytes > buf_bytes || buf_bytes > 0xFFFFFFFFull)
+        return fail("window must be a power of two of at least 1 MiB inside a buffer below 4 GiB");
+    if (shape < 0 || shape > 2 || workgroups <= 0 || workgroups > 65535 || steps <= 0 || steps > (1 << 20))
+        return fail("shape / workgroups / steps out of range");
+    if (lds_bytes < (to_lds ? 32768 : 0) || lds_bytes > 160 * 1024)
+        return fail("lds_bytes out of range (loads into LDS need 32 KiB)");
+    const uint32_t mask = static_cast<uint32_t>(window_bytes - 1) & ~15u;
+    const uint32_t spread_bytes = spread ? static_cast<uint32_t>(steps) * kIntakeStepBytes : 0u;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define HIPQ_INTAKE(SHAPE, LDS)                                                                                                                              \
+    do                                                                                                                                                       \
+    {                                                                                                                                                        \
+        auto k = probe_intake_kernel<SHAPE, LDS>;                                                                                                            \
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)                    \
+            return fail("cannot raise the LDS limit");                                                                                                       \
+        k<<<static_cast<unsigned>(workgroups), 256, static_cast<size_t>(lds_bytes), s>>>(static_cast<const uint8_t*>(buf), static_cast<uint32_t>(buf_bytes), mask, spread_bytes, steps, \
+                                                                                          static_cast<int*>(sink));                                          \
+    } while (0)
+    if (to_lds)
+    {
+        if (shape == 0)
+            HIPQ_INTAKE(0, true);
+        else if (shape == 1)
+            HIPQ_INTAKE(1, true);
+        else
+            HIPQ_INTAKE(2, true);
+    }
+    else
+    {
+        if (shape == 0)
+            HIPQ_INTAKE(0, false);
+        else if (shape == 1)
+            HIPQ_INTAKE(1, false);
+        else
+            HIPQ_INTAKE(2, false);
+    }
+#undef HIPQ_INTAKE
+    return check_launch("probe_intake");
+}
+
+int hipq_probe_atomic_tiles(void* dst, size_t dst_bytes, int32_t workgroups, int32_t share, int32_t same_die, int32_t rounds, void* stream)
+{
+    if (!dst)
+        return fail("null pointer");
+    if (workgroups <= 0 || workgroups > 65535 || share <= 0 || rounds <= 0 || rounds > 4096)
+        return fail("workgroups / share / rounds out of range");
+    if (workgroups % (same_die ? 8 * share : share) != 0)
+        return fail("workgroups must be a multiple of %d", same_die ? 8 * share : share);
+    const int groups = workgroups / share;
+    if (static_cast<size_t>(groups) * static_cast<size_t>(rounds) * 65536 > dst_bytes)
+        return fail("destination holds fewer than %d x %d tiles of 64 KiB", groups, rounds);
+    probe_atomic_tiles_kernel<<<static_cast<unsigned>(workgroups), 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<int*>(dst), share, same_die, rounds, groups);
+    return check_launch("probe_atomic_tiles");
+}
+
+uint32_t hipq_debug_fastdiv(uint32_t n, uint32_t d)
+{
+    return hipq::fastdiv(n, hipq::make_fastdiv(d));
+}
+}

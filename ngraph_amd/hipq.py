@@ -278,9 +278,9 @@ EXPORTS = [
     "hipq_memcpy_d2h",
     "hipq_memcpy_d2d",
     "hipq_fill_bytes",
-    "hipq_probe_mfma_i8",
     "hipq_stream_create",
     "hipq_stream_destroy",
+    "hipq_stream_release_scratch",
     "hipq_stream_sync",
     "hipq_capture_begin",
     "hipq_capture_end",
@@ -338,6 +338,35 @@ class HipqError(RuntimeError):
         self.code = code
 
 
+PROBE_LIB_PATH = os.path.join(os.path.dirname(LIB_PATH), "libhipq_probe.so")
+_probe = None
+
+
+def load_probe():
+    """dlopen libhipq_probe.so, the measurement aids (ngraph_amd/csrc/probe/hipq_probe.h): bench.py's
+    device ceilings and the host-side index-division check.  Not part of the product library."""
+    global _probe
+    if _probe is not None:
+        return _probe
+    if not os.path.exists(PROBE_LIB_PATH):
+        raise RuntimeError(f"{PROBE_LIB_PATH} is missing: build it first (python -c 'import __graft_entry__ as g; g.build()')")
+    lib = C.CDLL(PROBE_LIB_PATH)
+    vp, i32, sz = C.c_void_p, C.c_int32, C.c_size_t
+    lib.hipq_probe_last_error.restype = C.c_char_p
+    lib.hipq_probe_mfma_i8.argtypes = [vp, vp, i32, i32, vp]
+    lib.hipq_probe_intake.argtypes = [vp, sz, sz, i32, i32, i32, i32, i32, i32, vp, vp]
+    lib.hipq_probe_atomic_tiles.argtypes = [vp, sz, i32, i32, i32, i32, vp]
+    lib.hipq_debug_fastdiv.restype = C.c_uint32
+    lib.hipq_debug_fastdiv.argtypes = [C.c_uint32] * 2
+    _probe = lib
+    return lib
+
+
+def check_probe(rc):
+    if rc:
+        raise RuntimeError("libhipq_probe: " + load_probe().hipq_probe_last_error().decode())
+
+
 def load():
     """dlopen libhipq.so (built by __graft_entry__.build()); raises if it is not there."""
     global _lib
@@ -361,9 +390,9 @@ def load():
     for n in ("hipq_memcpy_h2d", "hipq_memcpy_d2h", "hipq_memcpy_d2d"):
         getattr(lib, n).argtypes = [vp, vp, C.c_size_t, vp]
     lib.hipq_fill_bytes.argtypes = [vp, C.c_int, C.c_size_t, vp]
-    lib.hipq_probe_mfma_i8.argtypes = [vp, vp, C.c_int32, C.c_int32, vp]
     lib.hipq_stream_create.argtypes = [C.POINTER(vp)]
     lib.hipq_stream_destroy.argtypes = [vp]
+    lib.hipq_stream_release_scratch.argtypes = [vp]
     lib.hipq_stream_sync.argtypes = [vp]
     lib.hipq_event_create.argtypes = [C.POINTER(vp)]
     lib.hipq_event_destroy.argtypes = [vp]

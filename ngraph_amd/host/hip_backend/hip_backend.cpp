@@ -205,6 +205,7 @@ namespace
         vector<void*> m_value_ptr;                  // persistent device pointer, or null when bound per call
         vector<size_t> m_value_bytes;
         vector<int> m_value_uses;
+        vector<bool> m_value_external; // a Parameter's or Constant's memory: never redirected into a caller's output tensor
         vector<int> m_param_value, m_result_value;
         vector<Step> m_steps;
         vector<shared_ptr<DeviceBlock>> m_blocks;
@@ -314,12 +315,25 @@ namespace
     {
         return (is_type<op::v0::QuantizedConvolutionBiasAdd>(n) || is_type<op::v0::QuantizedConvolutionBiasSignedAdd>(n)) ? 3 : -1;
     }
+    // A pool that leaves no spatial extent (a global average): its output has the same bytes in
+    // either layout, so it reads whatever layout its input has and ties nothing -- a Reshape or a
+    // GEMM behind it must not pull the network in front of it back into nGraph's layout.
+    static bool pool_to_points(const Node* n)
+    {
+        if (!(is_type<op::v0::MaxPool>(n) || is_type<op::v0::AvgPool>(n)) || n->get_output_size() != 1)
+            return false;
+        const Shape& s = n->get_output_shape(0);
+        size_t spatial = 1;
+        for (size_t i = 2; i < s.size(); ++i)
+            spatial *= s[i];
+        return s.size() >= 3 && spatial == 1;
+    }
     // inputs of a layout-agnostic op that must share its output's layout (empty: not such an op)
     static vector<size_t> tied_inputs(const Node* n)
     {
         vector<size_t> r;
         const size_t rank = n->get_output_size() == 1 ? n->get_output_shape(0).size() : 0;
-        if (rank < 3)
+        if (rank < 3 || pool_to_points(n))
             return r;
         if (is_type<op::v0::Relu>(n) || is_type<op::v0::Abs>(n) || is_type<op::v0::Convert>(n) || is_type<op::v0::MaxPool>(n) || is_type<op::v0::AvgPool>(n))
             r.push_back(0);
@@ -468,6 +482,21 @@ namespace
             const Node* dot = n->input_value(0).get_node();
             if (!is_type<op::v0::QuantizedDotBias>(dot) || !single_user(dot) || dot->get_output_element_type(0) != element::f32 || !dot->get_argument(1)->is_constant())
                 continue;
+            {
+                // the fused entry point needs the weights lower_dot prepacks: shapes the library does not
+                // pack (a reduction that is not a multiple of 16, ...) keep Gelu and Quantize as they are
+                hipq_dot_desc_t d;
+                memset(&d, 0, sizeof(d));
+                d.a_t = dtype_of(dot->get_input_element_type(0));
+                d.b_t = dtype_of(dot->get_input_element_type(1));
+                d.out_t = dtype_of(dot->get_output_element_type(0));
+                d.b_layout = HIPQ_B_NK;
+                d.M = static_cast<int64_t>(dot->get_input_shape(0).at(0));
+                d.K = static_cast<int64_t>(dot->get_input_shape(0).at(1));
+                d.N = static_cast<int64_t>(dot->get_input_shape(1).at(0));
+                if (hipq_dot_packed_bytes(&d) == 0)
+                    continue;
+            }
             QuantizedCopy copy = qc->second;
             copy.through_gelu = true;
             m_quantized_copy.erase(qc);
@@ -515,7 +544,7 @@ namespace
                 pin(p);
             for (size_t i = 0; i < p->get_input_size(); ++i)
             {
-                const bool free_read = conv && (i == 0 || static_cast<int>(i) == conv_sum_input(p));
+                const bool free_read = (conv && (i == 0 || static_cast<int>(i) == conv_sum_input(p))) || (i == 0 && pool_to_points(p));
                 const bool tied_read = find(p->input_value(i).get_node()) == find(p) && !tied.empty();
                 if (!free_read && !tied_read)
                     pin(p->input_value(i).get_node());
@@ -733,7 +762,8 @@ namespace
             pa = &ap->get_padding_above();
         }
         d.dtype = dtype_of(n->get_output_element_type(0));
-        d.layout = nxc(n.get()) ? HIPQ_LAYOUT_NXC : HIPQ_LAYOUT_NCX; // input and output share a class
+        // input and output share a class, except where the output is points (the same bytes either way)
+        d.layout = nxc(pool_to_points(n.get()) ? n->input_value(0).get_node() : n.get()) ? HIPQ_LAYOUT_NXC : HIPQ_LAYOUT_NCX;
         d.n_spatial = static_cast<int32_t>(in.size() - 2);
         d.N = static_cast<int64_t>(in[0]);
         d.C = static_cast<int64_t>(in[1]);
@@ -794,10 +824,45 @@ namespace
             m_value_uses[value_of(n->input_value(0))] += 1;
             return;
         }
+        // Ops that change what the bytes are called, not the bytes: Convert between the two 8-bit
+        // integer types (a static_cast keeps the bits; the reference's CPU backend runs it in place,
+        // src/ngraph/runtime/cpu/pass/cpu_assignment.cpp:983-997) and Reshape without a transposition.
+        // The node shares its input's value: no launch, no memory.
+        {
+            bool same_bytes = false;
+            if (is_type<op::v0::Convert>(n))
+            {
+                const auto it = n->get_input_element_type(0);
+                same_bytes = (it == element::i8 || it == element::u8) && (et == element::i8 || et == element::u8);
+            }
+            else if (auto r = as_type_ptr<op::v0::Reshape>(n))
+            {
+                same_bytes = true;
+                const auto& order = r->get_input_order();
+                for (size_t i = 0; i < order.size(); ++i)
+                    same_bytes = same_bytes && order[i] == i;
+                // a transposition-free Reshape of a tensor kept channels-last would change the element
+                // order nGraph defines for it unless the tensor has no spatial extent left
+                if (same_bytes && nxc(n->input_value(0).get_node()))
+                {
+                    const Shape& is = n->get_input_shape(0);
+                    size_t spatial = 1;
+                    for (size_t i = 2; i < is.size(); ++i)
+                        spatial *= is[i];
+                    same_bytes = spatial == 1 || is.at(1) == 1;
+                }
+            }
+            if (same_bytes)
+            {
+                m_value_of[n.get()] = value_of(n->input_value(0));
+                return;
+            }
+        }
         m_value_of[n.get()] = id;
         m_value_ptr.push_back(nullptr);
         m_value_bytes.push_back(bytes);
         m_value_uses.push_back(0);
+        m_value_external.push_back(n->is_parameter() || n->is_constant());
         if (n->is_parameter())
             return; // bound per call
         if (auto c = as_type_ptr<op::v0::Constant>(n))
@@ -841,6 +906,7 @@ namespace
             m_value_ptr.push_back(alloc(obytes)->ptr);
             m_value_bytes.push_back(obytes);
             m_value_uses.push_back(0);
+            m_value_external.push_back(false);
             st.inputs.push_back(id + static_cast<int>(o)); // written, not read: no use counted
         }
         // glue fusion: the second addend of a folded Add, then the quantized copy a folded Quantize stands for
@@ -866,6 +932,7 @@ namespace
                 m_value_ptr.push_back(alloc(qbytes)->ptr);
                 m_value_bytes.push_back(qbytes);
                 m_value_uses.push_back(0);
+                m_value_external.push_back(false);
                 qcopy_at = static_cast<int>(st.inputs.size());
                 st.inputs.push_back(qid); // written, not read: no use counted
                 auto scalars = alloc(8);
@@ -1224,8 +1291,7 @@ namespace
                 throw runtime_error("HIP backend: output " + to_string(i) + " is not a tensor of this backend");
             out_ptr[i] = t->device_ptr();
             const int v = m_result_value[i];
-            const Node* producer = m_function->get_results()[i]->input_value(0).get_node();
-            if (m_value_uses[v] == 1 && !producer->is_parameter() && !producer->is_constant())
+            if (m_value_uses[v] == 1 && !m_value_external[v])
             {
                 ptr[v] = out_ptr[i];
                 direct[i] = true;

@@ -2,6 +2,7 @@
 of the quantized ops this library implements, the way nGraph's quantized graphs express it after
 the fusion passes:
 
+  input       Quantize f32 [N,3,224,224] (N(0,1) images) -> u8, scale 1/32, zero point 128, round half to even
   stem        QuantizedConvolutionBias(relu) 7x7/2, 3 -> 64          u8 [N,3,224,224] -> u8
               MaxPool 3x3/2, pad 1
   bottleneck  QuantizedConvolutionBias(relu) 1x1, in -> mid
@@ -9,11 +10,11 @@ the fusion passes:
               identity block:   QuantizedConvolutionBiasAdd(relu) 1x1, mid -> out, sum = block input (u8)
               first of a stage: QuantizedConvolutionBias 1x1/s, in -> out (i8, no relu) on the shortcut,
                                 QuantizedConvolutionBiasSignedAdd(relu) 1x1 (i8), Convert -> u8
-  head        AvgPool 7x7, QuantizedDotBias 2048 -> 1000 (f32 logits)
+  head        AvgPool 7x7, QuantizedDotBias 2048 -> 1000 requantized to i8, Dequantize -> f32 logits
 
 Weights, biases and scales are seeded pseudo-random numbers (there is no trained checkpoint here);
 scales are chosen so that activations keep using the 8-bit range through all 16 blocks.  The layer
-list is plain data: `run` executes it through any provider of the five ops (the HIP library's numpy
+list is plain data: `run` executes it through any provider of the ops (the HIP library's numpy
 conveniences, or a CPU implementation of the same ops), `DevicePlan` executes it with every tensor
 resident on the GPU, channels-last, for timing.
 """
@@ -27,19 +28,26 @@ from . import synth
 
 STAGES = [(64, 256, 3, 1), (128, 512, 4, 2), (256, 1024, 6, 2), (512, 2048, 3, 2)]
 CLASSES = 1000
+INPUT_SCALE, INPUT_ZP = 1.0 / 32, 128  # N(0,1) images: +-4 sigma fill the 8-bit range around 128
+LOGIT_SCALE = 0.05                      # scale of the i8 logits the Dequantize at the tail undoes
 
 
-def _conv(name, seed, Cc, K, R, stride, relu, src, sum_src=None, signed_sum=False, gain=1.0):
+def _conv(name, seed, Cc, K, R, stride, relu, src, sum_src=None, signed_sum=False, gain=1.0, in_rms=None, fold_zp=0):
     kred = Cc * R * R
-    # u8 activations (mean ~ 60, spread ~ 50) against uniform +-127 weights: accumulator spread ~ 73 * 80 * sqrt(kred)
-    scale = gain * 48.0 / (73.0 * 80.0 * math.sqrt(kred))
+    # Weights are uniform in -127 .. 127 (rms 73.3).  With inputs of root mean square a the accumulators
+    # have spread 73.3 a sqrt(kred); a ReLU output of spread s has root mean square s / sqrt(2): the scale
+    # sqrt(2) / (73.3 sqrt(kred)) hands the next layer the root mean square this layer was given, so the
+    # activations neither die out nor saturate over 16 blocks.  `in_rms` (the stem): the input's spread
+    # is known, the output is given a spread of 36 (the max pool behind it raises the level again).
+    scale = gain * math.sqrt(2.0) / (73.3 * math.sqrt(kred)) if in_rms is None else gain * 36.0 / (in_rms * 73.3 * math.sqrt(kred))
     return dict(op="conv", name=name, seed=seed, C=Cc, K=K, R=R, stride=stride, pad=R // 2, relu=relu, src=src, sum_src=sum_src, signed_sum=signed_sum, scale=scale,
-                sum_scale=0.5 if sum_src is not None else None)
+                sum_scale=0.5 if sum_src is not None else None, fold_zp=fold_zp)
 
 
 def layers():
     """the network as a list of ops; every op names its input(s) by the `name` of an earlier op ("input" for the image)"""
-    ops = [_conv("stem", 1, 3, 64, 7, 2, True, "input", gain=0.6), dict(op="maxpool", name="pool1", src="stem", window=3, stride=2, pad=1)]
+    ops = [dict(op="quantize", name="input_q", src="input", scale=INPUT_SCALE, zp=INPUT_ZP),
+           _conv("stem", 1, 3, 64, 7, 2, True, "input_q", in_rms=1.0 / INPUT_SCALE, fold_zp=INPUT_ZP), dict(op="maxpool", name="pool1", src="stem", window=3, stride=2, pad=1)]
     prev, cin, seed = "pool1", 64, 10
     for si, (mid, cout, blocks, stride) in enumerate(STAGES):
         for b in range(blocks):
@@ -49,19 +57,24 @@ def layers():
             ops.append(_conv(p + "c2", seed + 1, mid, mid, 3, s, True, p + "c1"))
             if b == 0:
                 ops.append(_conv(p + "down", seed + 2, cin, cout, 1, s, False, prev, gain=0.5))
-                ops.append(_conv(p + "c3", seed + 3, mid, cout, 1, 1, True, p + "c2", sum_src=p + "down", signed_sum=True, gain=0.7))
+                ops.append(_conv(p + "c3", seed + 3, mid, cout, 1, 1, True, p + "c2", sum_src=p + "down", signed_sum=True, gain=0.85))
                 ops.append(dict(op="convert_u8", name=p + "out", src=p + "c3"))
             else:
-                ops.append(_conv(p + "out", seed + 3, mid, cout, 1, 1, True, p + "c2", sum_src=prev, gain=0.7))
+                ops.append(_conv(p + "out", seed + 3, mid, cout, 1, 1, True, p + "c2", sum_src=prev, gain=0.85))
             prev, cin, seed = p + "out", cout, seed + 4
     ops.append(dict(op="avgpool", name="pool5", src=prev, window=7, stride=1, pad=0))
-    ops.append(dict(op="fc", name="logits", seed=seed, K=2048, N=CLASSES, src="pool5", scale=1.0 / 4000))
+    ops.append(dict(op="fc", name="fc", seed=seed, K=2048, N=CLASSES, src="pool5", scale=1.0 / 400))
+    ops.append(dict(op="dequantize", name="logits", src="fc", scale=LOGIT_SCALE))
     return ops
 
 
 def conv_weights(op):
     filt = synth.uniform_int(1000 + op["seed"], (op["K"], op["C"], op["R"], op["R"]), -127, 127, np.int8)
     bias = synth.uniform_int(5000 + op["seed"], (op["K"],), -3000, 3000, np.int32)
+    if op["fold_zp"]:
+        # the input's zero point folded into the bias, as quantized graphs do for an asymmetric u8 input:
+        # sum((x - zp) w) = sum(x w) - zp sum(w)
+        bias = (bias - op["fold_zp"] * filt.astype(np.int32).sum(axis=(1, 2, 3))).astype(np.int32)
     scales = (synth.uniform_f32(7000 + op["seed"], (op["K"],), 0.8, 1.2) * np.float32(op["scale"])).astype(np.float32)
     return filt, bias, scales
 
@@ -74,7 +87,9 @@ def fc_weights(op):
 
 
 def synthetic_images(N, seed=42, hw=224):
-    return synth.uniform_int(seed, (N, 3, hw, hw), 0, 255, np.uint8)
+    """N(0,1) f32 images [N,3,hw,hw]; image i depends on (seed, i) only, so a batch's first images are
+    the images of a smaller batch"""
+    return np.stack([synth.normal_f32(seed * 1000 + i, (3, hw, hw)) for i in range(N)])
 
 
 def out_hw(hw, R, stride, pad):
@@ -83,14 +98,19 @@ def out_hw(hw, R, stride, pad):
 
 def run(provider, images, ops=None):
     """executes the network on NCHW numpy tensors through `provider`, which offers
-    conv(desc, fused_desc, data, filt, bias, sum_in, scales, sum_scale), pool(desc, x),
-    dot_bias(desc, fused_desc, a, w, bias, scales); returns {name: tensor} of every op"""
+    quantize(x, scale, zp, quant_t), conv(desc, fused_desc, data, filt, bias, sum_in, scales, sum_scale),
+    pool(desc, x), dot_bias(desc, fused_desc, a, w, bias, scales), dequantize(q, scale, zp);
+    returns {name: tensor} of every op"""
     ops = layers() if ops is None else ops
     t = {"input": np.ascontiguousarray(images)}
     for op in ops:
         x = t[op["src"]]
         N, hw = x.shape[0], x.shape[2] if x.ndim == 4 else 1
-        if op["op"] == "conv":
+        if op["op"] == "quantize":
+            t[op["name"]] = provider.quantize(x, np.float32(op["scale"]), np.uint8(op["zp"]), "u8")
+        elif op["op"] == "dequantize":
+            t[op["name"]] = provider.dequantize(x, np.float32(op["scale"]), np.int8(0))
+        elif op["op"] == "conv":
             signed = op["signed_sum"] or not op["relu"]
             out_t = "i8" if signed else "u8"
             d = H.make_conv_desc(N, op["C"], op["K"], (hw, hw), (op["R"], op["R"]), stride=(op["stride"],) * 2, pad_below=(op["pad"],) * 2, pad_above=(op["pad"],) * 2, out_t=out_t)
@@ -105,7 +125,7 @@ def run(provider, images, ops=None):
             t[op["name"]] = x.view(np.uint8)  # static_cast between the 8-bit types keeps the bits
         elif op["op"] == "fc":
             w, bias, scales = fc_weights(op)
-            d = H.make_dot_desc(N, op["K"], op["N"], out_t="f32", b_layout=H.B_NK)
+            d = H.make_dot_desc(N, op["K"], op["N"], out_t="i8", b_layout=H.B_NK)
             f = H.make_fused_desc(has_bias=True, with_relu=False, scale_count=op["N"])
             t[op["name"]] = provider.dot_bias(d, f, x.reshape(N, op["K"]), w, bias, scales)
     return t
@@ -113,6 +133,14 @@ def run(provider, images, ops=None):
 
 class HipProvider:
     """the HIP library through its numpy-in / numpy-out conveniences (one upload and download per op)"""
+
+    @staticmethod
+    def quantize(x, scale, zp, quant_t):
+        return H.quantize(x, scale, zp, quant_t)
+
+    @staticmethod
+    def dequantize(q, scale, zp):
+        return H.dequantize(q, scale, zp, "f32")
 
     @staticmethod
     def conv(d, f, x, filt, bias, sum_in, scales, sum_scale):
@@ -128,26 +156,40 @@ class HipProvider:
 
 
 class DevicePlan:
-    """The network with every tensor resident in HBM, channels-last, weights packed once: `launch()`
-    issues the 71 kernel launches of one forward pass on `stream`; `capture()` turns them into one
-    HIP graph for `replay()`."""
+    """The network with every tensor resident in HBM, weights packed once: the f32 images arrive in the
+    reference's NCHW order, Quantize writes u8 NCHW, the stem reads that and writes channels-last, and
+    everything up to the logits stays channels-last.  `launch()` issues the kernel launches of one
+    forward pass on `stream`; `capture()` turns them into one HIP graph for `replay()`."""
 
     def __init__(self, lib, stream, N, hw=224):
         self.lib, self.stream, self.N = lib, stream, N
         self._replay = None
         self.calls, self.keep, self.graph = [], [], None
         dev = lambda a: self._keep(H.DeviceBuffer.from_numpy(np.ascontiguousarray(a)))
-        buf = {"input": self._keep(H.DeviceBuffer(N * hw * hw * 3))}
+        buf = {"input": self._keep(H.DeviceBuffer(N * hw * hw * 3 * 4))}
         shape = {"input": (3, hw)}
         self.input = buf["input"]
         self.ops_per_image = 0
         for op in layers():
             Cc, h = shape[op["src"]]
             src = buf[op["src"]]
-            if op["op"] == "conv":
+            if op["op"] == "quantize":
+                d = H.make_quant_desc((N, Cc, h, h), (), "f32", "u8")
+                out = self._keep(H.DeviceBuffer(N * Cc * h * h))
+                bs, bz = dev(np.asarray([op["scale"]], np.float32)), dev(np.asarray([op["zp"]], np.uint8))
+                self.calls.append((lib.hipq_quantize, (self._keep(d), src, bs, bz, out)))
+                buf[op["name"]], shape[op["name"]] = out, (Cc, h)
+            elif op["op"] == "dequantize":
+                d = H.make_quant_desc((N, CLASSES), (), "f32", "i8")
+                out = self._keep(H.DeviceBuffer(N * CLASSES * 4))
+                bs, bz = dev(np.asarray([op["scale"]], np.float32)), dev(np.zeros(1, np.int8))
+                self.calls.append((lib.hipq_dequantize, (self._keep(d), src, bs, bz, out)))
+                buf[op["name"]] = out
+            elif op["op"] == "conv":
                 signed = op["signed_sum"] or not op["relu"]
+                # the stem reads the Quantize's NCHW bytes itself; every later layer is channels-last
                 d = H.make_conv_desc(N, op["C"], op["K"], (h, h), (op["R"], op["R"]), stride=(op["stride"],) * 2, pad_below=(op["pad"],) * 2, pad_above=(op["pad"],) * 2,
-                                     out_t="i8" if signed else "u8", data_layout=H.NXC, out_layout=H.NXC)
+                                     out_t="i8" if signed else "u8", data_layout=H.NCX if op["src"] == "input_q" else H.NXC, out_layout=H.NXC)
                 has_sum = op["sum_src"] is not None
                 f = H.make_fused_desc(has_bias=True, has_sum=has_sum, sum_t="i8" if op["signed_sum"] else "u8", with_relu=op["relu"], scale_count=op["K"])
                 filt, bias, scales = conv_weights(op)
@@ -170,13 +212,13 @@ class DevicePlan:
                 buf[op["name"]], shape[op["name"]] = src, (Cc, h)  # same bits: the buffer is shared
             elif op["op"] == "fc":
                 w, bias, scales = fc_weights(op)
-                d = H.make_dot_desc(N, op["K"], op["N"], out_t="f32", b_layout=H.B_NK)
+                d = H.make_dot_desc(N, op["K"], op["N"], out_t="i8", b_layout=H.B_NK)
                 f = H.make_fused_desc(has_bias=True, with_relu=False, scale_count=op["N"])
                 bw, bb, bs = dev(w), dev(bias), dev(scales)
                 packed = self._keep(H.pack_dot(d, bw))
-                out = self._keep(H.DeviceBuffer(N * op["N"] * 4))
+                out = self._keep(H.DeviceBuffer(N * op["N"]))
                 self.calls.append((lib.hipq_quantized_dot_bias, (self._keep(d), self._keep(f), src, bw, packed, bb, bs, out)))
-                buf[op["name"]] = out
+                buf[op["name"]], shape[op["name"]] = out, (op["N"], 1)
                 self.ops_per_image += 2 * op["K"] * op["N"]
         self.logits = buf["logits"]
         self.buffers = buf
@@ -186,8 +228,9 @@ class DevicePlan:
         return x
 
     def set_images_nchw(self, images):
-        """uploads [N,3,H,W] images as the channels-last tensor the plan reads"""
-        x = np.ascontiguousarray(np.moveaxis(images, 1, -1))
+        """uploads f32 [N,3,H,W] images, the tensor the Quantize at the head reads"""
+        x = np.ascontiguousarray(images, dtype=np.float32)
+        assert x.nbytes == self.input.nbytes
         H.check(self.lib.hipq_memcpy_h2d(self.input.ptr, x.ctypes.data, x.nbytes, None))
 
     def launch(self):

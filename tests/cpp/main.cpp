@@ -1,8 +1,13 @@
 // hip_backend_tests [--cpu | --gpu | --all] [--list] [--exact] [substring or, with --exact, suite.name]
+// hip_backend_tests --bench [--calls N] [--warmup N] [--only conv|resnet50]   (bench_backend.cpp)
 #include "mini_test.hpp"
+
+int run_backend_bench(int argc, char** argv);
 
 int main(int argc, char** argv)
 {
+    if (argc > 1 && std::string(argv[1]) == "--bench")
+        return run_backend_bench(argc, argv);
     bool want_cpu = true, want_gpu = false, list = false, exact = false;
     std::string filter;
     for (int i = 1; i < argc; ++i)

@@ -432,3 +432,45 @@ GPU_TEST(HIP, glue_fusion_dot_bias_with_gelu_and_quantize)
         }
     }
 }
+
+GPU_TEST(HIP, glue_fusion_dot_bias_gelu_quantize_unpacked_shapes)
+{
+    // Shapes whose weights the library does not prepack (a reduction of 100 bytes is not a multiple of
+    // 16) cannot take the fused entry point: the product keeps its own launch and only the Quantize
+    // folds into the Gelu.  A narrow product (8 columns) that is packed takes the workspace route.
+    struct Case
+    {
+        size_t rows, K, N, fused_launches;
+    };
+    for (const Case c : {Case{48, 100, 24, 3}, Case{300, 100, 128, 3}, Case{64, 64, 8, 2}})
+    {
+        auto x = make_shared<op::v0::Parameter>(element::f32, Shape{c.rows, c.K});
+        auto xs = op::v0::Constant::create(element::f32, Shape{}, {0.02f});
+        auto xz = op::v0::Constant::create(element::i8, Shape{}, {0});
+        auto x8 = make_shared<op::v0::Quantize>(x, xs, xz, element::i8, AxisSet{}, op::v0::Quantize::RoundMode::ROUND_NEAREST_TOWARD_EVEN);
+        vector<int8_t> w(c.N * c.K);
+        for (size_t i = 0; i < w.size(); ++i)
+            w[i] = static_cast<int8_t>(static_cast<int>((i * 29 + i / c.K * 7) % 255) - 127);
+        vector<int32_t> b(c.N);
+        vector<float> s(c.N);
+        for (size_t i = 0; i < c.N; ++i)
+        {
+            b[i] = static_cast<int32_t>(i * 17) - 300;
+            s[i] = 0.0004f + 0.000002f * static_cast<float>(i);
+        }
+        auto W = op::v0::Constant::create(element::i8, Shape{c.N, c.K}, w);
+        auto B = op::v0::Constant::create(element::i32, Shape{c.N}, b);
+        auto S = op::v0::Constant::create(element::f32, Shape{c.N}, s);
+        auto dot = make_shared<op::v0::QuantizedDotBias>(x8, W, B, S, false, false);
+        auto gelu = make_shared<op::v0::Gelu>(dot);
+        auto qs = op::v0::Constant::create(element::f32, Shape{}, {0.03f});
+        auto qz = op::v0::Constant::create(element::i8, Shape{}, {2});
+        auto q = make_shared<op::v0::Quantize>(gelu, qs, qz, element::i8, AxisSet{}, op::v0::Quantize::RoundMode::ROUND_NEAREST_TOWARD_EVEN);
+        const auto data = wave(c.rows * c.K, 1.8f, 0.013f);
+        auto f = make_shared<Function>(OutputVector{q}, ParameterVector{x});
+        const auto plain = run_glue(f, {data}, false), fused = run_glue(f, {data}, true);
+        EXPECT_TRUE(plain.bytes == fused.bytes);
+        EXPECT_EQ(plain.launches, size_t(4));
+        EXPECT_EQ(fused.launches, c.fused_launches);
+    }
+}

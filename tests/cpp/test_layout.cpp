@@ -146,3 +146,75 @@ GPU_TEST(HIP, call_replays_hip_graph)
         }
     }
 }
+
+// A classifier tail behind residual blocks: QuantizedConvolutionBiasSignedAdd -> Convert (i8 -> u8) ->
+// QuantizedConvolutionBiasAdd -> global AvgPool -> Reshape [N, C, 1, 1] -> [N, C] -> QuantizedDotBias.
+// Reshape and the GEMM only know nGraph's layout, but a tensor without spatial extent has the same
+// bytes either way: the blocks in front stay channels-last (no transposition launches), the Convert
+// between the 8-bit types and the transposition-free Reshape are no launches at all, and the
+// results equal those of the pass-off run bit for bit.
+namespace
+{
+    shared_ptr<Function> classifier_tail(size_t N)
+    {
+        Lcg rng{4242u};
+        auto x = make_shared<op::v0::Parameter>(element::u8, Shape{N, 64, 7, 7});
+        auto scale = [](float v) { return op::v0::Constant::create(element::f32, Shape{}, {v}); };
+        auto weights = [&](size_t K, size_t C) { return random_constant<int8_t>(element::i8, Shape{K, C, 1, 1}, rng, -20, 20); };
+        auto bias = [&](size_t K) { return random_constant<int32_t>(element::i32, Shape{K}, rng, -2000, 2000); };
+        auto c1 = make_shared<op::v0::QuantizedConvolutionBias>(x, weights(64, 64), bias(64), Strides{1, 1}, Strides{1, 1}, CoordinateDiff{0, 0}, CoordinateDiff{0, 0}, Strides{1, 1},
+                                                                scale(1.0f / 900), true);
+        auto down = make_shared<op::v0::QuantizedConvolutionBias>(x, weights(128, 64), bias(128), Strides{1, 1}, Strides{1, 1}, CoordinateDiff{0, 0}, CoordinateDiff{0, 0}, Strides{1, 1},
+                                                                  scale(1.0f / 1800), false);
+        auto c3 = make_shared<op::v0::QuantizedConvolutionBiasSignedAdd>(c1, weights(128, 64), bias(128), down, Strides{1, 1}, Strides{1, 1}, CoordinateDiff{0, 0}, CoordinateDiff{0, 0},
+                                                                         Strides{1, 1}, scale(1.0f / 1100), scale(0.5f), true);
+        auto u = make_shared<op::v0::Convert>(c3, element::u8);
+        auto c4 = make_shared<op::v0::QuantizedConvolutionBias>(u, weights(64, 128), bias(64), Strides{1, 1}, Strides{1, 1}, CoordinateDiff{0, 0}, CoordinateDiff{0, 0}, Strides{1, 1},
+                                                                scale(1.0f / 1300), true);
+        auto c5 = make_shared<op::v0::QuantizedConvolutionBiasAdd>(c4, weights(128, 64), bias(128), u, Strides{1, 1}, Strides{1, 1}, CoordinateDiff{0, 0}, CoordinateDiff{0, 0}, Strides{1, 1},
+                                                                   scale(1.0f / 1100), scale(0.5f), true);
+        auto pool = make_shared<op::v0::AvgPool>(c5, Shape{7, 7}, Strides{1, 1}, Shape{0, 0}, Shape{0, 0}, false);
+        auto flat = make_shared<op::v0::Reshape>(pool, AxisVector{0, 1, 2, 3}, Shape{N, 128});
+        auto w = random_constant<int8_t>(element::i8, Shape{48, 128}, rng, -100, 100);
+        auto fc = make_shared<op::v0::QuantizedDotBias>(flat, w, bias(48), scale(1.0f / 300), true, false);
+        return make_shared<Function>(OutputVector{fc, u}, ParameterVector{x});
+    }
+}
+
+GPU_TEST(HIP, layout_pass_keeps_blocks_channels_last_in_front_of_a_classifier)
+{
+    const size_t N = 6;
+    vector<int8_t> logits[2];
+    vector<uint8_t> block[2];
+    size_t launches[2] = {0, 0};
+    for (int on = 0; on < 2; ++on)
+    {
+        setenv("NGRAPH_PASS_ENABLES", on ? "HIPLayout:1" : "HIPLayout:0", 1);
+        auto f = classifier_tail(N);
+        auto backend = runtime::Backend::create("HIP");
+        auto a = backend->create_tensor(element::u8, Shape{N, 64, 7, 7});
+        Lcg rng{31u};
+        vector<uint8_t> data(a->get_element_count());
+        for (auto& v : data)
+            v = static_cast<uint8_t>(rng.next(0, 255));
+        copy_data(a, data);
+        auto r = backend->create_tensor(element::i8, Shape{N, 48});
+        auto r2 = backend->create_tensor(element::u8, Shape{N, 128, 7, 7});
+        auto exec = backend->compile(f, true);
+        unsetenv("NGRAPH_PASS_ENABLES");
+        for (int i = 0; i < 3; ++i)
+            exec->call_with_validate({r, r2}, {a});
+        logits[on] = read_vector<int8_t>(r);
+        block[on] = read_vector<uint8_t>(r2);
+        launches[on] = exec->get_performance_data().size();
+    }
+    EXPECT_TRUE(logits[0] == logits[1]);
+    EXPECT_TRUE(block[0] == block[1]); // the Convert's value, returned in nGraph's layout either way
+    size_t distinct = 0, seen[256] = {0};
+    for (int8_t v : logits[1])
+        distinct += seen[static_cast<uint8_t>(v)]++ == 0;
+    EXPECT_TRUE(distinct > 20);
+    // five convolutions, the pool and the GEMM: Convert and Reshape launch nothing
+    EXPECT_EQ(launches[0], size_t(7));
+    EXPECT_EQ(launches[1], size_t(7));
+}

@@ -272,17 +272,22 @@ def resnet50_vectors():
     from ngraph_amd import resnet50 as R
 
     class Oracle:
+        quantize = staticmethod(lambda x, s, z, t: O.quantize(x, s, z, t))
+        dequantize = staticmethod(lambda q, s, z: O.dequantize(q, s, z, "f32"))
         conv = staticmethod(lambda d, f, x, filt, bias, s, sc, ss: O.quantized_convolution_fused(d, f, x, filt, bias, s, sc, ss))
         pool = staticmethod(lambda d, x: O.pool(d, x))
         dot_bias = staticmethod(lambda d, f, a, w, bias, sc: O.quantized_dot_bias(d, f, a, w, bias, sc))
 
     O.port().orc_set_threads(8)
-    t = R.run(Oracle, R.synthetic_images(1))
+    image = R.synthetic_images(1)
+    t = R.run(Oracle, image)
     O.port().orc_set_threads(1)
     sums = {op["name"]: int(t[op["name"]].view(np.uint8).astype(np.uint64).sum()) for op in R.layers()}
     np.savez_compressed(os.path.join(HERE, "resnet50_logits.npz"), logits=t["logits"])
     with open(os.path.join(HERE, "resnet50_logits.json"), "w") as f:
-        json.dump(dict(image_seed=42, byte_sums=sums, logits=[float(v) for v in t["logits"].ravel()]), f, indent=0)
+        # image_bit_sum: the f32 image is made with the host's log / cos / sin; a math library that rounds
+        # one value differently changes this sum, and the tests say so instead of reporting wrong logits
+        json.dump(dict(image_seed=42, image_bit_sum=int(image.view(np.uint32).astype(np.uint64).sum()), byte_sums=sums, logits=[float(v) for v in t["logits"].ravel()]), f, indent=0)
     print("resnet50_logits: 1000 logits,", len(sums), "byte sums")
 
 

@@ -25,6 +25,20 @@ def test_exports_match_header():
     assert sorted(H.EXPORTS) == names
 
 
+def test_product_library_exports_only_the_declared_abi():
+    """libhipq.so exports what include/hipq.h declares (plus hipq_last_kernel, the tests' window on the
+    dispatcher) and no development or measurement symbol; those live in libhipq_probe.so"""
+    import subprocess
+
+    out = subprocess.run(["nm", "-D", "--defined-only", H.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    exported = sorted(line.split()[-1] for line in out.splitlines() if " T " in line)
+    assert not [n for n in exported if "debug" in n or "probe" in n], exported
+    assert set(exported) - set(_declared()) <= {"hipq_last_kernel", "_init", "_fini"}, sorted(set(exported) - set(_declared()))
+    probe = H.load_probe()
+    for n in ("hipq_probe_mfma_i8", "hipq_probe_intake", "hipq_probe_atomic_tiles", "hipq_debug_fastdiv", "hipq_probe_last_error"):
+        assert hasattr(probe, n), n
+
+
 def test_struct_sizes_match_header():
     # sizes follow from the header's field lists (natural alignment)
     assert C.sizeof(H.QuantDesc) == 4 * 6 + 8 * 8
@@ -94,9 +108,7 @@ def test_packed_sizes_and_eligibility():
 
 
 def test_fastdiv_exact():
-    lib = H.load()
-    lib.hipq_debug_fastdiv.restype = C.c_uint32
-    lib.hipq_debug_fastdiv.argtypes = [C.c_uint32] * 2
+    lib = H.load_probe()  # the index division of the Quantize kernels, exported by the measurement-aid library
     rng = np.random.default_rng(0)
     ds = list(range(1, 130)) + [255, 256, 257, 1023, 1024, 1025, 65535, 65536, 65537, 2**30, 2**31 - 1] + rng.integers(1, 2**31, 50).tolist()
     for d in ds:

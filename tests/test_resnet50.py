@@ -1,4 +1,5 @@
-"""The synthetic int8 ResNet-50 (ngraph_amd/resnet50.py): every one of its 60 ops on the GPU against the
+"""The synthetic int8 ResNet-50 (ngraph_amd/resnet50.py: f32 N(0,1) images, Quantize, 53 fused
+convolutions, pools, the requantizing classifier GEMM, Dequantize): every one of its ops on the GPU against the
 CPU oracle on a full-size image, bit for bit, and the device-resident channels-last plan (with and
 without HIP-graph replay) against the op-by-op run."""
 import ctypes as C
@@ -12,6 +13,14 @@ from ngraph_amd import resnet50 as R
 
 
 class OracleProvider:
+    @staticmethod
+    def quantize(x, scale, zp, quant_t):
+        return O.quantize(x, scale, zp, quant_t)
+
+    @staticmethod
+    def dequantize(q, scale, zp):
+        return O.dequantize(q, scale, zp, "f32")
+
     @staticmethod
     def conv(d, f, x, filt, bias, sum_in, scales, sum_scale):
         return O.quantized_convolution_fused(d, f, x, filt, bias, sum_in, scales, sum_scale)
@@ -30,6 +39,7 @@ def test_layer_list_is_resnet50():
     convs = [o for o in ops if o["op"] == "conv"]
     assert len(convs) == 53 and sum(o["op"] == "fc" for o in ops) == 1
     assert sum(o["R"] == 3 for o in convs) == 16 and sum(o["R"] == 7 for o in convs) == 1
+    assert ops[0]["op"] == "quantize" and ops[-1]["op"] == "dequantize" and ops[-2]["op"] == "fc"  # BASELINE config 4: Quantize at the head, Dequantize at the tail
     names = {"input"}
     for o in ops:  # every op reads tensors that exist by then
         assert o["src"] in names and (o.get("sum_src") is None or o["sum_src"] in names)
@@ -60,11 +70,21 @@ def _golden():
     return meta, np.load(os.path.join(here, "resnet50_logits.npz"))["logits"]
 
 
+def _same_image_as_fixture(images, meta):
+    """The seeded f32 image comes out of numpy's log / cos / sin; the fixture records the sum of its bit
+    patterns.  A math library that rounds one value differently makes another image, for which the
+    committed logits do not hold (the live oracle comparison still does)."""
+    return int(images[:1].view(np.uint32).astype(np.uint64).sum()) == meta["image_bit_sum"]
+
+
 def test_oracle_reproduces_committed_logits():
     """the committed fixture (which the C++ backend test also uses) is what the restatement computes today"""
     meta, logits = _golden()
+    image = R.synthetic_images(1, seed=meta["image_seed"])
+    if not _same_image_as_fixture(image, meta):
+        pytest.skip("this host's math library makes a different f32 image than the fixture's")
     O.port().orc_set_threads(8)
-    t = R.run(OracleProvider, R.synthetic_images(1, seed=meta["image_seed"]))
+    t = R.run(OracleProvider, image)
     O.port().orc_set_threads(1)
     assert np.array_equal(t["logits"], logits)
     for name, total in meta["byte_sums"].items():
@@ -87,8 +107,13 @@ def test_resnet50_every_op_against_oracle(gpu_lib):
     # the network is alive to the end: the last block still uses the 8-bit range, the logits differ
     last = exp["s5_b2_out"]
     assert 0.2 < np.count_nonzero(last) / last.size and (last == 255).mean() < 0.2
-    assert np.unique(exp["logits"]).size > 900
-    assert np.array_equal(got["logits"], _golden()[1])
+    assert np.unique(exp["fc"]).size > 100 and np.abs(exp["fc"].astype(np.int32)).max() < 127  # spread over the 8-bit range, not saturated
+    assert exp["input_q"].dtype == np.uint8 and 100 < exp["input_q"].mean() < 156 and exp["logits"].dtype == np.float32
+    meta, golden = _golden()
+    if _same_image_as_fixture(images, meta):
+        assert np.array_equal(got["logits"], golden)
+    else:
+        print("[note] this host's math library makes a different f32 image than the fixture's: committed logits not compared", flush=True)
 
 
 @pytest.mark.gpu
@@ -133,7 +158,8 @@ def test_resnet50_benchmarked_batches_against_oracle(gpu_lib, N):
     O.port().orc_set_threads(8)
     exp = R.run(OracleProvider, four)
     O.port().orc_set_threads(1)
-    assert np.array_equal(exp["logits"][:1], golden)
+    if _same_image_as_fixture(four, meta):
+        assert np.array_equal(exp["logits"][:1], golden)
     images = np.ascontiguousarray(np.tile(four, (N // 4, 1, 1, 1)))
     sp = C.c_void_p()
     H.check(lib.hipq_stream_create(C.byref(sp)))

@@ -105,3 +105,64 @@ def test_noalloc_refuses_what_does_not_fit(gpu_lib, monkeypatch):
     # the regular entry point takes the same call
     H.check(lib.hipq_quantized_convolution(C.byref(d), data.ptr, filt.ptr, packed.ptr, s[0].ptr, z[0].ptr, s[1].ptr, z[1].ptr, s[2].ptr, z[2].ptr, out.ptr, None))
     H.check(lib.hipq_stream_sync(None))
+
+
+@pytest.mark.gpu
+def test_noalloc_first_on_a_fresh_stream_allocates_nothing_and_replays_from_a_graph(gpu_lib, monkeypatch):
+    """The entry point is the first thing a new stream ever sees (no regular call has sized any scratch
+    for that stream): the library's allocation epoch must not move.  Then the same call recorded into
+    a HIP graph and replayed three times, with eager work of the program between the replays, gives
+    the regular entry point's bytes every time (the layout copy into the scratch array is inside the
+    graph)."""
+    monkeypatch.setenv("HIPQ_NO_REGW", "1")
+    lib = gpu_lib
+    lib.hipq_workspace_epoch.restype = C.c_uint64
+    d = H.make_conv_desc(2, 64, 64, (28, 28), (3, 3), pad_below=(1, 1), pad_above=(1, 1))
+    nin, nout = int(np.prod(d.data_shape())), int(np.prod(d.out_shape()))
+    filt = H.DeviceBuffer.from_numpy(synth.uniform_int(3501, d.filter_shape(), -127, 127, np.int8))
+    packed = H.pack_filter(d, filt)
+    s = [H.DeviceBuffer.from_numpy(np.float32(v)) for v in (0.02, 0.005, 0.3)]
+    z = [H.DeviceBuffer.from_numpy(np.zeros(1, t)) for t in (np.uint8, np.int8, np.int8)]
+    data, out, ref = H.DeviceBuffer(nin), H.DeviceBuffer(nout), H.DeviceBuffer(nout)
+    sp = C.c_void_p()
+    H.check(lib.hipq_stream_create(C.byref(sp)))
+    stream = sp.value
+
+    def upload(seed):
+        x = synth.uniform_int(seed, d.data_shape(), 0, 255, np.uint8)
+        H.check(lib.hipq_memcpy_h2d(data.ptr, x.ctypes.data, x.nbytes, None))
+
+    def call(fn, dst, st):
+        H.check(fn(C.byref(d), data.ptr, filt.ptr, packed.ptr, s[0].ptr, z[0].ptr, s[1].ptr, z[1].ptr, s[2].ptr, z[2].ptr, dst.ptr, st))
+
+    say("noalloc first on a fresh stream")
+    upload(3502)
+    epoch = lib.hipq_workspace_epoch()
+    call(lib.hipq_quantized_convolution_noalloc, out, stream)
+    H.check(lib.hipq_stream_sync(stream))
+    assert lib.hipq_workspace_epoch() == epoch, "the entry point that allocates nothing moved the allocation epoch"
+    call(lib.hipq_quantized_convolution, ref, None)
+    H.check(lib.hipq_stream_sync(None))
+    first = out.to_numpy(np.uint8, (nout,))
+    assert np.array_equal(first, ref.to_numpy(np.uint8, (nout,)))
+    assert len(np.unique(first)) > 50
+
+    say("noalloc recorded into a graph")
+    H.check(lib.hipq_capture_begin(stream))
+    call(lib.hipq_quantized_convolution_noalloc, out, stream)
+    graph = C.c_void_p()
+    H.check(lib.hipq_capture_end(stream, C.byref(graph)))
+    try:
+        for i in range(3):
+            upload(3510 + i)  # eager work and a synchronisation between the replays
+            call(lib.hipq_quantized_convolution, ref, None)
+            H.check(lib.hipq_stream_sync(None))
+            H.check(lib.hipq_fill_bytes(out.ptr, 0xA5, nout, stream))
+            say("replay", i)
+            H.check(lib.hipq_graph_launch(graph, stream))
+            H.check(lib.hipq_stream_sync(stream))
+            assert np.array_equal(out.to_numpy(np.uint8, (nout,)), ref.to_numpy(np.uint8, (nout,))), "replay %d differs from the eager result" % i
+        assert lib.hipq_workspace_epoch() >= epoch
+    finally:
+        H.check(lib.hipq_graph_destroy(graph))
+        H.check(lib.hipq_stream_destroy(stream))

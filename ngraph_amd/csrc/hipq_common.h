@@ -261,7 +261,8 @@ namespace hipq
                         const ZeroPoints& zp,
                         const Epilogue& epi,
                         void* out,
-                        hipStream_t s);
+                        hipStream_t s,
+                        const void* w_frag = nullptr); // fragment-ordered copy of the weights (prepacked blobs), or null
 
     int launch_rows_mfma(const void* a, bool a_unsigned, const int8_t* w_nk, const int32_t* wsum, int64_t M, int32_t N, int32_t K,
                          const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s, const char* name);
@@ -283,4 +284,9 @@ namespace hipq
     int launch_stage_rows(const ConvGeom& g, const RowPack& rp, const void* in, void* staged, const void* zp, int zp_t, hipStream_t s);
     int launch_conv_rowpack(const ConvGeom& g, const RowPack& rp, const void* staged, const void* packed, const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s);
     int launch_row_sums_i8(const void* w, int64_t rows, int64_t cols, int32_t* sums, hipStream_t s);
+    // [N][K] weights in the fragment order of v_mfma_i32_16x16x64_i8 (K a multiple of 64): ceil(N / 16) * K / 64 blocks of 1 KB
+    int launch_pack_dot_fragments(const void* w_nk, int64_t N, int64_t K, void* frag, hipStream_t s);
+    // whether a packed blob of this product carries the fragment-ordered copy, and its size
+    bool dot_fragments_eligible(const hipq_dot_desc_t& d);
+    size_t dot_fragment_bytes(const hipq_dot_desc_t& d);
 }

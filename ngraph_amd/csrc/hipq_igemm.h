@@ -102,6 +102,15 @@ namespace hipq
     {
         asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base), "v"(off), "s"(rsrc) : "memory");
     }
+    // The same load without the compiler-level memory barrier, for kernels that bracket their LDS
+    // traffic with barriers of their own (every fragment read sits behind a wait_vmcnt, every load
+    // that overwrites a region behind the waited-for reads of that region).  A barrier on every load
+    // makes the compiler treat all of memory as changed behind it: uniform loads that follow can no
+    // longer go through the scalar cache and land in the vector queue behind the operand stream.
+    __device__ __forceinline__ void lds_dma16_unfenced(v4i rsrc, int32_t off, uint32_t lds_base)
+    {
+        asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_base), "v"(off), "s"(rsrc));
+    }
     template <int N>
     __device__ __forceinline__ void wait_vmcnt()
     {
@@ -489,6 +498,73 @@ namespace hipq
         // |acc| <= 2^31, so |acc * scale| < 2^31 whenever |scale| < 1 (false for NaN)
         c.slow_cvt = !(fabsf(r.scale) < 1.0f);
         return c;
+    }
+
+    // The scalars of a kernel's head -- both accumulation zero points and everything epi_const reads
+    // -- fetched by loads that are all issued at once.  epi_const / load_zp branch on modes, types and
+    // null pointers, and a load behind a branch waits for the loads in front of it: a chain of
+    // memory latencies where one is enough.  Here a pointer the call does not use (or a null one) is
+    // replaced by `safe` (any readable, 4-byte aligned address) and its value discarded; a byte is
+    // read through the aligned word that holds it (the word lies in the byte's own page), so that
+    // every load is a uniform word load: those go through the scalar cache and its own counter,
+    // where they neither wait for nor hold up the vector loads around them.  8-bit data and filter
+    // zero points only (what the MFMA kernels take).
+    //   head_scalars_load    at the very top of a kernel (behind an asm statement the compiler can no
+    //                        longer prove memory unchanged and falls back to vector loads)
+    //   head_scalars_settle  where the kernel is ready to wait for them (behind its operand loads):
+    //                        pins the first use of the raw words to this point
+    //   head_scalars_finish  the arithmetic
+    struct HeadWords
+    {
+        uint32_t x, w, o, sd, sf, so, s0, ss; // raw words: zero points (data, filter, output), scales
+    };
+    struct HeadScalars
+    {
+        int32_t xzp, wzp;
+        EpiConst ec;
+    };
+    __device__ __forceinline__ HeadWords head_scalars_load(const ZeroPoints& zp, const Epilogue& e, const void* safe)
+    {
+        const bool interp = e.mode == EPI_INTERP;
+        auto word_at = [&](const void* p, bool used) {
+            const uint8_t* q = static_cast<const uint8_t*>((used && p != nullptr) ? p : safe);
+            return *reinterpret_cast<const uint32_t*>(q - (reinterpret_cast<uintptr_t>(q) & 3)); // (pointer arithmetic, not an integer cast: the load stays a global one)
+        };
+        HeadWords h;
+        h.x = word_at(zp.data_zp, true);
+        h.w = word_at(zp.filter_zp, true);
+        h.o = word_at(e.out_zp, interp);
+        h.sd = word_at(e.s_data, interp);
+        h.sf = word_at(e.s_filter, interp);
+        h.so = word_at(e.s_out, interp);
+        h.s0 = word_at(e.scale, !interp);
+        h.ss = word_at(e.sum_scale, !interp && e.sum_in != nullptr);
+        return h;
+    }
+    __device__ __forceinline__ void head_scalars_settle(HeadWords& h)
+    {
+        asm volatile("" : "+s"(h.x), "+s"(h.w), "+s"(h.o), "+s"(h.sd), "+s"(h.sf), "+s"(h.so), "+s"(h.s0), "+s"(h.ss));
+    }
+    __device__ __forceinline__ HeadScalars head_scalars_finish(const HeadWords& h, const ZeroPoints& zp, const Epilogue& e)
+    {
+        const bool interp = e.mode == EPI_INTERP;
+        auto as_zp = [](uint32_t word, const void* p, int t) {
+            const uint32_t b = (word >> (8 * static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p) & 3))) & 0xFFu;
+            return t == HIPQ_U8 ? static_cast<int32_t>(b) : static_cast<int32_t>(static_cast<int8_t>(b));
+        };
+        HeadScalars r;
+        r.xzp = zp.data_zp ? as_zp(h.x, zp.data_zp, zp.data_t) : 0;
+        r.wzp = zp.filter_zp ? as_zp(h.w, zp.filter_zp, zp.filter_t) : 0;
+        EpiConst& c = r.ec;
+        // src/ngraph/runtime/reference/convolution.hpp:254 : two f32 roundings, this order
+        c.scale = interp ? __fdiv_rn(__fmul_rn(__uint_as_float(h.sd), __uint_as_float(h.sf)), __uint_as_float(h.so)) : __uint_as_float(h.s0);
+        c.sum_scale = (!interp && e.sum_in != nullptr) ? __uint_as_float(h.ss) : 0.0f;
+        c.ozp = (interp && e.out_zp != nullptr) ? ((e.out_t == HIPQ_U8 || e.out_t == HIPQ_I8) ? as_zp(h.o, e.out_zp, e.out_t) : static_cast<int32_t>(h.o)) : 0;
+        c.lo = (e.out_t == HIPQ_U8) ? 0.0f : (e.out_t == HIPQ_I8 ? -128.0f : -2147483648.0f);
+        c.hi = (e.out_t == HIPQ_U8) ? 255.0f : (e.out_t == HIPQ_I8 ? 127.0f : 2147483520.0f);
+        c.relu_floor = e.relu ? 0.0f : -__builtin_huge_valf();
+        c.slow_cvt = !(fabsf(c.scale) < 1.0f);
+        return r;
     }
 
     // INTERPRETER: (OUT) roundf(float(acc) * scale) + ozp; the caller keeps the low byte for 8-bit types

@@ -1,8 +1,12 @@
 // Layout helpers: batched 2-D transposes (NCX <-> NXC), filter repacking, row sums.
+#include <algorithm>
+
 #include "hipq_common.h"
 
 namespace hipq
 {
+    typedef int v4i_t __attribute__((ext_vector_type(4)));
+
     // in [B][R][Cc] -> out [B][Cc][R], elements of EB bytes, through a padded LDS tile
     template <typename T>
     __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ in, T* __restrict__ out, int64_t R, int64_t Cc)
@@ -151,6 +155,41 @@ namespace hipq
             return HIPQ_OK;
         row_sums_i8_kernel<<<static_cast<unsigned>((rows + 3) / 4), 256, 0, s>>>(static_cast<const int8_t*>(w), rows, cols, sums);
         return check_launch("row_sums_i8");
+    }
+
+    // weights [N][K] -> fragment order of v_mfma_i32_16x16x64_i8's B operand: the 1 KB block of
+    // (column block cb, 64-byte reduction step ks) holds, at 16 * lane, what lane (column lane % 16,
+    // chunk lane / 16) feeds the instruction: bytes ks * 64 + 16 * (lane / 16) ... of row cb * 16 +
+    // lane % 16 (zeros beyond N).  A wavefront then fetches a fragment as 1 KB of contiguous memory
+    // -- eight whole cache lines, consecutive lanes in one line -- where the row-major matrix makes
+    // consecutive lanes touch sixteen different lines.
+    __global__ __launch_bounds__(256) void pack_dot_fragments_kernel(const int8_t* __restrict__ w, int64_t N, int64_t K, v4i_t* __restrict__ frag)
+    {
+        const int64_t steps = K >> 6;
+        const int64_t total = ((N + 15) >> 4) * steps * 64;
+        int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+        const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+        for (; i < total; i += stride)
+        {
+            const int lane = static_cast<int>(i & 63);
+            const int64_t blk = i >> 6;
+            const int64_t cb = blk / steps, ks = blk - cb * steps;
+            const int64_t n = cb * 16 + (lane & 15);
+            v4i_t v = {0, 0, 0, 0};
+            if (n < N)
+                v = *reinterpret_cast<const v4i_t*>(w + n * K + ks * 64 + (lane >> 4) * 16);
+            frag[i] = v;
+        }
+    }
+
+    int launch_pack_dot_fragments(const void* w_nk, int64_t N, int64_t K, void* frag, hipStream_t s)
+    {
+        const int64_t total = ((N + 15) / 16) * (K / 64) * 64;
+        if (total == 0)
+            return HIPQ_OK;
+        const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((total + 255) / 256, 8192));
+        pack_dot_fragments_kernel<<<blocks, 256, 0, s>>>(static_cast<const int8_t*>(w_nk), N, K, static_cast<v4i_t*>(frag));
+        return check_launch("pack_dot_fragments");
     }
 
     // filter [K][C][taps] -> packed [K][taps][Cp], channels C .. Cp-1 zero

@@ -170,22 +170,34 @@ namespace hipq
         return HIPQ_OK;
     }
 
+    static int dot_pack(const hipq_dot_desc_t& d, const void* b, void* packed, bool with_fragments, hipStream_t s);
+
+    // Layout of a packed dot operand: [N][K] weights (only when the caller's are [K][N]), the column
+    // sums, and -- for products the weight-streaming kernels take -- the weights once more in MFMA
+    // fragment order.  Each part starts on a 256-byte boundary.
+    static size_t dot_blob_weights(const hipq_dot_desc_t& d) { return d.b_layout == HIPQ_B_KN ? align_up(static_cast<size_t>(d.N * d.K), 256) : 0; }
+    static size_t dot_blob_sums(const hipq_dot_desc_t& d) { return align_up(static_cast<size_t>(d.N) * sizeof(int32_t), 256); }
+
     // weights [N,K] + column sums for the MFMA dot, either prepacked or built in the workspace
-    static int dot_operands(const hipq_dot_desc_t& d, const void* b, const void* packed, const void** w, const int32_t** wsum, hipStream_t s)
+    // (built on the fly there is no fragment-ordered copy: making one costs more than it saves a call)
+    static int dot_operands(const hipq_dot_desc_t& d, const void* b, const void* packed, const void** w, const int32_t** wsum, const void** wfrag, hipStream_t s)
     {
-        const size_t wbytes = d.b_layout == HIPQ_B_KN ? align_up(static_cast<size_t>(d.N * d.K), 256) : 0;
+        const size_t wbytes = dot_blob_weights(d);
         const uint8_t* blob = static_cast<const uint8_t*>(packed);
+        *wfrag = nullptr;
         if (!blob)
         {
             uint8_t* ws = nullptr;
-            int rc = workspace(wbytes + static_cast<size_t>(d.N) * sizeof(int32_t), s, reinterpret_cast<void**>(&ws));
+            int rc = workspace(wbytes + dot_blob_sums(d), s, reinterpret_cast<void**>(&ws));
             if (rc)
                 return rc;
-            rc = hipq_dot_pack(&d, b, ws, s);
+            rc = dot_pack(d, b, ws, false, s);
             if (rc)
                 return rc;
             blob = ws;
         }
+        else if (dot_fragments_eligible(d))
+            *wfrag = blob + wbytes + dot_blob_sums(d);
         *w = d.b_layout == HIPQ_B_KN ? static_cast<const void*>(blob) : b;
         *wsum = reinterpret_cast<const int32_t*>(blob + wbytes);
         return HIPQ_OK;
@@ -207,11 +219,30 @@ namespace hipq
             (reinterpret_cast<uintptr_t>(out) & 15))
             return launch_dot_direct(d, a, b, zp, epi, out, s);
         const void* w = nullptr;
+        const void* wfrag = nullptr;
         const int32_t* wsum = nullptr;
-        int rc = dot_operands(d, b, packed, &w, &wsum, s);
+        int rc = dot_operands(d, b, packed, &w, &wsum, &wfrag, s);
         if (rc)
             return rc;
-        return launch_dot_mfma(d, a, w, wsum, zp, epi, out, s);
+        return launch_dot_mfma(d, a, w, wsum, zp, epi, out, s, wfrag);
+    }
+
+    static int dot_pack(const hipq_dot_desc_t& d, const void* b, void* packed, bool with_fragments, hipStream_t s)
+    {
+        uint8_t* blob = static_cast<uint8_t*>(packed);
+        const void* w = b;
+        const size_t wbytes = dot_blob_weights(d);
+        if (d.b_layout == HIPQ_B_KN)
+        {
+            int rc = launch_transpose(b, blob, 1, d.K, d.N, 1, s); // [K][N] -> [N][K]
+            if (rc)
+                return rc;
+            w = blob;
+        }
+        int rc = launch_row_sums_i8(w, d.N, d.K, reinterpret_cast<int32_t*>(blob + wbytes), s);
+        if (rc || !with_fragments || !dot_fragments_eligible(d))
+            return rc;
+        return launch_pack_dot_fragments(w, d.N, d.K, blob + wbytes + dot_blob_sums(d), s);
     }
 }
 
@@ -323,8 +354,7 @@ size_t hipq_dot_packed_bytes(const hipq_dot_desc_t* d)
 {
     if (!d || !dot_mfma_eligible(*d))
         return 0;
-    size_t wbytes = d->b_layout == HIPQ_B_KN ? align_up(static_cast<size_t>(d->N * d->K), 256) : 0;
-    return wbytes + static_cast<size_t>(d->N) * sizeof(int32_t);
+    return dot_blob_weights(*d) + dot_blob_sums(*d) + (dot_fragments_eligible(*d) ? dot_fragment_bytes(*d) : 0);
 }
 
 int hipq_dot_pack(const hipq_dot_desc_t* d, const void* b, void* packed, void* stream)
@@ -332,19 +362,7 @@ int hipq_dot_pack(const hipq_dot_desc_t* d, const void* b, void* packed, void* s
     HIPQ_REQUIRE(d && b && packed, "null pointer");
     if (!dot_mfma_eligible(*d))
         return fail(HIPQ_ERR_UNSUPPORTED, "shape is not eligible for the MFMA path (hipq_dot_packed_bytes is 0)");
-    hipStream_t s = as_stream(stream);
-    uint8_t* blob = static_cast<uint8_t*>(packed);
-    const void* w = b;
-    size_t wbytes = 0;
-    if (d->b_layout == HIPQ_B_KN)
-    {
-        wbytes = align_up(static_cast<size_t>(d->N * d->K), 256);
-        int rc = launch_transpose(b, blob, 1, d->K, d->N, 1, s); // [K][N] -> [N][K]
-        if (rc)
-            return rc;
-        w = blob;
-    }
-    return launch_row_sums_i8(w, d->N, d->K, reinterpret_cast<int32_t*>(blob + wbytes), s);
+    return dot_pack(*d, b, packed, true, as_stream(stream));
 }
 
 int hipq_quantized_dot(const hipq_dot_desc_t* d,
@@ -439,8 +457,9 @@ int hipq_quantized_dot_bias_gelu_quantize(const hipq_dot_desc_t* d,
     if (dot_mfma_eligible(*d) && d->M > 256 && (reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0 && (reinterpret_cast<uintptr_t>(quant->out) & 15) == 0)
     {
         const void* wn = nullptr;
+        const void* wfrag = nullptr;
         const int32_t* wsum = nullptr;
-        rc = dot_operands(*d, w, packed_w, &wn, &wsum, s);
+        rc = dot_operands(*d, w, packed_w, &wn, &wsum, &wfrag, s);
         if (rc)
             return rc;
         Epilogue post = e;

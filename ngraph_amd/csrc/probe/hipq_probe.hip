@@ -96,7 +96,7 @@ namespace
         // spread: every workgroup has a region of its own; else a start of its own inside the shared
         // window (4 KiB-aligned, scattered), so that the compute units do not walk the same L2
         // channel in step
-        const uint32_t base = spread_bytes ? static_cast<uint32_t>(blockIdx.x) * spread_bytes : (static_cast<uint32_t>(blockIdx.x) * 0x9E3779B1u) & ~0xFFFu;
+        const uint32_t base = spread_bytes == 1u ? 0u : spread_bytes ? static_cast<uint32_t>(blockIdx.x) * spread_bytes : (static_cast<uint32_t>(blockIdx.x) * 0x9E3779B1u) & ~0xFFFu;
         pv4i acc = {0, 0, 0, 0};
         if (TO_LDS)
         {
@@ -198,7 +198,7 @@ int hipq_probe_intake(const void* buf, size_t buf_bytes, size_t window_bytes, in
     if (lds_bytes < (to_lds ? 32768 : 0) || lds_bytes > 160 * 1024)
         return fail("lds_bytes out of range (loads into LDS need 32 KiB)");
     const uint32_t mask = static_cast<uint32_t>(window_bytes - 1) & ~15u;
-    const uint32_t spread_bytes = spread ? static_cast<uint32_t>(steps) * kIntakeStepBytes : 0u;
+    const uint32_t spread_bytes = spread == 2 ? 1u : spread ? static_cast<uint32_t>(steps) * kIntakeStepBytes : 0u; // 2: every workgroup walks the same addresses in step
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define HIPQ_INTAKE(SHAPE, LDS)                                                                                                                              \
     do                                                                                                                                                       \

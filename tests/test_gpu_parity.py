@@ -926,8 +926,9 @@ def test_dot_bias_config2_benchmarked_form(gpu_lib, M):
         exp = cases.dot_bias_closed_form(a, w, bias, scales, out_t, relu)
         assert np.array_equal(got, exp), (out_t, relu, kernel, int(np.sum(got != exp)))
         if out_t == "i8":
-            # the kernels bench.py's gemm_config2 entries name: weight-streaming up to 64 rows, 64 x 64 tiles with the whole reduction above
-            assert kernel == ("dot_skinny_i8_16x16x64" if M <= 64 else "dot_rows64_i8_16x16x64"), kernel
+            # the kernels bench.py's gemm_config2 entries name (prepacked weights: the fragment-ordered copy):
+            # weight-streaming up to 32 rows, 64 x 64 tiles with the whole reduction above
+            assert kernel == ("dot_skinnyf_i8_16x16x64" if M <= 32 else "dot_rows64w_i8_16x16x64"), kernel
             assert len(np.unique(exp)) > 100 and (exp == 127).any() and (exp == -128).any()
 
 
@@ -938,30 +939,48 @@ def test_dot_skinny(gpu_lib, M):
     both requantization policies, f32 output, and the exact path for a non-zero weight zero point"""
     say("dot skinny M", M)
     O.port().orc_set_threads(8)
-    for K, N in ((320, 40), (1024, 100), (256, 16)):
+
+    def kernel_of(tiles, K, prepacked):
+        # prepacked weights carry a fragment-ordered copy, which the kernels for up to 32 rows (reductions
+        # up to 4096 bytes; 8192 with at most 16 rows) and for 65-256 rows read; weights packed on the fly
+        # take the kernels that read the row-major matrix
+        if M > 64 and K >= 1024:
+            return "dot_rows64w_" if prepacked else "dot_rows64_"
+        if tiles:
+            return "dot_mfma"
+        if prepacked and (M <= 16 and K <= 8192 or M <= 32 and K <= 4096):
+            return "dot_skinnyf_"
+        return "dot_skinny_"
+
+    # (a reduction of five 64-byte steps, one that splits evenly, the shortest one, and -- for the
+    # fragment-ordered kernels -- one of two 1 KB segments a wavefront and one that leaves a wavefront
+    # a partial segment)
+    shapes = ((320, 40), (1024, 100), (256, 16)) + (((8192, 24), (2880, 20)) if M <= 32 else ())
+    for K, N in shapes:
         w = synth.uniform_int(802, (N, K), -128, 127, np.int8)
         for a_t, lo, hi in (("u8", 0, 255), ("i8", -128, 127)):
             a = synth.uniform_int(801, (M, K), lo, hi, H.NP_OF[H.dtype_code(a_t)])
-            for out_t, s, z in (("i32", (1.0, 1.0, 1.0), (0, 0, 0)), ("i8", (0.01, 0.01, 2.5), (5 if a_t == "u8" else -5, 0, 4)), ("u8", (0.01, 0.01, 2.5), (0, 3, 9))):
-                d = H.make_dot_desc(M, K, N, a_t=a_t, out_t=out_t, b_layout=H.B_NK)
-                exp = O.quantized_dot(d, a, w, s[0], z[0], s[1], z[1], s[2], z[2])
-                got = H.quantized_dot(d, a, w, s[0], z[0], s[1], z[1], s[2], z[2])
-                # (more than 64 rows with an 8-bit output in whole 16-byte rows go to the tile kernels)
-                tiles = M > 64 and out_t != "i32" and N % 16 == 0
-                rows64 = M > 64 and K >= 1024
-                assert H.last_kernel().startswith("dot_rows64" if rows64 else "dot_mfma" if tiles else "dot_skinny"), H.last_kernel()
-                assert np.array_equal(got, exp), (K, N, a_t, out_t, z)
-            bias = synth.uniform_int(803, (N,), -(2**15), 2**15, np.int32)
-            scales = synth.uniform_f32(804, (N,), 0.001, 0.01) * np.float32(0.05)
-            for out_t, relu in (("i8", False), ("u8", True), ("f32", True)):
-                d = H.make_dot_desc(M, K, N, a_t=a_t, out_t=out_t, b_layout=H.B_NK)
-                f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
-                exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
-                got = H.quantized_dot_bias(d, f, a, w, bias, scales)
-                tiles = M > 64 and N % 16 == 0
-                rows64 = M > 64 and K >= 1024
-                assert H.last_kernel().startswith("dot_rows64" if rows64 else "dot_mfma" if tiles else "dot_skinny"), H.last_kernel()
-                assert np.array_equal(got, exp), (K, N, a_t, out_t, relu)
+            for prepacked in (True, False):
+                if not prepacked and K > 1024:
+                    continue
+                for out_t, s, z in (("i32", (1.0, 1.0, 1.0), (0, 0, 0)), ("i8", (0.01, 0.01, 2.5), (5 if a_t == "u8" else -5, 0, 4)), ("u8", (0.01, 0.01, 2.5), (0, 3, 9))):
+                    d = H.make_dot_desc(M, K, N, a_t=a_t, out_t=out_t, b_layout=H.B_NK)
+                    exp = O.quantized_dot(d, a, w, s[0], z[0], s[1], z[1], s[2], z[2])
+                    got = H.quantized_dot(d, a, w, s[0], z[0], s[1], z[1], s[2], z[2], prepare=prepacked)
+                    # (more than 64 rows with an 8-bit output in whole 16-byte rows go to the tile kernels)
+                    want = kernel_of(M > 64 and out_t != "i32" and N % 16 == 0, K, prepacked)
+                    assert H.last_kernel().startswith(want), (H.last_kernel(), want)
+                    assert np.array_equal(got, exp), (K, N, a_t, out_t, z, prepacked)
+                bias = synth.uniform_int(803, (N,), -(2**15), 2**15, np.int32)
+                scales = synth.uniform_f32(804, (N,), 0.001, 0.01) * np.float32(0.05)
+                for out_t, relu in (("i8", False), ("u8", True), ("f32", True)):
+                    d = H.make_dot_desc(M, K, N, a_t=a_t, out_t=out_t, b_layout=H.B_NK)
+                    f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
+                    exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
+                    got = H.quantized_dot_bias(d, f, a, w, bias, scales, prepare=prepacked)
+                    want = kernel_of(M > 64 and N % 16 == 0, K, prepacked)
+                    assert H.last_kernel().startswith(want), (H.last_kernel(), want)
+                    assert np.array_equal(got, exp), (K, N, a_t, out_t, relu, prepacked)
     O.port().orc_set_threads(1)
 
 
@@ -1011,9 +1030,10 @@ def test_mfma_requant_ties(gpu_lib):
         assert np.array_equal(H.quantized_dot(d, a, w, s, 0, 1.0, 0, 1.0, 5), O.quantized_dot(d, a, w, s, 0, 1.0, 0, 1.0, 5)), s
 
 
-@pytest.mark.parametrize("shape", [(65, 1088, 64), (200, 1152, 130), (256, 2048, 48), (129, 1024, 1000), (192, 3008, 200)])
+@pytest.mark.parametrize("shape", [(65, 1088, 64), (200, 1152, 130), (256, 2048, 48), (129, 1024, 1000), (192, 3008, 200), (72, 4096, 40), (130, 4160, 72)])
 def test_dot_rows64(gpu_lib, shape):
-    """the whole-reduction kernel for 65-256 rows: ragged row and column tiles, reductions that end in
+    """the whole-reduction kernels for 65-256 rows (prepacked weights: the one that reads their
+    fragment-ordered copy; weights packed on the fly: the one that reads the row-major matrix): ragged row and column tiles, reductions that end in
     half a 128-byte piece (K % 128 == 64) or leave wavefronts without a piece, signed and unsigned
     data with zero points, both requantization policies, every output type, and the exact path for a
     non-zero weight zero point"""
@@ -1026,18 +1046,20 @@ def test_dot_rows64(gpu_lib, shape):
         for out_t, s, z in (("i32", (1.0, 1.0, 1.0), (0, 0, 0)), ("i8", (0.01, 0.01, 2.5), (5 if a_t == "u8" else -5, 0, 4)), ("u8", (0.01, 0.01, 2.5), (0, 3, 9))):
             d = H.make_dot_desc(M, K, N, a_t=a_t, out_t=out_t, b_layout=H.B_NK)
             exp = O.quantized_dot(d, a, w, s[0], z[0], s[1], z[1], s[2], z[2])
-            got = H.quantized_dot(d, a, w, s[0], z[0], s[1], z[1], s[2], z[2])
-            assert H.last_kernel().startswith("dot_rows64"), H.last_kernel()
-            assert np.array_equal(got, exp), (a_t, out_t, z)
+            for prepacked, name in ((True, "dot_rows64w_" if K <= 4096 else "dot_rows64_"), (False, "dot_rows64_")):  # (the fragment-ordered kernel holds a reduction of 4096 bytes in registers)
+                got = H.quantized_dot(d, a, w, s[0], z[0], s[1], z[1], s[2], z[2], prepare=prepacked)
+                assert H.last_kernel().startswith(name), H.last_kernel()
+                assert np.array_equal(got, exp), (a_t, out_t, z, prepacked)
         bias = synth.uniform_int(1503, (N,), -(2**15), 2**15, np.int32)
         scales = synth.uniform_f32(1504, (N,), 0.001, 0.01) * np.float32(0.05)
         for out_t, relu in (("i8", False), ("u8", True), ("f32", True)):
             d = H.make_dot_desc(M, K, N, a_t=a_t, out_t=out_t, b_layout=H.B_NK)
             f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
             exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
-            got = H.quantized_dot_bias(d, f, a, w, bias, scales)
-            assert H.last_kernel().startswith("dot_rows64"), H.last_kernel()
-            assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), (a_t, out_t, relu)
+            for prepacked, name in ((True, "dot_rows64w_" if K <= 4096 else "dot_rows64_"), (False, "dot_rows64_")):  # (the fragment-ordered kernel holds a reduction of 4096 bytes in registers)
+                got = H.quantized_dot_bias(d, f, a, w, bias, scales, prepare=prepacked)
+                assert H.last_kernel().startswith(name), H.last_kernel()
+                assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), (a_t, out_t, relu, prepacked)
     O.port().orc_set_threads(1)
 
 

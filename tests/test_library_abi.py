@@ -100,10 +100,13 @@ def test_packed_sizes_and_eligibility():
     assert lib.hipq_conv_packed_filter_bytes(C.byref(d40)) == 0
     du = H.make_conv_desc(1, 64, 64, (8, 8), (1, 1), filter_t="u8", out_t="u8")
     assert lib.hipq_conv_packed_filter_bytes(C.byref(du)) == 0
+    # column sums, plus (up to 256 rows, reductions in whole 64-byte steps) the weights once more in fragment order
     dd = H.make_dot_desc(32, 4096, 4096, b_layout=H.B_NK)
-    assert lib.hipq_dot_packed_bytes(C.byref(dd)) == 4096 * 4
+    assert lib.hipq_dot_packed_bytes(C.byref(dd)) == 4096 * 4 + 4096 * 4096
     dk = H.make_dot_desc(32, 4096, 4096, b_layout=H.B_KN)
-    assert lib.hipq_dot_packed_bytes(C.byref(dk)) == 4096 * 4096 + 4096 * 4
+    assert lib.hipq_dot_packed_bytes(C.byref(dk)) == 4096 * 4096 + 4096 * 4 + 4096 * 4096
+    assert lib.hipq_dot_packed_bytes(C.byref(H.make_dot_desc(512, 4096, 4096, b_layout=H.B_NK))) == 4096 * 4
+    assert lib.hipq_dot_packed_bytes(C.byref(H.make_dot_desc(32, 4000, 100, b_layout=H.B_NK))) == 512  # 100 sums, padded to 256 bytes
     assert lib.hipq_dot_packed_bytes(C.byref(H.make_dot_desc(1, 30, 8))) == 0
 
 

@@ -429,6 +429,27 @@ def bench_backend(calls=100, warmup=10):
                          "host stopwatch around the calls; a call returns when its results are in the output tensors" % (warmup, calls), rows=rows)
 
 
+def bench_launch_floor(lib, stream, timer, launches=(58, 85)):
+    """What a pass of n dependent launches costs before any of them computes: n launches in a row of a
+    kernel that does nothing (256 workgroups; and 1 workgroup), eagerly and replayed as one HIP graph.
+    58 = the launches of a ResNet-50 pass, 85 = of a BERT-base pass."""
+    probe = H.load_probe()
+    sink = H.DeviceBuffer(65536 * 4)
+    out = []
+    for n in launches:
+        for wgs in (1, 256):
+            def chain():
+                H.check_probe(probe.hipq_probe_empty_chain(sink.ptr, n, wgs, 1, stream))
+
+            _, eager = timer.run(chain, 20, 3)
+            replay = H.GraphReplay(lib, stream, chain)
+            replay.capture()
+            _, graph = timer.run(replay.replay, 20, 3)
+            replay.close()
+            out.append(dict(launches=n, workgroups=wgs, ms_eager=eager, ms_graph=graph, us_per_launch_eager=eager * 1e3 / n, us_per_launch_graph=graph * 1e3 / n))
+    return out
+
+
 def under_profiler():
     """rocprofv3 (and its predecessors) announce themselves in the environment of the program they run"""
     pre = os.environ.get("LD_PRELOAD", "")
@@ -611,7 +632,8 @@ def main():
         print(json.dumps({"quantize_dequantize_config3": bench_qdq(lib, stream, timer, args.steps, args.warmup), "copy_calibration": copy_calibration(lib, stream, timer)}))
         return
     if args.only == "intake":
-        print(json.dumps({"l2_intake_per_cu": bench_intake(lib, stream, timer, info.compute_units), "atomic_tiles": bench_atomic_tiles(lib, stream, timer, info.compute_units)}))
+        print(json.dumps({"l2_intake_per_cu": bench_intake(lib, stream, timer, info.compute_units), "atomic_tiles": bench_atomic_tiles(lib, stream, timer, info.compute_units),
+                          "launch_floor": bench_launch_floor(lib, stream, timer)}))
         return
     if args.only == "glue":
         print(json.dumps({"fp32_glue": bench_fp32_glue(lib, stream, timer, args.steps, args.warmup), "copy_calibration": copy_calibration(lib, stream, timer)}))
@@ -649,6 +671,7 @@ def main():
         results["pool_resnet50_u8"] = bench_pool(lib, stream, timer, small, 5, args.batch)
         results["glue_resnet50_u8"] = bench_glue(lib, stream, timer, small, 5, args.batch)
         results["fp32_glue_bert_base"] = bench_fp32_glue(lib, stream, timer, small, 5)
+        results["launch_floor"] = bench_launch_floor(lib, stream, timer)
         if not args.skip_models:
             results["bert_base_int8"] = bench_bert(lib, stream, timer, use_graph=not args.no_graph)
             results["resnet50_int8"] = bench_resnet50(lib, stream, timer, use_graph=not args.no_graph)

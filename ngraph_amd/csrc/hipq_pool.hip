@@ -189,20 +189,43 @@ namespace hipq
         window_range(o0, g.st[0], g.pb[0], g.win[0], g.in[0], lo0, hi0);
         window_range(o1, g.st[1], g.pb[1], g.win[1], g.in[1], lo1, hi1);
         window_range(o2, g.st[2], g.pb[2], g.win[2], g.in[2], lo2, hi2);
+        // The cells of the two inner window axes are fetched kBatch at a time, all loads of a batch in
+        // flight together: a loop that loads a cell, waits and reduces pays one memory latency a cell
+        // (49 in a row for a 7 x 7 average).  A slot past the window's end holds the reduction's
+        // identity (the byte pattern whose biased form is zero).
+        constexpr int kBatch = VEC == 4 ? 8 : 16;
         Bytes4<AVG> acc[VEC];
+        const int span2 = hi2 - lo2;
+        const int cells = (hi1 - lo1) * span2;
         for (int w0 = lo0; w0 < hi0; ++w0)
-            for (int w1 = lo1; w1 < hi1; ++w1)
+        {
+            const size_t plane = static_cast<size_t>(n) * g.in[0] + (o0 * g.st[0] - g.pb[0] + w0);
+            int r = lo1, c = lo2; // cell (r, c) is slot `first` of the next batch
+            for (int first = 0; first < cells; first += kBatch)
             {
-                const size_t line = (static_cast<size_t>(n) * g.in[0] + (o0 * g.st[0] - g.pb[0] + w0)) * g.in[1] + (o1 * g.st[1] - g.pb[1] + w1);
-                const vec_t* p = reinterpret_cast<const vec_t*>(in) + (line * g.in[2] + (o2 * g.st[2] - g.pb[2] + lo2)) * groups + cg;
-                for (int w2 = lo2; w2 < hi2; ++w2, p += groups)
+                vec_t v[kBatch];
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u)
                 {
-                    const vec_t v = *p;
+                    const bool in_window = first + u < cells;
+                    const size_t line = plane * g.in[1] + (o1 * g.st[1] - g.pb[1] + r);
+                    const vec_t* p = reinterpret_cast<const vec_t*>(in) + (line * g.in[2] + (o2 * g.st[2] - g.pb[2] + c)) * groups + cg;
+                    vec_t ident;
 #pragma unroll
                     for (int j = 0; j < VEC; ++j)
-                        acc[j].add(v[j] ^ bias);
+                        ident[j] = bias;
+                    v[u] = in_window ? *p : ident;
+                    const bool wrap = c + 1 == hi2;
+                    c = wrap ? lo2 : c + 1;
+                    r += (wrap && in_window) ? 1 : 0; // (a row past the window is never formed: its address would lie outside the tensor)
                 }
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u)
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j)
+                        acc[j].add(v[u][j] ^ bias);
             }
+        }
         vec_t r;
         if (AVG)
         {

@@ -50,6 +50,12 @@ HIPQ_PROBE_API int hipq_probe_intake(const void* buf, size_t buf_bytes, size_t w
  * `dst`: workgroups / share x rounds tiles of 64 KiB, zeroed by the caller. */
 HIPQ_PROBE_API int hipq_probe_atomic_tiles(void* dst, size_t dst_bytes, int32_t workgroups, int32_t share, int32_t same_die, int32_t rounds, void* stream);
 
+/* The floor under a sequence of dependent launches: `kernels` launches in a row on `stream` of a
+ * kernel that does nothing (`workgroups` workgroups of 256 lanes; touch != 0: lane 0 of each writes a
+ * word of `sink`, workgroups ints).  Timed eagerly and as a replayed graph it says what a pass of that
+ * many launches costs before any of them computes anything. */
+HIPQ_PROBE_API int hipq_probe_empty_chain(void* sink, int32_t kernels, int32_t workgroups, int32_t touch, void* stream);
+
 /* host-only: n / d by the multiply-shift the Quantize kernels use for their scale index
  * (0 <= n < 2^31, 1 <= d < 2^31) */
 HIPQ_PROBE_API uint32_t hipq_debug_fastdiv(uint32_t n, uint32_t d);

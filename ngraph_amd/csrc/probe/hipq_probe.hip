@@ -139,6 +139,13 @@ namespace
         sink[blockIdx.x * 256 + threadIdx.x] = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
     }
 
+    // a kernel that does nothing but exist: `touch` != 0 makes lane 0 of every workgroup write one word
+    __global__ __launch_bounds__(256) void probe_empty_kernel(int* __restrict__ sink, int touch)
+    {
+        if (touch && threadIdx.x == 0)
+            sink[blockIdx.x] = touch;
+    }
+
     // a workgroup of 256 lanes holds a 128 x 128 int32 tile as 64 values a lane; value j of lane t is
     // element j * 256 + t of the tile (a wavefront instruction covers 256 contiguous bytes)
     __global__ __launch_bounds__(256) void probe_atomic_tiles_kernel(int* __restrict__ dst, int share, int same_die, int rounds, int groups)
@@ -244,6 +251,15 @@ int hipq_probe_atomic_tiles(void* dst, size_t dst_bytes, int32_t workgroups, int
         return fail("destination holds fewer than %d x %d tiles of 64 KiB", groups, rounds);
     probe_atomic_tiles_kernel<<<static_cast<unsigned>(workgroups), 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<int*>(dst), share, same_die, rounds, groups);
     return check_launch("probe_atomic_tiles");
+}
+
+int hipq_probe_empty_chain(void* sink, int32_t kernels, int32_t workgroups, int32_t touch, void* stream)
+{
+    if (!sink || kernels <= 0 || kernels > 4096 || workgroups <= 0 || workgroups > 65535)
+        return fail("kernels / workgroups out of range");
+    for (int i = 0; i < kernels; ++i)
+        probe_empty_kernel<<<static_cast<unsigned>(workgroups), 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<int*>(sink), touch);
+    return check_launch("probe_empty");
 }
 
 uint32_t hipq_debug_fastdiv(uint32_t n, uint32_t d)

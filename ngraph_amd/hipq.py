@@ -356,6 +356,7 @@ def load_probe():
     lib.hipq_probe_mfma_i8.argtypes = [vp, vp, i32, i32, vp]
     lib.hipq_probe_intake.argtypes = [vp, sz, sz, i32, i32, i32, i32, i32, i32, vp, vp]
     lib.hipq_probe_atomic_tiles.argtypes = [vp, sz, i32, i32, i32, i32, vp]
+    lib.hipq_probe_empty_chain.argtypes = [vp, i32, i32, i32, vp]
     lib.hipq_debug_fastdiv.restype = C.c_uint32
     lib.hipq_debug_fastdiv.argtypes = [C.c_uint32] * 2
     _probe = lib

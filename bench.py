@@ -354,7 +354,8 @@ def mfma_ceiling(lib, stream, timer, compute_units):
 def bench_intake(lib, stream, timer, compute_units):
     """What a compute unit takes in: 1 / 2 / 4 workgroups of four wavefronts a compute unit (by their LDS
     allocation) each read 8 MiB in 16-byte pieces -- a wavefront instruction covering 1 KiB contiguous,
-    8 rows x 128 bytes or 16 rows x 64 bytes (rows 4096 bytes apart) -- into registers or straight into
+    8 rows x 128 bytes, 16 rows x 64 bytes (rows 4096 bytes apart) or 64 rows x 16 bytes (every lane in
+    a cache line of its own, rows 1024 bytes apart) -- into registers or straight into
     LDS, out of a 2 MiB window (served by the L2s after the first pass) or out of 2 GiB with a region
     per workgroup (served by HBM).  No division in the address stream; the launch is below 2 % of a sample."""
     probe = H.load_probe()
@@ -365,10 +366,10 @@ def bench_intake(lib, stream, timer, compute_units):
     sink = H.DeviceBuffer(4 * cus * 256 * 4)
     steps = 256  # x 32 KiB = 8 MiB a workgroup
     out = []
-    shapes = {0: "1024 B contiguous", 1: "8 rows x 128 B", 2: "16 rows x 64 B"}
+    shapes = {0: "1024 B contiguous", 1: "8 rows x 128 B", 2: "16 rows x 64 B", 3: "64 rows x 16 B"}
     for source, window, spread in (("l2", 2 << 20, 0), ("hbm", total, 1)):
         for to_lds in (0, 1):
-            for shape in (0, 1, 2):
+            for shape in (0, 1, 2, 3):
                 for per_cu in (1, 2, 4):
                     wgs = cus * per_cu
                     lds_bytes = {1: 160 * 1024, 2: 80 * 1024, 4: 40 * 1024}[per_cu]

@@ -35,6 +35,8 @@ HIPQ_PROBE_API int hipq_probe_mfma_i8(const void* operands_8k, void* sink, int32
  *   shape 0: a wavefront instruction covers 1024 contiguous bytes
  *   shape 1: 8 rows x 128 bytes (rows `pitch` = 4096 bytes apart: whole cache lines)
  *   shape 2: 16 rows x 64 bytes (half lines)
+ *   shape 3: 64 rows x 16 bytes, rows 1024 bytes apart (every lane in a line of its own: the MFMA
+ *            fragment read of a row-major matrix)
  *   to_lds 0: into registers (xor-reduced into `sink`); 1: straight into LDS (buffer_load ... lds)
  * Addresses wrap inside `window_bytes` (a power of two >= 1 MiB): a window of a few MiB is served
  * by the L2s after the first pass, a window of GiBs with `spread` != 0 (every workgroup starts

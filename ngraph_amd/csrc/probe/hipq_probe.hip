@@ -73,17 +73,19 @@ namespace
     {
         if (SHAPE == 0) // 1 KiB contiguous an instruction, a step is 32 KiB contiguous
             return base + step * kIntakeStepBytes + static_cast<uint32_t>((wave * kIntakeLoads + u) * 1024 + lane * 16);
-        // row pieces out of rows 4096 bytes apart: a workgroup's step is a block of 256 (128-byte
-        // pieces) or 512 (64-byte pieces) rows at one column; 32 (64) steps sweep the 4096 columns,
-        // then the block moves on by its rows
-        constexpr int PIECE = SHAPE == 1 ? 128 : 64;
+        // row pieces out of rows kPitch bytes apart: a workgroup's step is a block of 256 (128-byte
+        // pieces), 512 (64-byte pieces) or 2048 (16-byte pieces: every lane in a line of its own,
+        // what a wavefront reading MFMA fragments out of a row-major matrix does) rows at one column;
+        // the steps sweep the columns of a row, then the block moves on by its rows
+        constexpr int PIECE = SHAPE == 1 ? 128 : SHAPE == 2 ? 64 : 16;
+        constexpr uint32_t kPitch = SHAPE == 3 ? 1024u : 4096u;
         constexpr int LANES = PIECE / 16;      // lanes a row piece
         constexpr int ROWS = 64 / LANES;       // rows an instruction
         constexpr int BLOCK_ROWS = 4 * kIntakeLoads * ROWS;
-        constexpr int SWEEP = 4096 / PIECE;    // steps until the columns wrap (a power of two)
+        constexpr int SWEEP = kPitch / PIECE;  // steps until the columns wrap (a power of two)
         const uint32_t row = static_cast<uint32_t>((wave * kIntakeLoads + u) * ROWS + lane / LANES);
         const uint32_t col = (step & (SWEEP - 1)) * PIECE + static_cast<uint32_t>(lane % LANES) * 16;
-        return base + (step / SWEEP) * (BLOCK_ROWS * 4096u) + row * 4096u + col;
+        return base + (step / SWEEP) * (BLOCK_ROWS * kPitch) + row * kPitch + col;
     }
 
     template <int SHAPE, bool TO_LDS>
@@ -200,7 +202,7 @@ int hipq_probe_intake(const void* buf, size_t buf_bytes, size_t window_bytes, in
         return fail("buffer must be 16-byte aligned");
     if (window_bytes < (1u << 20) || (window_bytes & (window_bytes - 1)) != 0 || window_bytes > buf_bytes || buf_bytes > 0xFFFFFFFFull)
         return fail("window must be a power of two of at least 1 MiB inside a buffer below 4 GiB");
-    if (shape < 0 || shape > 2 || workgroups <= 0 || workgroups > 65535 || steps <= 0 || steps > (1 << 20))
+    if (shape < 0 || shape > 3 || workgroups <= 0 || workgroups > 65535 || steps <= 0 || steps > (1 << 20))
         return fail("shape / workgroups / steps out of range");
     if (lds_bytes < (to_lds ? 32768 : 0) || lds_bytes > 160 * 1024)
         return fail("lds_bytes out of range (loads into LDS need 32 KiB)");
@@ -222,8 +224,10 @@ int hipq_probe_intake(const void* buf, size_t buf_bytes, size_t window_bytes, in
             HIPQ_INTAKE(0, true);
         else if (shape == 1)
             HIPQ_INTAKE(1, true);
-        else
+        else if (shape == 2)
             HIPQ_INTAKE(2, true);
+        else
+            HIPQ_INTAKE(3, true);
     }
     else
     {
@@ -231,8 +235,10 @@ int hipq_probe_intake(const void* buf, size_t buf_bytes, size_t window_bytes, in
             HIPQ_INTAKE(0, false);
         else if (shape == 1)
             HIPQ_INTAKE(1, false);
-        else
+        else if (shape == 2)
             HIPQ_INTAKE(2, false);
+        else
+            HIPQ_INTAKE(3, false);
     }
 #undef HIPQ_INTAKE
     return check_launch("probe_intake");

@@ -500,6 +500,29 @@ typedef struct
 HIPQ_API int hipq_pool_infer_output(hipq_pool_desc_t* desc);
 HIPQ_API int hipq_pool(const hipq_pool_desc_t* desc, const void* in, void* out, void* stream);
 
+/*
+ * MaxPool(QuantizedConvolutionBias(...)) in one launch, for the pairs a first layer makes: the
+ * convolution is the one hipq_quantized_convolution_fused would run with these descriptors (no
+ * residual input; src/ngraph/runtime/cpu/builder/quantized_conv.cpp:332-766), the pool the one
+ * hipq_pool would run over its result (src/ngraph/runtime/reference/max_pool.hpp:127-222); `out`
+ * is the pooled tensor and the convolution's own result is never written.  The bytes equal the two
+ * calls'.  Eligible pairs (hipq_conv_max_pool_fusable returns 1): [N][C][H][W] u8 / i8 data with at
+ * most four channels and a width that is a multiple of four, 64 output channels, a filter of up to
+ * 8 x 8 taps with a column stride of two, u8 channels-last output, a pool window of up to 3 x 3.
+ * `packed_filter` is required (hipq_conv_pack_filter); `data` must be 4-byte aligned.
+ * HIPQ_ERR_UNSUPPORTED for any other pair: the caller then makes the two calls.
+ */
+HIPQ_API int hipq_conv_max_pool_fusable(const hipq_conv_desc_t* desc, const hipq_fused_desc_t* fused, const hipq_pool_desc_t* pool);
+HIPQ_API int hipq_quantized_convolution_fused_max_pool(const hipq_conv_desc_t* desc,
+                                                       const hipq_fused_desc_t* fused,
+                                                       const hipq_pool_desc_t* pool,
+                                                       const void* data,
+                                                       const void* packed_filter,
+                                                       const int32_t* bias,
+                                                       const float* scale,
+                                                       void* out,
+                                                       void* stream);
+
 /* op::v0::Concat (src/ngraph/runtime/reference/concat.hpp): piece i is [outer][extent[i]][inner]
  * elements, the result [outer][sum extent][inner]; `inputs` and `extents` are host arrays of
  * device pointers / axis extents. */

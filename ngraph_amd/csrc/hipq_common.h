@@ -283,6 +283,17 @@ namespace hipq
     bool conv_rowpack_eligible(const ConvGeom& g, RowPack* rp);
     int launch_stage_rows(const ConvGeom& g, const RowPack& rp, const void* in, void* staged, const void* zp, int zp_t, hipStream_t s);
     int launch_conv_rowpack(const ConvGeom& g, const RowPack& rp, const void* staged, const void* packed, const ZeroPoints& zp, const Epilogue& epi, void* out, hipStream_t s);
+    // first layers with 64 output channels and a stride of two along the rows of pixels, fused
+    // policy, u8 output: the band kernel that reads [N][C][H][W] bytes itself, and optionally reduces
+    // a MaxPool over its own output before anything is written (hipq_conv_stem.hip)
+    struct PoolFuse
+    {
+        int64_t wh, ww, sh, sw; // window, strides
+        int64_t pt, pl;         // padding above / left
+        int64_t out_h, out_w;   // extent of the pooled result
+    };
+    bool conv_stem_eligible(const ConvGeom& g, const Epilogue& epi, const ZeroPoints& zp, const PoolFuse* pool);
+    int launch_conv_stem(const ConvGeom& g, const void* data, const void* packed, const ZeroPoints& zp, const Epilogue& epi, const PoolFuse* pool, void* out, hipStream_t s);
     int launch_row_sums_i8(const void* w, int64_t rows, int64_t cols, int32_t* sums, hipStream_t s);
     // [N][K] weights in the fragment order of v_mfma_i32_16x16x64_i8 (K a multiple of 64): ceil(N / 16) * K / 64 blocks of 1 KB
     int launch_pack_dot_fragments(const void* w_nk, int64_t N, int64_t K, void* frag, hipStream_t s);

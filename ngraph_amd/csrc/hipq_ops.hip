@@ -35,6 +35,9 @@ namespace hipq
     {
         // the MFMA kernels have no fused-policy instantiation with int32 output (no nGraph op asks for one)
         RowPack rp;
+        // a first layer the band kernel takes whole: it reads the [N][C][H][W] bytes itself
+        if (packed && (reinterpret_cast<uintptr_t>(data) & 3) == 0 && conv_rowpack_eligible(g, &rp) && conv_stem_eligible(g, epi, zp, nullptr))
+            return launch_conv_stem(g, data, packed, zp, epi, nullptr, out, s);
         if (packed && conv_rowpack_eligible(g, &rp))
         {
             // a first layer's three or four channels: a copy with the padding materialised, whose
@@ -348,6 +351,76 @@ int hipq_quantized_convolution_fused(const hipq_conv_desc_t* desc,
         return rc;
     ZeroPoints zp{nullptr, nullptr, g.data_t, g.filter_t};
     return run_conv(g, data, filter, packed_filter, zp, e, out, as_stream(stream));
+}
+
+// MaxPool over the output of a fused convolution, as the pair of descriptors the two calls would take
+static int conv_pool_pair(const hipq_conv_desc_t* desc, const hipq_fused_desc_t* fused, const hipq_pool_desc_t* pool, ConvGeom* g, PoolFuse* pf)
+{
+    int rc = make_geom(desc, g);
+    if (rc)
+        return rc;
+    rc = check_conv_types(*g, true);
+    if (rc)
+        return rc;
+    HIPQ_REQUIRE(fused && pool, "descriptor is null");
+    if (g->in[0] != 1 || pool->op != HIPQ_POOL_MAX || pool->n_spatial != 2 || desc->n_spatial != 2 || pool->dtype != g->out_t || pool->layout != g->out_layout || pool->N != g->N ||
+        pool->C != g->K || pool->in_sp[0] != g->out[1] || pool->in_sp[1] != g->out[2] || fused->has_sum)
+        return fail(HIPQ_ERR_UNSUPPORTED, "not a 2-D MaxPool over this convolution's output");
+    hipq_pool_desc_t pd = *pool;
+    rc = hipq_pool_infer_output(&pd);
+    if (rc)
+        return rc;
+    pf->wh = pool->window[0];
+    pf->ww = pool->window[1];
+    pf->sh = pool->stride[0];
+    pf->sw = pool->stride[1];
+    pf->pt = pool->pad_below[0];
+    pf->pl = pool->pad_below[1];
+    pf->out_h = pd.out_sp[0];
+    pf->out_w = pd.out_sp[1];
+    return HIPQ_OK;
+}
+
+int hipq_conv_max_pool_fusable(const hipq_conv_desc_t* desc, const hipq_fused_desc_t* fused, const hipq_pool_desc_t* pool)
+{
+    ConvGeom g;
+    PoolFuse pf;
+    if (!desc || !fused || !pool || conv_pool_pair(desc, fused, pool, &g, &pf) != HIPQ_OK)
+        return 0;
+    Epilogue e;
+    memset(&e, 0, sizeof(e));
+    e.mode = EPI_FUSED;
+    e.out_t = g.out_t;
+    ZeroPoints zp{nullptr, nullptr, g.data_t, g.filter_t};
+    RowPack rp;
+    return conv_rowpack_eligible(g, &rp) && conv_stem_eligible(g, e, zp, &pf) ? 1 : 0;
+}
+
+int hipq_quantized_convolution_fused_max_pool(const hipq_conv_desc_t* desc,
+                                              const hipq_fused_desc_t* fused,
+                                              const hipq_pool_desc_t* pool,
+                                              const void* data,
+                                              const void* packed_filter,
+                                              const int32_t* bias,
+                                              const float* scale,
+                                              void* out,
+                                              void* stream)
+{
+    ConvGeom g;
+    PoolFuse pf;
+    int rc = conv_pool_pair(desc, fused, pool, &g, &pf);
+    if (rc)
+        return rc;
+    HIPQ_REQUIRE(data && packed_filter && out, "null tensor pointer");
+    Epilogue e;
+    rc = fused_epilogue(fused, g.out_t, g.K, bias, nullptr, scale, nullptr, &e);
+    if (rc)
+        return rc;
+    ZeroPoints zp{nullptr, nullptr, g.data_t, g.filter_t};
+    RowPack rp;
+    if (!conv_rowpack_eligible(g, &rp) || !conv_stem_eligible(g, e, zp, &pf))
+        return fail(HIPQ_ERR_UNSUPPORTED, "this convolution / MaxPool pair has no fused kernel (hipq_conv_max_pool_fusable is 0)");
+    return launch_conv_stem(g, data, packed_filter, zp, e, &pf, out, as_stream(stream));
 }
 
 size_t hipq_dot_packed_bytes(const hipq_dot_desc_t* d)

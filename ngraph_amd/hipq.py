@@ -300,6 +300,8 @@ EXPORTS = [
     "hipq_quantized_convolution",
     "hipq_quantized_convolution_noalloc",
     "hipq_quantized_convolution_fused",
+    "hipq_conv_max_pool_fusable",
+    "hipq_quantized_convolution_fused_max_pool",
     "hipq_dot_packed_bytes",
     "hipq_dot_pack",
     "hipq_quantized_dot",
@@ -407,6 +409,8 @@ def load():
     lib.hipq_quantized_convolution.argtypes = [C.POINTER(ConvDesc)] + [vp] * 11
     lib.hipq_quantized_convolution_noalloc.argtypes = [C.POINTER(ConvDesc)] + [vp] * 11
     lib.hipq_quantized_convolution_fused.argtypes = [C.POINTER(ConvDesc), C.POINTER(FusedDesc)] + [vp] * 9
+    lib.hipq_conv_max_pool_fusable.argtypes = [C.POINTER(ConvDesc), C.POINTER(FusedDesc), C.POINTER(PoolDesc)]
+    lib.hipq_quantized_convolution_fused_max_pool.argtypes = [C.POINTER(ConvDesc), C.POINTER(FusedDesc), C.POINTER(PoolDesc)] + [vp] * 6
     lib.hipq_dot_packed_bytes.restype = C.c_size_t
     lib.hipq_dot_packed_bytes.argtypes = [C.POINTER(DotDesc)]
     lib.hipq_dot_pack.argtypes = [C.POINTER(DotDesc), vp, vp, vp]
@@ -568,6 +572,24 @@ def quantized_convolution_fused(desc, fused, data, filt, bias, sum_in, scale, su
             C.byref(desc), C.byref(fused), bd.ptr, bf.ptr, _p(packed), _p(bb), _p(bsum), bsc.ptr, _p(bss), out.ptr, None
         )
     )
+    check(lib.hipq_stream_sync(None))
+    return out.to_numpy(NP_OF[desc.out_t], oshape)
+
+
+def conv_max_pool_fusable(desc, fused, pool_desc) -> bool:
+    return bool(load().hipq_conv_max_pool_fusable(C.byref(desc), C.byref(fused), C.byref(pool_desc)))
+
+
+def quantized_convolution_fused_max_pool(desc, fused, pool_desc, data, filt, bias, scale):
+    """MaxPool(fused convolution) in one launch; raises HipqError (UNSUPPORTED) for pairs without a fused kernel"""
+    lib = load()
+    bd, bf = _dev(data), _dev(filt)
+    packed = pack_filter(desc, bf)
+    bb = _dev(None if bias is None else np.asarray(bias, dtype=np.int32))
+    bsc = _dev(np.asarray(scale, dtype=np.float32))
+    oshape = pool_desc.out_shape()
+    out = DeviceBuffer(int(np.prod(oshape)) * np.dtype(NP_OF[desc.out_t]).itemsize)
+    check(lib.hipq_quantized_convolution_fused_max_pool(C.byref(desc), C.byref(fused), C.byref(pool_desc), bd.ptr, _p(packed), _p(bb), bsc.ptr, out.ptr, None))
     check(lib.hipq_stream_sync(None))
     return out.to_numpy(NP_OF[desc.out_t], oshape)
 

@@ -61,6 +61,10 @@ namespace hipq
             // pool (window wh x ww, strides, padding above / left) and its result's extent
             int32_t PH, PW, wh, ww, psh, psw, ppt, ppl;
             FastDiv by_pw;
+            // epilogue (fused policy, u8 output): bias may be null
+            const int32_t* bias;
+            const float* scale;
+            int32_t per_channel, relu;
         };
 
         // byte-wise unsigned maximum of dwords: even and odd bytes in 16-bit lanes (the low byte of
@@ -83,7 +87,7 @@ namespace hipq
         // rows past R weigh zero and read LDS rows the band holds for that purpose)
         // UNIT: bytes a lane stages per load (16 when the image rows are whole 16-byte pieces, else 4)
         template <bool POOL, int KS, int UNIT>
-        __global__ __launch_bounds__(kStemThreads) void conv_stem_kernel(const StemParams p, const Epilogue epi)
+        __global__ __launch_bounds__(kStemThreads) void conv_stem_kernel(const StemParams p)
         {
             extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
             const int tid = static_cast<int>(threadIdx.x);
@@ -102,9 +106,9 @@ namespace hipq
                 int32_t b = 0;
                 if (tid < 64)
                 {
-                    b = epi.bias ? epi.bias[tid] : 0;
+                    b = p.bias ? p.bias[tid] : 0;
                     consts[tid] = (p.x_unsigned ? 128 : 0) * p.wsum[tid] + b;
-                    reinterpret_cast<float*>(consts)[64 + tid] = epi.per_channel ? epi.scale[tid] : epi.scale[0];
+                    reinterpret_cast<float*>(consts)[64 + tid] = p.per_channel ? p.scale[tid] : p.scale[0];
                 }
                 fold = __syncthreads_and(b >= -(1 << 24) && b <= (1 << 24)) != 0;
             }
@@ -124,6 +128,13 @@ namespace hipq
                 for (int ni = 0; ni < 2; ++ni)
                     wf[r][ni] = r < p.R ? *reinterpret_cast<const v4i*>(p.w + (ni * 32 + (lane & 31)) * p.kp + r * 32 + half * 16) : v4i{0, 0, 0, 0};
             // a lane's accumulator register 4 g + e of block ni is channel 32 ni + 8 g + 4 half + e
+            // the fragments have arrived before the first tile: a wait for them inside the tile loop
+            // would also wait for the next band's rows, which the compiler does not know are in flight
+#pragma unroll
+            for (int r = 0; r < KS; ++r)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+                    asm volatile("" ::"v"(wf[r][ni]));
             // (the start values stay in registers; the scales are read back from LDS tile by tile)
             v16i start[2];
 #pragma unroll
@@ -201,8 +212,16 @@ namespace hipq
             };
 
             // ---- the slow, exact band (a bias the accumulators cannot carry) ---------------------
-            const EpiRegs er = epi_load(epi);
             auto slow_band = [&](int n, int cy0) {
+                Epilogue epi;
+                memset(&epi, 0, sizeof(epi));
+                epi.mode = EPI_FUSED;
+                epi.out_t = HIPQ_U8;
+                epi.bias = p.bias;
+                epi.scale = p.scale;
+                epi.per_channel = p.per_channel;
+                epi.relu = p.relu;
+                const EpiRegs er = epi_load(epi);
                 const uint8_t* const src = lds;
                 const int total = p.CR * p.Q * 64;
                 for (int i = tid; i < total; i += kStemThreads)
@@ -475,6 +494,10 @@ namespace hipq
         p.w = static_cast<const int8_t*>(packed);
         p.wsum = reinterpret_cast<const int32_t*>(static_cast<const uint8_t*>(packed) + align_up(static_cast<size_t>(g.K) * p.kp, 256));
         p.out = static_cast<uint8_t*>(out);
+        p.bias = epi.bias;
+        p.scale = epi.scale;
+        p.per_channel = epi.per_channel;
+        p.relu = epi.relu;
         const unsigned grid = static_cast<unsigned>(std::min<int64_t>(p.items, device_compute_units()));
         int rc = HIPQ_OK;
         auto go = [&](auto kernel, int slot) {
@@ -494,7 +517,7 @@ namespace hipq
                 }
                 configured[slot][dev] = true;
             }
-            kernel<<<grid, kStemThreads, lds_bytes, s>>>(p, epi);
+            kernel<<<grid, kStemThreads, lds_bytes, s>>>(p);
         };
         const int ks = stem_steps(p.R);
         const bool wide = p.W % 16 == 0 && (reinterpret_cast<uintptr_t>(data) & 15) == 0; // image rows in whole 16-byte pieces

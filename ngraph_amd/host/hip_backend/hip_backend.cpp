@@ -158,6 +158,17 @@ namespace
         void lower_conv(const shared_ptr<Node>& n, Step& st);
         void lower_dot(const shared_ptr<Node>& n, Step& st, const hipq_quant_out_t* gelu_quantize = nullptr, int gelu_quantize_at = -1);
         void lower_pool(const shared_ptr<Node>& n, Step& st);
+        // the library call a convolution node stands for: descriptors and the positions of its inputs
+        struct ConvCall
+        {
+            hipq_conv_desc_t d;
+            hipq_fused_desc_t f;
+            int bias_i = -1, sum_i = -1, scale_i = -1, sum_scale_i = -1;
+            bool plain = false;
+        };
+        ConvCall conv_call(const shared_ptr<Node>& n) const;
+        hipq_pool_desc_t pool_desc(const shared_ptr<Node>& n) const;
+        shared_ptr<DeviceBlock> packed_filter(const shared_ptr<Node>& n, const ConvCall& c);
         void assign_layouts();
         void plan_glue_fusion();
         bool nxc(const Node* n) const { return m_nxc.count(n) != 0; }
@@ -193,6 +204,9 @@ namespace
         };
         unordered_map<const Node*, Attention> m_attention;
         unordered_map<const Node*, pair<Output<Node>, Output<Node>>> m_layer_norm_of_sum;
+        // ... a MaxPool that also runs the convolution in front of it (a network's first two layers):
+        // one launch, the convolution's own output is never written
+        unordered_map<const Node*, shared_ptr<Node>> m_pool_of_conv;
         struct QuantizedCopy
         {
             shared_ptr<Node> quantize;
@@ -395,6 +409,32 @@ namespace
         auto single_user = [&](const Node* n) { return users[n].size() == 1; };
         for (const auto& n : m_function->get_ordered_ops())
         {
+            if (is_type<op::v0::MaxPool>(n))
+            {
+                // MaxPool(QuantizedConvolutionBias / Relu) with a constant filter, for the pairs the
+                // library has a fused kernel for (a network's first two layers)
+                const auto conv = n->input_value(0).get_node_shared_ptr();
+                if ((is_type<op::v0::QuantizedConvolutionBias>(conv) || is_type<op::v0::QuantizedConvolutionRelu>(conv)) && single_user(conv.get()) &&
+                    !conv->is_output() && conv->get_argument(1)->is_constant())
+                {
+                    const ConvCall c = conv_call(conv);
+                    hipq_pool_desc_t pd;
+                    try
+                    {
+                        pd = pool_desc(n);
+                    }
+                    catch (const exception&)
+                    {
+                        continue; // (lowering the pool by itself reports what is wrong with it)
+                    }
+                    if (hipq_conv_max_pool_fusable(&c.d, &c.f, &pd))
+                    {
+                        m_pool_of_conv[n.get()] = conv;
+                        m_folded.insert(conv.get());
+                    }
+                }
+                continue;
+            }
             if (auto sm = as_type_ptr<op::v0::Softmax>(n))
             {
                 auto mul = as_type_ptr<op::v1::Multiply>(n->input_value(0).get_node_shared_ptr());
@@ -557,59 +597,78 @@ namespace
                 m_nxc[n.get()] = true;
     }
 
-    void HIPExecutable::lower_conv(const shared_ptr<Node>& n, Step& st)
+    HIPExecutable::ConvCall HIPExecutable::conv_call(const shared_ptr<Node>& n) const
     {
+        ConvCall c;
         ConvAttrs attrs;
         // input positions per op (src/ngraph/op/experimental/quantized_conv_bias.cpp, quantized_conv_relu.cpp)
-        int bias_i = -1, sum_i = -1, scale_i = -1, sum_scale_i = -1;
-        bool relu = false, plain = false;
-        int sum_t = HIPQ_U8;
+        bool relu = false;
         if (auto q = as_type_ptr<op::v0::QuantizedConvolution>(n))
         {
             attrs = conv_attrs(*q);
-            plain = true;
+            c.plain = true;
         }
         else if (auto qb = as_type_ptr<op::v0::QuantizedConvolutionBias>(n))
         {
             attrs = conv_attrs(*qb);
-            bias_i = 2, scale_i = 3, relu = qb->with_relu();
+            c.bias_i = 2, c.scale_i = 3, relu = qb->with_relu();
         }
         else if (auto qr = as_type_ptr<op::v0::QuantizedConvolutionRelu>(n))
         {
             attrs = conv_attrs(*qr);
-            scale_i = 2, relu = true;
+            c.scale_i = 2, relu = true;
         }
         else if (auto qa = as_type_ptr<op::v0::QuantizedConvolutionBiasAdd>(n))
         {
             attrs = conv_attrs(*qa);
-            bias_i = 2, sum_i = 3, scale_i = 4, sum_scale_i = 5, relu = qa->with_relu();
+            c.bias_i = 2, c.sum_i = 3, c.scale_i = 4, c.sum_scale_i = 5, relu = qa->with_relu();
         }
         else if (auto qs = as_type_ptr<op::v0::QuantizedConvolutionBiasSignedAdd>(n))
         {
             attrs = conv_attrs(*qs);
-            bias_i = 2, sum_i = 3, scale_i = 4, sum_scale_i = 5, relu = qs->with_relu();
+            c.bias_i = 2, c.sum_i = 3, c.scale_i = 4, c.sum_scale_i = 5, relu = qs->with_relu();
         }
-        hipq_conv_desc_t d;
-        fill_conv_desc(d, *n, attrs);
-        d.data_layout = nxc(n->input_value(0).get_node()) ? HIPQ_LAYOUT_NXC : HIPQ_LAYOUT_NCX;
-        d.out_layout = nxc(n.get()) ? HIPQ_LAYOUT_NXC : HIPQ_LAYOUT_NCX; // the sum input is in the output's class
-        if (sum_i >= 0)
-            sum_t = dtype_of(n->get_input_element_type(sum_i));
+        fill_conv_desc(c.d, *n, attrs);
+        c.d.data_layout = nxc(n->input_value(0).get_node()) ? HIPQ_LAYOUT_NXC : HIPQ_LAYOUT_NCX;
+        c.d.out_layout = nxc(n.get()) ? HIPQ_LAYOUT_NXC : HIPQ_LAYOUT_NCX; // the sum input is in the output's class
+        memset(&c.f, 0, sizeof(c.f));
+        if (c.plain)
+            return c;
+        c.f.has_bias = c.bias_i >= 0;
+        c.f.has_sum = c.sum_i >= 0;
+        c.f.sum_t = c.sum_i >= 0 ? dtype_of(n->get_input_element_type(c.sum_i)) : HIPQ_U8;
+        c.f.with_relu = relu;
+        c.f.scale_count = static_cast<int64_t>(shape_size(n->get_input_shape(c.scale_i)));
+        if (c.f.scale_count != 1 && c.f.scale_count != c.d.K)
+            throw ngraph_error("HIP backend: requantization scale must be a scalar or have one entry per output channel");
+        if (c.sum_scale_i >= 0 && shape_size(n->get_input_shape(c.sum_scale_i)) != 1)
+            throw ngraph_error("HIP backend: sum scale must be a scalar");
+        return c;
+    }
 
-        // A constant filter whose zero point is a constant 0 (the fused ops have none) is packed
-        // once here; the nGraph CPU backend makes the same demand of its fast path
-        // (src/ngraph/runtime/cpu/pass/cpu_assignment.cpp:801-825).
+    // A constant filter whose zero point is a constant 0 (the fused ops have none) is packed once at
+    // compile time; the nGraph CPU backend makes the same demand of its fast path
+    // (src/ngraph/runtime/cpu/pass/cpu_assignment.cpp:801-825).  Null when there is nothing to pack.
+    shared_ptr<DeviceBlock> HIPExecutable::packed_filter(const shared_ptr<Node>& n, const ConvCall& c)
+    {
         shared_ptr<DeviceBlock> packed;
         const bool filter_const = n->get_argument(1)->is_constant();
-        const bool zp_zero = plain ? constant_is_zero(n->input_value(5)) : true;
-        size_t packed_bytes = hipq_conv_packed_filter_bytes(&d);
+        const bool zp_zero = c.plain ? constant_is_zero(n->input_value(5)) : true;
+        const size_t packed_bytes = hipq_conv_packed_filter_bytes(&c.d);
         if (filter_const && zp_zero && packed_bytes)
         {
             packed = alloc(packed_bytes);
-            check(hipq_conv_pack_filter(&d, constant_ptr(n->input_value(1)), packed->ptr, m_stream), "filter packing");
+            check(hipq_conv_pack_filter(&c.d, constant_ptr(n->input_value(1)), packed->ptr, m_stream), "filter packing");
         }
+        return packed;
+    }
 
-        if (plain)
+    void HIPExecutable::lower_conv(const shared_ptr<Node>& n, Step& st)
+    {
+        const ConvCall c = conv_call(n);
+        const hipq_conv_desc_t d = c.d;
+        const shared_ptr<DeviceBlock> packed = packed_filter(n, c);
+        if (c.plain)
         {
             st.launch = [d, packed](const vector<void*>& in, void* out, void* stream) {
                 check(hipq_quantized_convolution(&d, in[0], in[1], packed ? packed->ptr : nullptr, static_cast<const float*>(in[2]), in[3],
@@ -618,17 +677,8 @@ namespace
             };
             return;
         }
-        hipq_fused_desc_t f;
-        memset(&f, 0, sizeof(f));
-        f.has_bias = bias_i >= 0;
-        f.has_sum = sum_i >= 0;
-        f.sum_t = sum_t;
-        f.with_relu = relu;
-        f.scale_count = static_cast<int64_t>(shape_size(n->get_input_shape(scale_i)));
-        if (f.scale_count != 1 && f.scale_count != d.K)
-            throw ngraph_error("HIP backend: requantization scale must be a scalar or have one entry per output channel");
-        if (sum_scale_i >= 0 && shape_size(n->get_input_shape(sum_scale_i)) != 1)
-            throw ngraph_error("HIP backend: sum scale must be a scalar");
+        const hipq_fused_desc_t f = c.f;
+        const int bias_i = c.bias_i, sum_i = c.sum_i, scale_i = c.scale_i, sum_scale_i = c.sum_scale_i;
         const string name = n->get_type_name();
         st.launch = [d, f, packed, bias_i, sum_i, scale_i, sum_scale_i, name](const vector<void*>& in, void* out, void* stream) {
             check(hipq_quantized_convolution_fused(&d, &f, in[0], in[1], packed ? packed->ptr : nullptr,
@@ -734,7 +784,7 @@ namespace
     }
 
     // MaxPool / AvgPool over [N, C, spatial...] (src/ngraph/runtime/reference/max_pool.hpp:127-222, avg_pool.hpp:128-250)
-    void HIPExecutable::lower_pool(const shared_ptr<Node>& n, Step& st)
+    hipq_pool_desc_t HIPExecutable::pool_desc(const shared_ptr<Node>& n) const
     {
         hipq_pool_desc_t d;
         memset(&d, 0, sizeof(d));
@@ -780,6 +830,30 @@ namespace
         for (int i = 0; i < d.n_spatial; ++i)
             if (d.out_sp[i] != static_cast<int64_t>(out[2 + i]))
                 throw runtime_error("HIP backend: pooling output shape disagrees with the node's");
+        return d;
+    }
+
+    void HIPExecutable::lower_pool(const shared_ptr<Node>& n, Step& st)
+    {
+        const hipq_pool_desc_t d = pool_desc(n);
+        const auto fused = m_pool_of_conv.find(n.get());
+        if (fused != m_pool_of_conv.end())
+        {
+            // the step's inputs are the convolution's (lower): data, filter, bias / scale
+            const ConvCall c = conv_call(fused->second);
+            const shared_ptr<DeviceBlock> packed = packed_filter(fused->second, c);
+            if (!packed)
+                throw runtime_error("HIP backend: fused convolution + MaxPool without a packed filter");
+            const hipq_conv_desc_t cd = c.d;
+            const hipq_fused_desc_t cf = c.f;
+            const int bias_i = c.bias_i, scale_i = c.scale_i;
+            st.launch = [cd, cf, d, packed, bias_i, scale_i](const vector<void*>& in, void* out, void* stream) {
+                check(hipq_quantized_convolution_fused_max_pool(&cd, &cf, &d, in[0], packed->ptr, bias_i >= 0 ? static_cast<const int32_t*>(in[bias_i]) : nullptr,
+                                                                static_cast<const float*>(in[scale_i]), out, stream),
+                      "QuantizedConvolutionBias + MaxPool");
+            };
+            return;
+        }
         st.launch = [d](const vector<void*>& in, void* out, void* stream) { check(hipq_pool(&d, in[0], out, stream), "pooling"); };
     }
 
@@ -887,7 +961,17 @@ namespace
                 m_value_uses[st.inputs.back()] += 1;
             }
         }
-        for (size_t i = 0; attention == m_attention.end() && i < n->get_input_size(); ++i)
+        const auto pool_of_conv = m_pool_of_conv.find(n.get());
+        if (pool_of_conv != m_pool_of_conv.end())
+        {
+            // the folded convolution in front of input 0: the launch reads its data, filter, bias and scale
+            for (size_t i = 0; i < pool_of_conv->second->get_input_size(); ++i)
+            {
+                st.inputs.push_back(value_of(pool_of_conv->second->input_value(i)));
+                m_value_uses[st.inputs.back()] += 1;
+            }
+        }
+        for (size_t i = 0; attention == m_attention.end() && pool_of_conv == m_pool_of_conv.end() && i < n->get_input_size(); ++i)
         {
             // (a folded Multiply / Add in front of input 0: the consumer reads the folded node's inputs instead)
             const auto sp = m_softmax_of_product.find(n.get());

@@ -161,7 +161,7 @@ class DevicePlan:
     everything up to the logits stays channels-last.  `launch()` issues the kernel launches of one
     forward pass on `stream`; `capture()` turns them into one HIP graph for `replay()`."""
 
-    def __init__(self, lib, stream, N, hw=224):
+    def __init__(self, lib, stream, N, hw=224, fuse_pool=True):
         self.lib, self.stream, self.N = lib, stream, N
         self._replay = None
         self.calls, self.keep, self.graph = [], [], None
@@ -170,9 +170,16 @@ class DevicePlan:
         shape = {"input": (3, hw)}
         self.input = buf["input"]
         self.ops_per_image = 0
-        for op in layers():
+        ops = layers()
+        readers = {}
+        for op in ops:
+            for key in ("src", "sum_src"):
+                if op.get(key) is not None:
+                    readers[op[key]] = readers.get(op[key], 0) + 1
+        pending = None  # a convolution whose only reader is the MaxPool behind it, held back for the fused call
+        for i, op in enumerate(ops):
             Cc, h = shape[op["src"]]
-            src = buf[op["src"]]
+            src = buf.get(op["src"])
             if op["op"] == "quantize":
                 d = H.make_quant_desc((N, Cc, h, h), (), "f32", "u8")
                 out = self._keep(H.DeviceBuffer(N * Cc * h * h))
@@ -196,17 +203,30 @@ class DevicePlan:
                 bf, bb, bs = dev(filt), dev(bias), dev(scales)
                 packed = self._keep(H.pack_filter(d, bf))
                 ho = out_hw(h, op["R"], op["stride"], op["pad"])
+                self.ops_per_image += 2 * op["K"] * op["C"] * op["R"] * op["R"] * ho * ho
+                shape[op["name"]] = (op["K"], ho)
+                nxt = ops[i + 1] if i + 1 < len(ops) else None
+                if nxt is not None and nxt["op"] == "maxpool" and nxt["src"] == op["name"] and readers.get(op["name"], 0) == 1 and not has_sum and fuse_pool:
+                    pd = H.make_pool_desc("max", "u8", N, op["K"], [ho, ho], [nxt["window"]] * 2, [nxt["stride"]] * 2, [nxt["pad"]] * 2, [nxt["pad"]] * 2, False, H.NXC)
+                    if H.conv_max_pool_fusable(d, f, pd):
+                        # MaxPool(convolution) in one launch: the convolution's own output is never written
+                        pending = (op["name"], self._keep(d), self._keep(f), self._keep(pd), src, packed, bb, bs)
+                        continue
                 out = self._keep(H.DeviceBuffer(N * op["K"] * ho * ho))
                 ss = dev(np.asarray(op["sum_scale"], np.float32)) if has_sum else None
                 sm = buf[op["sum_src"]] if has_sum else None
                 self.calls.append((lib.hipq_quantized_convolution_fused, (self._keep(d), self._keep(f), src, bf, packed, bb, sm, bs, ss, out)))
-                buf[op["name"]], shape[op["name"]] = out, (op["K"], ho)
-                self.ops_per_image += 2 * op["K"] * op["C"] * op["R"] * op["R"] * ho * ho
+                buf[op["name"]] = out
             elif op["op"] in ("maxpool", "avgpool"):
-                d = H.make_pool_desc("max" if op["op"] == "maxpool" else "avg", "u8", N, Cc, [h, h], [op["window"]] * 2, [op["stride"]] * 2, [op["pad"]] * 2, [op["pad"]] * 2, False, H.NXC)
                 ho = out_hw(h, op["window"], op["stride"], op["pad"])
                 out = self._keep(H.DeviceBuffer(N * Cc * ho * ho))
-                self.calls.append((lib.hipq_pool, (self._keep(d), src, out)))
+                if pending is not None and pending[0] == op["src"]:
+                    _, cd, cf, pd, csrc, cpacked, cbias, cscale = pending
+                    self.calls.append((lib.hipq_quantized_convolution_fused_max_pool, (cd, cf, pd, csrc, cpacked, cbias, cscale, out)))
+                    pending = None
+                else:
+                    d = H.make_pool_desc("max" if op["op"] == "maxpool" else "avg", "u8", N, Cc, [h, h], [op["window"]] * 2, [op["stride"]] * 2, [op["pad"]] * 2, [op["pad"]] * 2, False, H.NXC)
+                    self.calls.append((lib.hipq_pool, (self._keep(d), src, out)))
                 buf[op["name"]], shape[op["name"]] = out, (Cc, ho)
             elif op["op"] == "convert_u8":
                 buf[op["name"]], shape[op["name"]] = src, (Cc, h)  # same bits: the buffer is shared

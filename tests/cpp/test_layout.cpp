@@ -218,3 +218,59 @@ GPU_TEST(HIP, layout_pass_keeps_blocks_channels_last_in_front_of_a_classifier)
     EXPECT_EQ(launches[0], size_t(7));
     EXPECT_EQ(launches[1], size_t(7));
 }
+
+// A network's first two layers: QuantizedConvolutionBias (3 -> 64 channels, 7 x 7, stride 2, ReLU) over
+// an NCHW parameter, then MaxPool 3 x 3 / 2.  With the glue fusion on the pair is one launch (the
+// convolution's own output is never written); with NGRAPH_PASS_ENABLES "HIPGlueFusion:0" it is two.
+// The bytes of the 1 x 1 convolution behind the pool are the same either way.  (The pool itself is not
+// returned: a tensor a Result reads is kept in nGraph's layout, and the fused kernel writes channels-last.)
+namespace
+{
+    shared_ptr<Function> first_layers(size_t N, size_t H, size_t W)
+    {
+        Lcg rng{2024u};
+        auto x = make_shared<op::v0::Parameter>(element::u8, Shape{N, 3, H, W});
+        auto scale = [](float v) { return op::v0::Constant::create(element::f32, Shape{}, {v}); };
+        auto w = random_constant<int8_t>(element::i8, Shape{64, 3, 7, 7}, rng, -100, 100);
+        auto b = random_constant<int32_t>(element::i32, Shape{64}, rng, -20000, 20000);
+        auto stem = make_shared<op::v0::QuantizedConvolutionBias>(x, w, b, Strides{2, 2}, Strides{1, 1}, CoordinateDiff{3, 3}, CoordinateDiff{3, 3}, Strides{1, 1}, scale(1.0f / 600), true);
+        auto pool = make_shared<op::v0::MaxPool>(stem, Shape{3, 3}, Strides{2, 2}, Shape{1, 1}, Shape{1, 1});
+        auto w2 = random_constant<int8_t>(element::i8, Shape{32, 64, 1, 1}, rng, -20, 20);
+        auto b2 = random_constant<int32_t>(element::i32, Shape{32}, rng, -2000, 2000);
+        auto c2 = make_shared<op::v0::QuantizedConvolutionBias>(pool, w2, b2, Strides{1, 1}, Strides{1, 1}, CoordinateDiff{0, 0}, CoordinateDiff{0, 0}, Strides{1, 1}, scale(1.0f / 100), true);
+        return make_shared<Function>(OutputVector{c2}, ParameterVector{x});
+    }
+}
+
+GPU_TEST(HIP, first_convolution_and_max_pool_are_one_launch)
+{
+    const size_t N = 3, H = 64, W = 48;
+    vector<uint8_t> out[2];
+    size_t launches[2] = {0, 0};
+    for (int on = 0; on < 2; ++on)
+    {
+        setenv("NGRAPH_PASS_ENABLES", on ? "HIPGlueFusion:1" : "HIPGlueFusion:0", 1);
+        auto f = first_layers(N, H, W);
+        auto backend = runtime::Backend::create("HIP");
+        auto a = backend->create_tensor(element::u8, Shape{N, 3, H, W});
+        Lcg rng{5u};
+        vector<uint8_t> data(a->get_element_count());
+        for (auto& v : data)
+            v = static_cast<uint8_t>(rng.next(0, 255));
+        copy_data(a, data);
+        auto r = backend->create_tensor(element::u8, f->get_output_shape(0));
+        auto exec = backend->compile(f, true);
+        unsetenv("NGRAPH_PASS_ENABLES");
+        for (int i = 0; i < 3; ++i)
+            exec->call_with_validate({r}, {a});
+        out[on] = read_vector<uint8_t>(r);
+        launches[on] = exec->get_performance_data().size();
+    }
+    EXPECT_TRUE(out[0] == out[1]);
+    size_t distinct = 0, seen[256] = {0};
+    for (uint8_t v : out[1])
+        distinct += seen[v]++ == 0;
+    EXPECT_TRUE(distinct > 50);
+    EXPECT_EQ(launches[0], size_t(3)); // convolution, pool, convolution
+    EXPECT_EQ(launches[1], size_t(2)); // convolution + pool, convolution
+}

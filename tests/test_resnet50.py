@@ -129,7 +129,9 @@ def test_resnet50_device_plan_and_graph_replay(gpu_lib):
     print("[case] resnet50 plan launch", flush=True)
     plan.launch()
     assert np.array_equal(plan.read_logits(), ref["logits"])
+    assert np.array_equal(plan.read("pool1", 64, 56), ref["pool1"])  # written by the launch that also runs the stem convolution
     assert np.array_equal(plan.read("s3_b0_out", 512, 28), ref["s3_b0_out"])
+    assert any(fn is lib.hipq_quantized_convolution_fused_max_pool or getattr(fn, "__name__", "") == "hipq_quantized_convolution_fused_max_pool" for fn, _ in plan.calls)
     print("[case] resnet50 plan capture", flush=True)
     plan.capture()
     for seed in (8, 9, 10):  # new images before every replay, an eager op-by-op run in between
@@ -171,7 +173,7 @@ def test_resnet50_benchmarked_batches_against_oracle(gpu_lib, N):
     def check_all(tag):
         logits = plan.read_logits()
         assert np.array_equal(logits, np.tile(exp["logits"], (N // 4, 1))), tag
-        for name, ch, hw in (("s2_b0_out", 256, 56), ("s3_b0_out", 512, 28), ("s4_b5_out", 1024, 14), ("s5_b2_out", 2048, 7)):
+        for name, ch, hw in (("pool1", 64, 56), ("s2_b0_out", 256, 56), ("s3_b0_out", 512, 28), ("s4_b5_out", 1024, 14), ("s5_b2_out", 2048, 7)):
             got = plan.read(name, ch, hw)
             assert got.shape == (N, ch, hw, hw)
             assert np.array_equal(got, np.tile(exp[name], (N // 4, 1, 1, 1))), (tag, name)

@@ -25,55 +25,6 @@
 
 #include "hipq_igemm.h"
 
-// Optional phase clocks (development builds only): the first lane of either group of workgroup 0
-// records the shader clock at each HIPQ_PHASE(i); hipq_debug_band_phases copies them out.
-#ifdef HIPQ_PHASE_CLOCKS
-static __device__ long long g_phase_clock[32];
-#define HIPQ_PHASE(i)                                                                              \
-    do                                                                                             \
-    {                                                                                              \
-        if (blockIdx.x == 0 && (threadIdx.x & 255) == 0 && (i) < 16 && threadIdx.x < 512)                               \
-            g_phase_clock[(threadIdx.x >> 8) * 16 + (i)] = clock64();                              \
-    } while (0)
-static __device__ long long g_block_times[256][4];
-static __device__ long long g_wave_clock[12][12][2]; // [phase][wave][arrive at barrier, leave barrier]
-#define HIPQ_WAVE_MARK(phase, which)                                                               \
-    do                                                                                             \
-    {                                                                                              \
-        if (blockIdx.x == 0 && (threadIdx.x & 63) == 0 && (phase) < 12)                             \
-            g_wave_clock[phase][threadIdx.x >> 6][which] = clock64();                              \
-    } while (0)
-extern "C" HIPQ_API int hipq_debug_band_waves(long long* out288)
-{
-    return hipMemcpyFromSymbol(out288, HIP_SYMBOL(g_wave_clock), sizeof(long long) * 288) == hipSuccess ? 0 : 1;
-}
-#define HIPQ_BLOCK_BEGIN()                                                                         \
-    long long blk_w0 = wall_clock64(), blk_c0 = clock64()
-#define HIPQ_BLOCK_END()                                                                           \
-    do                                                                                             \
-    {                                                                                              \
-        if (threadIdx.x == 0 && blockIdx.x < 256)                                                  \
-        {                                                                                          \
-            g_block_times[blockIdx.x][0] = blk_w0;                                                 \
-            g_block_times[blockIdx.x][1] = wall_clock64();                                         \
-            g_block_times[blockIdx.x][2] = clock64() - blk_c0;                                     \
-            g_block_times[blockIdx.x][3] = __builtin_amdgcn_s_getreg(((32 - 1) << 11) | 4);        \
-        }                                                                                          \
-    } while (0)
-extern "C" HIPQ_API int hipq_debug_band_blocks(long long* out1024)
-{
-    return hipMemcpyFromSymbol(out1024, HIP_SYMBOL(g_block_times), sizeof(long long) * 1024) == hipSuccess ? 0 : 1;
-}
-extern "C" HIPQ_API int hipq_debug_band_phases(long long* out32)
-{
-    return hipMemcpyFromSymbol(out32, HIP_SYMBOL(g_phase_clock), sizeof(long long) * 32) == hipSuccess ? 0 : 1;
-}
-#else
-#define HIPQ_PHASE(i) ((void)0)
-#define HIPQ_BLOCK_BEGIN() ((void)0)
-#define HIPQ_BLOCK_END() ((void)0)
-#define HIPQ_WAVE_MARK(phase, which) ((void)0)
-#endif
 
 namespace hipq
 {
@@ -398,8 +349,6 @@ namespace hipq
         const int l32 = lane & 31;
         const int xs_off = p.x_lds + grp * p.band_bytes;
 
-        HIPQ_BLOCK_BEGIN();
-        HIPQ_PHASE(0);
         // ---- small loads first: they must not queue behind the bulk loads ------------------------
         const int32_t xzp = load_zp(zp.data_zp, zp.data_t);
         const int32_t wzp = load_zp(zp.filter_zp, zp.filter_t);
@@ -526,7 +475,6 @@ namespace hipq
                         }
         };
 
-        HIPQ_PHASE(1);
         for (int u0 = 0; u0 * 8 < taps * 4; u0 += kBandBatch)
         {
             if (u0)
@@ -538,7 +486,6 @@ namespace hipq
         if (grp == 0 && 0 < my_items)
             band_store(xb0, 0);
         __syncthreads();
-        HIPQ_PHASE(2);
 
         // Phase p multiplies item p and requantizes item p - 1; item j belongs to group j % 2.  Both
         // groups run the same multiply / barrier / requantize / barrier loop over their own items,
@@ -549,9 +496,7 @@ namespace hipq
         {
             if (phases_done == grp - 1 && grp < my_items)
                 band_store(xb0, grp);
-            HIPQ_WAVE_MARK(phases_done, 0);
             __syncthreads();
-            HIPQ_WAVE_MARK(phases_done, 1);
         }
         // staging holds a whole wavefront tile (two groups) or half of one (three groups: LDS is short)
         constexpr bool kStageHalf = G == 3;
@@ -582,7 +527,6 @@ namespace hipq
                 // requantizing wavefront fills the gaps.
                 __builtin_amdgcn_s_setprio(3);
                 {
-                    if (sp <= 1) HIPQ_PHASE(10);
                     item_geom(sp, img, p0, rows);
                     const int npix = rows * p.Q;
                     const int ntiles = (npix + 31) >> 5;
@@ -610,26 +554,20 @@ namespace hipq
                             xcol0[ti] = pix - py * p.Q;
                         }
                         const int woff = band_cell(l32, half, 0);
-                        if (sp <= 1) HIPQ_PHASE(11);
                         if (U == 0)
                             band_reduce_33<T, !kCorrLate>(acc, lds, woff, xrow0, xcol0, half, corr);
                         else
                             band_reduce<T, U == 0 ? 1 : U>(acc, lds, woff, xrow0, xcol0, half, p.R, p.S, p.BW);
-                        if (sp <= 1) HIPQ_PHASE(12);
                     }
                 }
             }
             __builtin_amdgcn_s_setprio(0);
             if (!kEarlyFetch && sp + G < my_items)
                 band_fetch(nb, sp + G);
-            HIPQ_WAVE_MARK(phases_done, 0);
             __syncthreads();
-            HIPQ_WAVE_MARK(phases_done, 1);
             ++phases_done;
-            if (phases_done < 6) HIPQ_PHASE(2 + phases_done);
             {
                 // ================= requantize and write out: item sp =================
-                if (sp <= 1) HIPQ_PHASE(13);
                 // per-lane indices are recomputed from an opaque copy of the lane id: hoisted out of the
                 // item loop they would occupy registers through the multiply phase and spill
                 int lane_v = lane;
@@ -743,7 +681,6 @@ namespace hipq
                         }
                     }
                 };
-                if (sp <= 1) HIPQ_PHASE(14);
                 using std::false_type;
                 using std::true_type;
                 auto requantize = [&](auto ti0, auto ti1) {
@@ -808,9 +745,7 @@ namespace hipq
                     __builtin_amdgcn_sched_barrier(0);
                     if (G == 3) // the second half of the tile is the group's third phase
                     {
-                        HIPQ_WAVE_MARK(phases_done, 0);
                         __syncthreads();
-                        HIPQ_WAVE_MARK(phases_done, 1);
                         ++phases_done;
                     }
                     if (kStageHalf) // the first half leaves the staging area before the second half enters
@@ -820,7 +755,6 @@ namespace hipq
                     }
                     requantize(std::integral_constant<int, T / 2>{}, std::integral_constant<int, T>{});
                     __builtin_amdgcn_sched_barrier(0);
-                    if (sp <= 1) HIPQ_PHASE(15);
                     if (!kStageHalf)
                         stage_write_out(0);
                     stage_read(1);
@@ -836,28 +770,19 @@ namespace hipq
                         ++phases_done;
                     }
                     requantize(std::integral_constant<int, T / 2>{}, std::integral_constant<int, T>{});
-                    if (sp <= 1) HIPQ_PHASE(15);
                 }
-                if (sp <= 1) HIPQ_PHASE(9);
                 if (!kEarlyFetch && sp + G < my_items)
                     band_store(nb, sp + G);
                 if (kCarryFetch && sp + G < my_items)
                     band_store(nb, sp + G);
-                if (sp <= 1) HIPQ_PHASE(8);
             }
-            HIPQ_WAVE_MARK(phases_done, 0);
             __syncthreads();
-            HIPQ_WAVE_MARK(phases_done, 1);
             ++phases_done;
-            if (phases_done < 6) HIPQ_PHASE(2 + phases_done);
         }
         for (; phases_done < my_items + G - 1; ++phases_done)
         {
-            HIPQ_WAVE_MARK(phases_done, 0);
             __syncthreads();
-            HIPQ_WAVE_MARK(phases_done, 1);
         }
-        HIPQ_BLOCK_END();
     }
 
     // rows per band and LDS bytes; false when the layer does not fit this kernel

@@ -26,23 +26,6 @@
 
 #include "hipq_igemm.h"
 
-// Optional clock stamps (development builds only): wavefronts of workgroup 0 record the shader clock
-// at HIPQ_RW_MARK(i); hipq_debug_regw_clocks copies them out.
-#ifdef HIPQ_REGW_CLOCKS
-static __device__ long long g_rw_clock[8][64];
-#define HIPQ_RW_MARK(i)                                                                            \
-    do                                                                                             \
-    {                                                                                              \
-        if (blockIdx.x == 0 && (threadIdx.x & 63) == 0 && (i) < 64)                                \
-            g_rw_clock[threadIdx.x >> 6][i] = clock64();                                           \
-    } while (0)
-extern "C" HIPQ_API int hipq_debug_regw_clocks(long long* out512)
-{
-    return hipMemcpyFromSymbol(out512, HIP_SYMBOL(g_rw_clock), sizeof(long long) * 512) == hipSuccess ? 0 : 1;
-}
-#else
-#define HIPQ_RW_MARK(i) ((void)0)
-#endif
 
 namespace hipq
 {
@@ -129,11 +112,6 @@ namespace hipq
         const int npix = rows * W_;
         const int PQ = p.H * W_;
 
-        HIPQ_RW_MARK(0);
-#ifdef HIPQ_REGW_CLOCKS
-        if (blockIdx.x == 0 && (threadIdx.x & 63) == 0)
-            g_rw_clock[threadIdx.x >> 6][63] = __builtin_amdgcn_s_getreg(((32 - 1) << 11) | 4);
-#endif
         const __amdgpu_buffer_rsrc_t xrs = make_rsrc(p.x, p.x_bytes);
         const __amdgpu_buffer_rsrc_t ors = make_rsrc(out, p.out_bytes);
         const bool loader = wave >= 8 - kRwLoaders; // uniform
@@ -312,9 +290,7 @@ namespace hipq
                 *reinterpret_cast<v4i*>(wlds + (((ks * 2 + (n >> 5)) * 2 + hf) * 32 + (n & 31)) * 16) = fpiece[i];
             }
         }
-        HIPQ_RW_MARK(1);
         __syncthreads();
-        HIPQ_RW_MARK(2);
 
         if (*reinterpret_cast<volatile uint32_t*>(slow_flag) != 0) // uniform; w - wzp does not fit a signed byte: exact, slow, one output a lane
         {
@@ -372,7 +348,6 @@ namespace hipq
                     }
                 }
             }
-            HIPQ_RW_MARK(3);
             xzp = load_zp(zp.data_zp, zp.data_t);
         }
 
@@ -653,14 +628,11 @@ namespace hipq
 
         auto run = [&](auto fast_c) {
             v16i acc_a[2], acc_b[2];
-            int mark = 8;
             int ta = grab();
             if (ta >= ntiles)
                 return;
             await_rows(ta);
-            HIPQ_RW_MARK(5);
             tile_mfma(ta, acc_a);
-            HIPQ_RW_MARK(6);
             if (SUM) // the residual's loads and conversions leave no registers for a second accumulator set
             {
                 for (;;)
@@ -676,34 +648,24 @@ namespace hipq
             }
             for (;;)
             {
-                HIPQ_RW_MARK(mark);
                 const int tb = grab();
                 if (tb >= ntiles)
                 {
                     tile_store(ta, acc_a, fast_c);
                     break;
                 }
-                HIPQ_RW_MARK(mark + 1);
                 await_rows(tb);
-                HIPQ_RW_MARK(mark + 2);
                 tile_both(tb, acc_b, ta, acc_a, fast_c);
-                HIPQ_RW_MARK(mark + 3);
                 ta = grab();
                 if (ta >= ntiles)
                 {
                     tile_store(tb, acc_b, fast_c);
                     break;
                 }
-                HIPQ_RW_MARK(mark + 4);
                 await_rows(ta);
-                HIPQ_RW_MARK(mark + 5);
                 tile_both(ta, acc_a, tb, acc_b, fast_c);
-                HIPQ_RW_MARK(mark + 6);
-                mark += 7;
             }
-            HIPQ_RW_MARK(mark);
         };
-        HIPQ_RW_MARK(4);
         if (MODE == EPI_INTERP && fast_interp) // uniform
             run(std::true_type{});
         else

@@ -980,19 +980,6 @@ namespace hipq
     }
 
 
-    // Optional clocks (development builds only): the first lane of every wavefront of workgroup 0
-    // records the shader clock at points of its first 12 slices.
-#ifdef HIPQ_PIPE_CLOCKS
-    static __device__ long long g_pipe_clock[12][4][8];
-#define HIPQ_PIPE_MARK(step, point)                                                                \
-    do                                                                                             \
-    {                                                                                              \
-        if (blockIdx.x == 0 && (threadIdx.x & 63) == 0 && (step) < 12)                              \
-            g_pipe_clock[step][threadIdx.x >> 6][point] = clock64();                                \
-    } while (0)
-#else
-#define HIPQ_PIPE_MARK(step, point) ((void)0)
-#endif
 
     // ---- persistent, software-pipelined variant ---------------------------------------------------
     // For 8-bit channels-last / row-major outputs whose rows are whole 16-byte pieces.  A workgroup
@@ -1688,16 +1675,13 @@ namespace hipq
                 compute(buf, std::false_type{});
         };
         auto step = [&](int s, int buf, const Regs& next, Regs& free_regs) {
-            HIPQ_PIPE_MARK(s, 0);
             const bool tile_done = ckt + 1 == KT;
             if (tile_done) // uniform; the residual is fetched and used inside one branch
             {
                 if (has_sum)
                     sum_fetch();
                 gload(free_regs);
-                HIPQ_PIPE_MARK(s, 1);
                 multiply(buf);
-                HIPQ_PIPE_MARK(s, 2);
                 if (splits == 1 || (cm0 < M && gather_splits())) // uniform
                 {
                     run_epilogue();
@@ -1711,16 +1695,11 @@ namespace hipq
             else
             {
                 gload(free_regs);
-                HIPQ_PIPE_MARK(s, 1);
                 multiply(buf);
-                HIPQ_PIPE_MARK(s, 2);
                 ++ckt;
             }
-            HIPQ_PIPE_MARK(s, 3);
             lstore(next, buf ^ 1);
-            HIPQ_PIPE_MARK(s, 4);
             __syncthreads();
-            HIPQ_PIPE_MARK(s, 5);
             if (tile_done && cj < my_tiles && cn0 != params_n0) // uniform
             {
                 load_params(cn0);
@@ -1772,14 +1751,11 @@ namespace hipq
                 int t, ks = 0;
                 if (splits > 1)
                     tile_index(cj, t, ks);
-                HIPQ_PIPE_MARK(s, 0);
                 if (has_sum && KT == 1) // ahead of the operand loads, so that waiting for it leaves them in flight
                     sum_fetch();
                 issue();
-                HIPQ_PIPE_MARK(s, 1);
                 corr_load(ks != 0); // the correction enters a split reduction once
                 compute(cb, std::true_type{});
-                HIPQ_PIPE_MARK(s, 2);
                 if (KT > 1) // uniform
                 {
                     slice_end();
@@ -1803,7 +1779,6 @@ namespace hipq
                 {
                     run_epilogue();
                 }
-                HIPQ_PIPE_MARK(s, 3);
                 if (cj + 1 < my_tiles)
                     tile_origin(cj + 1, cm0, cn0);
                 slice_end();

@@ -1091,10 +1091,3 @@ namespace hipq
                                 out, s, "dot_mfma_i8_32x32x32");
     }
 }
-
-#ifdef HIPQ_PIPE_CLOCKS
-extern "C" HIPQ_API int hipq_debug_pipe_clocks_rows(long long* out384)
-{
-    return hipMemcpyFromSymbol(out384, HIP_SYMBOL(hipq::g_pipe_clock), sizeof(long long) * 384) == hipSuccess ? 0 : 1;
-}
-#endif

@@ -938,17 +938,67 @@ namespace ngraph
                                                                   AxisSet{})};
             }
 
-            // builder/matmul_factory.cpp:71-150: operands of rank <= 2 are one dot; stacks of matrices are
-            // collapsed to rank 3, multiplied matrix by matrix (Slice, squeeze, dot, expand) and
-            // concatenated, then given their stack axes back.  Both operands must carry the same stack
-            // here: the reference also broadcasts the stack axes numpy-style.
+            // builder/matmul_factory.cpp:71-150: operands of rank <= 2 are one dot; stacks of matrices get
+            // their stack axes broadcast numpy-style against each other (builder/autobroadcast.cpp:95-110,
+            // 138-184, 285-318: a Reshape that drops the axes of length 1 to be repeated, then a
+            // Broadcast over them), are collapsed to rank 3, multiplied matrix by matrix (Slice, squeeze,
+            // dot, expand) and concatenated, then given their stack axes back.
             OutputVector matmul_of(const OnnxNode& node, Output<Node> left, Output<Node> right, const function<Output<Node>(const Output<Node>&, const Output<Node>&)>& make_dot)
             {
-                const Shape left_shape = left.get_shape(), right_shape = right.get_shape();
-                if (left_shape.size() <= 2 && right_shape.size() <= 2)
+                if (left.get_shape().size() <= 2 && right.get_shape().size() <= 2)
                     return {make_dot(left, right)};
-                if (left_shape.size() != right_shape.size() || !equal(left_shape.begin(), left_shape.end() - 2, right_shape.begin()))
-                    throw ngraph_error(node.description() + ": stacks of matrices of different stack shapes (numpy broadcasting) are not supported here");
+                // (the reference slices nothing out of a vector and multiplies it with every matrix of
+                // the other operand's stack; the quantized dot of this library takes matrices)
+                if (left.get_shape().size() < 2 || right.get_shape().size() < 2)
+                    throw ngraph_error(node.description() + ": a vector against a stack of matrices is not supported here");
+                auto identity_order = [](size_t rank) {
+                    AxisVector order(rank);
+                    for (size_t i = 0; i < rank; ++i)
+                        order[i] = i;
+                    return order;
+                };
+                {
+                    const Shape ls = left.get_shape(), rs = right.get_shape();
+                    const Shape lstack(ls.begin(), ls.end() - 2), rstack(rs.begin(), rs.end() - 2);
+                    // the stack both operands are repeated to: axes aligned at the right, lengths equal or 1
+                    const size_t rank = max(lstack.size(), rstack.size());
+                    Shape lfull(rank - lstack.size(), 1), rfull(rank - rstack.size(), 1), target(rank);
+                    lfull.insert(lfull.end(), lstack.begin(), lstack.end());
+                    rfull.insert(rfull.end(), rstack.begin(), rstack.end());
+                    for (size_t i = 0; i < rank; ++i)
+                    {
+                        if (lfull[i] != rfull[i] && lfull[i] != 1 && rfull[i] != 1)
+                            throw ngraph_error(node.description() + ": the stack shapes of the operands cannot be broadcast against each other (axis " + to_string(i) + ": " +
+                                               to_string(lfull[i]) + " and " + to_string(rfull[i]) + ")");
+                        target[i] = lfull[i] == 1 ? rfull[i] : lfull[i];
+                    }
+                    auto repeat = [&](const Output<Node>& x, Shape full) -> Output<Node> {
+                        const Shape& xs = x.get_shape();
+                        Shape out = target;
+                        out.insert(out.end(), xs.end() - 2, xs.end());
+                        full.insert(full.end(), xs.end() - 2, xs.end());
+                        if (out == xs)
+                            return x;
+                        AxisSet repeated;
+                        Shape squeezed;
+                        for (size_t i = 0; i < out.size(); ++i)
+                        {
+                            if (full[i] == 1 && out[i] != 1)
+                                repeated.insert(i);
+                            else
+                                squeezed.push_back(full[i]);
+                        }
+                        Output<Node> y = x;
+                        if (squeezed != xs)
+                            y = make_shared<op::v0::Reshape>(y, identity_order(xs.size()), squeezed);
+                        if (!repeated.empty())
+                            y = make_shared<op::v0::Broadcast>(y, out, repeated);
+                        return y;
+                    };
+                    left = repeat(left, lfull);
+                    right = repeat(right, rfull);
+                }
+                const Shape left_shape = left.get_shape(), right_shape = right.get_shape();
                 auto reshape = [](const Output<Node>& x, const Shape& to) {
                     AxisVector order(x.get_shape().size());
                     for (size_t i = 0; i < order.size(); ++i)

@@ -250,9 +250,8 @@ CPU_TEST(onnx_import, errors_and_operator_queries)
     for (const char* format : kFormats)
     {
         EXPECT_TRUE(what_of([&] { load("unsupported_operator", format); }).find("unsupported operator Softplus (opset 10)") != string::npos);
-        // stacks of matrices multiply when both operands carry the same stack; numpy broadcasting of the
-        // stack axes (builder/autobroadcast.cpp:285-318) is not offered
-        EXPECT_TRUE(what_of([&] { load("matmul_integer_stacks_differ", format); }).find("different stack shapes") != string::npos);
+        // stack axes are broadcast numpy-style (builder/autobroadcast.cpp:285-318); stacks of 2 and of 3 matrices do not fit
+        EXPECT_TRUE(what_of([&] { load("matmul_integer_stacks_clash", format); }).find("cannot be broadcast") != string::npos);
     }
     EXPECT_TRUE(onnx_import::is_operator_supported("QLinearConv", 10, "ai.onnx"));
     EXPECT_TRUE(onnx_import::is_operator_supported("QuantizeLinear", 10, ""));
@@ -449,6 +448,74 @@ GPU_TEST(onnx_import, stacked_matmul_vectors)
     expect_output<int32_t>("matmul_integer_4d_no_zero_point", {in(ramp), in(ramp)}, Shape{1, 2, 3, 3}, plain);
     // (not from the reference's tests) two groups of one channel under 1 x 1 filters 2 and 3
     expect_output<int8_t>("qlinear_conv_groups", {in<uint8_t>({1, 2, 3, 4, 5, 6, 7, 8})}, Shape{1, 2, 2, 2}, {2, 4, 6, 8, 15, 18, 21, 24});
+}
+
+// builder/matmul_factory.cpp:88-105 with builder/autobroadcast.cpp:285-318: the stack axes of the two
+// operands are broadcast against each other numpy-style before the stack is multiplied matrix by matrix.
+// Expected values: the products written out as loops here (numpy.matmul's definition).
+namespace
+{
+    // a [.., M, K] by b [.., K, N] with the stack axes of both already repeated to `stack` (row-major);
+    // la / lb give, for every matrix of the result, which matrix of a / b it multiplies
+    vector<int32_t> stacked_product(const vector<uint8_t>& a, const vector<uint8_t>& b, const vector<size_t>& la, const vector<size_t>& lb, size_t M, size_t K, size_t N, int azp, int bzp)
+    {
+        vector<int32_t> y(la.size() * M * N);
+        for (size_t g = 0; g < la.size(); ++g)
+            for (size_t m = 0; m < M; ++m)
+                for (size_t n = 0; n < N; ++n)
+                {
+                    int32_t acc = 0;
+                    for (size_t k = 0; k < K; ++k)
+                        acc += (static_cast<int>(a[(la[g] * M + m) * K + k]) - azp) * (static_cast<int>(b[(lb[g] * K + k) * N + n]) - bzp);
+                    y[(g * M + m) * N + n] = acc;
+                }
+        return y;
+    }
+}
+
+CPU_TEST(onnx_import, stack_axes_are_broadcast)
+{
+    for (const char* format : kFormats)
+    {
+        // [2, 3, 4] x [1, 4, 3]: the right operand loses its axis of length 1 (Reshape) and is repeated (Broadcast)
+        auto f = load("matmul_integer_broadcast_3d", format);
+        EXPECT_EQ(f->get_output_shape(0), (Shape{2, 3, 3}));
+        EXPECT_EQ(count_ops_of_type<op::v0::Broadcast>(f), size_t(1));
+        EXPECT_EQ(count_ops_of_type<op::v0::QuantizedDot>(f), size_t(2));
+        // [2, 1, 3, 4] x [1, 3, 4, 2]: both repeated to a [2, 3] stack, six products
+        auto g = load("matmul_integer_broadcast_4d", format);
+        EXPECT_EQ(g->get_output_shape(0), (Shape{2, 3, 3, 2}));
+        EXPECT_EQ(count_ops_of_type<op::v0::Broadcast>(g), size_t(2));
+        EXPECT_EQ(count_ops_of_type<op::v0::QuantizedDot>(g), size_t(6));
+        // [3, 4] x [2, 4, 3]: the matrix is repeated for every matrix of the stack
+        auto h = load("matmul_integer_matrix_by_stack", format);
+        EXPECT_EQ(h->get_output_shape(0), (Shape{2, 3, 3}));
+        EXPECT_EQ(count_ops_of_type<op::v0::Broadcast>(h), size_t(1));
+    }
+}
+
+GPU_TEST(onnx_import, stack_axes_are_broadcast_vectors)
+{
+    auto ramp = [](size_t n, int step, int start) {
+        vector<uint8_t> v(n);
+        for (size_t i = 0; i < n; ++i)
+            v[i] = static_cast<uint8_t>((start + static_cast<int>(i) * step) & 0xFF);
+        return v;
+    };
+    {
+        const auto a = ramp(24, 7, 3), b = ramp(12, 11, 5);
+        expect_output<int32_t>("matmul_integer_broadcast_3d", {in(a), in(b), in<uint8_t>({2}), in<uint8_t>({9})}, Shape{2, 3, 3}, stacked_product(a, b, {0, 1}, {0, 0}, 3, 4, 3, 2, 9));
+    }
+    {
+        // result stack [2, 3]: matrix (i, j) is a[i] x b[j]
+        const auto a = ramp(24, 13, 1), b = ramp(24, 5, 200);
+        expect_output<int32_t>("matmul_integer_broadcast_4d", {in(a), in(b), in<uint8_t>({100}), in<uint8_t>({0})}, Shape{2, 3, 3, 2},
+                               stacked_product(a, b, {0, 0, 0, 1, 1, 1}, {0, 1, 2, 0, 1, 2}, 3, 4, 2, 100, 0));
+    }
+    {
+        const auto a = ramp(12, 17, 9), b = ramp(24, 3, 50);
+        expect_output<int32_t>("matmul_integer_matrix_by_stack", {in(a), in(b), in<uint8_t>({0}), in<uint8_t>({60})}, Shape{2, 3, 3}, stacked_product(a, b, {0, 0}, {0, 1}, 3, 4, 3, 0, 60));
+    }
 }
 
 // not from the reference's tests: window sums worked by hand (a 4 x 4 ramp 0..15 under a 3 x 3 window

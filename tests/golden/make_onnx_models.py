@@ -218,7 +218,11 @@ MODELS = {
     "matmul_integer_scalar": matmul_integer([1, 1], [1, 1], [1, 1]),
     "matmul_integer_4d": matmul_integer([1, 2, 3, 4], [1, 2, 4, 3], [1, 2, 3, 3]),
     "matmul_integer_4d_no_zero_point": matmul_integer([1, 2, 3, 4], [1, 2, 4, 3], [1, 2, 3, 3], zero_points=False),
-    "matmul_integer_stacks_differ": matmul_integer([2, 3, 4], [1, 4, 3], [2, 3, 3]),
+    # stack axes broadcast numpy-style: a stack of one matrix against two, two stack axes against each other, a matrix against a stack; stacks that do not fit
+    "matmul_integer_broadcast_3d": matmul_integer([2, 3, 4], [1, 4, 3], [2, 3, 3]),
+    "matmul_integer_broadcast_4d": matmul_integer([2, 1, 3, 4], [1, 3, 4, 2], [2, 3, 3, 2]),
+    "matmul_integer_matrix_by_stack": matmul_integer([3, 4], [2, 4, 3], [2, 3, 3]),
+    "matmul_integer_stacks_clash": matmul_integer([2, 3, 4], [3, 4, 3], [2, 3, 3]),
     # QLinearConv in two groups: a 1 x 1 filter a channel (unit scales, zero zero points)
     "qlinear_conv_groups": qlinear_conv(
         [1, 2, 2, 2], [2, 1, 1, 1], [1, 2, 2, 2], w_type=INT8, y_type=INT8,

@@ -294,6 +294,10 @@ namespace hipq
     };
     bool conv_stem_eligible(const ConvGeom& g, const Epilogue& epi, const ZeroPoints& zp, const PoolFuse* pool);
     int launch_conv_stem(const ConvGeom& g, const void* data, const void* packed, const ZeroPoints& zp, const Epilogue& epi, const PoolFuse* pool, void* out, hipStream_t s);
+    // 1 x 1 layers from 64 to a multiple of 256 channels over many pixels, fused policy, channels-last:
+    // weights in registers, tile loads one tile ahead (hipq_conv_pw.hip)
+    bool conv_pw64_eligible(const ConvGeom& g, const Epilogue& epi, const ZeroPoints& zp);
+    int launch_conv_pw64(const ConvGeom& g, const void* data, const void* packed, const Epilogue& epi, void* out, hipStream_t s);
     int launch_row_sums_i8(const void* w, int64_t rows, int64_t cols, int32_t* sums, hipStream_t s);
     // [N][K] weights in the fragment order of v_mfma_i32_16x16x64_i8 (K a multiple of 64): ceil(N / 16) * K / 64 blocks of 1 KB
     int launch_pack_dot_fragments(const void* w_nk, int64_t N, int64_t K, void* frag, hipStream_t s);

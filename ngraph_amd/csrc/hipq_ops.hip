@@ -68,6 +68,10 @@ namespace hipq
         if (!packed || !conv_mfma_eligible(g) || (epi.mode == EPI_FUSED && g.out_t == HIPQ_I32))
             return launch_conv_direct(g, data, filter, zp, epi, out, s);
 
+        // layers bound by HBM traffic that widen 64 channels: weights in registers, loads a tile ahead
+        if (conv_pw64_eligible(g, epi, zp))
+            return launch_conv_pw64(g, data, packed, epi, out, s);
+
         // 3x3 layers over 64 channels with an NCHW output keep their filter in registers and read the
         // input in whichever layout it has: no transposition, no scratch
         if (conv_regw_eligible(g, g.out_layout == HIPQ_LAYOUT_NCX && g.K > 1))

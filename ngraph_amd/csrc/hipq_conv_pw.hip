@@ -1,12 +1,12 @@
-// 1 x 1 convolutions that widen 64 channels to a multiple of 256 (a bottleneck block's last layer and
-// its projection shortcut at the first stage of a ResNet), fused policy, channels-last, optionally
+// 1 x 1 convolutions that widen 64 or 128 channels to a multiple of 256 (a bottleneck block's last layer
+// and its projection shortcut at the first stages of a ResNet), fused policy, channels-last, optionally
 // with the residual input: layers that move 9 bytes through HBM for every 64 multiply-adds and are
 // bound by that traffic.  What the general tile kernel leaves on the table there is overlap -- a
 // workgroup loads, multiplies, requantizes and stores one tile after the other -- so this kernel is
 // arranged around keeping the memory system busy:
 //
-//   * the weights of a wavefront's 128 output channels (8 KiB) stay in its registers as MFMA
-//     fragments for the whole launch; a tile's operands are 64 pixels x 64 bytes of data (4 KiB,
+//   * the weights of a wavefront's 128 output channels (8 or 16 KiB) stay in its registers as MFMA
+//     fragments for the whole launch; a tile's operands are 64 pixels x C bytes of data (4 or 8 KiB,
 //     shared by the four wavefronts through LDS) and, per wavefront, 32 pixels x 128 bytes of
 //     residual;
 //   * both arrive by loads straight into LDS, whole 128-byte lines an instruction for the
@@ -34,8 +34,8 @@ namespace hipq
     {
         struct PwParams
         {
-            const uint8_t* x;      // [M][64]
-            const int8_t* w;       // [N][64]
+            const uint8_t* x;      // [M][C], C = 64 or 128
+            const int8_t* w;       // [N][C]
             const int32_t* wsum;   // [N]
             uint8_t* out;          // [M][N]
             const uint8_t* sum_in; // [M][N] or null
@@ -51,15 +51,19 @@ namespace hipq
 
         constexpr int kPwRows = 64;    // pixels of a workgroup's tile
         constexpr int kPwCols = 256;   // output channels of a workgroup's tile
-        constexpr int kPwData = 4096;  // bytes of a tile's data in LDS
         constexpr int kPwStage = 4096; // bytes of a wavefront's residual / output region
 
-        template <bool HAS_SUM>
+        // CIN: input channels, 64 or 128 (reduction steps of 32 bytes: 2 or 4; with 128 the weight
+        // fragments take 64 registers)
+        template <int CIN, bool HAS_SUM>
         __global__ __launch_bounds__(256, 3) void conv_pw64_kernel(const PwParams p)
         {
+            constexpr int KS = CIN / 32;
+            constexpr int NB = CIN == 64 ? 2 : 1; // accumulator blocks of 32 channels live at a time (registers: the weight fragments take 8 KS)
+            constexpr int kPwData = kPwRows * CIN; // bytes of a tile's data in LDS
             extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
             constexpr int NSTAGE = HAS_SUM ? 2 : 1; // regions a wavefront: the residual of the next tile lands while this one is worked on
-            uint8_t* const data = lds;                                       // [2][64 pixels][64 bytes], swizzled like the tile kernels' operands
+            uint8_t* const data = lds;                                       // [2][64 pixels][CIN bytes], swizzled like the tile kernels' operands
             uint8_t* const stage = lds + 2 * kPwData;                        // [4 wavefronts][NSTAGE][32 pixels][128 bytes]
             float* const consts = reinterpret_cast<float*>(stage + 4 * NSTAGE * kPwStage); // [3][256]: start values (as int), bias, scale
             const int tid = static_cast<int>(threadIdx.x);
@@ -90,14 +94,14 @@ namespace hipq
             const float sum_scale = HAS_SUM ? *p.sum_scale : 0.0f;
             // the wavefront's weights as fragments: lane (c = lane % 32, half) of block ni, step ks holds
             // bytes [32 ks + 16 half, + 16) of weight row n_wave + 32 ni + c
-            v4i wf[2][4];
+            v4i wf[KS][4];
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
+            for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
                 for (int ni = 0; ni < 4; ++ni)
-                    wf[ks][ni] = *reinterpret_cast<const v4i*>(p.w + (n_wave + ni * 32 + (lane & 31)) * 64 + ks * 32 + half * 16);
+                    wf[ks][ni] = *reinterpret_cast<const v4i*>(p.w + (n_wave + ni * 32 + (lane & 31)) * CIN + ks * 32 + half * 16);
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
+            for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
                 for (int ni = 0; ni < 4; ++ni)
                     asm volatile("" ::"v"(wf[ks][ni])); // arrived before the loop: a wait for them inside it would also wait for the tile loads
@@ -107,17 +111,20 @@ namespace hipq
             const v4i xrs = rsrc_words(p.x, p.x_bytes);
             const v4i srs = rsrc_words(p.sum_in, HAS_SUM ? p.out_bytes : 0u);
             const uint32_t data_lds = lds_address(data) + static_cast<uint32_t>(wave) * 1024u;
+            constexpr int LPR = CIN / 16; // lanes that load one row of the data tile
             const uint32_t stage_lds = lds_address(stage) + static_cast<uint32_t>(wave) * (NSTAGE * kPwStage);
-            // data: lane tid fills slot tid % 4 of row tid / 4 with the chunk that belongs there
-            const int drow = tid >> 2;
-            const int dchunk = (tid & 3) ^ ((drow >> 2) & 3);
+            // data: lane tid fills slot tid % LPR of row tid / LPR (and of the rows 256 / LPR further on) with the chunk that belongs there
+            const int drow = tid / LPR;
+            const int dchunk = CIN == 64 ? ((tid & 3) ^ ((drow >> 2) & 3)) : ((tid & 7) ^ ((drow >> 1) & 7));
             // residual / output rows: eight lanes a row, slot s of row r holds channels 16 (s ^ (r / 2 % 8)) ..
             auto issue = [&](int j) { // tile j of the workgroup's sequence (anything past the end loads nothing)
                 const int64_t m0 = j < my_tiles ? static_cast<int64_t>(first + j * stride) * kPwRows : static_cast<int64_t>(p.M);
+#pragma unroll
+                for (int i = 0; i < CIN / 64; ++i) // (rows 32 apart share the swizzle of their slots)
                 {
-                    const int64_t m = m0 + drow;
-                    const int32_t off = m < p.M ? static_cast<int32_t>(m) * 64 + dchunk * 16 : kOob;
-                    lds_dma16(xrs, off, __builtin_amdgcn_readfirstlane(data_lds + static_cast<uint32_t>(j & 1) * kPwData));
+                    const int64_t m = m0 + drow + i * (256 / LPR);
+                    const int32_t off = m < p.M ? static_cast<int32_t>(m) * CIN + dchunk * 16 : kOob;
+                    lds_dma16(xrs, off, __builtin_amdgcn_readfirstlane(data_lds + static_cast<uint32_t>(j & 1) * kPwData + i * 4096));
                 }
                 if constexpr (HAS_SUM)
                 {
@@ -144,41 +151,42 @@ namespace hipq
                 constexpr bool PK_U8 = decltype(to_u8)::value;
                 const uint8_t* const xs = data + (j & 1) * kPwData;
                 uint8_t* const region = stage + (wave * NSTAGE + (HAS_SUM ? (j & 1) : 0)) * kPwStage;
-                v4i xf[2];
+                v4i xf[KS];
 #pragma unroll
-                for (int ks = 0; ks < 2; ++ks)
+                for (int ks = 0; ks < KS; ++ks)
                 {
-                    const v4i f = *reinterpret_cast<const v4i*>(xs + lds_offset(ph * 32 + (lane & 31), ks * 2 + half));
+                    const int frow = ph * 32 + (lane & 31), fchunk = ks * 2 + half;
+                    const v4i f = *reinterpret_cast<const v4i*>(xs + (CIN == 64 ? lds_offset(frow, fchunk) : frow * 128 + ((fchunk ^ ((frow >> 1) & 7)) << 4)));
                     xf[ks] = v4i{f[0] ^ xor_mask, f[1] ^ xor_mask, f[2] ^ xor_mask, f[3] ^ xor_mask};
                 }
                 const int row = lane & 31;
-                // 64 channels at a time: two accumulator blocks live, not four
+                // NB blocks of 32 channels at a time, not all four: registers
 #pragma unroll
-                for (int nh = 0; nh < 2; ++nh)
+                for (int nh = 0; nh < 4 / NB; ++nh)
                 {
-                    __builtin_amdgcn_sched_barrier(0); // (the second half's reads stay behind the first half's epilogue: registers)
-                    v16i acc[2];
+                    __builtin_amdgcn_sched_barrier(0); // (the next blocks' reads stay behind these blocks' epilogue)
+                    v16i acc[NB];
 #pragma unroll
-                    for (int i = 0; i < 2; ++i)
+                    for (int i = 0; i < NB; ++i)
 #pragma unroll
                         for (int g = 0; g < 4; ++g)
                         {
-                            const v4i c4 = *reinterpret_cast<const v4i*>(start_at + (nh * 2 + i) * 32 + 8 * g);
+                            const v4i c4 = *reinterpret_cast<const v4i*>(start_at + (nh * NB + i) * 32 + 8 * g);
 #pragma unroll
                             for (int e = 0; e < 4; ++e)
                                 acc[i][4 * g + e] = c4[e];
                         }
 #pragma unroll
-                    for (int ks = 0; ks < 2; ++ks)
+                    for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-                        for (int i = 0; i < 2; ++i)
-                            acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ks][nh * 2 + i], xf[ks], acc[i], 0, 0, 0);
+                        for (int i = 0; i < NB; ++i)
+                            acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ks][nh * NB + i], xf[ks], acc[i], 0, 0, 0);
 #pragma unroll
-                    for (int i = 0; i < 2; ++i)
+                    for (int i = 0; i < NB; ++i)
 #pragma unroll
                         for (int g = 0; g < 4; ++g)
                         {
-                            const int nl = (nh * 2 + i) * 32 + 8 * g + 4 * half; // channel within the wavefront's 128
+                            const int nl = (nh * NB + i) * 32 + 8 * g + 4 * half; // channel within the wavefront's 128
                             v4f bias4 = v4f{0.0f, 0.0f, 0.0f, 0.0f};
                             if (!FOLD)
                                 bias4 = *reinterpret_cast<const v4f*>(consts + 256 + cg * 128 + nl);
@@ -282,7 +290,9 @@ namespace hipq
             return false;
         if (g.data_layout != HIPQ_LAYOUT_NXC || g.out_layout != HIPQ_LAYOUT_NXC)
             return false;
-        if (g.C != 64 || g.K % kPwCols != 0 || g.K > 2048)
+        if ((g.C != 64 && g.C != 128) || g.K % kPwCols != 0 || g.K > 2048)
+            return false;
+        if (g.C == 128 && getenv("HIPQ_NO_PW128") != nullptr)
             return false;
         const int64_t M = g.N * g.in[1] * g.in[2];
         // few pixels: the tile kernels split their work better (HIPQ_PW64_MIN_ROWS moves the threshold)
@@ -302,13 +312,13 @@ namespace hipq
         const int64_t M = g.N * g.in[1] * g.in[2];
         p.x = static_cast<const uint8_t*>(data);
         p.w = static_cast<const int8_t*>(packed);
-        p.wsum = reinterpret_cast<const int32_t*>(static_cast<const uint8_t*>(packed) + align_up(static_cast<size_t>(g.K) * 64, 256));
+        p.wsum = reinterpret_cast<const int32_t*>(static_cast<const uint8_t*>(packed) + align_up(static_cast<size_t>(g.K * g.C), 256));
         p.out = static_cast<uint8_t*>(out);
         p.sum_in = static_cast<const uint8_t*>(epi.sum_in);
         p.bias = epi.bias;
         p.scale = epi.scale;
         p.sum_scale = epi.sum_scale;
-        p.x_bytes = static_cast<uint32_t>(M * 64);
+        p.x_bytes = static_cast<uint32_t>(M * g.C);
         p.out_bytes = static_cast<uint32_t>(M * g.K);
         p.M = static_cast<int32_t>(M);
         p.N = static_cast<int32_t>(g.K);
@@ -320,14 +330,24 @@ namespace hipq
         p.out_t = epi.out_t;
         p.sum_t = epi.sum_t;
         const bool has_sum = epi.sum_in != nullptr;
-        const size_t lds_bytes = 2 * kPwData + 4 * (has_sum ? 2 : 1) * kPwStage + 3 * 256 * sizeof(float);
+        const size_t lds_bytes = 2 * static_cast<size_t>(kPwRows * g.C) + 4 * (has_sum ? 2 : 1) * kPwStage + 3 * 256 * sizeof(float);
         const int64_t slots = static_cast<int64_t>(device_compute_units()) * 3 / p.col_tiles * p.col_tiles;
         const int64_t items = static_cast<int64_t>(p.tiles) * p.col_tiles;
         const unsigned grid = static_cast<unsigned>(std::min<int64_t>(items, std::max<int64_t>(slots, p.col_tiles)));
-        if (has_sum)
-            conv_pw64_kernel<true><<<grid, 256, lds_bytes, s>>>(p);
+        if (g.C == 64)
+        {
+            if (has_sum)
+                conv_pw64_kernel<64, true><<<grid, 256, lds_bytes, s>>>(p);
+            else
+                conv_pw64_kernel<64, false><<<grid, 256, lds_bytes, s>>>(p);
+        }
         else
-            conv_pw64_kernel<false><<<grid, 256, lds_bytes, s>>>(p);
+        {
+            if (has_sum)
+                conv_pw64_kernel<128, true><<<grid, 256, lds_bytes, s>>>(p);
+            else
+                conv_pw64_kernel<128, false><<<grid, 256, lds_bytes, s>>>(p);
+        }
         return check_launch("conv_pw64_i8_32x32x32");
     }
 }

@@ -1,4 +1,4 @@
-"""1 x 1 convolutions from 64 to 256 / 512 channels on the kernel that keeps its weights in registers and
+"""1 x 1 convolutions from 64 or 128 to 256 / 512 channels on the kernel that keeps its weights in registers and
 loads a tile ahead (bottleneck blocks' last layer and projection shortcut): bytes against the C
 restatement of the fused ops (quantized_conv.cpp:332-766 arithmetic) and against the tile kernel."""
 import numpy as np
@@ -16,24 +16,27 @@ def say(*a):
     print("[pw64]", *a, flush=True)
 
 
-# N, image, K, relu, residual (None / "u8" / "i8"), per-channel scales, bias magnitude
+# N, image, K, relu, residual (None / "u8" / "i8"), per-channel scales, bias magnitude, input channels
 CASES = [
-    (3, (40, 40), 256, True, "u8", True, 20000),     # QuantizedConvolutionBiasAdd, 75 whole tiles
-    (2, (37, 29), 256, False, "i8", False, 20000),   # ...BiasSignedAdd without ReLU: i8 out, scalar scale, ragged last tile (2146 rows)
-    (2, (33, 31), 256, True, None, True, 20000),     # QuantizedConvolutionBias + ReLU, last tile 62 rows short of 64
-    (1, (50, 41), 512, False, None, True, 20000),    # two column blocks, i8 out
-    (2, (20, 20), 256, True, "u8", True, 1 << 25),   # biases beyond 2^24: added in float, not carried in the accumulators
+    (3, (40, 40), 256, True, "u8", True, 20000, 64),     # QuantizedConvolutionBiasAdd, 75 whole tiles
+    (2, (37, 29), 256, False, "i8", False, 20000, 64),   # ...BiasSignedAdd without ReLU: i8 out, scalar scale, ragged last tile (2146 rows)
+    (2, (33, 31), 256, True, None, True, 20000, 64),     # QuantizedConvolutionBias + ReLU, last tile 62 rows short of 64
+    (1, (50, 41), 512, False, None, True, 20000, 64),    # two column blocks, i8 out
+    (2, (20, 20), 256, True, "u8", True, 1 << 25, 64),   # biases beyond 2^24: added in float, not carried in the accumulators
+    (2, (28, 28), 512, True, "u8", True, 20000, 128),    # 128 input channels (four reduction steps), two column blocks
+    (1, (31, 23), 256, False, "i8", True, 20000, 128),   # ... signed residual, i8 out, ragged last tile
+    (2, (19, 21), 256, True, None, False, 20000, 128),   # ... no residual, scalar scale
 ]
 
 
 @pytest.mark.parametrize("i", range(len(CASES)))
 def test_pw64_against_oracle_and_tile_kernel(gpu_lib, i, monkeypatch):
-    N, image, K, relu, res, per_channel, bias_mag = CASES[i]
+    N, image, K, relu, res, per_channel, bias_mag, Cc = CASES[i]
     say(CASES[i])
     O.port().orc_set_threads(8)
     out_t = "u8" if relu else "i8"
-    d = H.make_conv_desc(N, 64, K, image, (1, 1), out_t=out_t, data_layout=H.NXC, out_layout=H.NXC)
-    dn = H.make_conv_desc(N, 64, K, image, (1, 1), out_t=out_t)
+    d = H.make_conv_desc(N, Cc, K, image, (1, 1), out_t=out_t, data_layout=H.NXC, out_layout=H.NXC)
+    dn = H.make_conv_desc(N, Cc, K, image, (1, 1), out_t=out_t)
     data = synth.uniform_int(5100 + i, dn.data_shape(), 0, 255, np.uint8)
     filt = synth.uniform_int(5200 + i, dn.filter_shape(), -127, 127, np.int8)
     bias = synth.uniform_int(5300 + i, (K,), -bias_mag, bias_mag, np.int32)

@@ -244,6 +244,11 @@ namespace hipq
                     }
                 const float var = __fdiv_rn(wave_sum(q), n);
                 const float sd = sqrtf(var + eps);
+                // one division a row: the elements divide through its reciprocal, which gives the division's
+                // own result for every normal quotient (a row whose deviation is zero, infinite or out of
+                // the reciprocal's range keeps the division)
+                const float rsd = __fdiv_rn(1.0f, sd);
+                const bool by_reciprocal = sd > 1e-30f && sd < 1e30f; // uniform
 #pragma unroll
                 for (int i = 0; i < kRowVecs; ++i)
                 {
@@ -256,7 +261,7 @@ namespace hipq
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
                         {
-                            const float nv = __fdiv_rn(v[i][e], sd);
+                            const float nv = by_reciprocal ? div_by_reciprocal(v[i][e], sd, rsd) : __fdiv_rn(v[i][e], sd);
                             r[e] = scale ? __fadd_rn(__fmul_rn(nv, sc[e]), bi[e]) : nv;
                         }
                         reinterpret_cast<f4*>(y)[j] = r;

@@ -51,13 +51,29 @@ namespace hipq
         s = wave_sum<W>(s);
         return row_f4{v[0] / s, v[1] / s, v[2] / s, v[3] / s};
     }
+    // a / b rounded as the division rounds it, from r = fl(1 / b): q0 = a r, e = a - b q0 (exact in a fused
+    // multiply-add), q = q0 + e r -- three instructions where the division sequence takes eleven.
+    // (Markstein's correction: with a correctly rounded reciprocal the result is the correctly rounded
+    // quotient as long as nothing overflows or goes subnormal; checked on the CPU against the division
+    // for all 2^23 mantissas of a with b = float(sqrt(2)), and for 2 x 10^8 random pairs.)  Callers keep
+    // infinities and zero divisors away from it.
+    __device__ __forceinline__ float div_by_reciprocal(float a, float b, float r)
+    {
+        const float q0 = __fmul_rn(a, r);
+        return fmaf(fmaf(-b, q0, a), r, q0);
+    }
+
     // Gelu as the reference decomposes it (src/ngraph/op/gelu.cpp:46-60):
     // (0.5 * x) * (1 + erf(x / float(sqrt(2.0)))), every step rounded to f32.  Shared by the Gelu
     // kernel and by the GEMM epilogue that applies Gelu to what it has just computed.
     __device__ __forceinline__ float gelu1(float x)
     {
         const float sqrt_two = 1.41421354f; // float(std::sqrt(2.0))
-        return __fmul_rn(__fmul_rn(0.5f, x), __fadd_rn(1.0f, erff(__fdiv_rn(x, sqrt_two))));
+        const float r = 0.70710677f;        // fl(1 / sqrt_two)
+        // x / sqrt_two, bit for bit; an infinite x stays itself, and where the quotient would be
+        // subnormal erf's argument is so small that 1 + erf is 1 either way
+        const float t = __builtin_isinf(x) ? x : div_by_reciprocal(x, sqrt_two, r);
+        return __fmul_rn(__fmul_rn(0.5f, x), __fadd_rn(1.0f, erff(t)));
     }
 
 }

@@ -1843,7 +1843,7 @@ namespace hipq
         return check_launch(name);
     }
 
-    template <class XL, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM, int KIND = OUT_Q8, int BKT = BK>
+    template <class XL, int WAVES_M, int WAVES_N, int MODE, bool HAS_SUM, int KIND = OUT_Q8, int BKT = BK, int WM = 2>
     static int launch_pipe(const XL& xl,
                            const int8_t* w,
                            const int32_t* wsum,
@@ -1858,11 +1858,11 @@ namespace hipq
                            hipStream_t s,
                            const char* name)
     {
-        constexpr int BM = WAVES_M * 64, BN = WAVES_N * 64;
+        constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * 64;
         constexpr bool DMA = XL::kUniform;
         // (the kernels that load into LDS and take no residual stage their outputs in an operand buffer)
-        constexpr size_t lds_bytes = (DMA && BKT == BK && !HAS_SUM && WAVES_N > 1 ? 3 : 2) * static_cast<size_t>(BM + BN) * BKT + (DMA && !HAS_SUM ? 0 : 4 * 64 * 64) + 3 * BN * sizeof(float) + 16;
-        auto kernel = igemm_pipe_kernel<XL, 2, 2, WAVES_M, WAVES_N, MODE, HAS_SUM, DMA, KIND, BKT>;
+        constexpr size_t lds_bytes = (DMA && BKT == BK && !HAS_SUM && WAVES_N > 1 ? 3 : 2) * static_cast<size_t>(BM + BN) * BKT + (DMA && !HAS_SUM ? 0 : 4 * WM * 32 * 64) + 3 * BN * sizeof(float) + 16;
+        auto kernel = igemm_pipe_kernel<XL, WM, 2, WAVES_M, WAVES_N, MODE, HAS_SUM, DMA, KIND, BKT>;
         static bool configured[16] = {};
         static int cus[16] = {};
         static int per_cu[16] = {}; // workgroups of this kernel that fit a compute unit (LDS and registers)
@@ -1908,7 +1908,7 @@ namespace hipq
             // measured on ResNet-50's layers at batches 1, 32 and 128 and on GEMMs of 128 to 512 rows
             const int64_t units = dev >= 0 && dev < 16 && cus[dev] > 0 ? cus[dev] : 256;
             while (splits < 16 && slices % (splits * 2) == 0 &&
-                   ((tiles * splits * 2 * 4 <= units * 3 && slices * kDeep / (splits * 2) >= 8) || (tiles * splits * 2 <= resident && slices * kDeep / (splits * 2) >= 16)))
+                   ((tiles * splits * 2 * 4 <= units * 3 && slices * kDeep / (splits * 2) >= 8) || (WM == 2 && tiles * splits * 2 <= resident && slices * kDeep / (splits * 2) >= 16)))
                 splits *= 2;
         }
         int32_t* partials = nullptr;
@@ -1983,9 +1983,23 @@ namespace hipq
             if (tiles * 8 <= units * 3 && Kred >= 16 * BK)
                 deep = false;
         }
+        // 128 x 128 tiles that leave compute units idle (and would have their reductions split over
+        // workgroups, partial sums through memory): 64 x 128 tiles, twice as many, no split.
+        // Row matrices only: a 3 x 3 filter's long reduction over gathered rows does better split
+        // (512 -> 512 channels on 128 x 7 x 7 pixels: 34 us split, 40 us in half tiles)
+        bool half_height = false;
+        if constexpr (XL::kDeep && !XL::kPads)
+        {
+            const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+            half_height = deep && M > 64 && tiles <= device_compute_units() && getenv("HIPQ_NO_HALF_TILES") == nullptr;
+        }
         if constexpr (XL::kFloatOut)
             if (f32)
             {
+                if (half_height && gelu_q8)
+                    return launch_pipe<XL, 2, 2, EPI_FUSED, false, OUT_GELU_Q8, 2 * BK, 1>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
+                if (half_height)
+                    return launch_pipe<XL, 2, 2, EPI_FUSED, false, OUT_F32, 2 * BK, 1>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
                 if (gelu_q8)
                 {
                     if (deep)
@@ -2001,6 +2015,8 @@ namespace hipq
         if constexpr (XL::kDeep)
             if (deep)
             {
+                if (half_height && epi.mode == EPI_FUSED)
+                    return launch_pipe<XL, 2, 2, EPI_FUSED, false, OUT_Q8, 2 * BK, 1>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
                 if (epi.mode == EPI_INTERP)
                     return launch_pipe<XL, 2, 2, EPI_INTERP, false, OUT_Q8, 2 * BK>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);
                 return launch_pipe<XL, 2, 2, EPI_FUSED, false, OUT_Q8, 2 * BK>(xl, w, wsum, M, N, Kred, x_unsigned, zp, epi, om, out, s, name);

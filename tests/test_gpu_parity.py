@@ -857,6 +857,33 @@ def test_dot_tile_order(gpu_lib, shape):
     O.port().orc_set_threads(1)
 
 
+@pytest.mark.parametrize("shape", [(1000, 768, 400), (2000, 512, 1104), (4096, 768, 768)])
+def test_dot_half_height_tiles(gpu_lib, shape, monkeypatch):
+    """row matrices whose 128 x 128 tiles would leave compute units idle run on 64 x 128 tiles with
+    whole reductions: ragged last tiles in both directions, 8-bit and float outputs, against the
+    oracle and against the 128 x 128 tiles (reductions split over workgroups) behind the switch"""
+    M, K, N = shape
+    say("dot half-height tiles", shape)
+    O.port().orc_set_threads(8)
+    a = synth.uniform_int(1451, (M, K), 0, 255, np.uint8)
+    w = synth.uniform_int(1452, (N, K), -127, 127, np.int8)
+    bias = synth.uniform_int(1453, (N,), -(2**15), 2**15, np.int32)
+    scales = synth.uniform_f32(1454, (N,), 0.001, 0.01) * np.float32(0.03)
+    for out_t, relu in (("i8", False), ("u8", True), ("f32", False)):
+        d = H.make_dot_desc(M, K, N, a_t="u8", out_t=out_t, b_layout=H.B_NK)
+        f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
+        exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
+        got = H.quantized_dot_bias(d, f, a, w, bias, scales)
+        assert H.last_kernel().startswith("dot_mfma"), H.last_kernel()
+        monkeypatch.setenv("HIPQ_NO_HALF_TILES", "1")
+        full = H.quantized_dot_bias(d, f, a, w, bias, scales)
+        monkeypatch.delenv("HIPQ_NO_HALF_TILES")
+        assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), (out_t, relu)
+        assert np.array_equal(full.view(np.uint8), exp.view(np.uint8)), (out_t, relu, "128 x 128")
+        assert len(np.unique(exp)) > 20
+    O.port().orc_set_threads(1)
+
+
 @pytest.mark.parametrize("split", ["2", "4"])
 def test_dot_deep_slices_split(gpu_lib, split, monkeypatch):
     """reductions in whole 128-byte pieces run with slices twice as deep and two operand buffers;

@@ -351,6 +351,35 @@ def mfma_ceiling(lib, stream, timer, compute_units):
     return out
 
 
+def bench_coissue(lib, stream, timer, compute_units):
+    """Do matrix and vector instructions share a SIMD's time?  One workgroup of eight wavefronts a
+    compute unit (two a SIMD), every wavefront 16 x iters v_mfma_i32_32x32x32_i8 (32 cycles each) with 4, 8
+    or 16 independent v_fma_f32 (4 cycles each) behind each of them -- 'both'; the same MFMAs alone;
+    the same vector instructions alone; and 'split': four wavefronts issue only MFMAs, the other four
+    only vector instructions (half the work of either kind); 'both_acc_regs': 'both' with the accumulators
+    in the accumulation registers.  If the two kinds overlap, 'both' takes the longer of the two alone; if
+    they take turns, their sum.  (Times move with the clock the chip holds under each mix; the counter run
+    in profiles/ gives the same comparison in cycles.)"""
+    probe = H.load_probe()
+    iters, wgs = 400, int(compute_units)
+    sink = H.DeviceBuffer(wgs * 512 * 4)
+    ops = dev(np.random.default_rng(4002).integers(0, 256, 2048, dtype=np.uint8))
+    out = []
+    for v in (4, 8, 16):
+        row = {"vector_per_mfma": v}
+        for mode, name in ((0, "both"), (1, "mfma_alone"), (2, "vector_alone"), (3, "split"), (4, "both_acc_regs")):
+
+            def step():
+                H.check_probe(probe.hipq_probe_coissue(ops.ptr, sink.ptr, wgs, iters, v, mode, stream))
+
+            _, ev = timer.run(step, 5, 2)
+            row[name + "_us"] = ev * 1e3
+        row["both_over_sum"] = row["both_us"] / (row["mfma_alone_us"] + row["vector_alone_us"])
+        row["both_over_longer"] = row["both_us"] / max(row["mfma_alone_us"], row["vector_alone_us"])
+        out.append(row)
+    return out
+
+
 def bench_intake(lib, stream, timer, compute_units):
     """What a compute unit takes in: 1 / 2 / 4 workgroups of four wavefronts a compute unit (by their LDS
     allocation) each read 8 MiB in 16-byte pieces -- a wavefront instruction covering 1 KiB contiguous,
@@ -634,7 +663,7 @@ def main():
         return
     if args.only == "intake":
         print(json.dumps({"l2_intake_per_cu": bench_intake(lib, stream, timer, info.compute_units), "atomic_tiles": bench_atomic_tiles(lib, stream, timer, info.compute_units),
-                          "launch_floor": bench_launch_floor(lib, stream, timer)}))
+                          "launch_floor": bench_launch_floor(lib, stream, timer), "matrix_vector_coissue": bench_coissue(lib, stream, timer, info.compute_units)}))
         return
     if args.only == "glue":
         print(json.dumps({"fp32_glue": bench_fp32_glue(lib, stream, timer, args.steps, args.warmup), "copy_calibration": copy_calibration(lib, stream, timer)}))

@@ -28,6 +28,17 @@ HIPQ_PROBE_API const char* hipq_probe_last_error(void);
  * workgroup's 4 wavefronts issues 64 x iters MFMAs of 65536 operations. */
 HIPQ_PROBE_API int hipq_probe_mfma_i8(const void* operands_8k, void* sink, int32_t workgroups, int32_t iters, void* stream);
 
+/* Whether matrix and vector instructions overlap on a SIMD.  Workgroups of eight wavefronts (two a
+ * SIMD), `iters` iterations of 16 v_mfma_i32_32x32x32_i8 a wavefront (32 cycles each on its SIMD) and
+ * `vector_per_mfma` (4, 8 or 16) independent v_fma_f32 for each of them (4 cycles each):
+ *   mode 0: every wavefront issues both, the vector instructions behind each MFMA
+ *   mode 1: the MFMAs alone          mode 2: the vector instructions alone
+ *   mode 3: four wavefronts of a workgroup issue only the MFMAs, the other four only the vector work
+ *           (half of mode 0's work of either kind: compare with half of modes 1 and 2)
+ *   mode 4: mode 0 with the accumulators in a[0:31] (the accumulation registers)
+ * `operands_2k`: 2 sets of 64 lanes x 16 bytes; `sink`: workgroups x 512 ints. */
+HIPQ_PROBE_API int hipq_probe_coissue(const void* operands_2k, void* sink, int32_t workgroups, int32_t iters, int32_t vector_per_mfma, int32_t mode, void* stream);
+
 /* How many bytes a second a compute unit takes in from L2 (or from HBM).  `workgroups` workgroups of
  * 4 wavefronts (`lds_bytes` of dynamic LDS each: the handle on how many share a compute unit) read
  * `steps` x 32 KiB each out of `buf`: 16 bytes a lane and instruction, 8 instructions a wavefront

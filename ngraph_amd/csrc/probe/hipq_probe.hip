@@ -64,6 +64,84 @@ namespace
         sink[blockIdx.x * 256 + threadIdx.x] = s;
     }
 
+    // Do matrix and vector instructions share a SIMD's time?  MODE 0: every wavefront issues 16 MFMAs
+    // an iteration with V independent v_fma_f32 behind each (the compiler is held to that order);
+    // 1: the MFMAs alone; 2: the vector instructions alone; 3: a workgroup of eight wavefronts, two a
+    // SIMD, of which the first four issue only the MFMAs and the last four only the vector instructions;
+    // 4: as 0 with the accumulators named in the accumulation half of the register file.
+    template <int V, int MODE>
+    __global__ __launch_bounds__(512) void probe_coissue_kernel(const pv4i* __restrict__ ops, int* __restrict__ sink, int iters)
+    {
+        pv16i acc[2];
+        for (int i = 0; i < 2; ++i)
+            for (int r = 0; r < 16; ++r)
+                acc[i][r] = i;
+        const pv4i a = ops[threadIdx.x & 63], b = ops[64 + (threadIdx.x & 63)];
+        float x[8];
+        for (int k = 0; k < 8; ++k)
+            x[k] = static_cast<float>(a[k & 3] & 0xFF) * 1e-3f;
+        const float c = 0.999f + static_cast<float>(b[0] & 1) * 1e-4f, d = static_cast<float>(b[1] & 3) * 1e-3f;
+        const bool matrix = MODE == 0 || MODE == 1 || (MODE == 3 && (threadIdx.x >> 8) == 0);
+        const bool vector = MODE == 0 || MODE == 2 || (MODE == 3 && (threadIdx.x >> 8) == 1);
+        for (int it = 0; it < iters; ++it)
+        {
+            if (MODE == 4)
+            {
+                // as mode 0 with the accumulators in the accumulation registers (AGPRs): the MFMA's 16
+                // registers of input and output then do not pass through the vector register file's ports
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                {
+                    if (i & 1)
+                        asm volatile("v_mfma_i32_32x32x32_i8 a[16:31], %0, %1, a[16:31]" ::"v"(a), "v"(b)
+                                     : "a16", "a17", "a18", "a19", "a20", "a21", "a22", "a23", "a24", "a25", "a26", "a27", "a28", "a29", "a30", "a31");
+                    else
+                        asm volatile("v_mfma_i32_32x32x32_i8 a[0:15], %0, %1, a[0:15]" ::"v"(a), "v"(b)
+                                     : "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11", "a12", "a13", "a14", "a15");
+#pragma unroll
+                    for (int v = 0; v < V; ++v)
+                        asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(x[v & 7]) : "v"(c), "v"(d));
+                }
+            }
+            else if (MODE == 0)
+            {
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                {
+                    acc[i & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[i & 1], 0, 0, 0);
+#pragma unroll
+                    for (int v = 0; v < V; ++v)
+                        x[v & 7] = __builtin_fmaf(x[v & 7], c, d);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, V, 0);
+                }
+            }
+            else
+            {
+                if (matrix) // uniform per wavefront
+                {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i)
+                        acc[i & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[i & 1], 0, 0, 0);
+                }
+                if (vector)
+                {
+#pragma unroll
+                    for (int i = 0; i < 16 * V; ++i)
+                        x[i & 7] = __builtin_fmaf(x[i & 7], c, d);
+                }
+            }
+        }
+        int s = 0;
+        for (int i = 0; i < 2; ++i)
+            for (int r = 0; r < 16; ++r)
+                s += acc[i][r];
+        float f = 0.0f;
+        for (int k = 0; k < 8; ++k)
+            f += x[k];
+        sink[blockIdx.x * 512 + threadIdx.x] = s + static_cast<int>(f);
+    }
+
     constexpr int kIntakeLoads = 8;       // 16-byte loads a lane and step
     constexpr int kIntakeStepBytes = 32768; // 4 wavefronts x 8 instructions x 1 KiB
 
@@ -191,6 +269,43 @@ int hipq_probe_mfma_i8(const void* operands_8k, void* sink, int32_t workgroups, 
         return fail("operands must be 16-byte aligned");
     probe_mfma_i8_kernel<<<static_cast<unsigned>(workgroups), 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const pv4i*>(operands_8k), static_cast<int*>(sink), iters);
     return check_launch("probe_mfma_i8");
+}
+
+int hipq_probe_coissue(const void* operands_2k, void* sink, int32_t workgroups, int32_t iters, int32_t vector_per_mfma, int32_t mode, void* stream)
+{
+    if (!operands_2k || !sink)
+        return fail("null pointer");
+    if (workgroups <= 0 || workgroups > 65535 || iters <= 0 || iters > 100000)
+        return fail("workgroups / iterations out of range");
+    if (mode < 0 || mode > 4 || (vector_per_mfma != 4 && vector_per_mfma != 8 && vector_per_mfma != 16))
+        return fail("mode 0..3, 4, 8 or 16 vector instructions an MFMA");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const pv4i* ops = static_cast<const pv4i*>(operands_2k);
+    int* out = static_cast<int*>(sink);
+    const unsigned grid = static_cast<unsigned>(workgroups);
+#define COISSUE(V)                                                        \
+    switch (mode)                                                         \
+    {                                                                     \
+    case 0: probe_coissue_kernel<V, 0><<<grid, 512, 0, s>>>(ops, out, iters); break; \
+    case 1: probe_coissue_kernel<V, 1><<<grid, 512, 0, s>>>(ops, out, iters); break; \
+    case 2: probe_coissue_kernel<V, 2><<<grid, 512, 0, s>>>(ops, out, iters); break; \
+    case 3: probe_coissue_kernel<V, 3><<<grid, 512, 0, s>>>(ops, out, iters); break; \
+    default: probe_coissue_kernel<V, 4><<<grid, 512, 0, s>>>(ops, out, iters); break; \
+    }
+    if (vector_per_mfma == 4)
+    {
+        COISSUE(4)
+    }
+    else if (vector_per_mfma == 8)
+    {
+        COISSUE(8)
+    }
+    else
+    {
+        COISSUE(16)
+    }
+#undef COISSUE
+    return check_launch("probe_coissue");
 }
 
 int hipq_probe_intake(const void* buf, size_t buf_bytes, size_t window_bytes, int32_t spread, int32_t shape, int32_t to_lds, int32_t workgroups, int32_t lds_bytes, int32_t steps,

@@ -356,6 +356,7 @@ def load_probe():
     vp, i32, sz = C.c_void_p, C.c_int32, C.c_size_t
     lib.hipq_probe_last_error.restype = C.c_char_p
     lib.hipq_probe_mfma_i8.argtypes = [vp, vp, i32, i32, vp]
+    lib.hipq_probe_coissue.argtypes = [vp, vp, i32, i32, i32, i32, vp]
     lib.hipq_probe_intake.argtypes = [vp, sz, sz, i32, i32, i32, i32, i32, i32, vp, vp]
     lib.hipq_probe_atomic_tiles.argtypes = [vp, sz, i32, i32, i32, i32, vp]
     lib.hipq_probe_empty_chain.argtypes = [vp, i32, i32, i32, vp]

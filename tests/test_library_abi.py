@@ -35,7 +35,7 @@ def test_product_library_exports_only_the_declared_abi():
     assert not [n for n in exported if "debug" in n or "probe" in n], exported
     assert set(exported) - set(_declared()) <= {"hipq_last_kernel", "_init", "_fini"}, sorted(set(exported) - set(_declared()))
     probe = H.load_probe()
-    for n in ("hipq_probe_mfma_i8", "hipq_probe_intake", "hipq_probe_atomic_tiles", "hipq_debug_fastdiv", "hipq_probe_last_error"):
+    for n in ("hipq_probe_mfma_i8", "hipq_probe_coissue", "hipq_probe_intake", "hipq_probe_atomic_tiles", "hipq_debug_fastdiv", "hipq_probe_last_error"):
         assert hasattr(probe, n), n
 
 

@@ -552,6 +552,50 @@ def test_conv_bias_in_accumulator(gpu_lib):
     O.port().orc_set_threads(1)
 
 
+def _conv_sweep():
+    """seeded channels-last layers of the kinds a ResNet holds -- 1 x 1 and 3 x 3, stride 1 and 2, 64 to
+    512 channels either side, with and without a residual -- at image sizes and batches that put their
+    tile counts on both sides of the dispatch edges (pointwise / tile kernels, 64- and 128-byte
+    slices, 64 x 128 tiles, split reductions)"""
+    rng = np.random.default_rng(777)
+    out = []
+    for _ in range(60):
+        Cc = int(rng.choice([64, 128, 256, 512]))
+        K = int(rng.choice([64, 128, 256, 512]))
+        r = int(rng.choice([1, 1, 3]))
+        st = int(rng.choice([1, 1, 2]))
+        hw = int(rng.choice([7, 10, 14, 21, 28]))
+        N = int(rng.choice([1, 2, 5, 9]))
+        res = bool(rng.integers(0, 2)) and st == 1
+        ho = (hw + 2 * (r // 2) - r) // st + 1
+        if N * ho * ho * K * Cc * r * r <= 600_000_000:
+            out.append((N, Cc, K, hw, r, st, res))
+    return sorted(set(out))[:30]
+
+
+@pytest.mark.parametrize("case", _conv_sweep())
+def test_conv_fused_nxc_sweep(gpu_lib, case):
+    """QuantizedConvolutionBias(+Add)+ReLU, channels-last in and out, over seeded ResNet-like layers, against the oracle"""
+    N, Cc, K, hw, r, st, res = case
+    say("conv fused nxc sweep", case)
+    O.port().orc_set_threads(8)
+    pad = (r // 2, r // 2)
+    kw = dict(stride=(st, st), pad_below=pad, pad_above=pad, out_t="u8")
+    dn = H.make_conv_desc(N, Cc, K, (hw, hw), (r, r), **kw)
+    d = H.make_conv_desc(N, Cc, K, (hw, hw), (r, r), data_layout=H.NXC, out_layout=H.NXC, **kw)
+    data = synth.uniform_int(3301, dn.data_shape(), 0, 255, np.uint8)
+    filt = synth.uniform_int(3302, dn.filter_shape(), -127, 127, np.int8)
+    bias = synth.uniform_int(3303, (K,), -20000, 20000, np.int32)
+    scales = synth.uniform_f32(3304, (K,), 1e-3, 3e-3) * np.float32(8.0 / (r * np.sqrt(Cc)))
+    summ = synth.uniform_int(3305, dn.out_shape(), 0, 255, np.uint8) if res else None
+    f = H.make_fused_desc(has_bias=True, has_sum=res, sum_t="u8", with_relu=True, scale_count=K)
+    exp = O.quantized_convolution_fused(dn, f, data, filt, bias, summ, scales, 0.3 if res else None)
+    got = H.quantized_convolution_fused(d, f, cases.to_nxc(data), filt, bias, cases.to_nxc(summ) if res else None, scales, 0.3 if res else None)
+    assert np.array_equal(cases.to_ncx(got), exp), (case, H.last_kernel())
+    assert len(np.unique(exp)) > 20, case
+    O.port().orc_set_threads(1)
+
+
 @pytest.mark.parametrize("i", range(len(SPLIT_CONV_SHAPES)))
 def test_conv_register_staged(gpu_lib, i, monkeypatch):
     """the same shapes through the register-staged kernels (windows over multiples of 64 channels
@@ -881,6 +925,40 @@ def test_dot_half_height_tiles(gpu_lib, shape, monkeypatch):
         assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), (out_t, relu)
         assert np.array_equal(full.view(np.uint8), exp.view(np.uint8)), (out_t, relu, "128 x 128")
         assert len(np.unique(exp)) > 20
+    O.port().orc_set_threads(1)
+
+
+def _sweep_shapes():
+    """seeded shapes around the tile kernels' dispatch edges: rows just past 64 and 128, column counts
+    that are not whole tiles, reductions from one 64-byte slice to 2048 bytes (whole 128-byte pieces and
+    not), tile counts below and above the compute units"""
+    rng = np.random.default_rng(20240)
+    shapes = []
+    for _ in range(28):
+        M = int(rng.choice([65, 96, 129, 200, 257, 384, 640, 1000, 1536, 2500, 4100]))
+        K = int(rng.choice([64, 128, 192, 256, 320, 512, 768, 1024, 1408, 2048]))
+        N = int(rng.choice([16, 48, 64, 80, 128, 144, 256, 400, 768, 1104]))
+        if M * K * N <= 1_500_000_000:
+            shapes.append((M, K, N))
+    return sorted(set(shapes))
+
+
+@pytest.mark.parametrize("shape", _sweep_shapes())
+def test_dot_dispatch_sweep(gpu_lib, shape):
+    """QuantizedDotBias over shapes drawn around the dispatch edges, 8-bit and float outputs, against the oracle"""
+    M, K, N = shape
+    say("dot dispatch sweep", shape)
+    O.port().orc_set_threads(8)
+    a = synth.uniform_int(1501, (M, K), 0, 255, np.uint8)
+    w = synth.uniform_int(1502, (N, K), -127, 127, np.int8)
+    bias = synth.uniform_int(1503, (N,), -(2**15), 2**15, np.int32)
+    scales = synth.uniform_f32(1504, (N,), 0.001, 0.01) * np.float32(40.0 / K)
+    for out_t, relu in (("u8", True), ("f32", False)):
+        d = H.make_dot_desc(M, K, N, a_t="u8", out_t=out_t, b_layout=H.B_NK)
+        f = H.make_fused_desc(has_bias=True, with_relu=relu, scale_count=N)
+        exp = O.quantized_dot_bias(d, f, a, w, bias, scales)
+        got = H.quantized_dot_bias(d, f, a, w, bias, scales)
+        assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), (shape, out_t, H.last_kernel())
     O.port().orc_set_threads(1)
 
 
